@@ -1,0 +1,130 @@
+// Host side of the C ABI: error text, device sanity, argument checks of
+// cw_gemm_ksteps. The other entry points live beside their kernels.
+#include <cstdarg>
+#include <cstdio>
+#include <cstring>
+
+#include "cw_common.h"
+#include "gemm.h"
+
+namespace cw {
+
+namespace {
+thread_local char g_error[512] = "";
+thread_local char g_arch[128] = "";
+}  // namespace
+
+int fail(int code, const char* fmt, ...) {
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(g_error, sizeof(g_error), fmt, ap);
+    va_end(ap);
+    return code;
+}
+
+int check_launch(const char* what) {
+    const hipError_t e = hipGetLastError();
+    if (e == hipSuccess) return CW_OK;
+    return fail(CW_ERR_LAUNCH, "%s: launch failed: %s", what, hipGetErrorString(e));
+}
+
+}  // namespace cw
+
+using namespace cw;
+
+extern "C" const char* cw_version(void) { return "cubework-hip 0.1.0 (gfx950)"; }
+
+extern "C" const char* cw_last_error(void) { return g_error; }
+
+extern "C" const char* cw_device_arch(void) {
+    g_arch[0] = '\0';
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess) {
+        (void)hipGetLastError();
+        return g_arch;
+    }
+    hipDeviceProp_t prop;
+    if (hipGetDeviceProperties(&prop, dev) != hipSuccess) {
+        (void)hipGetLastError();
+        return g_arch;
+    }
+    strncpy(g_arch, prop.gcnArchName, sizeof(g_arch) - 1);
+    g_arch[sizeof(g_arch) - 1] = '\0';
+    return g_arch;
+}
+
+extern "C" int cw_gemm_ksteps(int layout, int64_t M, int64_t N, int64_t K, int n_steps, const void* const* A_steps,
+                              int64_t lda, const void* const* B_steps, int64_t ldb, const void* bias, int epilogue,
+                              void* C, int64_t ldc, void* preact, int64_t ldp, const void* const* addends,
+                              int n_addends, int64_t ldadd, int io_dtype, void* stream) {
+    if (layout != CW_NN && layout != CW_NT && layout != CW_TN)
+        return fail(CW_ERR_INVALID, "cw_gemm_ksteps: bad layout %d", layout);
+    if (epilogue < CW_EPI_NONE || epilogue > CW_EPI_BIAS_RELU)
+        return fail(CW_ERR_INVALID, "cw_gemm_ksteps: bad epilogue %d", epilogue);
+    if (io_dtype != CW_BF16 && io_dtype != CW_F32)
+        return fail(CW_ERR_INVALID, "cw_gemm_ksteps: bad io_dtype %d", io_dtype);
+    if (M < 0 || N < 0 || K < 0 || M > INT32_MAX || N > INT32_MAX || K > INT32_MAX)
+        return fail(CW_ERR_INVALID, "cw_gemm_ksteps: bad shape M=%lld N=%lld K=%lld", (long long)M, (long long)N,
+                    (long long)K);
+    if (n_steps < 0 || n_steps > CW_MAX_KSTEPS)
+        return fail(CW_ERR_INVALID, "cw_gemm_ksteps: n_steps=%d outside [0, %d]", n_steps, CW_MAX_KSTEPS);
+    if (n_addends < 0 || n_addends > CW_MAX_ADDENDS)
+        return fail(CW_ERR_INVALID, "cw_gemm_ksteps: n_addends=%d outside [0, %d]", n_addends, CW_MAX_ADDENDS);
+    if (M == 0 || N == 0) return CW_OK;
+    if (C == nullptr || ldc < N) return fail(CW_ERR_INVALID, "cw_gemm_ksteps: C is NULL or ldc < N");
+    if (preact != nullptr && ldp < N) return fail(CW_ERR_INVALID, "cw_gemm_ksteps: ldp < N");
+    if (K == 0) n_steps = 0;
+    if (n_steps > 0) {
+        if (A_steps == nullptr || B_steps == nullptr)
+            return fail(CW_ERR_INVALID, "cw_gemm_ksteps: operand pointer tables are NULL");
+        const int64_t a_cols = (layout == CW_TN) ? M : K;  // contiguous extent of A's rows
+        const int64_t b_cols = (layout == CW_NT) ? K : N;
+        if (lda < a_cols || ldb < b_cols)
+            return fail(CW_ERR_INVALID, "cw_gemm_ksteps: leading dimension smaller than the row (lda=%lld ldb=%lld)",
+                        (long long)lda, (long long)ldb);
+    }
+    if (n_addends > 0 && (addends == nullptr || ldadd < N))
+        return fail(CW_ERR_INVALID, "cw_gemm_ksteps: addends table is NULL or ldadd < N");
+
+    GemmArgs args;
+    memset(&args, 0, sizeof(args));
+    const int vec = (io_dtype == CW_BF16) ? 8 : 4;       // elements per 16 bytes
+    const uintptr_t out_mask = (io_dtype == CW_BF16) ? 7u : 15u;  // bf16 outputs move 8 bytes at a time
+    const int out_vec = 4;
+    args.vec_a = args.vec_b = 1;
+    for (int i = 0; i < n_steps; ++i) {
+        if (A_steps[i] == nullptr || B_steps[i] == nullptr)
+            return fail(CW_ERR_INVALID, "cw_gemm_ksteps: operand pointer of step %d is NULL", i);
+        args.A[i] = A_steps[i];
+        args.B[i] = B_steps[i];
+        if (!aligned16(A_steps[i])) args.vec_a = 0;
+        if (!aligned16(B_steps[i])) args.vec_b = 0;
+    }
+    if (lda % vec != 0) args.vec_a = 0;
+    if (ldb % vec != 0) args.vec_b = 0;
+    args.vec_add = 1;
+    for (int j = 0; j < n_addends; ++j) {
+        if (addends[j] == nullptr) return fail(CW_ERR_INVALID, "cw_gemm_ksteps: addend %d is NULL", j);
+        args.addend[j] = addends[j];
+        if ((reinterpret_cast<uintptr_t>(addends[j]) & out_mask) != 0) args.vec_add = 0;
+    }
+    if (ldadd % out_vec != 0) args.vec_add = 0;
+    args.bias = bias;
+    args.vec_bias = (bias == nullptr || (reinterpret_cast<uintptr_t>(bias) & out_mask) == 0) ? 1 : 0;
+    args.C = C;
+    args.vec_c = ((reinterpret_cast<uintptr_t>(C) & out_mask) == 0 && ldc % out_vec == 0) ? 1 : 0;
+    args.preact = preact;
+    args.vec_p = (preact == nullptr || ((reinterpret_cast<uintptr_t>(preact) & out_mask) == 0 && ldp % out_vec == 0)) ? 1 : 0;
+    args.lda = lda;
+    args.ldb = ldb;
+    args.ldc = ldc;
+    args.ldp = ldp;
+    args.ldadd = ldadd;
+    args.M = (int)M;
+    args.N = (int)N;
+    args.K = (int)K;
+    args.n_steps = n_steps;
+    args.n_addends = n_addends;
+    hipStream_t s = (hipStream_t)stream;
+    return io_dtype == CW_BF16 ? gemm_bf16_launch(args, layout, epilogue, s) : gemm_f32_launch(args, layout, epilogue, s);
+}

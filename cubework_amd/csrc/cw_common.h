@@ -1,0 +1,143 @@
+// Shared device/host helpers for the gfx950 kernels of libcubework_hip.so.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "../../include/cubework_hip.h"
+
+namespace cw {
+
+// ---- host side: thread-local error text --------------------------------
+int fail(int code, const char* fmt, ...);
+int check_launch(const char* what);
+
+inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+
+// ---- element types -------------------------------------------------------
+struct bf16_t {
+    uint16_t bits;
+};
+
+template <typename T>
+struct elem;
+
+template <>
+struct elem<bf16_t> {
+    static constexpr int kVec = 8;  // elements per 16-byte vector
+};
+template <>
+struct elem<float> {
+    static constexpr int kVec = 4;
+};
+
+__device__ __forceinline__ float bf16_bits_to_f32(uint32_t h) { return __uint_as_float(h << 16); }
+
+// Round-to-nearest-even, the rounding torch uses for float -> bfloat16
+// (lowers to v_cvt_pk_bf16_f32 on gfx950).
+__device__ __forceinline__ uint32_t f32_to_bf16_bits(float f) {
+    __bf16 b = static_cast<__bf16>(f);
+    return static_cast<uint32_t>(__builtin_bit_cast(uint16_t, b));
+}
+
+__device__ __forceinline__ uint32_t pack_bf16x2(float lo, float hi) {
+    return f32_to_bf16_bits(lo) | (f32_to_bf16_bits(hi) << 16);
+}
+
+__device__ __forceinline__ float load_elem(const bf16_t* p) { return bf16_bits_to_f32(p->bits); }
+__device__ __forceinline__ float load_elem(const float* p) { return *p; }
+__device__ __forceinline__ void store_elem(bf16_t* p, float v) { p->bits = static_cast<uint16_t>(f32_to_bf16_bits(v)); }
+__device__ __forceinline__ void store_elem(float* p, float v) { *p = v; }
+
+// 16-byte vector load of kVec consecutive elements into floats. p must be
+// 16-byte aligned.
+__device__ __forceinline__ void load_vec(const bf16_t* p, float (&v)[8]) {
+    const uint4 u = *reinterpret_cast<const uint4*>(p);
+    v[0] = __uint_as_float(u.x << 16);
+    v[1] = __uint_as_float(u.x & 0xffff0000u);
+    v[2] = __uint_as_float(u.y << 16);
+    v[3] = __uint_as_float(u.y & 0xffff0000u);
+    v[4] = __uint_as_float(u.z << 16);
+    v[5] = __uint_as_float(u.z & 0xffff0000u);
+    v[6] = __uint_as_float(u.w << 16);
+    v[7] = __uint_as_float(u.w & 0xffff0000u);
+}
+__device__ __forceinline__ void load_vec(const float* p, float (&v)[4]) {
+    const float4 u = *reinterpret_cast<const float4*>(p);
+    v[0] = u.x;
+    v[1] = u.y;
+    v[2] = u.z;
+    v[3] = u.w;
+}
+__device__ __forceinline__ void store_vec(bf16_t* p, const float (&v)[8]) {
+    uint4 u;
+    u.x = pack_bf16x2(v[0], v[1]);
+    u.y = pack_bf16x2(v[2], v[3]);
+    u.z = pack_bf16x2(v[4], v[5]);
+    u.w = pack_bf16x2(v[6], v[7]);
+    *reinterpret_cast<uint4*>(p) = u;
+}
+__device__ __forceinline__ void store_vec(float* p, const float (&v)[4]) {
+    *reinterpret_cast<float4*>(p) = make_float4(v[0], v[1], v[2], v[3]);
+}
+
+// ---- wavefront (64 lanes) reductions ------------------------------------
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off, 64);
+    return v;
+}
+__device__ __forceinline__ float wave_max(float v) {
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) v = fmaxf(v, __shfl_xor(v, off, 64));
+    return v;
+}
+
+constexpr float kLog2e = 1.4426950408889634f;
+constexpr float kLn2 = 0.6931471805599453f;
+
+// exp(x) through the hardware exp2; x <= 0 in every use here.
+__device__ __forceinline__ float fast_exp(float x) { return __builtin_amdgcn_exp2f(x * kLog2e); }
+
+// ---- activations ---------------------------------------------------------
+__device__ __forceinline__ float tanh_fast(float x) {
+    // tanh(x) = 1 - 2 / (exp(2x) + 1); saturates cleanly for |x| large.
+    const float e = __builtin_amdgcn_exp2f(x * (2.0f * kLog2e));
+    return 1.0f - 2.0f * __builtin_amdgcn_rcpf(e + 1.0f);
+}
+__device__ __forceinline__ float gelu_tanh(float x) {
+    const float k0 = 0.7978845608028654f, k1 = 0.044715f;
+    const float u = k0 * (x + k1 * x * x * x);
+    return 0.5f * x * (1.0f + tanh_fast(u));
+}
+__device__ __forceinline__ float gelu_tanh_grad(float x) {
+    const float k0 = 0.7978845608028654f, k1 = 0.044715f;
+    const float u = k0 * (x + k1 * x * x * x);
+    const float t = tanh_fast(u);
+    const float du = k0 * (1.0f + 3.0f * k1 * x * x);
+    return 0.5f * (1.0f + t) + 0.5f * x * (1.0f - t * t) * du;
+}
+__device__ __forceinline__ float gelu_erf(float x) { return 0.5f * x * (1.0f + erff(x * 0.7071067811865476f)); }
+__device__ __forceinline__ float gelu_erf_grad(float x) {
+    const float cdf = 0.5f * (1.0f + erff(x * 0.7071067811865476f));
+    const float pdf = 0.3989422804014327f * __expf(-0.5f * x * x);
+    return cdf + x * pdf;
+}
+
+template <int ACT>
+__device__ __forceinline__ float apply_act(float x) {
+    if constexpr (ACT == CW_ACT_GELU_TANH) return gelu_tanh(x);
+    if constexpr (ACT == CW_ACT_GELU_ERF) return gelu_erf(x);
+    if constexpr (ACT == CW_ACT_RELU) return x > 0.0f ? x : 0.0f;
+    return x;
+}
+__device__ __forceinline__ float act_grad(int act, float x) {
+    switch (act) {
+        case CW_ACT_GELU_TANH: return gelu_tanh_grad(x);
+        case CW_ACT_GELU_ERF: return gelu_erf_grad(x);
+        case CW_ACT_RELU: return x > 0.0f ? 1.0f : 0.0f;
+        default: return 1.0f;
+    }
+}
+
+}  // namespace cw

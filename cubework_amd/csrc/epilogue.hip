@@ -1,0 +1,200 @@
+// Bias-gradient column sums and the backward of the fused activation
+// epilogue, for gfx950. Streaming kernels: a block owns a slab of rows and a
+// tile of 64 vectors of columns, lanes keep their columns' sums in registers,
+// wavefronts are combined in a fixed-order LDS tree, slabs by a finalize
+// kernel (no atomics: bit-reproducible).
+#include "cw_common.h"
+#include "reduce_cols.h"
+
+namespace cw {
+
+namespace {
+
+constexpr int kColWaves = 16;  // 1024 threads per block on the vector path
+constexpr int64_t kGenericSlabRows = 64;
+
+template <typename T, int MODE>
+__global__ __launch_bounds__(kColWaves * 64) void colsum_vec_kernel(
+    int64_t M, int64_t N, const T* __restrict__ dY, int64_t ld_dy, const T* __restrict__ pre, int64_t ld_pre,
+    T* __restrict__ dPre, int64_t ld_dpre, int act, float* __restrict__ ws, int64_t rows_per_slab, int want_sum) {
+    constexpr int V = elem<T>::kVec;
+    extern __shared__ float lds_red[];
+    const int lane = threadIdx.x & 63;
+    const int wave = threadIdx.x >> 6;
+    const int64_t c0 = ((int64_t)blockIdx.x * 64 + lane) * V;
+    const bool valid = c0 < N;
+    const int64_t r0 = (int64_t)blockIdx.y * rows_per_slab;
+    const int64_t r1 = (r0 + rows_per_slab < M) ? r0 + rows_per_slab : M;
+    float acc[V];
+#pragma unroll
+    for (int e = 0; e < V; ++e) acc[e] = 0.0f;
+    if (valid) {
+        for (int64_t row = r0 + wave; row < r1; row += kColWaves) {
+            float dy[V];
+            load_vec(dY + row * ld_dy + c0, dy);
+            if constexpr (MODE == 1) {
+                float p[V];
+                load_vec(pre + row * ld_pre + c0, p);
+#pragma unroll
+                for (int e = 0; e < V; ++e) dy[e] *= act_grad(act, p[e]);
+                store_vec(dPre + row * ld_dpre + c0, dy);
+            }
+#pragma unroll
+            for (int e = 0; e < V; ++e) acc[e] += dy[e];
+        }
+    }
+    if (!want_sum) return;
+    block_tree_reduce<V, kColWaves>(acc, lds_red, wave, lane);
+    if (wave == 0 && valid) {
+        float* out = ws + (int64_t)blockIdx.y * N + c0;
+#pragma unroll
+        for (int e = 0; e < V; e += 4)
+            *reinterpret_cast<float4*>(out + e) = make_float4(acc[e], acc[e + 1], acc[e + 2], acc[e + 3]);
+    }
+}
+
+template <typename T, int MODE>
+__global__ __launch_bounds__(256) void colsum_generic_kernel(int64_t M, int64_t N, const T* __restrict__ dY,
+                                                             int64_t ld_dy, const T* __restrict__ pre,
+                                                             int64_t ld_pre, T* __restrict__ dPre, int64_t ld_dpre,
+                                                             int act, float* __restrict__ ws,
+                                                             int64_t rows_per_slab, int want_sum) {
+    const int64_t c = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (c >= N) return;
+    const int64_t r0 = (int64_t)blockIdx.y * rows_per_slab;
+    const int64_t r1 = (r0 + rows_per_slab < M) ? r0 + rows_per_slab : M;
+    float acc = 0.0f;
+    for (int64_t row = r0; row < r1; ++row) {
+        float d = load_elem(dY + row * ld_dy + c);
+        if constexpr (MODE == 1) {
+            d *= act_grad(act, load_elem(pre + row * ld_pre + c));
+            store_elem(dPre + row * ld_dpre + c, d);
+        }
+        acc += d;
+    }
+    if (want_sum) ws[(int64_t)blockIdx.y * N + c] = acc;
+}
+
+// grid (ceil(C/64), nsets); 4 groups of 64 threads split the partials.
+__global__ __launch_bounds__(256) void finalize_cols_kernel(const float* __restrict__ ws, int64_t nparts,
+                                                            int64_t part_stride, int64_t C, float* __restrict__ out0,
+                                                            float* __restrict__ out1) {
+    __shared__ float red[4][64];
+    const int lane = threadIdx.x & 63;
+    const int grp = threadIdx.x >> 6;
+    const int64_t c = (int64_t)blockIdx.x * 64 + lane;
+    const int k = blockIdx.y;
+    float acc = 0.0f;
+    if (c < C) {
+        const float* base = ws + (int64_t)k * C + c;
+        for (int64_t p = grp; p < nparts; p += 4) acc += base[p * part_stride];
+    }
+    red[grp][lane] = acc;
+    __syncthreads();
+    if (grp == 0 && c < C) {
+        const float total = ((red[0][lane] + red[1][lane]) + red[2][lane]) + red[3][lane];
+        float* out = (k == 0) ? out0 : out1;
+        if (out != nullptr) out[c] = total;
+    }
+}
+
+template <typename T, int MODE>
+int colsum_impl(int64_t M, int64_t N, const void* dY, int64_t ld_dy, const void* pre, int64_t ld_pre, void* dPre,
+                int64_t ld_dpre, int act, float* out, void* workspace, int64_t workspace_bytes, hipStream_t s) {
+    constexpr int V = elem<T>::kVec;
+    const int want_sum = out != nullptr ? 1 : 0;
+    bool vec = aligned16(dY) && (ld_dy % V) == 0 && (N % V) == 0;
+    if (MODE == 1) vec = vec && aligned16(pre) && (ld_pre % V) == 0 && aligned16(dPre) && (ld_dpre % V) == 0;
+    int64_t slabs, rows_per_slab;
+    if (vec) {
+        const int64_t coltiles = (N + 64 * V - 1) / (64 * V);
+        slabs = 512 / coltiles;
+        const int64_t max_slabs = (M + kColWaves - 1) / kColWaves;
+        if (slabs > max_slabs) slabs = max_slabs;
+        if (slabs < 1) slabs = 1;
+        rows_per_slab = (M + slabs - 1) / slabs;
+        slabs = (M + rows_per_slab - 1) / rows_per_slab;
+        if (want_sum && workspace_bytes < slabs * N * (int64_t)sizeof(float))
+            return fail(CW_ERR_INVALID, "column sum: workspace too small (%lld bytes)", (long long)workspace_bytes);
+        const size_t lds = tree_reduce_lds_bytes(V, kColWaves);
+        hipLaunchKernelGGL((colsum_vec_kernel<T, MODE>), dim3((unsigned)coltiles, (unsigned)slabs),
+                           dim3(kColWaves * 64), lds, s, M, N, (const T*)dY, ld_dy, (const T*)pre, ld_pre, (T*)dPre,
+                           ld_dpre, act, (float*)workspace, rows_per_slab, want_sum);
+    } else {
+        rows_per_slab = kGenericSlabRows;
+        slabs = (M + rows_per_slab - 1) / rows_per_slab;
+        if (want_sum && workspace_bytes < slabs * N * (int64_t)sizeof(float))
+            return fail(CW_ERR_INVALID, "column sum: workspace too small (%lld bytes)", (long long)workspace_bytes);
+        hipLaunchKernelGGL((colsum_generic_kernel<T, MODE>), dim3((unsigned)((N + 255) / 256), (unsigned)slabs),
+                           dim3(256), 0, s, M, N, (const T*)dY, ld_dy, (const T*)pre, ld_pre, (T*)dPre, ld_dpre, act,
+                           (float*)workspace, rows_per_slab, want_sum);
+    }
+    int rc = check_launch("colsum kernel");
+    if (rc != CW_OK || !want_sum) return rc;
+    return finalize_col_partials((const float*)workspace, slabs, N, 1, N, out, nullptr, s);
+}
+
+}  // namespace
+
+int finalize_col_partials(const float* ws, int64_t nparts, int64_t part_stride, int nsets, int64_t C, float* out0,
+                          float* out1, hipStream_t s) {
+    hipLaunchKernelGGL(finalize_cols_kernel, dim3((unsigned)((C + 63) / 64), (unsigned)nsets), dim3(256), 0, s, ws,
+                       nparts, part_stride, C, out0, out1);
+    return check_launch("finalize_cols_kernel");
+}
+
+int64_t colsum_workspace_bytes(int64_t M, int64_t N) {
+    int64_t parts = (M + kGenericSlabRows - 1) / kGenericSlabRows;
+    if (parts < 512) parts = 512;
+    return parts * N * (int64_t)sizeof(float);
+}
+
+}  // namespace cw
+
+using namespace cw;
+
+extern "C" int64_t cw_colsum_workspace_bytes(int64_t M, int64_t N) {
+    if (M < 0 || N < 0) return 0;
+    const int64_t a = colsum_workspace_bytes(M, N);
+    const int64_t b = ln_bwd_workspace_bytes(M, N);
+    return a > b ? a : b;
+}
+
+extern "C" int cw_colsum(int64_t M, int64_t N, const void* dY, int64_t ld, float* out, void* workspace,
+                         int64_t workspace_bytes, int io_dtype, void* stream) {
+    if (M < 0 || N <= 0) return fail(CW_ERR_INVALID, "cw_colsum: bad shape M=%lld N=%lld", (long long)M, (long long)N);
+    if (io_dtype != CW_BF16 && io_dtype != CW_F32) return fail(CW_ERR_INVALID, "cw_colsum: bad io_dtype %d", io_dtype);
+    if (out == nullptr) return fail(CW_ERR_INVALID, "cw_colsum: out is NULL");
+    hipStream_t s = (hipStream_t)stream;
+    if (M == 0) return finalize_col_partials(nullptr, 0, N, 1, N, out, nullptr, s);  // zero fill
+    if (dY == nullptr || workspace == nullptr || ld < N)
+        return fail(CW_ERR_INVALID, "cw_colsum: null pointer or ld < N");
+    return io_dtype == CW_BF16
+               ? colsum_impl<bf16_t, 0>(M, N, dY, ld, nullptr, 0, nullptr, 0, 0, out, workspace, workspace_bytes, s)
+               : colsum_impl<float, 0>(M, N, dY, ld, nullptr, 0, nullptr, 0, 0, out, workspace, workspace_bytes, s);
+}
+
+extern "C" int cw_act_bwd_colsum(int activation, int64_t M, int64_t N, const void* dY, int64_t ld_dy,
+                                 const void* preact, int64_t ld_pre, void* dPre, int64_t ld_dpre, float* dbias,
+                                 void* workspace, int64_t workspace_bytes, int io_dtype, void* stream) {
+    if (M < 0 || N <= 0)
+        return fail(CW_ERR_INVALID, "cw_act_bwd_colsum: bad shape M=%lld N=%lld", (long long)M, (long long)N);
+    if (io_dtype != CW_BF16 && io_dtype != CW_F32)
+        return fail(CW_ERR_INVALID, "cw_act_bwd_colsum: bad io_dtype %d", io_dtype);
+    if (activation != CW_ACT_NONE && activation != CW_ACT_GELU_TANH && activation != CW_ACT_GELU_ERF &&
+        activation != CW_ACT_RELU)
+        return fail(CW_ERR_INVALID, "cw_act_bwd_colsum: bad activation %d", activation);
+    hipStream_t s = (hipStream_t)stream;
+    if (M == 0) {
+        if (dbias == nullptr) return CW_OK;
+        return finalize_col_partials(nullptr, 0, N, 1, N, dbias, nullptr, s);  // zero fill
+    }
+    if (dY == nullptr || preact == nullptr || dPre == nullptr || ld_dy < N || ld_pre < N || ld_dpre < N)
+        return fail(CW_ERR_INVALID, "cw_act_bwd_colsum: null pointer or leading dimension < N");
+    if (dbias != nullptr && workspace == nullptr)
+        return fail(CW_ERR_INVALID, "cw_act_bwd_colsum: workspace is NULL");
+    return io_dtype == CW_BF16 ? colsum_impl<bf16_t, 1>(M, N, dY, ld_dy, preact, ld_pre, dPre, ld_dpre, activation, dbias,
+                                                        workspace, workspace_bytes, s)
+                               : colsum_impl<float, 1>(M, N, dY, ld_dy, preact, ld_pre, dPre, ld_dpre, activation, dbias,
+                                                       workspace, workspace_bytes, s);
+}

@@ -1,0 +1,26 @@
+// Kernel argument block shared by the bf16 and fp32 block-GEMM kernels.
+#pragma once
+
+#include "cw_common.h"
+
+namespace cw {
+
+struct GemmArgs {
+    const void* A[CW_MAX_KSTEPS];
+    const void* B[CW_MAX_KSTEPS];
+    const void* addend[CW_MAX_ADDENDS];
+    const void* bias;
+    void* C;
+    void* preact;
+    int64_t lda, ldb, ldc, ldp, ldadd;
+    int M, N, K;  // K: reduction length of one step
+    int n_steps, n_addends;
+    // 1 when the operand's base and leading dimension allow 16-byte (bf16: 8
+    // elements, fp32: 4 elements) row accesses; C/preact/addends/bias: 8-byte.
+    int vec_a, vec_b, vec_c, vec_p, vec_add, vec_bias;
+};
+
+int gemm_bf16_launch(const GemmArgs& args, int layout, int epilogue, hipStream_t s);
+int gemm_f32_launch(const GemmArgs& args, int layout, int epilogue, hipStream_t s);
+
+}  // namespace cw

@@ -1,0 +1,545 @@
+// LayerNorm2D / LayerNorm3D per-rank kernels for gfx950: partial statistics,
+// normalise (+ affine), backward partials (row sums + dgamma/dbeta column
+// partials) and dx. All are HBM-streaming kernels: one 64-lane wavefront owns
+// a row, every lane moves 16-byte vectors, row reductions are wavefront
+// shuffles, column reductions go through registers -> LDS tree -> a small
+// per-block partial in global memory (no atomics, so results are
+// deterministic).
+#include "cw_common.h"
+#include "reduce_cols.h"
+
+namespace cw {
+
+namespace {
+
+constexpr int kLnBlock = 256;  // 4 wavefronts; one row per wavefront per trip
+
+// Sum of (x-mu) and (x-mu)^2 over one row; every lane returns the full sums.
+template <typename T>
+__device__ __forceinline__ void row_moments(const T* __restrict__ xr, int64_t C, float mu, bool vec_ok,
+                                            int lane, float& s1, float& s2) {
+    constexpr int V = elem<T>::kVec;
+    float a1 = 0.0f, a2 = 0.0f;
+    if (vec_ok) {
+        const int64_t nvec = C / V;
+        for (int64_t i = lane; i < nvec; i += 64) {
+            float v[V];
+            load_vec(xr + i * V, v);
+#pragma unroll
+            for (int e = 0; e < V; ++e) {
+                const float d = v[e] - mu;
+                a1 += d;
+                a2 += d * d;
+            }
+        }
+        for (int64_t c = nvec * V + lane; c < C; c += 64) {
+            const float d = load_elem(xr + c) - mu;
+            a1 += d;
+            a2 += d * d;
+        }
+    } else {
+        for (int64_t c = lane; c < C; c += 64) {
+            const float d = load_elem(xr + c) - mu;
+            a1 += d;
+            a2 += d * d;
+        }
+    }
+    s1 = wave_sum(a1);
+    s2 = wave_sum(a2);
+}
+
+template <typename T>
+__global__ __launch_bounds__(kLnBlock) void ln_stats_kernel(int64_t R, int64_t C, const T* __restrict__ x,
+                                                            int64_t ld, int mode, const float* __restrict__ mean,
+                                                            float* __restrict__ stats, int vec_ok) {
+    const int lane = threadIdx.x & 63;
+    const int64_t wave = (int64_t)blockIdx.x * (kLnBlock / 64) + (threadIdx.x >> 6);
+    const int64_t nwaves = (int64_t)gridDim.x * (kLnBlock / 64);
+    for (int64_t row = wave; row < R; row += nwaves) {
+        const float mu = (mode == CW_LN_TWO_PASS && mean != nullptr) ? mean[row] : 0.0f;
+        float s1, s2;
+        row_moments(x + row * ld, C, mu, vec_ok != 0, lane, s1, s2);
+        if (lane == 0) {
+            stats[2 * row] = s1;
+            stats[2 * row + 1] = (mode == CW_LN_TWO_PASS && mean == nullptr) ? 0.0f : s2;
+        }
+    }
+}
+
+// mean / rstd from whole-hidden-size statistics.
+__device__ __forceinline__ void finish_stats(int mode, float s1, float s2, float inv_h, float eps, float& mean,
+                                             float& rstd) {
+    float var;
+    if (mode == CW_LN_ONE_PASS) {
+        mean = s1 * inv_h;
+        var = s2 * inv_h - mean * mean;
+    } else {
+        mean = s1;
+        var = s2 * inv_h;
+    }
+    rstd = 1.0f / sqrtf(var + eps);
+}
+
+template <typename T, bool FUSED>
+__global__ __launch_bounds__(kLnBlock) void ln_normalize_kernel(int64_t R, int64_t C, const T* __restrict__ x,
+                                                                int64_t ld, const float* __restrict__ stats,
+                                                                int mode, float inv_h, float eps,
+                                                                const T* __restrict__ gamma,
+                                                                const T* __restrict__ beta, T* __restrict__ y,
+                                                                int64_t ldy, float* __restrict__ mean_rstd,
+                                                                int vec_ok) {
+    constexpr int V = elem<T>::kVec;
+    const int lane = threadIdx.x & 63;
+    const int64_t wave = (int64_t)blockIdx.x * (kLnBlock / 64) + (threadIdx.x >> 6);
+    const int64_t nwaves = (int64_t)gridDim.x * (kLnBlock / 64);
+    for (int64_t row = wave; row < R; row += nwaves) {
+        const T* xr = x + row * ld;
+        T* yr = y + row * ldy;
+        float mean, rstd;
+        if constexpr (FUSED) {
+            float s1, s2;
+            row_moments(xr, C, 0.0f, vec_ok != 0, lane, s1, s2);
+            if (mode == CW_LN_TWO_PASS) {
+                const float mu = s1 * inv_h;
+                float d1, d2;
+                row_moments(xr, C, mu, vec_ok != 0, lane, d1, d2);
+                finish_stats(mode, mu, d2, inv_h, eps, mean, rstd);
+            } else {
+                finish_stats(mode, s1, s2, inv_h, eps, mean, rstd);
+            }
+        } else {
+            finish_stats(mode, stats[2 * row], stats[2 * row + 1], inv_h, eps, mean, rstd);
+        }
+        if (mean_rstd != nullptr && lane == 0) {
+            mean_rstd[2 * row] = mean;
+            mean_rstd[2 * row + 1] = rstd;
+        }
+        if (vec_ok) {
+            const int64_t nvec = C / V;
+            for (int64_t i = lane; i < nvec; i += 64) {
+                float v[V], g[V], b[V];
+                load_vec(xr + i * V, v);
+                if (gamma != nullptr) load_vec(gamma + i * V, g);
+                if (beta != nullptr) load_vec(beta + i * V, b);
+#pragma unroll
+                for (int e = 0; e < V; ++e) {
+                    float xh = (v[e] - mean) * rstd;
+                    if (gamma != nullptr) xh *= g[e];
+                    if (beta != nullptr) xh += b[e];
+                    v[e] = xh;
+                }
+                store_vec(yr + i * V, v);
+            }
+            for (int64_t c = nvec * V + lane; c < C; c += 64) {
+                float xh = (load_elem(xr + c) - mean) * rstd;
+                if (gamma != nullptr) xh *= load_elem(gamma + c);
+                if (beta != nullptr) xh += load_elem(beta + c);
+                store_elem(yr + c, xh);
+            }
+        } else {
+            for (int64_t c = lane; c < C; c += 64) {
+                float xh = (load_elem(xr + c) - mean) * rstd;
+                if (gamma != nullptr) xh *= load_elem(gamma + c);
+                if (beta != nullptr) xh += load_elem(beta + c);
+                store_elem(yr + c, xh);
+            }
+        }
+    }
+}
+
+// Backward partials, vector path. Lane `l` owns the columns of chunks
+// (j*64 + l)*V .. +V-1, j < NCH, for every row its wavefront visits, so the
+// dgamma/dbeta accumulators stay in registers for the whole kernel.
+template <typename T, int NCH, int NWAVES>
+__global__ __launch_bounds__(NWAVES * 64) void ln_bwd_partials_kernel(
+    int64_t R, int64_t C, const T* __restrict__ dY, int64_t ld_dy, const T* __restrict__ x, int64_t ld_x,
+    const float* __restrict__ mean_rstd, const T* __restrict__ gamma, float* __restrict__ row_sums,
+    float* __restrict__ col_ws, int want_cols) {
+    constexpr int V = elem<T>::kVec;
+    extern __shared__ float lds_red[];
+    const int lane = threadIdx.x & 63;
+    const int wave = threadIdx.x >> 6;
+
+    float gam[NCH][V];
+    float acc[2 * NCH * V];  // [0, NCH*V): dgamma, [NCH*V, 2*NCH*V): dbeta
+#pragma unroll
+    for (int j = 0; j < NCH; ++j) {
+        const int64_t c0 = ((int64_t)j * 64 + lane) * V;
+        if (gamma != nullptr && c0 < C) {
+            load_vec(gamma + c0, gam[j]);
+        } else {
+#pragma unroll
+            for (int e = 0; e < V; ++e) gam[j][e] = 1.0f;
+        }
+    }
+#pragma unroll
+    for (int i = 0; i < 2 * NCH * V; ++i) acc[i] = 0.0f;
+
+    for (int64_t row = (int64_t)blockIdx.x * NWAVES + wave; row < R; row += (int64_t)gridDim.x * NWAVES) {
+        const float mean = mean_rstd[2 * row];
+        const float rstd = mean_rstd[2 * row + 1];
+        const T* dyr = dY + row * ld_dy;
+        const T* xr = x + row * ld_x;
+        float s1 = 0.0f, s2 = 0.0f;
+#pragma unroll
+        for (int j = 0; j < NCH; ++j) {
+            const int64_t c0 = ((int64_t)j * 64 + lane) * V;
+            if (c0 < C) {
+                float dy[V], xv[V];
+                load_vec(dyr + c0, dy);
+                load_vec(xr + c0, xv);
+#pragma unroll
+                for (int e = 0; e < V; ++e) {
+                    const float xh = (xv[e] - mean) * rstd;
+                    const float g = dy[e] * gam[j][e];
+                    s1 += g;
+                    s2 += g * xh;
+                    acc[j * V + e] += dy[e] * xh;
+                    acc[NCH * V + j * V + e] += dy[e];
+                }
+            }
+        }
+        s1 = wave_sum(s1);
+        s2 = wave_sum(s2);
+        if (lane == 0) {
+            row_sums[2 * row] = s1;
+            row_sums[2 * row + 1] = s2;
+        }
+    }
+    if (!want_cols) return;
+
+    block_tree_reduce<2 * NCH * V, NWAVES>(acc, lds_red, wave, lane);
+    if (wave == 0) {
+        float* out = col_ws + (int64_t)blockIdx.x * 2 * C;
+#pragma unroll
+        for (int j = 0; j < NCH; ++j) {
+            const int64_t c0 = ((int64_t)j * 64 + lane) * V;
+            if (c0 < C) {
+#pragma unroll
+                for (int e = 0; e < V; e += 4) {
+                    *reinterpret_cast<float4*>(out + c0 + e) =
+                        make_float4(acc[j * V + e], acc[j * V + e + 1], acc[j * V + e + 2], acc[j * V + e + 3]);
+                    *reinterpret_cast<float4*>(out + C + c0 + e) =
+                        make_float4(acc[NCH * V + j * V + e], acc[NCH * V + j * V + e + 1],
+                                    acc[NCH * V + j * V + e + 2], acc[NCH * V + j * V + e + 3]);
+                }
+            }
+        }
+    }
+}
+
+// Backward partials for shapes the vector kernel does not take (ragged C,
+// unaligned rows, very wide rows). Row sums only; the column sums of this
+// path come from ln_bwd_cols_generic_kernel.
+template <typename T>
+__global__ __launch_bounds__(kLnBlock) void ln_bwd_rows_generic_kernel(
+    int64_t R, int64_t C, const T* __restrict__ dY, int64_t ld_dy, const T* __restrict__ x, int64_t ld_x,
+    const float* __restrict__ mean_rstd, const T* __restrict__ gamma, float* __restrict__ row_sums) {
+    const int lane = threadIdx.x & 63;
+    const int64_t wave = (int64_t)blockIdx.x * (kLnBlock / 64) + (threadIdx.x >> 6);
+    const int64_t nwaves = (int64_t)gridDim.x * (kLnBlock / 64);
+    for (int64_t row = wave; row < R; row += nwaves) {
+        const float mean = mean_rstd[2 * row];
+        const float rstd = mean_rstd[2 * row + 1];
+        float s1 = 0.0f, s2 = 0.0f;
+        for (int64_t c = lane; c < C; c += 64) {
+            const float xh = (load_elem(x + row * ld_x + c) - mean) * rstd;
+            const float g = load_elem(dY + row * ld_dy + c) * (gamma != nullptr ? load_elem(gamma + c) : 1.0f);
+            s1 += g;
+            s2 += g * xh;
+        }
+        s1 = wave_sum(s1);
+        s2 = wave_sum(s2);
+        if (lane == 0) {
+            row_sums[2 * row] = s1;
+            row_sums[2 * row + 1] = s2;
+        }
+    }
+}
+
+// Column partials of the generic path: thread = one column, block.y = a slab
+// of rows. ws[slab][2][C].
+template <typename T>
+__global__ __launch_bounds__(kLnBlock) void ln_bwd_cols_generic_kernel(
+    int64_t R, int64_t C, const T* __restrict__ dY, int64_t ld_dy, const T* __restrict__ x, int64_t ld_x,
+    const float* __restrict__ mean_rstd, float* __restrict__ col_ws, int64_t rows_per_slab) {
+    const int64_t c = (int64_t)blockIdx.x * kLnBlock + threadIdx.x;
+    if (c >= C) return;
+    const int64_t r0 = (int64_t)blockIdx.y * rows_per_slab;
+    const int64_t r1 = (r0 + rows_per_slab < R) ? r0 + rows_per_slab : R;
+    float dg = 0.0f, db = 0.0f;
+    for (int64_t row = r0; row < r1; ++row) {
+        const float xh = (load_elem(x + row * ld_x + c) - mean_rstd[2 * row]) * mean_rstd[2 * row + 1];
+        const float dy = load_elem(dY + row * ld_dy + c);
+        dg += dy * xh;
+        db += dy;
+    }
+    col_ws[(int64_t)blockIdx.y * 2 * C + c] = dg;
+    col_ws[(int64_t)blockIdx.y * 2 * C + C + c] = db;
+}
+
+template <typename T>
+__global__ __launch_bounds__(kLnBlock) void ln_bwd_dx_kernel(int64_t R, int64_t C, const T* __restrict__ dY,
+                                                             int64_t ld_dy, const T* __restrict__ x, int64_t ld_x,
+                                                             const float* __restrict__ mean_rstd,
+                                                             const T* __restrict__ gamma,
+                                                             const float* __restrict__ row_sums, float inv_h,
+                                                             T* __restrict__ dx, int64_t ld_dx, int vec_ok) {
+    constexpr int V = elem<T>::kVec;
+    const int lane = threadIdx.x & 63;
+    const int64_t wave = (int64_t)blockIdx.x * (kLnBlock / 64) + (threadIdx.x >> 6);
+    const int64_t nwaves = (int64_t)gridDim.x * (kLnBlock / 64);
+    for (int64_t row = wave; row < R; row += nwaves) {
+        const float mean = mean_rstd[2 * row];
+        const float rstd = mean_rstd[2 * row + 1];
+        const float c1 = row_sums[2 * row] * inv_h;
+        const float c2 = row_sums[2 * row + 1] * inv_h;
+        const T* dyr = dY + row * ld_dy;
+        const T* xr = x + row * ld_x;
+        T* dxr = dx + row * ld_dx;
+        if (vec_ok) {
+            const int64_t nvec = C / V;
+            for (int64_t i = lane; i < nvec; i += 64) {
+                float dy[V], xv[V], g[V];
+                load_vec(dyr + i * V, dy);
+                load_vec(xr + i * V, xv);
+                if (gamma != nullptr) load_vec(gamma + i * V, g);
+#pragma unroll
+                for (int e = 0; e < V; ++e) {
+                    const float xh = (xv[e] - mean) * rstd;
+                    const float gg = gamma != nullptr ? dy[e] * g[e] : dy[e];
+                    dy[e] = (gg - xh * c2 - c1) * rstd;
+                }
+                store_vec(dxr + i * V, dy);
+            }
+            for (int64_t c = nvec * V + lane; c < C; c += 64) {
+                const float xh = (load_elem(xr + c) - mean) * rstd;
+                const float gg = load_elem(dyr + c) * (gamma != nullptr ? load_elem(gamma + c) : 1.0f);
+                store_elem(dxr + c, (gg - xh * c2 - c1) * rstd);
+            }
+        } else {
+            for (int64_t c = lane; c < C; c += 64) {
+                const float xh = (load_elem(xr + c) - mean) * rstd;
+                const float gg = load_elem(dyr + c) * (gamma != nullptr ? load_elem(gamma + c) : 1.0f);
+                store_elem(dxr + c, (gg - xh * c2 - c1) * rstd);
+            }
+        }
+    }
+}
+
+int ln_grid(int64_t R) {
+    const int64_t blocks = (R + (kLnBlock / 64) - 1) / (kLnBlock / 64);
+    const int64_t cap = 256 * 8;  // 8 resident blocks of 4 wavefronts per CU
+    return (int)(blocks < cap ? (blocks > 0 ? blocks : 1) : cap);
+}
+
+template <typename T>
+bool rows_vec_ok(const void* p, int64_t ld) {
+    return aligned16(p) && (ld % elem<T>::kVec) == 0;
+}
+
+template <typename T>
+int stats_impl(int64_t R, int64_t C, const void* x, int64_t ld, int mode, const float* mean, float* stats,
+               hipStream_t s) {
+    const int vec_ok = rows_vec_ok<T>(x, ld);
+    hipLaunchKernelGGL(ln_stats_kernel<T>, dim3(ln_grid(R)), dim3(kLnBlock), 0, s, R, C, (const T*)x, ld, mode,
+                       mean, stats, vec_ok);
+    return check_launch("ln_stats_kernel");
+}
+
+template <typename T, bool FUSED>
+int normalize_impl(int64_t R, int64_t C, const void* x, int64_t ld, const float* stats, int mode, int64_t H,
+                   float eps, const void* gamma, const void* beta, void* y, int64_t ldy, float* mean_rstd,
+                   hipStream_t s) {
+    const int vec_ok = rows_vec_ok<T>(x, ld) && rows_vec_ok<T>(y, ldy) && (gamma == nullptr || aligned16(gamma)) &&
+                       (beta == nullptr || aligned16(beta));
+    hipLaunchKernelGGL((ln_normalize_kernel<T, FUSED>), dim3(ln_grid(R)), dim3(kLnBlock), 0, s, R, C, (const T*)x,
+                       ld, stats, mode, 1.0f / (float)H, eps, (const T*)gamma, (const T*)beta, (T*)y, ldy,
+                       mean_rstd, vec_ok);
+    return check_launch("ln_normalize_kernel");
+}
+
+// Number of blocks (= column partials) of the vector backward kernel.
+int64_t bwd_blocks(int64_t R, int nwaves) {
+    int64_t nb = (R + nwaves - 1) / nwaves;
+    if (nb > 256) nb = 256;
+    if (nb < 1) nb = 1;
+    return nb;
+}
+
+template <typename T, int NCH, int NWAVES>
+int bwd_partials_launch(int64_t R, int64_t C, const void* dY, int64_t ld_dy, const void* x, int64_t ld_x,
+                        const float* mean_rstd, const void* gamma, float* row_sums, float* ws, int want_cols,
+                        hipStream_t s) {
+    constexpr int V = elem<T>::kVec;
+    const int64_t nb = bwd_blocks(R, NWAVES);
+    const size_t lds = tree_reduce_lds_bytes(2 * NCH * V, NWAVES);
+    auto kern = ln_bwd_partials_kernel<T, NCH, NWAVES>;
+    if (lds > 48 * 1024) {
+        hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+        if (e != hipSuccess) return fail(CW_ERR_LAUNCH, "hipFuncSetAttribute(ln_bwd_partials): %s", hipGetErrorString(e));
+    }
+    hipLaunchKernelGGL(kern, dim3((unsigned)nb), dim3(NWAVES * 64), lds, s, R, C, (const T*)dY, ld_dy, (const T*)x,
+                       ld_x, mean_rstd, (const T*)gamma, row_sums, ws, want_cols);
+    return check_launch("ln_bwd_partials_kernel");
+}
+
+constexpr int64_t kGenericSlabRows = 64;
+
+template <typename T>
+int bwd_partials_impl(int64_t R, int64_t C, const void* dY, int64_t ld_dy, const void* x, int64_t ld_x,
+                      const float* mean_rstd, const void* gamma, float* row_sums, float* dgamma, float* dbeta,
+                      void* workspace, int64_t workspace_bytes, hipStream_t s) {
+    constexpr int V = elem<T>::kVec;
+    const int want_cols = (dgamma != nullptr || dbeta != nullptr) ? 1 : 0;
+    const bool vec = rows_vec_ok<T>(dY, ld_dy) && rows_vec_ok<T>(x, ld_x) && (gamma == nullptr || aligned16(gamma)) &&
+                     (C % V) == 0;
+    const int64_t nch = (C + 64 * V - 1) / (64 * V);
+    int64_t nparts = 0;
+    int rc;
+    if (vec && nch <= 8) {
+        int nwaves = nch <= 2 ? 16 : (nch <= 4 ? 8 : 4);
+        nparts = bwd_blocks(R, nwaves);
+        if (want_cols && workspace_bytes < nparts * 2 * C * (int64_t)sizeof(float))
+            return fail(CW_ERR_INVALID, "cw_ln_bwd_partials: workspace too small (%lld bytes)", (long long)workspace_bytes);
+        float* ws = (float*)workspace;
+        if (nch <= 1)
+            rc = bwd_partials_launch<T, 1, 16>(R, C, dY, ld_dy, x, ld_x, mean_rstd, gamma, row_sums, ws, want_cols, s);
+        else if (nch <= 2)
+            rc = bwd_partials_launch<T, 2, 16>(R, C, dY, ld_dy, x, ld_x, mean_rstd, gamma, row_sums, ws, want_cols, s);
+        else if (nch <= 4)
+            rc = bwd_partials_launch<T, 4, 8>(R, C, dY, ld_dy, x, ld_x, mean_rstd, gamma, row_sums, ws, want_cols, s);
+        else
+            rc = bwd_partials_launch<T, 8, 4>(R, C, dY, ld_dy, x, ld_x, mean_rstd, gamma, row_sums, ws, want_cols, s);
+        if (rc != CW_OK) return rc;
+    } else {
+        hipLaunchKernelGGL(ln_bwd_rows_generic_kernel<T>, dim3(ln_grid(R)), dim3(kLnBlock), 0, s, R, C,
+                           (const T*)dY, ld_dy, (const T*)x, ld_x, mean_rstd, (const T*)gamma, row_sums);
+        rc = check_launch("ln_bwd_rows_generic_kernel");
+        if (rc != CW_OK) return rc;
+        if (want_cols) {
+            nparts = (R + kGenericSlabRows - 1) / kGenericSlabRows;
+            if (workspace_bytes < nparts * 2 * C * (int64_t)sizeof(float))
+                return fail(CW_ERR_INVALID, "cw_ln_bwd_partials: workspace too small (%lld bytes)", (long long)workspace_bytes);
+            dim3 grid((unsigned)((C + kLnBlock - 1) / kLnBlock), (unsigned)nparts);
+            hipLaunchKernelGGL(ln_bwd_cols_generic_kernel<T>, grid, dim3(kLnBlock), 0, s, R, C, (const T*)dY, ld_dy,
+                               (const T*)x, ld_x, mean_rstd, (float*)workspace, kGenericSlabRows);
+            rc = check_launch("ln_bwd_cols_generic_kernel");
+            if (rc != CW_OK) return rc;
+        }
+    }
+    if (want_cols) {
+        // ws is [nparts][2][C]: dgamma partials are rows 2p, dbeta partials rows 2p+1.
+        rc = finalize_col_partials((const float*)workspace, nparts, 2 * C, 2, C, dgamma, dbeta, s);
+    }
+    return rc;
+}
+
+template <typename T>
+int bwd_dx_impl(int64_t R, int64_t C, const void* dY, int64_t ld_dy, const void* x, int64_t ld_x,
+                const float* mean_rstd, const void* gamma, const float* row_sums, int64_t H, void* dx, int64_t ld_dx,
+                hipStream_t s) {
+    const int vec_ok = rows_vec_ok<T>(dY, ld_dy) && rows_vec_ok<T>(x, ld_x) && rows_vec_ok<T>(dx, ld_dx) &&
+                       (gamma == nullptr || aligned16(gamma));
+    hipLaunchKernelGGL(ln_bwd_dx_kernel<T>, dim3(ln_grid(R)), dim3(kLnBlock), 0, s, R, C, (const T*)dY, ld_dy,
+                       (const T*)x, ld_x, mean_rstd, (const T*)gamma, row_sums, 1.0f / (float)H, (T*)dx, ld_dx,
+                       vec_ok);
+    return check_launch("ln_bwd_dx_kernel");
+}
+
+int check_rc(const char* fn, int64_t R, int64_t C, int io_dtype) {
+    if (R < 0 || C <= 0) return fail(CW_ERR_INVALID, "%s: bad shape R=%lld C=%lld", fn, (long long)R, (long long)C);
+    if (io_dtype != CW_BF16 && io_dtype != CW_F32) return fail(CW_ERR_INVALID, "%s: bad io_dtype %d", fn, io_dtype);
+    return CW_OK;
+}
+
+}  // namespace
+
+// Upper bound of the column-partial scratch cw_ln_bwd_partials can need.
+int64_t ln_bwd_workspace_bytes(int64_t R, int64_t C) {
+    int64_t parts = (R + kGenericSlabRows - 1) / kGenericSlabRows;
+    if (parts < 256) parts = 256;
+    return parts * 2 * C * (int64_t)sizeof(float);
+}
+
+}  // namespace cw
+
+using namespace cw;
+
+extern "C" int cw_ln_partial_stats(int64_t R, int64_t C, const void* x, int64_t ld, int mode, const float* mean,
+                                   float* stats, int io_dtype, void* stream) {
+    int rc = check_rc("cw_ln_partial_stats", R, C, io_dtype);
+    if (rc != CW_OK) return rc;
+    if (mode != CW_LN_ONE_PASS && mode != CW_LN_TWO_PASS) return fail(CW_ERR_INVALID, "cw_ln_partial_stats: bad mode %d", mode);
+    if (R == 0) return CW_OK;
+    if (x == nullptr || stats == nullptr || ld < C) return fail(CW_ERR_INVALID, "cw_ln_partial_stats: null pointer or ld < C");
+    hipStream_t s = (hipStream_t)stream;
+    return io_dtype == CW_BF16 ? stats_impl<bf16_t>(R, C, x, ld, mode, mean, stats, s)
+                               : stats_impl<float>(R, C, x, ld, mode, mean, stats, s);
+}
+
+extern "C" int cw_ln_normalize(int64_t R, int64_t C, const void* x, int64_t ld, const float* stats, int mode,
+                               int64_t H, float eps, const void* gamma, const void* beta, void* y, int64_t ldy,
+                               float* mean_rstd, int io_dtype, void* stream) {
+    int rc = check_rc("cw_ln_normalize", R, C, io_dtype);
+    if (rc != CW_OK) return rc;
+    if (mode != CW_LN_ONE_PASS && mode != CW_LN_TWO_PASS) return fail(CW_ERR_INVALID, "cw_ln_normalize: bad mode %d", mode);
+    if (H < C) return fail(CW_ERR_INVALID, "cw_ln_normalize: hidden size H=%lld smaller than local C=%lld", (long long)H, (long long)C);
+    if (R == 0) return CW_OK;
+    if (x == nullptr || y == nullptr || stats == nullptr || ld < C || ldy < C)
+        return fail(CW_ERR_INVALID, "cw_ln_normalize: null pointer or leading dimension < C");
+    hipStream_t s = (hipStream_t)stream;
+    return io_dtype == CW_BF16
+               ? normalize_impl<bf16_t, false>(R, C, x, ld, stats, mode, H, eps, gamma, beta, y, ldy, mean_rstd, s)
+               : normalize_impl<float, false>(R, C, x, ld, stats, mode, H, eps, gamma, beta, y, ldy, mean_rstd, s);
+}
+
+extern "C" int cw_ln_forward_fused(int64_t R, int64_t C, const void* x, int64_t ld, int mode, float eps,
+                                   const void* gamma, const void* beta, void* y, int64_t ldy, float* mean_rstd,
+                                   int io_dtype, void* stream) {
+    int rc = check_rc("cw_ln_forward_fused", R, C, io_dtype);
+    if (rc != CW_OK) return rc;
+    if (mode != CW_LN_ONE_PASS && mode != CW_LN_TWO_PASS) return fail(CW_ERR_INVALID, "cw_ln_forward_fused: bad mode %d", mode);
+    if (R == 0) return CW_OK;
+    if (x == nullptr || y == nullptr || ld < C || ldy < C)
+        return fail(CW_ERR_INVALID, "cw_ln_forward_fused: null pointer or leading dimension < C");
+    hipStream_t s = (hipStream_t)stream;
+    return io_dtype == CW_BF16
+               ? normalize_impl<bf16_t, true>(R, C, x, ld, nullptr, mode, C, eps, gamma, beta, y, ldy, mean_rstd, s)
+               : normalize_impl<float, true>(R, C, x, ld, nullptr, mode, C, eps, gamma, beta, y, ldy, mean_rstd, s);
+}
+
+extern "C" int cw_ln_bwd_partials(int64_t R, int64_t C, const void* dY, int64_t ld_dy, const void* x, int64_t ld_x,
+                                  const float* mean_rstd, const void* gamma, float* row_sums, float* dgamma,
+                                  float* dbeta, void* workspace, int64_t workspace_bytes, int io_dtype,
+                                  void* stream) {
+    int rc = check_rc("cw_ln_bwd_partials", R, C, io_dtype);
+    if (rc != CW_OK) return rc;
+    if ((dgamma == nullptr) != (dbeta == nullptr))
+        return fail(CW_ERR_INVALID, "cw_ln_bwd_partials: dgamma and dbeta must both be given or both be NULL");
+    if (R == 0) return CW_OK;
+    if (dY == nullptr || x == nullptr || mean_rstd == nullptr || row_sums == nullptr || ld_dy < C || ld_x < C)
+        return fail(CW_ERR_INVALID, "cw_ln_bwd_partials: null pointer or leading dimension < C");
+    if (dgamma != nullptr && workspace == nullptr) return fail(CW_ERR_INVALID, "cw_ln_bwd_partials: workspace is NULL");
+    hipStream_t s = (hipStream_t)stream;
+    return io_dtype == CW_BF16 ? bwd_partials_impl<bf16_t>(R, C, dY, ld_dy, x, ld_x, mean_rstd, gamma, row_sums, dgamma,
+                                                           dbeta, workspace, workspace_bytes, s)
+                               : bwd_partials_impl<float>(R, C, dY, ld_dy, x, ld_x, mean_rstd, gamma, row_sums, dgamma,
+                                                          dbeta, workspace, workspace_bytes, s);
+}
+
+extern "C" int cw_ln_bwd_dx(int64_t R, int64_t C, const void* dY, int64_t ld_dy, const void* x, int64_t ld_x,
+                            const float* mean_rstd, const void* gamma, const float* row_sums, int64_t H, void* dx,
+                            int64_t ld_dx, int io_dtype, void* stream) {
+    int rc = check_rc("cw_ln_bwd_dx", R, C, io_dtype);
+    if (rc != CW_OK) return rc;
+    if (H < C) return fail(CW_ERR_INVALID, "cw_ln_bwd_dx: hidden size H=%lld smaller than local C=%lld", (long long)H, (long long)C);
+    if (R == 0) return CW_OK;
+    if (dY == nullptr || x == nullptr || mean_rstd == nullptr || row_sums == nullptr || dx == nullptr || ld_dy < C ||
+        ld_x < C || ld_dx < C)
+        return fail(CW_ERR_INVALID, "cw_ln_bwd_dx: null pointer or leading dimension < C");
+    hipStream_t s = (hipStream_t)stream;
+    return io_dtype == CW_BF16
+               ? bwd_dx_impl<bf16_t>(R, C, dY, ld_dy, x, ld_x, mean_rstd, gamma, row_sums, H, dx, ld_dx, s)
+               : bwd_dx_impl<float>(R, C, dY, ld_dy, x, ld_x, mean_rstd, gamma, row_sums, H, dx, ld_dx, s);
+}

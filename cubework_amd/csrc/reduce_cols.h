@@ -1,0 +1,44 @@
+// Deterministic column reductions shared by the bias-gradient and LayerNorm
+// backward kernels: register accumulators -> LDS tree across the block's
+// wavefronts -> one partial row per block in global memory -> finalize kernel.
+#pragma once
+
+#include "cw_common.h"
+
+namespace cw {
+
+inline size_t tree_reduce_lds_bytes(int nreg, int nwaves) {
+    return (size_t)(nwaves / 2 > 0 ? nwaves / 2 : 1) * nreg * 64 * sizeof(float);
+}
+
+// Sums acc[] element-wise over the NWAVES wavefronts of a block into
+// wavefront 0, in a fixed order. Must be reached by every thread of the block.
+template <int NREG, int NWAVES>
+__device__ __forceinline__ void block_tree_reduce(float (&acc)[NREG], float* lds, int wave, int lane) {
+#pragma unroll
+    for (int half = NWAVES / 2; half >= 1; half >>= 1) {
+        if (wave >= half && wave < 2 * half) {
+            float* region = lds + (size_t)(wave - half) * NREG * 64;
+#pragma unroll
+            for (int i = 0; i < NREG; ++i) region[i * 64 + lane] = acc[i];
+        }
+        __syncthreads();
+        if (wave < half) {
+            const float* region = lds + (size_t)wave * NREG * 64;
+#pragma unroll
+            for (int i = 0; i < NREG; ++i) acc[i] += region[i * 64 + lane];
+        }
+        __syncthreads();
+    }
+}
+
+// out_k[c] = sum_p ws[p*part_stride + k*C + c], k < nsets (nsets is 1 or 2;
+// out1 is ignored when nsets == 1). Enqueued on `s`.
+int finalize_col_partials(const float* ws, int64_t nparts, int64_t part_stride, int nsets, int64_t C, float* out0,
+                          float* out1, hipStream_t s);
+
+// Scratch bounds of the two users, combined by cw_colsum_workspace_bytes.
+int64_t colsum_workspace_bytes(int64_t M, int64_t N);
+int64_t ln_bwd_workspace_bytes(int64_t R, int64_t C);
+
+}  // namespace cw

@@ -1,0 +1,282 @@
+// Vocab-parallel cross-entropy, one rank's vocabulary slice, for gfx950.
+// forward: one online pass (running max + rescaled sum of exponentials) over a
+// row per 256-thread block, 16-byte loads, wavefront-shuffle reductions, plus
+// the bit-exact target mask / shifted index / gather. backward: recomputes the
+// softmax from the logits and the global (max, sum) and writes the gradient;
+// the logits are never modified.
+#include "cw_common.h"
+
+namespace cw {
+
+namespace {
+
+constexpr int kCeBlock = 256;
+constexpr float kNegInf = -__builtin_huge_valf();
+
+// Running (max m, sum s of exp(x - m)) kept in the exp2 domain: m2 = m*log2(e).
+struct OnlineLse {
+    float m;   // running maximum of the logits seen (exact input value)
+    float m2;  // m * log2(e), or 0 while m is -inf
+    float s;   // sum of exp2(x*log2e - m2)
+};
+
+template <int V>
+__device__ __forceinline__ void lse_add_chunk(OnlineLse& st, const float (&v)[V]) {
+    float cm = v[0];
+#pragma unroll
+    for (int e = 1; e < V; ++e) cm = fmaxf(cm, v[e]);
+    const float m_new = fmaxf(st.m, cm);
+    const float m2_new = (m_new == kNegInf) ? 0.0f : m_new * kLog2e;
+    // rescale the old sum; an empty state (m == -inf) has s == 0 and stays 0
+    const float scale = (st.m == kNegInf) ? 0.0f : __builtin_amdgcn_exp2f(st.m2 - m2_new);
+    float s = st.s * scale;
+#pragma unroll
+    for (int e = 0; e < V; ++e) s += __builtin_amdgcn_exp2f(__builtin_fmaf(v[e], kLog2e, -m2_new));
+    st.m = m_new;
+    st.m2 = m2_new;
+    st.s = s;
+}
+
+__device__ __forceinline__ void lse_add_one(OnlineLse& st, float x) {
+    const float v[1] = {x};
+    lse_add_chunk<1>(st, v);
+}
+
+// Merge (m_b, s_b) into (m_a, s_a).
+__device__ __forceinline__ void lse_merge(float& m_a, float& s_a, float m_b, float s_b) {
+    const float m = fmaxf(m_a, m_b);
+    const float fa = (m_a == kNegInf) ? 0.0f : __builtin_amdgcn_exp2f((m_a - m) * kLog2e);
+    const float fb = (m_b == kNegInf) ? 0.0f : __builtin_amdgcn_exp2f((m_b - m) * kLog2e);
+    s_a = s_a * fa + s_b * fb;
+    m_a = m;
+}
+
+template <typename T>
+__global__ __launch_bounds__(kCeBlock) void vpce_fwd_kernel(int64_t T_rows, int64_t V_cols,
+                                                            const T* __restrict__ logits, int64_t ld,
+                                                            const int64_t* __restrict__ targets, int64_t vocab_start,
+                                                            float* __restrict__ out_max, float* __restrict__ out_sumexp,
+                                                            float* __restrict__ out_pred, uint8_t* __restrict__ out_mask,
+                                                            int vec_ok) {
+    constexpr int V = elem<T>::kVec;
+    __shared__ float red_m[kCeBlock / 64];
+    __shared__ float red_s[kCeBlock / 64];
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = tid >> 6;
+    for (int64_t row = blockIdx.x; row < T_rows; row += gridDim.x) {
+        const T* xr = logits + row * ld;
+        OnlineLse st{kNegInf, 0.0f, 0.0f};
+        if (vec_ok) {
+            const int64_t nvec = V_cols / V;
+            int64_t i = tid;
+            // two independent 16-byte loads in flight per trip
+            for (; i + kCeBlock < nvec; i += 2 * kCeBlock) {
+                float v0[V], v1[V];
+                load_vec(xr + i * V, v0);
+                load_vec(xr + (i + kCeBlock) * V, v1);
+                lse_add_chunk<V>(st, v0);
+                lse_add_chunk<V>(st, v1);
+            }
+            for (; i < nvec; i += kCeBlock) {
+                float v0[V];
+                load_vec(xr + i * V, v0);
+                lse_add_chunk<V>(st, v0);
+            }
+            for (int64_t c = nvec * V + tid; c < V_cols; c += kCeBlock) lse_add_one(st, load_elem(xr + c));
+        } else {
+            for (int64_t c = tid; c < V_cols; c += kCeBlock) lse_add_one(st, load_elem(xr + c));
+        }
+        // wavefront, then block
+        float m = st.m, s = st.s;
+#pragma unroll
+        for (int off = 32; off > 0; off >>= 1) {
+            const float mo = __shfl_xor(m, off, 64);
+            const float so = __shfl_xor(s, off, 64);
+            lse_merge(m, s, mo, so);
+        }
+        if (lane == 0) {
+            red_m[wave] = m;
+            red_s[wave] = s;
+        }
+        __syncthreads();
+        if (tid == 0) {
+            float gm = red_m[0], gs = red_s[0];
+#pragma unroll
+            for (int w = 1; w < kCeBlock / 64; ++w) lse_merge(gm, gs, red_m[w], red_s[w]);
+            out_max[row] = gm;
+            out_sumexp[row] = gs;
+            // target bookkeeping: integer-exact
+            const int64_t t = targets[row];
+            const bool masked = (t < vocab_start) || (t >= vocab_start + V_cols);
+            const int64_t idx = masked ? 0 : (t - vocab_start);
+            out_mask[row] = masked ? 1 : 0;
+            out_pred[row] = masked ? 0.0f : load_elem(xr + idx);
+        }
+        __syncthreads();
+    }
+}
+
+__global__ __launch_bounds__(256) void vpce_finalize_kernel(int64_t T_rows, int n_ranks,
+                                                            const float* __restrict__ max_all,
+                                                            const float* __restrict__ sumexp_all,
+                                                            const float* __restrict__ pred_all,
+                                                            const uint8_t* __restrict__ mask_all,
+                                                            float* __restrict__ loss, float* __restrict__ gmax,
+                                                            float* __restrict__ gsum) {
+    const int64_t t = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (t >= T_rows) return;
+    float m = max_all[t];
+    for (int r = 1; r < n_ranks; ++r) m = fmaxf(m, max_all[(int64_t)r * T_rows + t]);
+    float s = 0.0f, p = 0.0f;
+    for (int r = 0; r < n_ranks; ++r) {
+        const float mr = max_all[(int64_t)r * T_rows + t];
+        const float f = (mr == kNegInf) ? 0.0f : expf(mr - m);
+        s += sumexp_all[(int64_t)r * T_rows + t] * f;
+        if (mask_all[(int64_t)r * T_rows + t] == 0) p += pred_all[(int64_t)r * T_rows + t] - m;
+    }
+    loss[t] = logf(s) - p;
+    if (gmax != nullptr) gmax[t] = m;
+    if (gsum != nullptr) gsum[t] = s;
+}
+
+template <int V>
+__device__ __forceinline__ void store_grad(bf16_t* p, const float (&v)[V]) {
+    static_assert(V == 8, "bf16 gradients are written 8 at a time");
+    store_vec(p, v);
+}
+template <int V>
+__device__ __forceinline__ void store_grad(float* p, const float (&v)[V]) {
+#pragma unroll
+    for (int e = 0; e < V; e += 4)
+        *reinterpret_cast<float4*>(p + e) = make_float4(v[e], v[e + 1], v[e + 2], v[e + 3]);
+}
+
+template <typename T, typename G>
+__global__ __launch_bounds__(kCeBlock) void vpce_bwd_kernel(int64_t T_rows, int64_t V_cols,
+                                                            const T* __restrict__ logits, int64_t ld,
+                                                            const int64_t* __restrict__ targets, int64_t vocab_start,
+                                                            const float* __restrict__ gmax,
+                                                            const float* __restrict__ gsum,
+                                                            const float* __restrict__ dloss_rows, float dloss_scale,
+                                                            G* __restrict__ grad, int64_t ld_grad, int vec_ok) {
+    constexpr int V = elem<T>::kVec;
+    const int tid = threadIdx.x;
+    for (int64_t row = blockIdx.x; row < T_rows; row += gridDim.x) {
+        const T* xr = logits + row * ld;
+        G* gr = grad + row * ld_grad;
+        const float m2 = gmax[row] * kLog2e;
+        const float dl = (dloss_rows != nullptr ? dloss_rows[row] : 1.0f) * dloss_scale;
+        const float scale = dl / gsum[row];
+        const int64_t t = targets[row];
+        const bool masked = (t < vocab_start) || (t >= vocab_start + V_cols);
+        const int64_t tcol = masked ? -1 : (t - vocab_start);
+        if (vec_ok) {
+            const int64_t nvec = V_cols / V;
+            for (int64_t i = tid; i < nvec; i += kCeBlock) {
+                float v[V];
+                load_vec(xr + i * V, v);
+#pragma unroll
+                for (int e = 0; e < V; ++e) v[e] = __builtin_amdgcn_exp2f(__builtin_fmaf(v[e], kLog2e, -m2)) * scale;
+                const int64_t rel = tcol - i * V;
+                if (rel >= 0 && rel < V) {
+#pragma unroll
+                    for (int e = 0; e < V; ++e)
+                        if (e == rel) v[e] -= dl;
+                }
+                store_grad<V>(gr + i * V, v);
+            }
+            for (int64_t c = nvec * V + tid; c < V_cols; c += kCeBlock) {
+                float y = __builtin_amdgcn_exp2f(__builtin_fmaf(load_elem(xr + c), kLog2e, -m2)) * scale;
+                if (c == tcol) y -= dl;
+                store_elem(gr + c, y);
+            }
+        } else {
+            for (int64_t c = tid; c < V_cols; c += kCeBlock) {
+                float y = __builtin_amdgcn_exp2f(__builtin_fmaf(load_elem(xr + c), kLog2e, -m2)) * scale;
+                if (c == tcol) y -= dl;
+                store_elem(gr + c, y);
+            }
+        }
+    }
+}
+
+int ce_grid(int64_t T_rows) {
+    const int64_t cap = 256 * 16;
+    return (int)(T_rows < cap ? T_rows : cap);
+}
+
+template <typename T, typename G>
+int bwd_impl(int64_t T_rows, int64_t V_cols, const void* logits, int64_t ld, const int64_t* targets,
+             int64_t vocab_start, const float* gmax, const float* gsum, const float* dloss_rows, float dloss_scale,
+             void* grad, int64_t ld_grad, hipStream_t s) {
+    const int vec_ok = aligned16(logits) && (ld % elem<T>::kVec) == 0 && aligned16(grad) &&
+                       (ld_grad % (16 / (int)sizeof(G))) == 0;
+    hipLaunchKernelGGL((vpce_bwd_kernel<T, G>), dim3(ce_grid(T_rows)), dim3(kCeBlock), 0, s, T_rows, V_cols,
+                       (const T*)logits, ld, targets, vocab_start, gmax, gsum, dloss_rows, dloss_scale, (G*)grad,
+                       ld_grad, vec_ok);
+    return check_launch("vpce_bwd_kernel");
+}
+
+}  // namespace
+}  // namespace cw
+
+using namespace cw;
+
+extern "C" int cw_vpce_fwd_local(int64_t T, int64_t V, const void* logits, int64_t ld, const int64_t* targets,
+                                 int64_t vocab_start, float* out_max, float* out_sumexp, float* out_pred,
+                                 uint8_t* out_mask, int io_dtype, void* stream) {
+    if (T < 0 || V <= 0) return fail(CW_ERR_INVALID, "cw_vpce_fwd_local: bad shape T=%lld V=%lld", (long long)T, (long long)V);
+    if (io_dtype != CW_BF16 && io_dtype != CW_F32) return fail(CW_ERR_INVALID, "cw_vpce_fwd_local: bad io_dtype %d", io_dtype);
+    if (vocab_start < 0) return fail(CW_ERR_INVALID, "cw_vpce_fwd_local: negative vocab_start");
+    if (T == 0) return CW_OK;
+    if (logits == nullptr || targets == nullptr || out_max == nullptr || out_sumexp == nullptr ||
+        out_pred == nullptr || out_mask == nullptr || ld < V)
+        return fail(CW_ERR_INVALID, "cw_vpce_fwd_local: null pointer or ld < V");
+    hipStream_t s = (hipStream_t)stream;
+    if (io_dtype == CW_BF16) {
+        const int vec_ok = aligned16(logits) && (ld % 8) == 0;
+        hipLaunchKernelGGL(vpce_fwd_kernel<bf16_t>, dim3(ce_grid(T)), dim3(kCeBlock), 0, s, T, V,
+                           (const bf16_t*)logits, ld, targets, vocab_start, out_max, out_sumexp, out_pred, out_mask,
+                           vec_ok);
+    } else {
+        const int vec_ok = aligned16(logits) && (ld % 4) == 0;
+        hipLaunchKernelGGL(vpce_fwd_kernel<float>, dim3(ce_grid(T)), dim3(kCeBlock), 0, s, T, V,
+                           (const float*)logits, ld, targets, vocab_start, out_max, out_sumexp, out_pred, out_mask,
+                           vec_ok);
+    }
+    return check_launch("vpce_fwd_kernel");
+}
+
+extern "C" int cw_vpce_finalize(int64_t T, int n_ranks, const float* max_all, const float* sumexp_all,
+                                const float* pred_all, const uint8_t* mask_all, float* loss, float* gmax,
+                                float* gsum, void* stream) {
+    if (T < 0 || n_ranks < 1) return fail(CW_ERR_INVALID, "cw_vpce_finalize: bad T=%lld or n_ranks=%d", (long long)T, n_ranks);
+    if (T == 0) return CW_OK;
+    if (max_all == nullptr || sumexp_all == nullptr || pred_all == nullptr || mask_all == nullptr || loss == nullptr)
+        return fail(CW_ERR_INVALID, "cw_vpce_finalize: null pointer");
+    hipLaunchKernelGGL(vpce_finalize_kernel, dim3((unsigned)((T + 255) / 256)), dim3(256), 0, (hipStream_t)stream, T,
+                       n_ranks, max_all, sumexp_all, pred_all, mask_all, loss, gmax, gsum);
+    return check_launch("vpce_finalize_kernel");
+}
+
+extern "C" int cw_vpce_bwd(int64_t T, int64_t V, const void* logits, int64_t ld, const int64_t* targets,
+                           int64_t vocab_start, const float* gmax, const float* gsum, const float* dloss_rows,
+                           float dloss_scale, void* grad, int64_t ld_grad, int io_dtype, int grad_dtype,
+                           void* stream) {
+    if (T < 0 || V <= 0) return fail(CW_ERR_INVALID, "cw_vpce_bwd: bad shape T=%lld V=%lld", (long long)T, (long long)V);
+    if (io_dtype != CW_BF16 && io_dtype != CW_F32) return fail(CW_ERR_INVALID, "cw_vpce_bwd: bad io_dtype %d", io_dtype);
+    if (grad_dtype != CW_BF16 && grad_dtype != CW_F32) return fail(CW_ERR_INVALID, "cw_vpce_bwd: bad grad_dtype %d", grad_dtype);
+    if (io_dtype == CW_F32 && grad_dtype == CW_BF16)
+        return fail(CW_ERR_UNSUPPORTED, "cw_vpce_bwd: bf16 gradient of fp32 logits is not provided");
+    if (T == 0) return CW_OK;
+    if (logits == nullptr || targets == nullptr || gmax == nullptr || gsum == nullptr || grad == nullptr || ld < V ||
+        ld_grad < V)
+        return fail(CW_ERR_INVALID, "cw_vpce_bwd: null pointer or leading dimension < V");
+    hipStream_t s = (hipStream_t)stream;
+    if (io_dtype == CW_BF16 && grad_dtype == CW_BF16)
+        return bwd_impl<bf16_t, bf16_t>(T, V, logits, ld, targets, vocab_start, gmax, gsum, dloss_rows, dloss_scale, grad, ld_grad, s);
+    if (io_dtype == CW_BF16)
+        return bwd_impl<bf16_t, float>(T, V, logits, ld, targets, vocab_start, gmax, gsum, dloss_rows, dloss_scale, grad, ld_grad, s);
+    return bwd_impl<float, float>(T, V, logits, ld, targets, vocab_start, gmax, gsum, dloss_rows, dloss_scale, grad, ld_grad, s);
+}

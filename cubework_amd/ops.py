@@ -1,0 +1,330 @@
+"""Tensor-level wrappers of the C ABI: check shapes, allocate outputs with torch
+(device memory and streams are torch's; the arithmetic is the HIP library's),
+pass raw pointers and the current stream.
+
+Every function requires CUDA (ROCm) tensors of dtype bfloat16 or float32 and
+raises instead of falling back to torch arithmetic.
+"""
+import ctypes
+from typing import Optional, Sequence, Tuple
+
+import torch
+
+from . import _lib
+from ._lib import (CW_ACT_GELU_ERF, CW_ACT_GELU_TANH, CW_ACT_NONE, CW_ACT_RELU, CW_BF16, CW_EPI_BIAS,
+                   CW_EPI_BIAS_GELU_ERF, CW_EPI_BIAS_GELU_TANH, CW_EPI_BIAS_RELU, CW_EPI_NONE, CW_F32, CW_LN_ONE_PASS,
+                   CW_LN_TWO_PASS, CW_NN, CW_NT, CW_TN)
+
+ACTIVATIONS = {None: CW_ACT_NONE, "none": CW_ACT_NONE, "gelu_tanh": CW_ACT_GELU_TANH, "gelu": CW_ACT_GELU_ERF,
+               "gelu_erf": CW_ACT_GELU_ERF, "relu": CW_ACT_RELU}
+LAYOUTS = {"NN": CW_NN, "NT": CW_NT, "TN": CW_TN}
+
+
+def epilogue_code(has_bias: bool, activation: Optional[str]) -> int:
+    act = ACTIVATIONS[activation]
+    if act == CW_ACT_NONE:
+        return CW_EPI_BIAS if has_bias else CW_EPI_NONE
+    return {CW_ACT_GELU_TANH: CW_EPI_BIAS_GELU_TANH, CW_ACT_GELU_ERF: CW_EPI_BIAS_GELU_ERF,
+            CW_ACT_RELU: CW_EPI_BIAS_RELU}[act]
+
+
+def _dtype_code(t: torch.Tensor) -> int:
+    if t.dtype == torch.bfloat16:
+        return CW_BF16
+    if t.dtype == torch.float32:
+        return CW_F32
+    raise TypeError("cubework_amd kernels take bfloat16 or float32 tensors, got %s" % t.dtype)
+
+
+def _require_device(*tensors):
+    for t in tensors:
+        if t is not None and not t.is_cuda:
+            raise RuntimeError("cubework_amd operators run on the GPU only (got a %s tensor); "
+                               "there is no CPU fallback" % t.device)
+
+
+def _rows(t: torch.Tensor) -> torch.Tensor:
+    """View as [rows, cols] with unit column stride (copy only if unavoidable)."""
+    if t.dim() != 2:
+        t = t.reshape(-1, t.shape[-1])
+    if t.stride(1) != 1 or (t.shape[0] > 1 and t.stride(0) < t.shape[1]):
+        t = t.contiguous()
+    return t
+
+
+def _ld(t: torch.Tensor) -> int:
+    return t.stride(0) if t.shape[0] > 1 else max(t.shape[1], 1)
+
+
+def _stream() -> ctypes.c_void_p:
+    return ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+
+def _p(t: Optional[torch.Tensor]) -> ctypes.c_void_p:
+    return ctypes.c_void_p(0 if t is None else t.data_ptr())
+
+
+def _ptr_table(tensors: Sequence[torch.Tensor]):
+    arr = (ctypes.c_void_p * max(len(tensors), 1))()
+    for i, t in enumerate(tensors):
+        arr[i] = t.data_ptr()
+    return arr
+
+
+# --------------------------------------------------------------------------
+# block GEMM
+# --------------------------------------------------------------------------
+def gemm_ksteps(layout: str, A_steps: Sequence[torch.Tensor], B_steps: Sequence[torch.Tensor],
+                bias: Optional[torch.Tensor] = None, activation: Optional[str] = None,
+                addends: Sequence[torch.Tensor] = (), want_preact: bool = False,
+                out: Optional[torch.Tensor] = None):
+    """C = act(sum_i op(A_i) op(B_i) + sum_j addends_j + bias); see cw_gemm_ksteps.
+
+    layout "NN": A_i [M,K], B_i [K,N];  "NT": A_i [M,K], B_i [N,K];  "TN": A_i [K,M], B_i [K,N].
+    Returns C, or (C, preact) when want_preact.
+    """
+    lib = _lib.load()
+    if len(A_steps) != len(B_steps) or len(A_steps) == 0:
+        raise ValueError("need the same, non-zero number of A and B step operands")
+    A_steps = [_rows(a) for a in A_steps]
+    B_steps = [_rows(b) for b in B_steps]
+    _require_device(*A_steps, *B_steps, bias, *addends)
+    a0, b0 = A_steps[0], B_steps[0]
+    dt = _dtype_code(a0)
+    if layout == "NN":
+        M, K, N, Kb = a0.shape[0], a0.shape[1], b0.shape[1], b0.shape[0]
+    elif layout == "NT":
+        M, K, N, Kb = a0.shape[0], a0.shape[1], b0.shape[0], b0.shape[1]
+    elif layout == "TN":
+        M, K, N, Kb = a0.shape[1], a0.shape[0], b0.shape[1], b0.shape[0]
+    else:
+        raise ValueError("layout must be NN, NT or TN")
+    if K != Kb:
+        raise ValueError("reduction sizes differ: A %s, B %s for %s" % (tuple(a0.shape), tuple(b0.shape), layout))
+    for t in list(A_steps) + list(B_steps):
+        if t.dtype != a0.dtype:
+            raise TypeError("all GEMM operands must share one dtype")
+    lda, ldb = _ld(a0), _ld(b0)
+    for a in A_steps:
+        if a.shape != a0.shape or _ld(a) != lda:
+            raise ValueError("A step operands must share shape and leading dimension")
+    for b in B_steps:
+        if b.shape != b0.shape or _ld(b) != ldb:
+            raise ValueError("B step operands must share shape and leading dimension")
+    if bias is not None:
+        if bias.numel() != N:
+            raise ValueError("bias has %d elements, output width is %d" % (bias.numel(), N))
+        bias = bias.to(a0.dtype).contiguous()
+    addends = [_rows(t) for t in addends]
+    ldadd = 0
+    for t in addends:
+        if tuple(t.shape) != (M, N) or t.dtype != a0.dtype:
+            raise ValueError("addends must be [M,N] of the operand dtype")
+        ldadd = _ld(t)
+    if out is None:
+        out = torch.empty((M, N), dtype=a0.dtype, device=a0.device)
+    elif tuple(out.shape) != (M, N) or out.dtype != a0.dtype or out.stride(1) != 1:
+        raise ValueError("out must be a row-major [M,N] tensor of the operand dtype")
+    preact = torch.empty((M, N), dtype=a0.dtype, device=a0.device) if want_preact else None
+    epi = epilogue_code(bias is not None, activation)
+    ta, tb, tadd = _ptr_table(A_steps), _ptr_table(B_steps), _ptr_table(addends)
+    rc = lib.cw_gemm_ksteps(LAYOUTS[layout], M, N, K, len(A_steps), ta, lda, tb, ldb, _p(bias), epi, _p(out),
+                            _ld(out), _p(preact), _ld(preact) if preact is not None else 0, tadd, len(addends),
+                            ldadd, dt, _stream())
+    _lib.check(rc, "cw_gemm_ksteps")
+    return (out, preact) if want_preact else out
+
+
+def _workspace(M: int, N: int, device) -> torch.Tensor:
+    nbytes = _lib.load().cw_colsum_workspace_bytes(M, N)
+    return torch.empty(max(nbytes, 16), dtype=torch.uint8, device=device)
+
+
+def colsum(dy: torch.Tensor) -> torch.Tensor:
+    """fp32 column sums of a [M,N] tensor (bias gradient)."""
+    lib = _lib.load()
+    dy = _rows(dy)
+    _require_device(dy)
+    M, N = dy.shape
+    out = torch.empty(N, dtype=torch.float32, device=dy.device)
+    ws = _workspace(M, N, dy.device)
+    rc = lib.cw_colsum(M, N, _p(dy), _ld(dy), _p(out), _p(ws), ws.numel(), _dtype_code(dy), _stream())
+    _lib.check(rc, "cw_colsum")
+    return out
+
+
+def act_bwd_colsum(activation: Optional[str], dy: torch.Tensor, preact: torch.Tensor,
+                   want_dbias: bool = True) -> Tuple[torch.Tensor, Optional[torch.Tensor]]:
+    """dPre = dy * act'(preact) and (optionally) its fp32 column sums."""
+    lib = _lib.load()
+    dy, preact = _rows(dy), _rows(preact)
+    _require_device(dy, preact)
+    if dy.shape != preact.shape or dy.dtype != preact.dtype:
+        raise ValueError("dy and preact must agree in shape and dtype")
+    M, N = dy.shape
+    dpre = torch.empty((M, N), dtype=dy.dtype, device=dy.device)
+    dbias = torch.empty(N, dtype=torch.float32, device=dy.device) if want_dbias else None
+    ws = _workspace(M, N, dy.device) if want_dbias else None
+    rc = lib.cw_act_bwd_colsum(ACTIVATIONS[activation], M, N, _p(dy), _ld(dy), _p(preact), _ld(preact), _p(dpre),
+                               _ld(dpre), _p(dbias), _p(ws), ws.numel() if ws is not None else 0, _dtype_code(dy),
+                               _stream())
+    _lib.check(rc, "cw_act_bwd_colsum")
+    return dpre, dbias
+
+
+# --------------------------------------------------------------------------
+# LayerNorm
+# --------------------------------------------------------------------------
+def ln_partial_stats(x: torch.Tensor, mode: int = CW_LN_ONE_PASS, mean: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """[R,2] fp32 partial statistics of the local columns of x [R,C]."""
+    lib = _lib.load()
+    x = _rows(x)
+    _require_device(x, mean)
+    R, C = x.shape
+    stats = torch.empty((R, 2), dtype=torch.float32, device=x.device)
+    if mean is not None:
+        mean = mean.reshape(-1).to(torch.float32).contiguous()
+        if mean.numel() != R:
+            raise ValueError("mean must have one entry per row")
+    rc = lib.cw_ln_partial_stats(R, C, _p(x), _ld(x), mode, _p(mean), _p(stats), _dtype_code(x), _stream())
+    _lib.check(rc, "cw_ln_partial_stats")
+    return stats
+
+
+def ln_normalize(x: torch.Tensor, stats: torch.Tensor, hidden: int, eps: float,
+                 gamma: Optional[torch.Tensor] = None, beta: Optional[torch.Tensor] = None,
+                 mode: int = CW_LN_ONE_PASS, save_mean_rstd: bool = True):
+    """y = gamma*(x-mean)*rstd+beta from whole-hidden-size stats; returns (y, mean_rstd)."""
+    lib = _lib.load()
+    shape = x.shape
+    x = _rows(x)
+    _require_device(x, stats, gamma, beta)
+    R, C = x.shape
+    stats = stats.reshape(R, 2).to(torch.float32).contiguous()
+    gamma = None if gamma is None else gamma.to(x.dtype).contiguous()
+    beta = None if beta is None else beta.to(x.dtype).contiguous()
+    for v in (gamma, beta):
+        if v is not None and v.numel() != C:
+            raise ValueError("gamma/beta must have C elements")
+    y = torch.empty((R, C), dtype=x.dtype, device=x.device)
+    mr = torch.empty((R, 2), dtype=torch.float32, device=x.device) if save_mean_rstd else None
+    rc = lib.cw_ln_normalize(R, C, _p(x), _ld(x), _p(stats), mode, hidden, eps, _p(gamma), _p(beta), _p(y), _ld(y),
+                             _p(mr), _dtype_code(x), _stream())
+    _lib.check(rc, "cw_ln_normalize")
+    return y.reshape(shape), mr
+
+
+def ln_forward_fused(x: torch.Tensor, eps: float, gamma: Optional[torch.Tensor] = None,
+                     beta: Optional[torch.Tensor] = None, mode: int = CW_LN_ONE_PASS, save_mean_rstd: bool = True):
+    """LayerNorm over the last dimension when this rank holds the whole hidden size."""
+    lib = _lib.load()
+    shape = x.shape
+    x = _rows(x)
+    _require_device(x, gamma, beta)
+    R, C = x.shape
+    gamma = None if gamma is None else gamma.to(x.dtype).contiguous()
+    beta = None if beta is None else beta.to(x.dtype).contiguous()
+    y = torch.empty((R, C), dtype=x.dtype, device=x.device)
+    mr = torch.empty((R, 2), dtype=torch.float32, device=x.device) if save_mean_rstd else None
+    rc = lib.cw_ln_forward_fused(R, C, _p(x), _ld(x), mode, eps, _p(gamma), _p(beta), _p(y), _ld(y), _p(mr),
+                                 _dtype_code(x), _stream())
+    _lib.check(rc, "cw_ln_forward_fused")
+    return y.reshape(shape), mr
+
+
+def ln_bwd_partials(dy: torch.Tensor, x: torch.Tensor, mean_rstd: torch.Tensor,
+                    gamma: Optional[torch.Tensor] = None, want_param_grads: bool = True):
+    """Returns (row_sums [R,2] fp32, dgamma [C] fp32 or None, dbeta [C] fp32 or None)."""
+    lib = _lib.load()
+    dy, x = _rows(dy), _rows(x)
+    _require_device(dy, x, mean_rstd, gamma)
+    if dy.shape != x.shape or dy.dtype != x.dtype:
+        raise ValueError("dy and x must agree in shape and dtype")
+    R, C = x.shape
+    gamma = None if gamma is None else gamma.to(x.dtype).contiguous()
+    row_sums = torch.empty((R, 2), dtype=torch.float32, device=x.device)
+    dgamma = dbeta = ws = None
+    if want_param_grads:
+        dgamma = torch.empty(C, dtype=torch.float32, device=x.device)
+        dbeta = torch.empty(C, dtype=torch.float32, device=x.device)
+        ws = _workspace(R, C, x.device)
+    rc = lib.cw_ln_bwd_partials(R, C, _p(dy), _ld(dy), _p(x), _ld(x), _p(mean_rstd), _p(gamma), _p(row_sums),
+                                _p(dgamma), _p(dbeta), _p(ws), ws.numel() if ws is not None else 0, _dtype_code(x),
+                                _stream())
+    _lib.check(rc, "cw_ln_bwd_partials")
+    return row_sums, dgamma, dbeta
+
+
+def ln_bwd_dx(dy: torch.Tensor, x: torch.Tensor, mean_rstd: torch.Tensor, row_sums: torch.Tensor, hidden: int,
+              gamma: Optional[torch.Tensor] = None) -> torch.Tensor:
+    lib = _lib.load()
+    shape = x.shape
+    dy, x = _rows(dy), _rows(x)
+    _require_device(dy, x, mean_rstd, row_sums, gamma)
+    R, C = x.shape
+    gamma = None if gamma is None else gamma.to(x.dtype).contiguous()
+    row_sums = row_sums.reshape(R, 2).to(torch.float32).contiguous()
+    dx = torch.empty((R, C), dtype=x.dtype, device=x.device)
+    rc = lib.cw_ln_bwd_dx(R, C, _p(dy), _ld(dy), _p(x), _ld(x), _p(mean_rstd), _p(gamma), _p(row_sums), hidden,
+                          _p(dx), _ld(dx), _dtype_code(x), _stream())
+    _lib.check(rc, "cw_ln_bwd_dx")
+    return dx.reshape(shape)
+
+
+# --------------------------------------------------------------------------
+# vocab-parallel cross-entropy
+# --------------------------------------------------------------------------
+def vpce_fwd_local(logits: torch.Tensor, targets: torch.Tensor, vocab_start: int):
+    """Returns (max, sumexp, pred, mask) of this rank's slice; each [T]."""
+    lib = _lib.load()
+    logits = _rows(logits)
+    _require_device(logits, targets)
+    T, V = logits.shape
+    targets = targets.reshape(-1).to(torch.int64).contiguous()
+    if targets.numel() != T:
+        raise ValueError("one target per logits row is required")
+    dev = logits.device
+    mx = torch.empty(T, dtype=torch.float32, device=dev)
+    se = torch.empty(T, dtype=torch.float32, device=dev)
+    pr = torch.empty(T, dtype=torch.float32, device=dev)
+    mk = torch.empty(T, dtype=torch.uint8, device=dev)
+    rc = lib.cw_vpce_fwd_local(T, V, _p(logits), _ld(logits), _p(targets), vocab_start, _p(mx), _p(se), _p(pr), _p(mk),
+                               _dtype_code(logits), _stream())
+    _lib.check(rc, "cw_vpce_fwd_local")
+    return mx, se, pr, mk
+
+
+def vpce_finalize(max_all: torch.Tensor, sumexp_all: torch.Tensor, pred_all: torch.Tensor, mask_all: torch.Tensor):
+    """Inputs [n_ranks, T]; returns (loss, gmax, gsum), each [T] fp32."""
+    lib = _lib.load()
+    _require_device(max_all, sumexp_all, pred_all, mask_all)
+    n, T = max_all.shape
+    max_all, sumexp_all, pred_all = (t.to(torch.float32).contiguous() for t in (max_all, sumexp_all, pred_all))
+    mask_all = mask_all.to(torch.uint8).contiguous()
+    dev = max_all.device
+    loss = torch.empty(T, dtype=torch.float32, device=dev)
+    gmax = torch.empty(T, dtype=torch.float32, device=dev)
+    gsum = torch.empty(T, dtype=torch.float32, device=dev)
+    rc = lib.cw_vpce_finalize(T, n, _p(max_all), _p(sumexp_all), _p(pred_all), _p(mask_all), _p(loss), _p(gmax),
+                              _p(gsum), _stream())
+    _lib.check(rc, "cw_vpce_finalize")
+    return loss, gmax, gsum
+
+
+def vpce_bwd(logits: torch.Tensor, targets: torch.Tensor, vocab_start: int, gmax: torch.Tensor, gsum: torch.Tensor,
+             dloss_rows: Optional[torch.Tensor] = None, dloss_scale: float = 1.0,
+             grad_dtype: Optional[torch.dtype] = None) -> torch.Tensor:
+    lib = _lib.load()
+    shape = logits.shape
+    logits = _rows(logits)
+    _require_device(logits, targets, gmax, gsum, dloss_rows)
+    T, V = logits.shape
+    targets = targets.reshape(-1).to(torch.int64).contiguous()
+    grad_dtype = grad_dtype or logits.dtype
+    grad = torch.empty((T, V), dtype=grad_dtype, device=logits.device)
+    if dloss_rows is not None:
+        dloss_rows = dloss_rows.reshape(-1).to(torch.float32).contiguous()
+    rc = lib.cw_vpce_bwd(T, V, _p(logits), _ld(logits), _p(targets), vocab_start, _p(gmax), _p(gsum), _p(dloss_rows),
+                         dloss_scale, _p(grad), _ld(grad), _dtype_code(logits), _dtype_code(grad), _stream())
+    _lib.check(rc, "cw_vpce_bwd")
+    return grad.reshape(shape)

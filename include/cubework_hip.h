@@ -1,0 +1,238 @@
+/*
+ * cubework_hip.h — C ABI of libcubework_hip.so (gfx950 / MI355X).
+ *
+ * One rank's share of the compute inside Cubework's tensor-parallel layers:
+ * the SUMMA block-GEMM accumulation loop (+ bias + activation), LayerNorm
+ * partial statistics / normalise / backward, vocab-parallel cross-entropy.
+ * Operands a collective would have delivered are passed as extra device
+ * pointers ("pre-staged" peers); the library never communicates.
+ *
+ * Conventions for every entry point
+ *   - returns 0 on success, a negative cw_status on failure; the message for
+ *     the calling thread is available from cw_last_error();
+ *   - every data pointer is a DEVICE pointer owned by the caller, row-major,
+ *     with explicit leading dimensions counted in ELEMENTS;
+ *   - no allocation, no synchronisation, nothing on the null stream: work is
+ *     enqueued on `stream` (a hipStream_t passed as void*) and the call returns;
+ *   - re-entrant and callable from any thread (the autograd engine calls the
+ *     backward entry points from its own device thread);
+ *   - io_dtype selects the storage type of activations/weights (CW_BF16 or
+ *     CW_F32); statistics, losses and all accumulation are fp32.
+ *
+ * Citations name the reference code (kurisusnowdeng/Cubework) each entry
+ * point stands in for; paths are relative to the reference tree.
+ */
+#ifndef CUBEWORK_HIP_H
+#define CUBEWORK_HIP_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef enum {
+    CW_OK = 0,
+    CW_ERR_INVALID = -1,     /* bad argument (shape, enum, null pointer) */
+    CW_ERR_ALIGNMENT = -2,   /* pointer / leading dimension not usable   */
+    CW_ERR_UNSUPPORTED = -3, /* valid request this build cannot serve    */
+    CW_ERR_LAUNCH = -4,      /* HIP reported an error at launch          */
+    CW_ERR_DEVICE = -5       /* current device is not gfx950             */
+} cw_status;
+
+typedef enum { CW_BF16 = 0, CW_F32 = 1 } cw_dtype;
+
+/* Operand orientation of the block GEMM, per k-step i:
+ *   CW_NN: C[M,N] += A_i[M,K] * B_i[K,N]      (summa_AB,  Linear2D/3D forward)
+ *   CW_NT: C[M,N] += A_i[M,K] * B_i[N,K]^T    (summa_ABT, F.linear, dX, classifiers)
+ *   CW_TN: C[M,N] += A_i[K,M]^T * B_i[K,N]    (summa_ATB, dW)                       */
+typedef enum { CW_NN = 0, CW_NT = 1, CW_TN = 2 } cw_layout;
+
+typedef enum {
+    CW_EPI_NONE = 0,       /* C = acc (+ addends)                    */
+    CW_EPI_BIAS = 1,       /* C = acc + bias[N]                      */
+    CW_EPI_BIAS_GELU_TANH = 2,
+    CW_EPI_BIAS_GELU_ERF = 3,
+    CW_EPI_BIAS_RELU = 4
+} cw_epilogue;
+
+typedef enum { CW_ACT_NONE = 0, CW_ACT_GELU_TANH = 2, CW_ACT_GELU_ERF = 3, CW_ACT_RELU = 4 } cw_activation;
+
+/* LayerNorm statistics convention.
+ *   CW_LN_ONE_PASS : partials are (sum x, sum x^2); var = E[x^2] - E[x]^2
+ *                    (LayerNorm2D, parallel_2d/module.py:142-153)
+ *   CW_LN_TWO_PASS : first exchange gives the mean, second partial is
+ *                    sum (x-mean)^2 (LayerNorm3D, parallel_3d/_operation.py:273-276) */
+typedef enum { CW_LN_ONE_PASS = 0, CW_LN_TWO_PASS = 1 } cw_ln_mode;
+
+#define CW_MAX_KSTEPS 16
+#define CW_MAX_ADDENDS 8
+
+/* ---- sanity ------------------------------------------------------------ */
+const char* cw_version(void);
+/* gcnArchName of the current device ("gfx950:..."), or "" without a device. */
+const char* cw_device_arch(void);
+/* Message of the last failing call made by this thread ("" if none). */
+const char* cw_last_error(void);
+
+/* ---- block GEMM with k-step accumulation ------------------------------- */
+/*
+ * C = act( sum_{i<n_steps} op(A_i) * op(B_i) + sum_{j<n_addends} addend_j + bias )
+ *
+ * Replaces the per-rank math of
+ *   _SUMMA_AB.forward   cubework/module/parallel_2d/_operation.py:41-47  (CW_NN)
+ *   _SUMMA_ABT.forward  cubework/module/parallel_2d/_operation.py:117-125 (CW_NT)
+ *   _SUMMA_ATB.forward  cubework/module/parallel_2d/_operation.py:197-204 (CW_TN)
+ *   _SUMMAbias.forward  cubework/module/parallel_2d/_operation.py:271-274 (bias)
+ *   F.linear            cubework/module/parallel_1d/module.py:147,209,269,338 (CW_NT)
+ *   _Linear3D fwd/bwd   cubework/module/parallel_3d/_operation.py:34,39,53,65
+ *   _Classifier2D       cubework/module/parallel_2d/_operation.py:383,387,408-410
+ *   activation after the linear: benchmark/gpt2/gpt2.py:116-117, benchmark/opt/opt.py:200
+ * with A_steps[i]/B_steps[i] standing for what the row/column broadcast of
+ * step i delivers, and addends[j] for the peers' partial products a reduce
+ * delivers. A_steps/B_steps/addends are HOST arrays of device pointers.
+ * K is the reduction length of ONE step. bias (length N, io_dtype) may be
+ * NULL for any epilogue. preact (optional, [M,N], ld = ldp) receives the value
+ * before the activation, for the backward of a fused activation. Accumulation
+ * across k and across steps is fp32; the result is rounded once.
+ */
+int cw_gemm_ksteps(int layout, int64_t M, int64_t N, int64_t K, int n_steps,
+                   const void* const* A_steps, int64_t lda,
+                   const void* const* B_steps, int64_t ldb,
+                   const void* bias, int epilogue,
+                   void* C, int64_t ldc,
+                   void* preact, int64_t ldp,
+                   const void* const* addends, int n_addends, int64_t ldadd,
+                   int io_dtype, void* stream);
+
+/* ---- bias / activation backward ---------------------------------------- */
+/*
+ * Number of bytes of scratch cw_colsum / cw_act_bwd_colsum / cw_ln_bwd_partials
+ * need for an [M,N] operand.
+ */
+int64_t cw_colsum_workspace_bytes(int64_t M, int64_t N);
+
+/*
+ * out[N] (fp32) = sum over rows of dY[M,N].
+ * Replaces torch.sum(output_grad, dim=reduce_dim) in _SUMMAbias.backward
+ * (parallel_2d/_operation.py:285-286), _Classifier2D.backward (:414),
+ * _Linear3D.backward (parallel_3d/_operation.py:59). Two deterministic stages
+ * through `workspace` (no atomics).
+ */
+int cw_colsum(int64_t M, int64_t N, const void* dY, int64_t ld, float* out,
+              void* workspace, int64_t workspace_bytes, int io_dtype, void* stream);
+
+/*
+ * dPre[M,N] = dY * act'(preact); optionally dbias[N] (fp32) = column sums of
+ * dPre (dbias may be NULL, then workspace may be NULL). Backward of the fused
+ * activation epilogue of cw_gemm_ksteps; the reference runs it as autograd of
+ * nn.functional.gelu / nn.ReLU (benchmark/gpt2/gpt2.py:117, benchmark/opt/opt.py:200)
+ * followed by _SUMMAbias.backward.
+ */
+int cw_act_bwd_colsum(int activation, int64_t M, int64_t N,
+                      const void* dY, int64_t ld_dy, const void* preact, int64_t ld_pre,
+                      void* dPre, int64_t ld_dpre, float* dbias,
+                      void* workspace, int64_t workspace_bytes, int io_dtype, void* stream);
+
+/* ---- LayerNorm ---------------------------------------------------------- */
+/*
+ * Local partial statistics of x[R,C] (this rank's C of the H hidden columns).
+ *   CW_LN_ONE_PASS: stats[r] = (sum_c x, sum_c x^2)
+ *   CW_LN_TWO_PASS: stats[r] = (sum_c (x-mean[r]), sum_c (x-mean[r])^2); mean == NULL
+ *                   means "first exchange": stats[r] = (sum_c x, 0).
+ * Replaces torch.sum(x), torch.sum(x*x) in LayerNorm2D.forward
+ * (parallel_2d/module.py:144,148) and torch.sum(input_), torch.sum(mu**2) in
+ * _Layernorm3D.forward (parallel_3d/_operation.py:273,275).
+ */
+int cw_ln_partial_stats(int64_t R, int64_t C, const void* x, int64_t ld, int mode,
+                        const float* mean, float* stats, int io_dtype, void* stream);
+
+/*
+ * y = gamma * (x - mean) * rstd + beta from statistics summed over the whole
+ * hidden size H (after the peers' partials were added):
+ *   CW_LN_ONE_PASS: stats[r] = (sum x, sum x^2) over H
+ *   CW_LN_TWO_PASS: stats[r] = (mean, sum (x-mean)^2 over H)
+ * gamma/beta (length C, io_dtype) may be NULL (no affine). mean_rstd[R,2]
+ * (fp32, optional) receives (mean, rstd) for the backward.
+ * Replaces parallel_2d/module.py:145-153,170 + _Layernorm_2D.forward
+ * (parallel_2d/_operation.py:321-324) and parallel_3d/_operation.py:273-281.
+ */
+int cw_ln_normalize(int64_t R, int64_t C, const void* x, int64_t ld, const float* stats,
+                    int mode, int64_t H, float eps, const void* gamma, const void* beta,
+                    void* y, int64_t ldy, float* mean_rstd, int io_dtype, void* stream);
+
+/*
+ * Statistics and normalise in one launch for the case with no peers (H == C):
+ * what LayerNorm2D/3D compute at tensor-parallel size 1.
+ */
+int cw_ln_forward_fused(int64_t R, int64_t C, const void* x, int64_t ld, int mode, float eps,
+                        const void* gamma, const void* beta, void* y, int64_t ldy,
+                        float* mean_rstd, int io_dtype, void* stream);
+
+/*
+ * Backward partials. With g = dY * gamma and xhat = (x - mean) * rstd:
+ *   row_sums[r] = (sum_c g, sum_c g*xhat)                 (fp32 [R,2])
+ *   dgamma[c]   = sum_r dY*xhat, dbeta[c] = sum_r dY      (fp32 [C] each, optional)
+ * Replaces _Layernorm_2D.backward sums (parallel_2d/_operation.py:334,338), the
+ * autograd of torch.addcmul (parallel_2d/module.py:170) and the bias_grad /
+ * weight_grad sums of _Layernorm3D.backward (parallel_3d/_operation.py:294-301).
+ * dgamma == dbeta == NULL skips the column part (and needs no workspace).
+ */
+int cw_ln_bwd_partials(int64_t R, int64_t C, const void* dY, int64_t ld_dy,
+                       const void* x, int64_t ld_x, const float* mean_rstd, const void* gamma,
+                       float* row_sums, float* dgamma, float* dbeta,
+                       void* workspace, int64_t workspace_bytes, int io_dtype, void* stream);
+
+/*
+ * dx = (g - xhat * S2/H - S1/H) * rstd with (S1, S2) = row_sums summed over
+ * the whole hidden size H. Replaces parallel_2d/_operation.py:336-345 and
+ * parallel_3d/_operation.py:303-311.
+ */
+int cw_ln_bwd_dx(int64_t R, int64_t C, const void* dY, int64_t ld_dy,
+                 const void* x, int64_t ld_x, const float* mean_rstd, const void* gamma,
+                 const float* row_sums, int64_t H, void* dx, int64_t ld_dx,
+                 int io_dtype, void* stream);
+
+/* ---- vocab-parallel cross-entropy -------------------------------------- */
+/*
+ * One online pass over this rank's vocabulary slice logits[T,V] (columns
+ * [vocab_start, vocab_start+V) of the full vocabulary):
+ *   out_max[t]    = max_c logits[t,c]
+ *   out_sumexp[t] = sum_c exp(logits[t,c] - out_max[t])
+ *   out_mask[t]   = 1 if targets[t] is outside the slice else 0
+ *   out_pred[t]   = logits[t, targets[t]-vocab_start] as fp32 (0 where masked)
+ * Replaces loss_1d.py:17,23-42,47-49; loss_2d.py:39,45-59,62-63;
+ * loss_3d.py:43,48-60,64-65 (cubework/module/loss/). logits are not modified.
+ */
+int cw_vpce_fwd_local(int64_t T, int64_t V, const void* logits, int64_t ld,
+                      const int64_t* targets, int64_t vocab_start,
+                      float* out_max, float* out_sumexp, float* out_pred, uint8_t* out_mask,
+                      int io_dtype, void* stream);
+
+/*
+ * Combine the n_ranks slices' statistics (row r of *_all is rank r's output of
+ * cw_vpce_fwd_local; they stand for the MAX / SUM / SUM all-reduces of
+ * loss_1d.py:18,44,50):
+ *   gmax = max_r max_r[t];  gsum = sum_r sumexp_r[t] * exp(max_r[t] - gmax)
+ *   loss = log(gsum) - sum_r (mask_r ? 0 : pred_r[t] - gmax)      (loss_1d.py:53)
+ */
+int cw_vpce_finalize(int64_t T, int n_ranks, const float* max_all, const float* sumexp_all,
+                     const float* pred_all, const uint8_t* mask_all,
+                     float* loss, float* gmax, float* gsum, void* stream);
+
+/*
+ * grad[t,c] = (exp(logits[t,c]-gmax[t]) / gsum[t] - [c == target column, in slice]) * dloss
+ * with dloss = dloss_rows[t] * dloss_scale (dloss_rows may be NULL = all ones).
+ * Recomputes the softmax instead of keeping it (loss_1d.py:55-56,61-79).
+ * grad_dtype selects the storage type of grad (CW_BF16 or CW_F32).
+ */
+int cw_vpce_bwd(int64_t T, int64_t V, const void* logits, int64_t ld,
+                const int64_t* targets, int64_t vocab_start,
+                const float* gmax, const float* gsum,
+                const float* dloss_rows, float dloss_scale,
+                void* grad, int64_t ld_grad, int io_dtype, int grad_dtype, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* CUBEWORK_HIP_H */

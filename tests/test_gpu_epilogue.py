@@ -1,0 +1,54 @@
+"""GPU parity of the bias-gradient column sum and the fused-activation
+backward (through the C ABI) against the CPU oracle."""
+import pytest
+import torch
+
+from tests.util import assert_parity, randn
+
+pytestmark = pytest.mark.gpu
+
+DEV = "cuda:0"
+SHAPES = [(8192, 2048), (100, 1000), (33, 8), (5, 7), (1000, 520), (4096, 64)]
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("shape", SHAPES)
+def test_colsum(shape, dtype):
+    import oracle
+    from cubework_amd import ops
+
+    M, N = shape
+    dy = randn((M, N), dtype, 1)
+    got = ops.colsum(dy.to(DEV))
+    want = oracle.colsum(dy)
+    # relative to sqrt(M): the sums are of M unit-variance terms
+    assert_parity(got, want, torch.float32, "colsum", scale=100)
+    # determinism: two runs are bit identical
+    assert torch.equal(got, ops.colsum(dy.to(DEV)))
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("act", [None, "gelu_tanh", "gelu_erf", "relu"])
+@pytest.mark.parametrize("shape", [(1024, 512), (77, 130), (9, 5)])
+def test_act_bwd_colsum(shape, act, dtype):
+    import oracle
+    from cubework_amd import ops
+
+    M, N = shape
+    dy = randn((M, N), dtype, 2)
+    pre = randn((M, N), dtype, 3, std=1.5)
+    dpre, dbias = ops.act_bwd_colsum(act, dy.to(DEV), pre.to(DEV))
+    want_dpre, want_dbias = oracle.act_bwd_colsum(act, dy, pre)
+    assert_parity(dpre, want_dpre, dtype, "dPre", scale=10 if dtype == torch.float32 else 1)
+    assert_parity(dbias, want_dbias, torch.float32, "dbias", scale=200)
+    dpre2, none = ops.act_bwd_colsum(act, dy.to(DEV), pre.to(DEV), want_dbias=False)
+    assert none is None and torch.equal(dpre, dpre2)
+
+
+def test_colsum_padded_rows():
+    import oracle
+    from cubework_amd import ops
+
+    parent = randn((300, 136), torch.bfloat16, 4).to(DEV)
+    view = parent[:, :128]
+    assert_parity(ops.colsum(view), oracle.colsum(view.cpu()), torch.float32, "padded colsum", scale=100)

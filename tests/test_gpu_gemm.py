@@ -1,0 +1,157 @@
+"""GPU parity of cw_gemm_ksteps (through the C ABI) against the CPU oracle.
+
+Bars: <= 1e-2 relative for bf16 I/O with fp32 accumulation, <= 1e-5 relative
+for fp32 (relative to the largest magnitude of the expected result).
+"""
+import pytest
+import torch
+
+from tests.util import assert_parity, randn
+
+pytestmark = pytest.mark.gpu
+
+LAYOUTS = ["NN", "NT", "TN"]
+
+
+def _operands(layout, M, N, K, steps, dtype, seed, pad_a=0, pad_b=0):
+    """Step operands on the CPU; pad_* adds unused columns so that the leading
+    dimension differs from the row length."""
+    a_shape = (K, M) if layout == "TN" else (M, K)
+    b_shape = (N, K) if layout == "NT" else (K, N)
+    A, B = [], []
+    for s in range(steps):
+        a = randn((a_shape[0], a_shape[1] + pad_a), dtype, seed + 10 * s)
+        b = randn((b_shape[0], b_shape[1] + pad_b), dtype, seed + 10 * s + 1, std=0.05)
+        A.append(a[:, :a_shape[1]])
+        B.append(b[:, :b_shape[1]])
+    return A, B
+
+
+def _to_dev(t, pad, dev):
+    """Copy to the device keeping `pad` unused columns behind every row."""
+    if pad == 0:
+        return t.to(dev)
+    parent = torch.zeros((t.shape[0], t.shape[1] + pad), dtype=t.dtype, device=dev)
+    view = parent[:, :t.shape[1]]
+    view.copy_(t)
+    return view
+
+
+def _run(layout, M, N, K, steps, dtype, act=None, bias=True, n_add=0, preact=False, pad_a=0, pad_b=0, seed=0):
+    import oracle
+    from cubework_amd import ops
+
+    A, B = _operands(layout, M, N, K, steps, dtype, seed, pad_a, pad_b)
+    b = randn((N,), dtype, seed + 100, std=0.5) if bias else None
+    adds = [randn((M, N), dtype, seed + 200 + i) for i in range(n_add)]
+    want = oracle.gemm_ksteps(layout, A, B, b, act, adds, return_preact=preact)
+    dev = "cuda:0"
+    Ad = [_to_dev(a, pad_a, dev) for a in A]
+    Bd = [_to_dev(b_, pad_b, dev) for b_ in B]
+    got = ops.gemm_ksteps(layout, Ad, Bd, None if b is None else b.to(dev), act, [t.to(dev) for t in adds],
+                          want_preact=preact)
+    torch.cuda.synchronize()
+    tag = "%s %dx%dx%d steps=%d %s act=%s" % (layout, M, N, K, steps, dtype, act)
+    if preact:
+        assert_parity(got[0], want[0], dtype, tag + " out")
+        assert_parity(got[1], want[1], dtype, tag + " preact")
+    else:
+        assert_parity(got, want, dtype, tag)
+
+
+@pytest.mark.parametrize("layout", LAYOUTS)
+def test_bf16_exact_tiles_small_config(layout):
+    # 128x128 tiles, no guards
+    _run(layout, 256, 384, 192, 2, torch.bfloat16, act=None)
+
+
+@pytest.mark.parametrize("layout", LAYOUTS)
+def test_bf16_exact_tiles_big_config(layout):
+    # 256x256 tiles (>= 128 of them), two k-steps, fused bias + GeLU(tanh)
+    _run(layout, 4096, 2048, 256, 2, torch.bfloat16, act="gelu_tanh")
+
+
+@pytest.mark.parametrize("layout", LAYOUTS)
+@pytest.mark.parametrize("shape", [(300, 200, 100), (257, 264, 72), (1, 8, 8), (129, 1, 3), (64, 130, 520)])
+def test_bf16_ragged(layout, shape):
+    M, N, K = shape
+    _run(layout, M, N, K, 3, torch.bfloat16, act="relu", seed=3)
+
+
+@pytest.mark.parametrize("layout", LAYOUTS)
+def test_bf16_ragged_big_config(layout):
+    # guarded 256x256 path: 4100 x 2056 is not a multiple of the tile
+    _run(layout, 4100, 2056, 136, 2, torch.bfloat16, act="gelu_erf", seed=5)
+
+
+@pytest.mark.parametrize("act", [None, "gelu_tanh", "gelu_erf", "relu"])
+def test_bf16_epilogues_with_preact_and_addends(act):
+    _run("NN", 384, 256, 128, 2, torch.bfloat16, act=act, n_add=2, preact=True, seed=7)
+
+
+def test_bf16_no_bias_no_act():
+    _run("NT", 512, 256, 64, 1, torch.bfloat16, act=None, bias=False, seed=9)
+
+
+@pytest.mark.parametrize("layout", LAYOUTS)
+def test_bf16_padded_leading_dimensions(layout):
+    _run(layout, 256, 256, 128, 2, torch.bfloat16, act=None, pad_a=8, pad_b=16, seed=11)
+    _run(layout, 130, 70, 50, 2, torch.bfloat16, act=None, pad_a=3, pad_b=5, seed=12)
+
+
+@pytest.mark.parametrize("layout", LAYOUTS)
+def test_fp32_exact_and_ragged(layout):
+    _run(layout, 256, 384, 128, 2, torch.float32, act="gelu_tanh", seed=13)
+    _run(layout, 300, 200, 100, 3, torch.float32, act=None, n_add=1, preact=True, seed=14)
+    _run(layout, 7, 5, 3, 1, torch.float32, act="relu", seed=15)
+
+
+def test_fp32_linear1d_col_shape():
+    # BASELINE config 1: x [8,512,1024] fp32, W [4096,1024], b zeros -> F.linear
+    import oracle
+    from cubework_amd import ops
+
+    x = randn((8 * 512, 1024), torch.float32, 0)
+    bound = (6.0 / (1024 + 4096)) ** 0.5
+    g = torch.Generator().manual_seed(1)
+    W = (torch.rand((4096, 1024), generator=g) * 2 - 1) * bound
+    b = torch.zeros(4096)
+    want = torch.nn.functional.linear(x, W, b)
+    got = ops.gemm_ksteps("NT", [x.cuda()], [W.cuda()], b.cuda())
+    assert_parity(got, want, torch.float32, "Linear1D_Col forward")
+    assert_parity(got, oracle.gemm_ksteps("NT", [x], [W], b), torch.float32, "oracle")
+
+
+def test_kstep_sum_equals_concatenated_gemm():
+    # size-independent property at the BASELINE config-2 shape: two k-steps ==
+    # one GEMM over the concatenated operands (both through the HIP path)
+    from cubework_amd import ops
+
+    dev = "cuda:0"
+    A = [randn((8192, 2048), torch.bfloat16, s, device=dev) for s in (0, 1)]
+    B = [randn((2048, 2048), torch.bfloat16, s, std=0.02, device=dev) for s in (2, 3)]
+    bias = randn((2048,), torch.bfloat16, 4, std=0.02, device=dev)
+    two = ops.gemm_ksteps("NN", A, B, bias, "gelu_tanh")
+    one = ops.gemm_ksteps("NN", [torch.cat(A, dim=1)], [torch.cat(B, dim=0)], bias, "gelu_tanh")
+    torch.cuda.synchronize()
+    assert torch.equal(two, one)
+    # and a sampled check of rows against the oracle
+    import oracle
+    rows = torch.tensor([0, 1, 255, 256, 4095, 8191])
+    want = oracle.gemm_ksteps("NN", [a[rows].cpu() for a in A], [b.cpu() for b in B], bias.cpu(), "gelu_tanh")
+    assert_parity(two[rows.to(dev)], want, torch.bfloat16, "config-2 sampled rows")
+
+
+def test_rejects_bad_arguments():
+    from cubework_amd import ops, _lib
+
+    a = torch.zeros((8, 8), dtype=torch.bfloat16, device="cuda:0")
+    with pytest.raises(ValueError):
+        ops.gemm_ksteps("NN", [a], [torch.zeros((4, 8), dtype=torch.bfloat16, device="cuda:0")])
+    with pytest.raises(RuntimeError):
+        ops.gemm_ksteps("NN", [a.cpu()], [a.cpu()])
+    with pytest.raises(TypeError):
+        ops.gemm_ksteps("NN", [a.half()], [a.half()])
+    lib = _lib.load()
+    rc = lib.cw_gemm_ksteps(7, 8, 8, 8, 1, None, 8, None, 8, None, 0, None, 8, None, 0, None, 0, 0, 0, None)
+    assert rc < 0 and b"layout" in lib.cw_last_error()

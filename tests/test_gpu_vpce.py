@@ -1,0 +1,139 @@
+"""GPU parity of the vocab-parallel cross-entropy entry points (through the C
+ABI) against the CPU oracle and against F.cross_entropy on the concatenated
+slices (the reference tests' own oracle, tests/test_1d/check_1d_modules.py:499-523).
+Mask, shifted index and gathered logit must be bit-exact.
+"""
+import pytest
+import torch
+
+from tests.util import assert_parity, randn
+
+pytestmark = pytest.mark.gpu
+
+DEV = "cuda:0"
+
+
+def _targets(T, vocab, seed):
+    g = torch.Generator().manual_seed(seed)
+    return torch.randint(0, vocab, (T,), generator=g, dtype=torch.int64)
+
+
+def _run_all_ranks(T, V, p, dtype, seed, grad_dtype=None, targets=None):
+    """Run every slice through the HIP kernels; compare each with the oracle
+    and the combination with F.cross_entropy."""
+    import oracle
+    from cubework_amd import ops
+
+    full = randn((T, V * p), dtype, seed, std=2.0)
+    t = _targets(T, V * p, seed + 1) if targets is None else targets
+    slices = list(torch.chunk(full, p, dim=-1))
+    stats_got, stats_want = [], []
+    for r, s in enumerate(slices):
+        s_dev = s.contiguous().to(DEV)
+        got = ops.vpce_fwd_local(s_dev, t.to(DEV), r * V)
+        want = oracle.vpce_fwd_local(s, t, r * V)
+        # integer / gather part: bit exact
+        assert torch.equal(got[3].cpu(), want[3]), "mask"
+        assert torch.equal(got[2].cpu(), want[2]), "gathered logit"
+        assert torch.equal(got[0].cpu(), want[0]), "row max"
+        assert_parity(got[1], want[1], torch.float32, "sum exp rank %d" % r, scale=10)
+        stats_got.append(got)
+        stats_want.append(want)
+    stk = lambda lst, k: torch.stack([x[k] for x in lst])  # noqa: E731
+    loss_g, gmax_g, gsum_g = ops.vpce_finalize(*(stk(stats_got, k) for k in range(4)))
+    loss_w, gmax_w, gsum_w = oracle.vpce_finalize(*(stk(stats_want, k) for k in range(4)))
+    assert torch.equal(gmax_g.cpu(), gmax_w)
+    assert_parity(gsum_g, gsum_w, torch.float32, "global sum", scale=10)
+    assert_parity(loss_g, loss_w, torch.float32, "loss", scale=10)
+    # the reference tests' oracle
+    logits_ref = full.float().requires_grad_(True)
+    loss_ref = torch.nn.functional.cross_entropy(logits_ref, t, reduction="none")
+    assert_parity(loss_g, loss_ref.detach(), torch.float32, "loss vs F.cross_entropy", scale=10)
+    dl = torch.linspace(0.5, 1.5, T)
+    loss_ref.backward(dl)
+    gd = grad_dtype or dtype
+    for r, s in enumerate(slices):
+        grad = ops.vpce_bwd(s.contiguous().to(DEV), t.to(DEV), r * V, gmax_g, gsum_g, dl.to(DEV), 1.0, grad_dtype=gd)
+        want = oracle.vpce_bwd(s, t, r * V, gmax_w, gsum_w, dl)
+        assert grad.dtype == gd
+        assert_parity(grad, want, gd, "grad rank %d vs oracle" % r, scale=10 if gd == torch.float32 else 1)
+        ref = logits_ref.grad[:, r * V:(r + 1) * V]
+        assert_parity(grad, ref, gd, "grad rank %d vs autograd" % r, scale=10 if gd == torch.float32 else 1)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("shape", [(64, 1024, 4), (37, 1571 * 8, 2), (16, 100, 4), (5, 7, 3), (130, 4104, 1)])
+def test_vpce_all_ranks(shape, dtype):
+    T, V, p = shape
+    _run_all_ranks(T, V, p, dtype, seed=T + V)
+
+
+def test_vpce_bf16_logits_fp32_grad():
+    _run_all_ranks(32, 2048, 2, torch.bfloat16, seed=3, grad_dtype=torch.float32)
+
+
+def test_vpce_edge_targets():
+    """Targets on the slice borders: start-1, start, end-1, end, 0, V-1."""
+    V, p = 256, 4
+    edge = []
+    for r in range(p):
+        edge += [max(r * V - 1, 0), r * V, (r + 1) * V - 1, min((r + 1) * V, V * p - 1)]
+    edge += [0, V * p - 1]
+    t = torch.tensor(edge, dtype=torch.int64)
+    _run_all_ranks(len(edge), V, p, torch.bfloat16, seed=11, targets=t)
+    _run_all_ranks(len(edge), V, p, torch.float32, seed=12, targets=t)
+
+
+def test_vpce_does_not_modify_logits_and_handles_padding():
+    from cubework_amd import ops
+    import oracle
+
+    T, V = 24, 520
+    parent = randn((T, V + 24), torch.bfloat16, 5, std=2.0).to(DEV)
+    view = parent[:, :V]
+    before = parent.clone()
+    t = _targets(T, 2 * V, 6).to(DEV)
+    got = ops.vpce_fwd_local(view, t, V)
+    want = oracle.vpce_fwd_local(view.cpu(), t.cpu(), V)
+    assert torch.equal(got[2].cpu(), want[2]) and torch.equal(got[3].cpu(), want[3])
+    assert_parity(got[1], want[1], torch.float32, "sumexp", scale=10)
+    loss, gmax, gsum = ops.vpce_finalize(*(g.unsqueeze(0) for g in got))
+    ops.vpce_bwd(view, t, V, gmax, gsum, None, 0.25)
+    torch.cuda.synchronize()
+    assert torch.equal(parent, before)
+
+
+def test_vpce_baseline_shape_properties():
+    """BASELINE config 4 at full size (rank 1 of 4, V_loc = 12568): rows of the
+    softmax gradient sum to zero across the 4 slices; loss equals logsumexp
+    minus the target logit on sampled rows; grad = -dloss*(1-softmax) at the
+    target column."""
+    from cubework_amd import ops
+
+    T, V, p = 8192, 12568, 4
+    t = _targets(T, V * p, 1).to(DEV)
+    slices = [randn((T, V), torch.bfloat16, 10 + r, std=2.0, device=DEV) for r in range(p)]
+    stats = [ops.vpce_fwd_local(s, t, r * V) for r, s in enumerate(slices)]
+    loss, gmax, gsum = ops.vpce_finalize(*(torch.stack([st[k] for st in stats]) for k in range(4)))
+    # exactly one rank owns each target
+    owners = torch.stack([st[3] for st in stats]).to(torch.int32)
+    assert torch.equal((1 - owners).sum(dim=0), torch.ones(T, dtype=torch.int32, device=DEV))
+    rows = torch.arange(0, T, 257, device=DEV)
+    full = torch.cat([s[rows] for s in slices], dim=1).float().cpu()
+    want = torch.logsumexp(full.double(), dim=1) - full.double()[torch.arange(len(rows)), t[rows].cpu()]
+    assert_parity(loss[rows].cpu().double(), want, torch.float32, "loss on sampled rows", scale=10)
+    dl = 1.0 / T
+    total = torch.zeros(T, dtype=torch.float64, device=DEV)
+    for r, s in enumerate(slices):
+        g = ops.vpce_bwd(s, t, r * V, gmax, gsum, None, dl, grad_dtype=torch.float32)
+        total += g.double().sum(dim=1)
+    assert (total.abs() / dl).max().item() < 1e-4
+
+
+def test_vpce_empty():
+    from cubework_amd import ops
+
+    x = torch.zeros((0, 64), dtype=torch.bfloat16, device=DEV)
+    t = torch.zeros((0,), dtype=torch.int64, device=DEV)
+    out = ops.vpce_fwd_local(x, t, 0)
+    assert all(o.numel() == 0 for o in out)

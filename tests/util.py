@@ -1,0 +1,33 @@
+"""Helpers shared by the parity tests."""
+import torch
+
+# Parity bars: relative to the largest magnitude of the expected result.
+TOL = {torch.float32: 1e-5, torch.bfloat16: 1e-2}
+
+
+def rel_err(got: torch.Tensor, want: torch.Tensor) -> float:
+    got = got.detach().to("cpu").to(torch.float64)
+    want = want.detach().to("cpu").to(torch.float64)
+    assert got.shape == want.shape, (got.shape, want.shape)
+    if want.numel() == 0:
+        return 0.0
+    denom = max(want.abs().max().item(), 1e-30)
+    return (got - want).abs().max().item() / denom
+
+
+def assert_parity(got, want, dtype, what="", scale=1.0):
+    assert torch.isfinite(got.detach().float().cpu()).all(), "%s: non-finite values" % what
+    err = rel_err(got, want)
+    tol = TOL[dtype] * scale
+    assert err <= tol, "%s: relative error %.3e above %.1e" % (what, err, tol)
+    return err
+
+
+def randn(shape, dtype, seed, std=1.0, device="cpu"):
+    g = torch.Generator().manual_seed(seed)
+    return (torch.randn(shape, generator=g) * std).to(dtype).to(device)
+
+
+def rand_uniform(shape, dtype, seed, lo, hi, device="cpu"):
+    g = torch.Generator().manual_seed(seed)
+    return (torch.rand(shape, generator=g) * (hi - lo) + lo).to(dtype).to(device)
