@@ -1,407 +1,25 @@
-// SUMMA block GEMM for gfx950: C = act(sum_i op(A_i) op(B_i) + addends + bias),
-// bf16 operands, fp32 accumulation in v_mfma_f32_32x32x16_bf16.
-//
-// Shape of the kernel
-//   - one 256-thread block (4 wavefronts, 2x2) per BM x BN tile of C; a
-//     wavefront owns a (BM/2) x (BN/2) sub-tile as TM x TN MFMA tiles of 32x32
-//     (256x256 block: 4x4 tiles = 256 fp32 accumulators per lane);
-//   - the k loop runs over (step, k) flattened into tiles of 64, so the software
-//     pipeline does not drain where one k-step's operands end and the next
-//     step's (a different allocation) begin;
-//   - global -> registers -> LDS with the next tile's loads in flight during the
-//     current tile's MFMAs, two LDS stages, one barrier per tile;
-//   - both operands sit in LDS as [row][k] with k contiguous (pitch 72 elements
-//     = 144 bytes, which spreads eight consecutive rows over all banks for the
-//     16-byte fragment reads). An operand whose memory has k as the slow index
-//     (B of NN, both of TN) is transposed in registers on its way to LDS: each
-//     thread owns an 8x8 block;
-//   - the MFMA is issued with the B fragment as srcA and the A fragment as
-//     srcB, so a lane ends up with four consecutive output COLUMNS per register
-//     quad; the epilogue packs them and stages the tile through LDS so that
-//     global stores are whole rows of the tile;
-//   - workgroup ids are remapped so that the 8 XCDs (ids are dealt round-robin
-//     to them) each work on a compact patch of tiles and share A/B panels in
-//     their own L2.
-#include "cw_common.h"
-#include "gemm.h"
+// bf16 block GEMM: choice of tile configuration and kernel variant.
+#include "gemm_bf16_kernel.h"
 
 namespace cw {
 
-namespace {
-
-typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
-typedef float f32x16_t __attribute__((ext_vector_type(16)));
-
-constexpr int kBK = 64;         // k extent of an LDS tile
-constexpr int kPitch = 72;      // elements per LDS row (64 + 8 padding)
-constexpr int kThreads = 256;
-
-// Eight consecutive bf16 of row r starting at column c of a row-major
-// [rmax][cmax] operand; zero outside. vec_ok: rows are 16-byte aligned.
-__device__ __forceinline__ uint4 load8_guarded(const uint16_t* __restrict__ base, int64_t ld, int r, int c, int rmax,
-                                               int cmax, bool vec_ok) {
-    uint4 out = make_uint4(0u, 0u, 0u, 0u);
-    if (r >= rmax || c >= cmax) return out;
-    const uint16_t* p = base + (int64_t)r * ld + c;
-    if (vec_ok && c + 8 <= cmax) return *reinterpret_cast<const uint4*>(p);
-    uint32_t w[4] = {0u, 0u, 0u, 0u};
-#pragma unroll
-    for (int e = 0; e < 8; ++e)
-        if (c + e < cmax) w[e >> 1] |= (uint32_t)p[e] << ((e & 1) * 16);
-    return make_uint4(w[0], w[1], w[2], w[3]);
-}
-
-// Global -> registers for a ROWS x 64 operand tile.
-//   TRANS == false: memory is [rows][k] (k contiguous). 16-byte chunk c of the
-//     tile is (row c/8, k-chunk c%8); thread handles chunks tid, tid+256, ...
-//   TRANS == true : memory is [k][rows] (rows contiguous). Thread owns the 8x8
-//     block (k-block tid%8, row-block tid/8) and loads its 8 k-rows.
-template <int ROWS, bool TRANS, bool GUARD>
-__device__ __forceinline__ void tile_g2r(uint4 (&reg)[8], const uint16_t* __restrict__ base, int64_t ld, int row0,
-                                         int k0, int rmax, int kmax, int tid, bool vec_ok) {
-    if constexpr (!TRANS) {
-        constexpr int CH = ROWS * 8 / kThreads;
-#pragma unroll
-        for (int it = 0; it < CH; ++it) {
-            const int c = it * kThreads + tid;
-            const int row = row0 + (c >> 3);
-            const int k = k0 + (c & 7) * 8;
-            if constexpr (GUARD)
-                reg[it] = load8_guarded(base, ld, row, k, rmax, kmax, vec_ok);
-            else
-                reg[it] = *reinterpret_cast<const uint4*>(base + (int64_t)row * ld + k);
-        }
-    } else {
-        const int kb = tid & 7;
-        const int rb = tid >> 3;
-        if (rb < ROWS / 8) {
-#pragma unroll
-            for (int j = 0; j < 8; ++j) {
-                const int k = k0 + kb * 8 + j;
-                const int row = row0 + rb * 8;
-                if constexpr (GUARD)
-                    reg[j] = load8_guarded(base, ld, k, row, kmax, rmax, vec_ok);
-                else
-                    reg[j] = *reinterpret_cast<const uint4*>(base + (int64_t)k * ld + row);
-            }
-        }
-    }
-}
-
-__device__ __forceinline__ uint32_t pick_lo(uint32_t a, uint32_t b) { return (a & 0xffffu) | (b << 16); }
-__device__ __forceinline__ uint32_t pick_hi(uint32_t a, uint32_t b) { return (a >> 16) | (b & 0xffff0000u); }
-
-// Registers -> LDS tile [ROWS][kPitch].
-template <int ROWS, bool TRANS>
-__device__ __forceinline__ void tile_r2s(const uint4 (&reg)[8], uint16_t* __restrict__ lds, int tid) {
-    if constexpr (!TRANS) {
-        constexpr int CH = ROWS * 8 / kThreads;
-#pragma unroll
-        for (int it = 0; it < CH; ++it) {
-            const int c = it * kThreads + tid;
-            *reinterpret_cast<uint4*>(lds + (c >> 3) * kPitch + (c & 7) * 8) = reg[it];
-        }
-    } else {
-        const int kb = tid & 7;
-        const int rb = tid >> 3;
-        if (rb < ROWS / 8) {
-            // reg[j] = 8 rows' values at k-row j; dword d of it = rows (2d, 2d+1).
-            // out(row i) dword d' = (k = 2d', 2d'+1) of row i.
-#pragma unroll
-            for (int i = 0; i < 8; ++i) {
-                uint32_t w[4];
-#pragma unroll
-                for (int d = 0; d < 4; ++d) {
-                    const uint4& ra = reg[2 * d];
-                    const uint4& rb4 = reg[2 * d + 1];
-                    const uint32_t a = (i >> 1) == 0 ? ra.x : (i >> 1) == 1 ? ra.y : (i >> 1) == 2 ? ra.z : ra.w;
-                    const uint32_t b = (i >> 1) == 0 ? rb4.x : (i >> 1) == 1 ? rb4.y : (i >> 1) == 2 ? rb4.z : rb4.w;
-                    w[d] = (i & 1) ? pick_hi(a, b) : pick_lo(a, b);
-                }
-                *reinterpret_cast<uint4*>(lds + (rb * 8 + i) * kPitch + kb * 8) = make_uint4(w[0], w[1], w[2], w[3]);
-            }
-        }
-    }
-}
-
-template <int EPI>
-__device__ __forceinline__ float epi_act(float x) {
-    if constexpr (EPI == CW_EPI_BIAS_GELU_TANH) return gelu_tanh(x);
-    if constexpr (EPI == CW_EPI_BIAS_GELU_ERF) return gelu_erf(x);
-    if constexpr (EPI == CW_EPI_BIAS_RELU) return x > 0.0f ? x : 0.0f;
-    return x;
-}
-
-__device__ __forceinline__ void load4_bf16(const uint16_t* __restrict__ p, int n_valid, bool vec_ok, float (&v)[4]) {
-    if (vec_ok && n_valid >= 4) {
-        const uint2 u = *reinterpret_cast<const uint2*>(p);
-        v[0] = __uint_as_float(u.x << 16);
-        v[1] = __uint_as_float(u.x & 0xffff0000u);
-        v[2] = __uint_as_float(u.y << 16);
-        v[3] = __uint_as_float(u.y & 0xffff0000u);
-    } else {
-#pragma unroll
-        for (int e = 0; e < 4; ++e) v[e] = e < n_valid ? bf16_bits_to_f32(p[e]) : 0.0f;
-    }
-}
-
-// Stage a wavefront's sub-tile (values already final, fp32) into the block's
-// LDS C tile as bf16 and write the tile out row by row.
-// LDS C tile: [BM][BN + 4] bf16 (pitch = 8 bytes mod 128: the 8-byte writes of
-// 16 consecutive rows land in 16 different bank pairs).
-template <int BM, int BN>
-__device__ __forceinline__ void tile_store(uint16_t* __restrict__ lds_c, uint16_t* __restrict__ C, int64_t ldc,
-                                           int m0, int n0, int M, int N, int tid, bool vec_ok) {
-    constexpr int CP = BN + 4;
-    constexpr int QUADS_PER_ROW = BN / 4;
-    constexpr int TOTAL = BM * QUADS_PER_ROW;
-#pragma unroll 4
-    for (int q = tid; q < TOTAL; q += kThreads) {
-        const int r = q / QUADS_PER_ROW;
-        const int cq = q % QUADS_PER_ROW;
-        const int row = m0 + r;
-        const int col = n0 + cq * 4;
-        if (row < M && col < N) {
-            const uint2 v = *reinterpret_cast<const uint2*>(lds_c + r * CP + cq * 4);
-            uint16_t* dst = C + (int64_t)row * ldc + col;
-            if (vec_ok && col + 4 <= N) {
-                *reinterpret_cast<uint2*>(dst) = v;
-            } else {
-                const uint16_t e[4] = {(uint16_t)(v.x & 0xffffu), (uint16_t)(v.x >> 16), (uint16_t)(v.y & 0xffffu),
-                                       (uint16_t)(v.y >> 16)};
-#pragma unroll
-                for (int i = 0; i < 4; ++i)
-                    if (col + i < N) dst[i] = e[i];
-            }
-        }
-    }
-}
-
-template <int BM, int BN, bool TRANS_A, bool TRANS_B, bool GUARD, int EPI>
-__global__ __launch_bounds__(kThreads) void gemm_bf16_kernel(const GemmArgs args) {
-    constexpr int WTM = BM / 2, WTN = BN / 2;  // wavefront sub-tile
-    constexpr int TM = WTM / 32, TN = WTN / 32;
-    constexpr int A_ELEMS = BM * kPitch, B_ELEMS = BN * kPitch;
-    constexpr int STAGE = A_ELEMS + B_ELEMS;
-    extern __shared__ __attribute__((aligned(16))) uint16_t lds[];
-
-    const int tid = threadIdx.x;
-    const int lane = tid & 63;
-    const int wave = tid >> 6;
-    const int wm = wave >> 1, wn = wave & 1;
-
-    const int M = args.M, N = args.N, K = args.K;
-    const int tiles_m = (M + BM - 1) / BM;
-    const int tiles_n = (N + BN - 1) / BN;
-    const int total = tiles_m * tiles_n;
-    // XCD-aware remap: ids pid, pid+8, ... share an XCD; give each XCD a
-    // contiguous range of tile ids, and order tile ids in groups of 8 tile rows.
-    int tile;
-    {
-        const int pid = blockIdx.x;
-        const int per_xcd = (total + 7) / 8;
-        tile = (pid & 7) * per_xcd + (pid >> 3);
-        if (tile >= total) return;
-    }
-    constexpr int GROUP_M = 8;
-    const int group = tile / (GROUP_M * tiles_n);
-    const int first_m = group * GROUP_M;
-    const int gsz = (tiles_m - first_m) < GROUP_M ? (tiles_m - first_m) : GROUP_M;
-    const int in_group = tile - group * GROUP_M * tiles_n;
-    const int tile_m = first_m + in_group % gsz;
-    const int tile_n = in_group / gsz;
-    const int m0 = tile_m * BM, n0 = tile_n * BN;
-
-    const int kt_per_step = (K + kBK - 1) / kBK;
-    const int KT = kt_per_step * args.n_steps;
-    const bool vec_a = args.vec_a != 0, vec_b = args.vec_b != 0;
-
-    f32x16_t acc[TM][TN];
-#pragma unroll
-    for (int i = 0; i < TM; ++i)
-#pragma unroll
-        for (int j = 0; j < TN; ++j)
-#pragma unroll
-            for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.0f;
-
-    uint4 ra[8], rb[8];
-    // fragment read offsets (elements) within a stage
-    const int a_frag = (wm * WTM + (lane & 31)) * kPitch + (lane >> 5) * 8;
-    const int b_frag = A_ELEMS + (wn * WTN + (lane & 31)) * kPitch + (lane >> 5) * 8;
-
-    auto issue_loads = [&](int kt) {
-        const int step = kt / kt_per_step;
-        const int k0 = (kt - step * kt_per_step) * kBK;
-        const uint16_t* Ap = reinterpret_cast<const uint16_t*>(args.A[step]);
-        const uint16_t* Bp = reinterpret_cast<const uint16_t*>(args.B[step]);
-        tile_g2r<BM, TRANS_A, GUARD>(ra, Ap, args.lda, m0, k0, M, K, tid, vec_a);
-        tile_g2r<BN, TRANS_B, GUARD>(rb, Bp, args.ldb, n0, k0, N, K, tid, vec_b);
-    };
-    auto commit_loads = [&](int stage) {
-        uint16_t* s = lds + stage * STAGE;
-        tile_r2s<BM, TRANS_A>(ra, s, tid);
-        tile_r2s<BN, TRANS_B>(rb, s + A_ELEMS, tid);
-    };
-
-    if (KT > 0) {
-        issue_loads(0);
-        commit_loads(0);
-    }
-    __syncthreads();
-
-    for (int kt = 0; kt < KT; ++kt) {
-        const int cur = kt & 1;
-        if (kt + 1 < KT) issue_loads(kt + 1);
-        const uint16_t* s = lds + cur * STAGE;
-#pragma unroll
-        for (int ks = 0; ks < kBK / 16; ++ks) {
-            bf16x8_t af[TM], bfr[TN];
-#pragma unroll
-            for (int i = 0; i < TM; ++i)
-                af[i] = *reinterpret_cast<const bf16x8_t*>(s + a_frag + i * 32 * kPitch + ks * 16);
-#pragma unroll
-            for (int j = 0; j < TN; ++j)
-                bfr[j] = *reinterpret_cast<const bf16x8_t*>(s + b_frag + j * 32 * kPitch + ks * 16);
-#pragma unroll
-            for (int i = 0; i < TM; ++i)
-#pragma unroll
-                for (int j = 0; j < TN; ++j)
-                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(bfr[j], af[i], acc[i][j], 0, 0, 0);
-        }
-        if (kt + 1 < KT) commit_loads(cur ^ 1);
-        __syncthreads();
-    }
-
-    // ---- epilogue -------------------------------------------------------
-    // acc[i][j][v]: row  m = m0 + wm*WTM + i*32 + (lane & 31)
-    //               col  n = n0 + wn*WTN + j*32 + 8*(v/4) + 4*(lane>>5) + (v%4)
-    constexpr int CP = BN + 4;
-    uint16_t* lds_c = lds;  // the operand stages are dead after the last barrier
-    const int row_l = wm * WTM + (lane & 31);
-    const int col_l = wn * WTN + 4 * (lane >> 5);
-    const bool vec_c = args.vec_c != 0;
-    const uint16_t* bias = reinterpret_cast<const uint16_t*>(args.bias);
-
-    if (args.n_addends > 0 || (EPI != CW_EPI_NONE && bias != nullptr)) {
-#pragma unroll
-        for (int j = 0; j < TN; ++j)
-#pragma unroll
-            for (int g = 0; g < 4; ++g) {
-                const int ncol = n0 + col_l + j * 32 + 8 * g;
-                float bv[4] = {0.0f, 0.0f, 0.0f, 0.0f};
-                if (EPI != CW_EPI_NONE && bias != nullptr && ncol < N)
-                    load4_bf16(bias + ncol, N - ncol, args.vec_bias != 0, bv);
-#pragma unroll
-                for (int i = 0; i < TM; ++i) {
-                    const int mrow = m0 + row_l + i * 32;
-                    float add[4] = {bv[0], bv[1], bv[2], bv[3]};
-                    if (args.n_addends > 0 && mrow < M && ncol < N) {
-                        for (int a = 0; a < args.n_addends; ++a) {
-                            float t[4];
-                            load4_bf16(reinterpret_cast<const uint16_t*>(args.addend[a]) + (int64_t)mrow * args.ldadd + ncol,
-                                       N - ncol, args.vec_add != 0, t);
-#pragma unroll
-                            for (int e = 0; e < 4; ++e) add[e] += t[e];
-                        }
-                    }
-#pragma unroll
-                    for (int e = 0; e < 4; ++e) acc[i][j][4 * g + e] += add[e];
-                }
-            }
-    }
-
-    auto stage_tile = [&](bool activated) {
-#pragma unroll
-        for (int i = 0; i < TM; ++i)
-#pragma unroll
-            for (int j = 0; j < TN; ++j)
-#pragma unroll
-                for (int g = 0; g < 4; ++g) {
-                    float v[4];
-#pragma unroll
-                    for (int e = 0; e < 4; ++e) {
-                        const float x = acc[i][j][4 * g + e];
-                        v[e] = activated ? epi_act<EPI>(x) : x;
-                    }
-                    uint2 p;
-                    p.x = pack_bf16x2(v[0], v[1]);
-                    p.y = pack_bf16x2(v[2], v[3]);
-                    *reinterpret_cast<uint2*>(lds_c + (row_l + i * 32) * CP + col_l + j * 32 + 8 * g) = p;
-                }
-    };
-
-    if (args.preact != nullptr) {
-        stage_tile(false);
-        __syncthreads();
-        tile_store<BM, BN>(lds_c, reinterpret_cast<uint16_t*>(args.preact), args.ldp, m0, n0, M, N, tid,
-                           args.vec_p != 0);
-        __syncthreads();
-    }
-    stage_tile(true);
-    __syncthreads();
-    tile_store<BM, BN>(lds_c, reinterpret_cast<uint16_t*>(args.C), args.ldc, m0, n0, M, N, tid, vec_c);
-}
-
-template <int BM, int BN>
-constexpr size_t lds_bytes() {
-    const size_t stages = 2u * (BM + BN) * kPitch * sizeof(uint16_t);
-    const size_t ctile = (size_t)BM * (BN + 4) * sizeof(uint16_t);
-    return stages > ctile ? stages : ctile;
-}
-
-template <int BM, int BN, bool TA, bool TB, bool GUARD, int EPI>
-int launch_cfg(const GemmArgs& args, hipStream_t s) {
-    auto kern = gemm_bf16_kernel<BM, BN, TA, TB, GUARD, EPI>;
-    constexpr size_t lds = lds_bytes<BM, BN>();
-    static_assert(lds <= 160 * 1024, "LDS tile does not fit the CU");
-    if (lds > 48 * 1024) {
-        hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-        if (e != hipSuccess) return fail(CW_ERR_LAUNCH, "hipFuncSetAttribute(gemm_bf16): %s", hipGetErrorString(e));
-    }
-    const int tiles = ((args.M + BM - 1) / BM) * ((args.N + BN - 1) / BN);
-    const int grid = ((tiles + 7) / 8) * 8;
-    hipLaunchKernelGGL(kern, dim3(grid), dim3(kThreads), lds, s, args);
-    return check_launch("gemm_bf16_kernel");
-}
-
-template <int BM, int BN, bool TA, bool TB, bool GUARD>
-int launch_epi(const GemmArgs& args, int epilogue, hipStream_t s) {
-    switch (epilogue) {
-        case CW_EPI_NONE: return launch_cfg<BM, BN, TA, TB, GUARD, CW_EPI_NONE>(args, s);
-        case CW_EPI_BIAS: return launch_cfg<BM, BN, TA, TB, GUARD, CW_EPI_BIAS>(args, s);
-        case CW_EPI_BIAS_GELU_TANH: return launch_cfg<BM, BN, TA, TB, GUARD, CW_EPI_BIAS_GELU_TANH>(args, s);
-        case CW_EPI_BIAS_GELU_ERF: return launch_cfg<BM, BN, TA, TB, GUARD, CW_EPI_BIAS_GELU_ERF>(args, s);
-        case CW_EPI_BIAS_RELU: return launch_cfg<BM, BN, TA, TB, GUARD, CW_EPI_BIAS_RELU>(args, s);
-        default: return fail(CW_ERR_INVALID, "cw_gemm_ksteps: bad epilogue %d", epilogue);
-    }
-}
-
-template <int BM, int BN, bool GUARD>
-int launch_layout(const GemmArgs& args, int layout, int epilogue, hipStream_t s) {
-    switch (layout) {
-        case CW_NN: return launch_epi<BM, BN, false, true, GUARD>(args, epilogue, s);
-        case CW_NT: return launch_epi<BM, BN, false, false, GUARD>(args, epilogue, s);
-        case CW_TN: return launch_epi<BM, BN, true, true, GUARD>(args, epilogue, s);
-        default: return fail(CW_ERR_INVALID, "cw_gemm_ksteps: bad layout %d", layout);
-    }
-}
-
-}  // namespace
-
 int gemm_bf16_launch(const GemmArgs& args, int layout, int epilogue, hipStream_t s) {
-    const bool all_vec = args.vec_a && args.vec_b && args.vec_c && (args.preact == nullptr || args.vec_p) &&
+    // the unguarded kernels address operands with 32-bit byte offsets
+    const int64_t max_dim = args.M > args.N ? (args.M > args.K ? args.M : args.K) : (args.N > args.K ? args.N : args.K);
+    const bool fits32 = (max_dim + 64) * (args.lda > args.ldb ? args.lda : args.ldb) * 2 < ((int64_t)1 << 32);
+    const bool all_vec = fits32 && args.vec_a && args.vec_b && args.vec_c && (args.preact == nullptr || args.vec_p) &&
                          (args.bias == nullptr || args.vec_bias) && (args.n_addends == 0 || args.vec_add);
     // Large problems: 256x256 tiles (one per CU at 8192x2048). Small ones: 128x128.
     const int64_t tiles256 = (int64_t)((args.M + 255) / 256) * ((args.N + 255) / 256);
     const bool big = tiles256 >= 128;
-    if (big) {
-        const bool exact = all_vec && (args.M % 256) == 0 && (args.N % 256) == 0 && (args.K % kBK) == 0;
-        return exact ? launch_layout<256, 256, false>(args, layout, epilogue, s)
-                     : launch_layout<256, 256, true>(args, layout, epilogue, s);
+    const int tile = big ? 256 : 128;
+    const bool exact = all_vec && (args.M % tile) == 0 && (args.N % tile) == 0 && (args.K % gemm_bf16::kBK) == 0;
+    switch (layout) {
+        case CW_NN: return gemm_bf16_launch_nn(args, epilogue, big, exact, s);
+        case CW_NT: return gemm_bf16_launch_nt(args, epilogue, big, exact, s);
+        case CW_TN: return gemm_bf16_launch_tn(args, epilogue, big, exact, s);
+        default: return fail(CW_ERR_INVALID, "cw_gemm_ksteps: bad layout %d", layout);
     }
-    const bool exact = all_vec && (args.M % 128) == 0 && (args.N % 128) == 0 && (args.K % kBK) == 0;
-    return exact ? launch_layout<128, 128, false>(args, layout, epilogue, s)
-                 : launch_layout<128, 128, true>(args, layout, epilogue, s);
 }
 
 }  // namespace cw

@@ -25,7 +25,7 @@ Precision convention for bf16 inputs: evaluate the reference formulas in fp32
 """
 from .summa import (gemm_ksteps, summa_ab_rank, summa_abt_rank, summa_atb_rank, summa_ab_reference_dtype,  # noqa: F401
                     activation, activation_grad, act_bwd_colsum, colsum)
-from .layernorm import (ln2d_partial_stats, ln2d_normalize, ln2d_backward_partials, ln2d_backward_dx,  # noqa: F401
+from .layernorm import (ln2d_partial_stats, ln2d_mean_rstd, ln2d_normalize, ln2d_backward_partials, ln2d_backward_dx,  # noqa: F401
                         ln3d_forward, ln3d_backward, ln_forward_full, ln_backward_full)
 from .vpce import vpce_fwd_local, vpce_finalize, vpce_bwd, vpce_reference_full  # noqa: F401
 from . import grid  # noqa: F401
