@@ -1,0 +1,256 @@
+#!/usr/bin/env python3
+"""bench.py — the Linear2D per-rank block GEMM on one MI355X, next to the CPU path.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W]
+
+A "step" is one pass of the hot path over one batch of synthetic input: rank
+(0, 1) of a q = 2 SUMMA grid computing
+    out[8192, 2048] = GeLU_tanh(A_0 B_0 + A_1 B_1 + bias)        (bf16, fp32 accumulation)
+with the operands a row/column broadcast would deliver already resident in HBM
+(BASELINE.json configs[1]; 137,438,953,472 FLOP per step). One step is one call
+of cw_gemm_ksteps through the C ABI = one kernel launch.
+
+Prints ONE JSON line. `value` is TFLOP/s over the timed region (wall clock
+around K steps, synchronised on both sides). `roofline` prices the GEMM kernel
+against the MI355X dense bf16 MFMA peak with the average launch duration from
+HIP events on the launch stream. `aux` reports the bandwidth-bound kernels of
+the same path (LayerNorm2D, vocab-parallel CE; BASELINE.json configs[2], [3])
+against the 8 TB/s HBM peak, on buffers rotated through > 512 MiB so that the
+256 MiB Infinity Cache cannot serve them. `cpu_baseline` times the reference's
+CPU path (torch, gloo, world size 1) restated by oracle/ on the host cores, on
+a bounded sample of the same workload.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+MFMA_BF16_PEAK_TFLOPS = 2516.6  # 256 CU x 2.4 GHz x 4096 FLOP/clk/CU, dense
+HBM_PEAK_GBPS = 8000.0
+
+M, N, K, STEPS_K = 8192, 2048, 2048, 2
+GEMM_FLOP = 2 * M * N * K * STEPS_K
+
+
+def _seeded(shape, seed, std, dtype):
+    import torch
+    g = torch.Generator().manual_seed(seed)
+    return (torch.randn(shape, generator=g) * std).to(dtype)
+
+
+def make_gemm_inputs(n_sets, device):
+    """Seeded synthetic operands: A_i ~ N(0,1), B_i ~ N(0,0.02), bias ~ N(0,0.02), generated on the
+    CPU, rounded to bf16, then copied to the device."""
+    import torch
+    sets = []
+    for s in range(n_sets):
+        A = [_seeded((M, K), 1000 * s + i, 1.0, torch.bfloat16).to(device) for i in range(STEPS_K)]
+        B = [_seeded((K, N), 1000 * s + 10 + i, 0.02, torch.bfloat16).to(device) for i in range(STEPS_K)]
+        sets.append((A, B))
+    bias = _seeded((N,), 7, 0.02, torch.bfloat16).to(device)
+    return sets, bias
+
+
+def event_time_us(fn, iters, warmup):
+    """Average duration of fn() per call from events on the current stream."""
+    import torch
+    for _ in range(warmup):
+        fn()
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for _ in range(iters):
+        fn()
+    e1.record()
+    torch.cuda.synchronize()
+    return e0.elapsed_time(e1) * 1e3 / iters
+
+
+def bench_bandwidth_kernels(device):
+    """LayerNorm2D (config 3) and vocab-parallel CE (config 4) kernels: algorithmic
+    bytes per launch / average launch duration. Each call below is one C-ABI
+    entry point; outputs are preallocated by the wrappers per call (torch's
+    caching allocator, no device malloc in the loop after warm-up)."""
+    import torch
+    from cubework_amd import ops
+
+    out = {}
+    R, C, H = 16384, 1024, 2048
+    nb = 17  # 17 x 32 MiB = 544 MiB of distinct activations
+    xs = [_seeded((R, C), 100 + i, 1.0, torch.bfloat16).to(device) for i in range(nb)]
+    dys = [_seeded((R, C), 200 + i, 1.0, torch.bfloat16).to(device) for i in range(nb)]
+    g = torch.Generator().manual_seed(3)
+    gamma = (torch.rand(C, generator=g) * 0.2 + 0.9).to(torch.bfloat16).to(device)
+    beta = _seeded((C,), 4, 0.02, torch.bfloat16).to(device)
+    peer = _seeded((R, C), 5, 1.0, torch.bfloat16).to(device)
+    stats = ops.ln_partial_stats(xs[0]) + ops.ln_partial_stats(peer)
+    _, mr = ops.ln_normalize(xs[0], stats, H, 1e-5, gamma, beta)
+    rs = ops.ln_bwd_partials(dys[0], xs[0], mr, gamma)[0] * 2
+    i = [0]
+
+    def rot(lst):
+        i[0] += 1
+        return lst[i[0] % len(lst)]
+
+    cases = [
+        ("ln_partial_stats", 33554432 + 131072, lambda: ops.ln_partial_stats(rot(xs))),
+        ("ln_normalize", 2 * 33554432 + 2 * 131072 + 4096, lambda: ops.ln_normalize(rot(xs), stats, H, 1e-5, gamma, beta)),
+        ("ln_bwd_partials", 2 * 33554432 + 2 * 131072 + 8192, lambda: ops.ln_bwd_partials(rot(dys), xs[i[0] % nb], mr, gamma)),
+        ("ln_bwd_dx", 3 * 33554432 + 2 * 131072 + 2048, lambda: ops.ln_bwd_dx(rot(dys), xs[i[0] % nb], mr, rs, H, gamma)),
+    ]
+    for name, nbytes, fn in cases:
+        us = event_time_us(fn, 51, 6)
+        out[name] = {"us": round(us, 2), "GBps": round(nbytes / us / 1e3, 1), "frac": round(nbytes / us / 1e3 / HBM_PEAK_GBPS, 3),
+                     "bytes": nbytes}
+    del xs, dys
+    T, V, V0 = 8192, 12568, 12568
+    lg = [_seeded((T, V), 300 + k, 2.0, torch.bfloat16).to(device) for k in range(3)]  # 3 x 196 MiB
+    tg = torch.randint(0, 50272, (T,), generator=torch.Generator().manual_seed(9)).to(device)
+    st = ops.vpce_fwd_local(lg[0], tg, V0)
+    loss, gmax, gsum = ops.vpce_finalize(*(s.unsqueeze(0) for s in st))
+    cases = [
+        ("vpce_fwd_local", T * V * 2 + T * 8 + 4 * T * 4, lambda: ops.vpce_fwd_local(rot(lg), tg, V0)),
+        ("vpce_bwd_bf16_grad", 2 * T * V * 2 + T * 8 + 2 * T * 4, lambda: ops.vpce_bwd(rot(lg), tg, V0, gmax, gsum, None, 1.0 / T)),
+        ("vpce_bwd_fp32_grad", T * V * 2 + T * V * 4 + T * 8 + 2 * T * 4,
+         lambda: ops.vpce_bwd(rot(lg), tg, V0, gmax, gsum, None, 1.0 / T, grad_dtype=torch.float32)),
+    ]
+    for name, nbytes, fn in cases:
+        us = event_time_us(fn, 15, 3)
+        out[name] = {"us": round(us, 2), "GBps": round(nbytes / us / 1e3, 1), "frac": round(nbytes / us / 1e3 / HBM_PEAK_GBPS, 3),
+                     "bytes": nbytes}
+    return out
+
+
+def cpu_baseline():
+    """The reference's CPU path (torch on gloo, world size 1) for the same
+    workload, through the oracle's restatement of _SUMMA_AB.forward +
+    _SUMMAbias.forward + GeLU in the tensors' own dtype, on a bounded sample
+    of the rows (the k loop and the widths are the full ones)."""
+    import torch
+    import torch.distributed as dist
+    import oracle
+
+    inited = False
+    try:
+        if not dist.is_initialized():
+            import socket
+            s = socket.socket()
+            s.bind(("127.0.0.1", 0))
+            port = s.getsockname()[1]
+            s.close()
+            dist.init_process_group("gloo", init_method="tcp://127.0.0.1:%d" % port, rank=0, world_size=1)
+            inited = True
+    except Exception:  # the baseline still runs without the (unused at world size 1) group
+        inited = False
+    threads = torch.get_num_threads()
+
+    def run(rows, iters):
+        A = [_seeded((rows, K), i, 1.0, torch.bfloat16) for i in range(STEPS_K)]
+        B = [_seeded((K, N), 10 + i, 0.02, torch.bfloat16) for i in range(STEPS_K)]
+        bias = _seeded((N,), 7, 0.02, torch.bfloat16)
+        f = lambda: torch.nn.functional.gelu(oracle.summa_ab_reference_dtype(A, B, bias), approximate="tanh")  # noqa: E731
+        f()
+        t0 = time.perf_counter()
+        for _ in range(iters):
+            f()
+        return (time.perf_counter() - t0) / iters
+
+    rows = 1024
+    t = run(rows, 1)
+    # grow the sample to the full row count if that stays within ~15 s of CPU work
+    per_row = t / rows
+    if per_row * M * 3 <= 15.0:
+        rows = M
+    else:
+        rows = max(256, min(M, int(15.0 / (3 * per_row)) // 256 * 256))
+    iters = max(2, min(10, int(12.0 / max(per_row * rows, 1e-6))))
+    t = run(rows, iters)
+    if inited:
+        dist.destroy_process_group()
+    flop = 2.0 * rows * N * K * STEPS_K
+    return {"value": round(flop / t / 1e12, 4), "unit": "TFLOP/s", "cores": threads, "kind": "port",
+            "sample": "%d of %d rows, full K=%dx%d steps and N=%d, bf16 addmm per k-step + bias + GeLU(tanh) as "
+                      "parallel_2d/_operation.py:41-47,273 runs it on CPU tensors; %d timed passes, %.3f s each; "
+                      "os.cpu_count()=%d" % (rows, M, K, STEPS_K, N, iters, t, os.cpu_count())}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--no-aux", action="store_true", help="skip the LayerNorm / CE kernels")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
+    args = ap.parse_args()
+    if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
+        sys.stderr.write("bench.py measures one rank's share on ONE GPU; --gpus N with N > 1 is not part of this "
+                         "build (no collectives, no sharding across GPUs).\n")
+        sys.exit(2)
+
+    import torch
+    from cubework_amd import _lib, ops
+
+    if not torch.cuda.is_available():
+        sys.stderr.write("bench.py needs an MI355X; there is no CPU fallback of the product path.\n")
+        sys.exit(3)
+    device = torch.device("cuda", 0)
+    torch.cuda.set_device(device)
+    lib = _lib.load()
+    arch = lib.cw_device_arch().decode()
+
+    n_sets = 3  # 3 x 80 MiB of operands rotate so that no step finds its inputs in the Infinity Cache
+    sets, bias = make_gemm_inputs(n_sets, device)
+    outs = [torch.empty((M, N), dtype=torch.bfloat16, device=device) for _ in range(n_sets)]
+    it = [0]
+
+    def step():
+        A, B = sets[it[0] % n_sets]
+        ops.gemm_ksteps("NN", A, B, bias, "gelu_tanh", out=outs[it[0] % n_sets])
+        it[0] += 1
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    t0 = time.perf_counter()
+    e0.record()
+    for _ in range(args.steps):
+        step()
+    e1.record()
+    torch.cuda.synchronize()
+    t1 = time.perf_counter()
+    ms_per_step = (t1 - t0) * 1e3 / args.steps
+    kernel_us = e0.elapsed_time(e1) * 1e3 / args.steps
+    achieved = GEMM_FLOP / kernel_us / 1e6
+
+    result = {
+        "metric": "Linear2D per-rank TFLOP/s (%bf16 MFMA peak); LN/CE HBM GB/s (%peak)",
+        "value": round(GEMM_FLOP / ms_per_step / 1e9, 2),
+        "unit": "TFLOP/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 5),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "bf16",
+        "data": "synthetic",
+        "config": {"workload": "Linear2D one rank of a q=2 grid: X blocks [8192,2048] bf16, W blocks [2048,2048] bf16, "
+                               "2 SUMMA k-steps accumulated in fp32, fused bias+GeLU(tanh), out [8192,2048] bf16",
+                   "layout": "NN", "flop_per_step": GEMM_FLOP, "operand_sets_rotated": n_sets, "device_arch": arch},
+        "roofline": {"bound": "mfma", "achieved": round(achieved, 2), "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
+                     "frac": round(achieved / MFMA_BF16_PEAK_TFLOPS, 4), "traffic": None,
+                     "kernel": "gemm_bf16_kernel<256,256,NN,bias+gelu_tanh>", "avg_launch_us": round(kernel_us, 2)},
+    }
+    if not args.no_aux:
+        result["aux"] = bench_bandwidth_kernels(device)
+        result["aux"]["hbm_peak_GBps"] = HBM_PEAK_GBPS
+    if not args.no_cpu:
+        result["cpu_baseline"] = cpu_baseline()
+    print(json.dumps(result))
+
+
+if __name__ == "__main__":
+    main()

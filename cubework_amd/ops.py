@@ -135,6 +135,25 @@ def gemm_ksteps(layout: str, A_steps: Sequence[torch.Tensor], B_steps: Sequence[
     return (out, preact) if want_preact else out
 
 
+def bias_act(x: torch.Tensor, bias: Optional[torch.Tensor], activation: Optional[str] = None) -> torch.Tensor:
+    """act(x + bias) as the GEMM epilogue alone (zero k-steps, x as the addend)."""
+    lib = _lib.load()
+    shape = x.shape
+    x2 = _rows(x)
+    _require_device(x2, bias)
+    M, N = x2.shape
+    if bias is not None:
+        if bias.numel() != N:
+            raise ValueError("bias has %d elements, width is %d" % (bias.numel(), N))
+        bias = bias.to(x2.dtype).contiguous()
+    out = torch.empty((M, N), dtype=x2.dtype, device=x2.device)
+    tadd = _ptr_table([x2])
+    rc = lib.cw_gemm_ksteps(CW_NN, M, N, 0, 0, None, 0, None, 0, _p(bias), epilogue_code(bias is not None, activation),
+                            _p(out), _ld(out), None, 0, tadd, 1, _ld(x2), _dtype_code(x2), _stream())
+    _lib.check(rc, "cw_gemm_ksteps (bias/activation only)")
+    return out.reshape(shape)
+
+
 def _workspace(M: int, N: int, device) -> torch.Tensor:
     nbytes = _lib.load().cw_colsum_workspace_bytes(M, N)
     return torch.empty(max(nbytes, 16), dtype=torch.uint8, device=device)

@@ -1,0 +1,94 @@
+"""An OPT decoder layer built from the drop-in layers, used as the shape
+source of the "OPT-1.3B-shaped block" workload (hidden 2048, 32 heads, FFN
+8192) and by its parity test.
+
+Structure of benchmark/opt/opt.py:45-211 of the reference (OPTAttention +
+OPTDecoderLayer, pre-LayerNorm variant, dropout 0): LayerNorm -> qkv Linear ->
+causal attention -> out Linear -> residual -> LayerNorm -> fc1 -> activation ->
+fc2 -> residual. The four Linears and two LayerNorms are cubework_amd.module
+layers (HIP path); the attention core (scaled QK^T, causal mask, softmax, PV)
+is model code in the reference and stays a torch call here.
+"""
+from typing import Dict, Optional, Tuple
+
+import torch
+import torch.nn as nn
+import torch.nn.functional as F
+
+from . import module as cube_nn
+
+
+class OPTBlock(nn.Module):
+
+    def __init__(self, hidden: int = 2048, heads: int = 32, ffn: int = 8192, dtype=None,
+                 activation: str = "relu", fuse_activation: bool = True):
+        super().__init__()
+        self.hidden, self.heads, self.head_dim = hidden, heads, hidden // heads
+        self.activation = activation
+        self.fuse_activation = fuse_activation
+        self.self_attn_layer_norm = cube_nn.LayerNorm(hidden, dtype=dtype)
+        self.qkv_proj = cube_nn.Linear(hidden, 3 * hidden, dtype=dtype)
+        self.out_proj = cube_nn.Linear(hidden, hidden, dtype=dtype)
+        self.final_layer_norm = cube_nn.LayerNorm(hidden, dtype=dtype)
+        fc1_kwargs = {"activation": activation} if fuse_activation else {}
+        self.fc1 = cube_nn.Linear(hidden, ffn, dtype=dtype, **fc1_kwargs)
+        self.fc2 = cube_nn.Linear(ffn, hidden, dtype=dtype)
+
+    def _attention_core(self, qkv: torch.Tensor) -> torch.Tensor:
+        b, s, _ = qkv.shape
+        qkv = qkv.view(b, s, self.heads, 3 * self.head_dim).permute(0, 2, 1, 3)
+        q, k, v = torch.chunk(qkv, 3, dim=-1)
+        o = F.scaled_dot_product_attention(q, k, v, is_causal=True)
+        return o.transpose(1, 2).reshape(b, s, self.heads * self.head_dim)
+
+    def forward(self, x: torch.Tensor) -> torch.Tensor:
+        h = self.self_attn_layer_norm(x)
+        h = self.out_proj(self._attention_core(self.qkv_proj(h)))
+        x = x + h
+        shape = x.shape
+        r = x.reshape(-1, shape[-1])
+        h = self.fc1(self.final_layer_norm(r))
+        if not self.fuse_activation:
+            h = _ACT[self.activation](h)
+        h = self.fc2(h)
+        return (r + h).view(shape)
+
+
+_ACT = {"relu": F.relu, "gelu": F.gelu, "gelu_erf": F.gelu, "gelu_tanh": lambda t: F.gelu(t, approximate="tanh")}
+
+
+def opt_block_reference(block: OPTBlock, x: torch.Tensor) -> Tuple[torch.Tensor, Dict[str, torch.Tensor]]:
+    """The same layer in plain fp32 torch on the CPU, with leaf copies of the
+    block's parameters (returned by name so gradients can be compared).
+    Weights of the 2D/3D layers are [in, out]; 1D layers keep [out, in]."""
+    p = {n: t.detach().float().cpu().clone().requires_grad_(True) for n, t in block.named_parameters()}
+
+    def find(prefix: str, leaf: str) -> torch.Tensor:
+        for n, t in p.items():
+            if n.startswith(prefix + ".") and n.endswith(leaf):
+                return t
+        raise KeyError(prefix + "." + leaf)
+
+    def lin(prefix: str, t: torch.Tensor) -> torch.Tensor:
+        w, b = find(prefix, "weight"), find(prefix, "bias")
+        return t @ w + b if _is_in_out(block, prefix) else F.linear(t, w, b)
+
+    def ln(prefix: str, t: torch.Tensor) -> torch.Tensor:
+        return F.layer_norm(t, (t.shape[-1],), find(prefix, "weight"), find(prefix, "bias"), 1e-5)
+
+    heads, hd = block.heads, block.head_dim
+    h = ln("self_attn_layer_norm", x)
+    qkv = lin("qkv_proj", h)
+    b, s, _ = qkv.shape
+    qkv = qkv.view(b, s, heads, 3 * hd).permute(0, 2, 1, 3)
+    q, k, v = torch.chunk(qkv, 3, dim=-1)
+    o = F.scaled_dot_product_attention(q, k, v, is_causal=True).transpose(1, 2).reshape(b, s, heads * hd)
+    x1 = x + lin("out_proj", o)
+    h = _ACT[block.activation](lin("fc1", ln("final_layer_norm", x1)))
+    return x1 + lin("fc2", h), p
+
+
+def _is_in_out(block: OPTBlock, prefix: str) -> bool:
+    """True when the layer stores its weight as [in, out] (Linear2D / Linear3D)."""
+    inner = getattr(block, prefix).linear
+    return type(inner).__name__ in ("Linear2D", "Linear3D")

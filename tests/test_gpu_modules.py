@@ -1,0 +1,321 @@
+"""GPU tests of the layer API (the drop-in for cubework.module): forward and
+backward of each layer against the reference tests' own oracles — plain torch
+on the master tensors (tests/test_2d/check_2d_modules.py:77, tests/test_1d/
+check_1d_modules.py:74,144, tests/test_3d/check_3d_modules.py:132) — at
+tensor-parallel size 1, and as one rank of a 2 x 2 grid / of 4 vocabulary
+slices with the peers' data pre-staged.
+"""
+import pytest
+import torch
+import torch.nn.functional as F
+
+from tests.util import assert_parity, randn
+
+pytestmark = pytest.mark.gpu
+
+DEV = "cuda:0"
+
+
+def _leaf(t):
+    return t.detach().clone().requires_grad_(True)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("mode", ["1d", "2d", "3d"])
+def test_facade_linear_size1(mode, dtype):
+    from cubework_amd.distributed import initialize
+    import cubework_amd.module as cube_nn
+
+    initialize(mode, 1)
+    layer = cube_nn.Linear(96, 160, dtype=dtype).to(DEV)
+    second = cube_nn.Linear(160, 96, dtype=dtype).to(DEV)  # 1d: row-parallel after the column-parallel layer
+    x = _leaf(randn((4, 24, 96), dtype, 0).to(DEV))
+    dy = randn((4, 24, 96), dtype, 1).to(DEV)
+    y = second(layer(x))
+    y.backward(dy)
+    xr = _leaf(x.detach().float().cpu())
+    ws = []
+    h = xr
+    for lyr in (layer, second):
+        w = _leaf(lyr.weight.detach().float().cpu())
+        b = _leaf(lyr.bias.detach().float().cpu())
+        ws.append((w, b))
+        h_in = h if dtype == torch.float32 else h.to(dtype).float()
+        h = F.linear(h_in, w, b) if mode == "1d" else h_in @ w + b
+    h.backward(dy.float().cpu())
+    s = 30 if dtype == torch.float32 else 2
+    assert_parity(y, h.detach().to(dtype), dtype, "forward", scale=s)
+    assert_parity(x.grad, xr.grad.to(dtype), dtype, "dX", scale=s)
+    for lyr, (w, b) in zip((layer, second), ws):
+        assert_parity(lyr.weight.grad, w.grad.to(dtype), dtype, "dW", scale=s)
+        assert_parity(lyr.bias.grad, b.grad.to(dtype), dtype, "dbias", scale=s)
+    names = set(dict(layer.named_parameters()).keys())
+    assert names == {"linear.weight", "linear.bias"} or names == {"linear.linear.weight", "linear.linear.bias"}
+
+
+@pytest.mark.parametrize("act", ["gelu_tanh", "gelu", "relu"])
+def test_linear2d_fused_activation(act):
+    from cubework_amd.distributed import initialize
+    from cubework_amd.module.parallel_2d import Linear2D
+
+    initialize("2d", 1)
+    layer = Linear2D(128, 256, activation=act).to(torch.bfloat16).to(DEV)
+    x = _leaf(randn((64, 128), torch.bfloat16, 0).to(DEV))
+    dy = randn((64, 256), torch.bfloat16, 1).to(DEV)
+    y = layer(x)
+    y.backward(dy)
+    xr = _leaf(x.detach().float().cpu())
+    w = _leaf(layer.weight.detach().float().cpu())
+    b = _leaf(layer.bias.detach().float().cpu())
+    pre = xr @ w + b
+    ref = {"gelu_tanh": lambda t: F.gelu(t, approximate="tanh"), "gelu": F.gelu, "relu": F.relu}[act](pre)
+    ref.backward(dy.float().cpu())
+    assert_parity(y, ref.detach(), torch.bfloat16, "fused forward")
+    assert_parity(x.grad, xr.grad, torch.bfloat16, "dX", scale=2)
+    assert_parity(layer.weight.grad, w.grad, torch.bfloat16, "dW", scale=2)
+    assert_parity(layer.bias.grad, b.grad, torch.bfloat16, "dbias", scale=2)
+
+
+def test_skip_bias_add_and_errors():
+    from cubework_amd.distributed import initialize
+    from cubework_amd.module.parallel_1d import Linear1D_Col, Linear1D_Row
+    from cubework_amd.module.parallel_2d import Linear2D
+
+    initialize("2d", 1)
+    layer = Linear2D(64, 64, skip_bias_add=True).to(DEV)
+    out, bias = layer(randn((8, 64), torch.float32, 0).to(DEV))
+    assert out.shape == (8, 64) and torch.equal(bias, layer.bias.detach())
+    with pytest.raises(AssertionError):
+        layer(torch.zeros((8, 32), device=DEV))  # "Invalid shapes ... for AB."
+    initialize("1d", 1)
+    with pytest.raises(ValueError):
+        Linear1D_Col(8, 8, bias=False, skip_bias_add=True)
+    with pytest.raises(ValueError):
+        Linear1D_Row(8, 8, bias=False, skip_bias_add=True)
+    col = Linear1D_Col(64, 64, skip_bias_add=True).to(DEV)
+    o, b = col(randn((8, 64), torch.float32, 0).to(DEV))
+    assert b is col.bias and o.shape == (8, 64)
+    initialize(None, 1)
+    with pytest.raises(AssertionError):
+        Linear2D(8, 8)  # 2D groups not initialised
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("mode", ["2d", "3d"])
+def test_facade_layernorm_size1(mode, dtype):
+    from cubework_amd.distributed import initialize
+    import cubework_amd.module as cube_nn
+
+    initialize(mode, 1)
+    H = 512
+    norm = cube_nn.LayerNorm(H, eps=1e-5, dtype=dtype).to(DEV)
+    with torch.no_grad():
+        norm.weight.copy_(torch.rand(H) * 0.2 + 0.9)
+        norm.bias.copy_(torch.randn(H) * 0.02)
+    x = _leaf(randn((6, 20, H), dtype, 3).to(DEV))
+    dy = randn((6, 20, H), dtype, 4).to(DEV)
+    y = norm(x)
+    y.backward(dy)
+    xr = _leaf(x.detach().float().cpu())
+    g = _leaf(norm.weight.detach().float().cpu())
+    b = _leaf(norm.bias.detach().float().cpu())
+    ref = F.layer_norm(xr, (H,), g, b, 1e-5)
+    ref.backward(dy.float().cpu())
+    s = 20 if dtype == torch.float32 else 1
+    assert_parity(y, ref.detach(), dtype, "forward", scale=s)
+    assert_parity(x.grad, xr.grad, dtype, "dX", scale=s)
+    assert_parity(norm.weight.grad, g.grad, dtype, "dgamma", scale=100 if dtype == torch.float32 else 2)
+    assert_parity(norm.bias.grad, b.grad, dtype, "dbeta", scale=100 if dtype == torch.float32 else 2)
+
+
+@pytest.mark.parametrize("mode", ["1d", "2d", "3d"])
+@pytest.mark.parametrize("vocab_parallel", [False, True])
+def test_facade_classifier_and_loss_size1(mode, vocab_parallel):
+    from cubework_amd.distributed import initialize
+    from cubework_amd.global_vars import env
+    import cubework_amd.module as cube_nn
+
+    initialize(mode, 1)
+    env.vocab_parallel = vocab_parallel
+    head = cube_nn.Classifier(128, 520, dtype=torch.float32).to(DEV)
+    crit = cube_nn.CrossEntropyLoss()
+    x = _leaf(randn((48, 128), torch.float32, 5).to(DEV))
+    t = torch.randint(0, 520, (48,), generator=torch.Generator().manual_seed(6)).to(DEV)
+    loss = crit(head(x), t)
+    loss.backward()
+    xr = _leaf(x.detach().cpu())
+    w = _leaf(head.weight.detach().cpu())
+    b = _leaf(head.bias.detach().cpu())
+    ref = F.cross_entropy(F.linear(xr, w, b), t.cpu())
+    ref.backward()
+    assert_parity(loss, ref.detach(), torch.float32, "loss", scale=10)
+    assert_parity(x.grad, xr.grad, torch.float32, "dX", scale=30)
+    assert_parity(head.weight.grad, w.grad, torch.float32, "dW", scale=30)
+    assert_parity(head.bias.grad, b.grad, torch.float32, "dbias", scale=30)
+
+
+def test_linear2d_one_rank_of_2x2_grid():
+    """Rank (row 0, col 1) of a 2 x 2 grid, peers' operands pre-staged; checked
+    against the master computation with the reference test's shard layout
+    (tests/test_2d/check_2d_modules.py:38-110)."""
+    import oracle
+    from oracle.grid import bias_shard, shard
+    from cubework_amd.distributed import initialize, pm
+    from cubework_amd.module.parallel_2d import Linear2D
+
+    q, i, j = 2, 0, 1
+    B_, S_, IN, OUT = 8, 4, 256, 384
+    dt = torch.float32
+    A_master = randn((B_, S_, IN), dt, 0)
+    W_master = randn((IN, OUT), dt, 1, std=0.05)
+    b_master = randn((OUT,), dt, 2)
+    dC_master = randn((B_, S_, OUT), dt, 3)
+    A2, dC2 = A_master.reshape(-1, IN), dC_master.reshape(-1, OUT)
+
+    initialize("2d", q * q, row=i, col=j)
+    layer = Linear2D(IN, OUT).to(DEV)
+    assert layer.weight.shape == (IN // q, OUT // q) and layer.bias.shape == (OUT // q ** 2,)
+    with torch.no_grad():
+        layer.weight.copy_(shard(W_master, q, i, j))
+        layer.bias.copy_(bias_shard(b_master, q, i, j))
+    row, col = pm.PARALLEL_2D_ROW, pm.PARALLEL_2D_COL
+    d = lambda t: t.to(DEV)  # noqa: E731
+    # forward: step 0's A comes from the rank at column 0 of my row, step 0's B is mine? no: B_k comes from row k
+    row.stage("broadcast", d(shard(A2, q, i, 0)))           # A of step 0 (I am column 1)
+    col.stage("broadcast", d(shard(W_master, q, 1, j)))     # B of step 1 (I am row 0)
+    col.stage("all_gather", [None, d(bias_shard(b_master, q, 1, j))])
+    x = _leaf(d(shard(A2, q, i, j)))
+    out = layer(x)
+    C_master = A2 @ W_master + b_master
+    assert_parity(out, shard(C_master, q, i, j), dt, "Linear2D forward shard", scale=10)
+
+    # backward: every "collective" of the three backward operators, in the order they run
+    dC = shard(dC2, q, i, j)
+    gemm = oracle.gemm_ksteps
+    col.stage("reduce_scatter", [d(oracle.colsum(shard(dC2, q, 1, j)))])           # peers' bias-grad column sums
+    col.stage("broadcast", d(shard(W_master, q, 1, j)))                             # summa_ABT: B of step 1
+    row.stage("reduce", [d(gemm("NT", [shard(dC2, q, i, 0)], [shard(W_master, q, j, 0)]))])  # peer's product for my column
+    row.stage("broadcast", d(shard(A2, q, i, 0)))                                   # summa_ATB: A of step 0
+    col.stage("reduce", [d(gemm("TN", [shard(A2, q, 1, i)], [shard(dC2, q, 1, j)]))])        # peer's product for my row
+    out.backward(d(dC))
+    dA_master = dC2 @ W_master.t()
+    dW_master = A2.t() @ dC2
+    assert_parity(x.grad, shard(dA_master, q, i, j), dt, "dA shard", scale=10)
+    assert_parity(layer.weight.grad, shard(dW_master, q, i, j), dt, "dW shard", scale=10)
+    assert_parity(layer.bias.grad, bias_shard(dC2.sum(0), q, i, j), dt, "dbias shard", scale=30)
+    # what this rank would have sent: its products for the peers
+    sent_row = dict(row.outbox["reduce"])
+    assert_parity(sent_row[0], gemm("NT", [dC], [shard(W_master, q, 0, j)]), dt, "product sent to column 0", scale=10)
+    assert not any(row.inbox.values()) and not any(col.inbox.values())
+
+
+def test_linear2d_missing_peer_data_is_an_error():
+    from cubework_amd.distributed import MissingPeerData, initialize
+    from cubework_amd.module.parallel_2d import Linear2D
+
+    initialize("2d", 4, row=0, col=0)
+    layer = Linear2D(64, 64).to(DEV)
+    with pytest.raises(MissingPeerData):
+        layer(torch.zeros((4, 32), device=DEV))
+
+
+def test_layernorm2d_one_rank_of_2x2_grid():
+    """tests/test_2d/check_2d_modules.py:113-162 for one rank, with affine."""
+    from oracle.grid import bias_shard, shard
+    import oracle
+    from cubework_amd.distributed import initialize, pm
+    from cubework_amd.module.parallel_2d import LayerNorm2D
+
+    q, i, j = 2, 1, 0
+    R, H, eps = 16, 512, 1e-5
+    dt = torch.float32
+    A = randn((R, H), dt, 0)
+    dY = randn((R, H), dt, 1)
+    gamma = torch.rand(H, generator=torch.Generator().manual_seed(2)) * 0.2 + 0.9
+    beta = randn((H,), dt, 3, std=0.02)
+    initialize("2d", q * q, row=i, col=j)
+    norm = LayerNorm2D(H, eps).to(DEV)
+    assert norm.weight.shape == (H // q ** 2,)
+    with torch.no_grad():
+        norm.weight.copy_(bias_shard(gamma, q, i, j))
+        norm.bias.copy_(bias_shard(beta, q, i, j))
+    row, col = pm.PARALLEL_2D_ROW, pm.PARALLEL_2D_COL
+    d = lambda t: t.to(DEV)  # noqa: E731
+    peer_col = 1 - j
+    col.stage("all_gather", [d(bias_shard(gamma, q, 0, j)), None])
+    col.stage("all_gather", [d(bias_shard(beta, q, 0, j)), None])
+    row.stage("all_reduce", [d(oracle.ln2d_partial_stats(shard(A, q, i, peer_col)))])
+    x = _leaf(d(shard(A, q, i, j)))
+    y = norm(x)
+    Ar = _leaf(A)
+    ref = F.layer_norm(Ar, (H,), gamma, beta, eps)
+    ref.backward(dY)
+    assert_parity(y, shard(ref.detach(), q, i, j), dt, "LayerNorm2D forward shard", scale=20)
+    # backward: the row peer's partial sums, then the column peers' dgamma/dbeta sums
+    stats = oracle.ln2d_partial_stats(A)
+    mr = oracle.ln2d_mean_rstd(stats, H, eps)
+    g_peer = torch.chunk(gamma, q, dim=-1)[peer_col]
+    rs_peer, _, _ = oracle.ln2d_backward_partials(shard(dY, q, i, peer_col), shard(A, q, i, peer_col), mr[i * R // q:(i + 1) * R // q], g_peer)
+    row.stage("all_reduce", [d(rs_peer)])
+    other_row = 1 - i
+    _, dg_o, db_o = oracle.ln2d_backward_partials(shard(dY, q, other_row, j), shard(A, q, other_row, j),
+                                                  mr[other_row * R // q:(other_row + 1) * R // q], torch.chunk(gamma, q, dim=-1)[j])
+    col.stage("reduce_scatter", [d(dg_o)])
+    col.stage("reduce_scatter", [d(db_o)])
+    y.backward(d(shard(dY, q, i, j)))
+    assert_parity(x.grad, shard(Ar.grad, q, i, j), dt, "dX shard", scale=20)
+    xh = (A - mr[:, 0:1]) * mr[:, 1:2]
+    assert_parity(norm.weight.grad, bias_shard((dY * xh).sum(0), q, i, j), dt, "dgamma shard", scale=100)
+    assert_parity(norm.bias.grad, bias_shard(dY.sum(0), q, i, j), dt, "dbeta shard", scale=100)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+def test_vocab_parallel_loss_one_rank_of_four(dtype):
+    """Rank 1 of 4 vocabulary slices (tests/test_1d/check_1d_modules.py:491-524
+    with [tokens, vocab] logits)."""
+    import oracle
+    from cubework_amd.distributed import initialize, pm
+    from cubework_amd.module.loss import VocabParallelCrossEntropyLoss1D
+
+    p, r, T, V = 4, 1, 96, 1000
+    full = randn((T, V * p), dtype, 0, std=2.0)
+    t = torch.randint(0, V * p, (T,), generator=torch.Generator().manual_seed(1))
+    slices = list(torch.chunk(full, p, dim=-1))
+    initialize("1d", p, rank=r)
+    peers = [oracle.vpce_fwd_local(s, t, k * V) for k, s in enumerate(slices) if k != r]
+    pm.PARALLEL_1D.stage("vpce_stats", [torch.stack([pk[n] for pk in peers]).to(DEV) for n in range(4)])
+    crit = VocabParallelCrossEntropyLoss1D()
+    x = _leaf(slices[r].contiguous().to(DEV))
+    before = x.detach().clone()
+    loss = crit(x, t.to(DEV))
+    loss.backward()
+    fr = _leaf(full.float())
+    ref = F.cross_entropy(fr, t)
+    ref.backward()
+    assert_parity(loss, ref.detach(), torch.float32, "mean loss", scale=10)
+    assert_parity(x.grad, fr.grad[:, r * V:(r + 1) * V], dtype, "logits grad", scale=10 if dtype == torch.float32 else 1)
+    assert torch.equal(x.detach(), before), "the caller's logits must stay intact"
+
+
+def test_opt_block_shapes_small():
+    """A reduced OPT decoder layer (benchmark/opt/opt.py:135-211 shapes: pre-LN,
+    qkv/out/fc1/fc2 Linear2D, ReLU) at tensor-parallel size 1, forward+backward
+    in bf16 against the same block in fp32 torch."""
+    from cubework_amd.distributed import initialize
+    from cubework_amd.opt_block import OPTBlock, opt_block_reference
+
+    initialize("2d", 1)
+    torch.manual_seed(0)
+    blk = OPTBlock(hidden=256, heads=4, ffn=1024, dtype=torch.bfloat16, activation="relu").to(DEV)
+    x = _leaf(randn((2, 64, 256), torch.bfloat16, 1).to(DEV))
+    dy = randn((2, 64, 256), torch.bfloat16, 2).to(DEV)
+    y = blk(x)
+    y.backward(dy)
+    xr = _leaf(x.detach().float().cpu())
+    ref, params = opt_block_reference(blk, xr)
+    ref.backward(dy.float().cpu())
+    assert_parity(y, ref.detach(), torch.bfloat16, "block forward", scale=3)
+    assert_parity(x.grad, xr.grad, torch.bfloat16, "block dX", scale=5)
+    for name, prm in blk.named_parameters():
+        assert prm.grad is not None and torch.isfinite(prm.grad.float()).all(), name
+        assert_parity(prm.grad, params[name].grad, torch.bfloat16, name + ".grad", scale=5)
