@@ -309,20 +309,25 @@ __global__ __launch_bounds__(kThreads) void gemm_bf16_kernel(const GemmArgs args
         const int cur = kt & 1;
         if (kt + 1 < KT) issue_loads(kt + 1);
         const uint16_t* s = lds + cur * STAGE;
-#pragma unroll
-        for (int ks = 0; ks < kBK / 16; ++ks) {
-            bf16x8_t af[TM], bfr[TN];
+        // fragments of k-step ks+1 are read from LDS while the MFMAs of step ks run
+        bf16x8_t af[2][TM], bfr[2][TN];
+        auto read_frags = [&](int ks, int set) {
 #pragma unroll
             for (int i = 0; i < TM; ++i)
-                af[i] = *reinterpret_cast<const bf16x8_t*>(s + a_frag + i * 32 * kPitch + ks * 16);
+                af[set][i] = *reinterpret_cast<const bf16x8_t*>(s + a_frag + i * 32 * kPitch + ks * 16);
 #pragma unroll
             for (int j = 0; j < TN; ++j)
-                bfr[j] = *reinterpret_cast<const bf16x8_t*>(s + b_frag + j * 32 * kPitch + ks * 16);
+                bfr[set][j] = *reinterpret_cast<const bf16x8_t*>(s + b_frag + j * 32 * kPitch + ks * 16);
+        };
+        read_frags(0, 0);
+#pragma unroll
+        for (int ks = 0; ks < kBK / 16; ++ks) {
+            if (ks + 1 < kBK / 16) read_frags(ks + 1, (ks + 1) & 1);
 #pragma unroll
             for (int i = 0; i < TM; ++i)
 #pragma unroll
                 for (int j = 0; j < TN; ++j)
-                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(bfr[j], af[i], acc[i][j], 0, 0, 0);
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(bfr[ks & 1][j], af[ks & 1][i], acc[i][j], 0, 0, 0);
         }
         if (kt + 1 < KT) commit_loads(cur ^ 1);
         __syncthreads();
