@@ -1,0 +1,10 @@
+// bf16 block GEMM, LDS-DMA kernel, orientation NT.
+#include "gemm_bf16_dma.h"
+
+namespace cw {
+
+int gemm_bf16_dma_launch_nt(const GemmArgs& args, int epilogue, hipStream_t s) {
+    return gemm_dma::launch_dma<false, false>(args, epilogue, s);
+}
+
+}  // namespace cw

@@ -1,0 +1,10 @@
+// bf16 block GEMM, LDS-DMA kernel, orientation TN.
+#include "gemm_bf16_dma.h"
+
+namespace cw {
+
+int gemm_bf16_dma_launch_tn(const GemmArgs& args, int epilogue, hipStream_t s) {
+    return gemm_dma::launch_dma<true, true>(args, epilogue, s);
+}
+
+}  // namespace cw

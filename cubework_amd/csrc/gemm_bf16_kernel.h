@@ -220,6 +220,84 @@ __device__ __forceinline__ void tile_store(uint16_t* __restrict__ lds_c, uint16_
     }
 }
 
+// Epilogue shared by the block-GEMM kernels: adds the addends and the bias to
+// the fp32 accumulators, optionally stores the pre-activation, applies the
+// activation, packs to bf16, stages the tile in LDS (which must be free: all
+// waves past their last operand read) and writes it out row by row.
+// acc[i][j][v]: row  m = m0 + wm*(BM/2) + i*32 + (lane & 31)
+//               col  n = n0 + wn*(BN/2) + j*32 + 8*(v/4) + 4*(lane>>5) + (v%4)
+template <int BM, int BN, int TM, int TN, int EPI>
+__device__ __forceinline__ void gemm_epilogue(f32x16_t (&acc)[TM][TN], const GemmArgs& args, uint16_t* lds, int m0,
+                                              int n0, int wm, int wn, int lane, int tid) {
+    constexpr int WTM = BM / 2, WTN = BN / 2;
+    const int M = args.M, N = args.N;
+    constexpr int CP = BN + 4;
+    uint16_t* lds_c = lds;  // the operand stages are dead after the last barrier
+    const int row_l = wm * WTM + (lane & 31);
+    const int col_l = wn * WTN + 4 * (lane >> 5);
+    const bool vec_c = args.vec_c != 0;
+    const uint16_t* bias = reinterpret_cast<const uint16_t*>(args.bias);
+
+    if (args.n_addends > 0 || (EPI != CW_EPI_NONE && bias != nullptr)) {
+#pragma unroll
+        for (int j = 0; j < TN; ++j)
+#pragma unroll
+            for (int g = 0; g < 4; ++g) {
+                const int ncol = n0 + col_l + j * 32 + 8 * g;
+                float bv[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+                if (EPI != CW_EPI_NONE && bias != nullptr && ncol < N)
+                    load4_bf16(bias + ncol, N - ncol, args.vec_bias != 0, bv);
+#pragma unroll
+                for (int i = 0; i < TM; ++i) {
+                    const int mrow = m0 + row_l + i * 32;
+                    float add[4] = {bv[0], bv[1], bv[2], bv[3]};
+                    if (args.n_addends > 0 && mrow < M && ncol < N) {
+                        for (int a = 0; a < args.n_addends; ++a) {
+                            float t[4];
+                            load4_bf16(reinterpret_cast<const uint16_t*>(args.addend[a]) + (int64_t)mrow * args.ldadd + ncol,
+                                       N - ncol, args.vec_add != 0, t);
+#pragma unroll
+                            for (int e = 0; e < 4; ++e) add[e] += t[e];
+                        }
+                    }
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) acc[i][j][4 * g + e] += add[e];
+                }
+            }
+    }
+
+    auto stage_tile = [&](bool activated) {
+#pragma unroll
+        for (int i = 0; i < TM; ++i)
+#pragma unroll
+            for (int j = 0; j < TN; ++j)
+#pragma unroll
+                for (int g = 0; g < 4; ++g) {
+                    float v[4];
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) {
+                        const float x = acc[i][j][4 * g + e];
+                        v[e] = activated ? epi_act<EPI>(x) : x;
+                    }
+                    u32x2_t p;
+                    p.x = pack_bf16x2(v[0], v[1]);
+                    p.y = pack_bf16x2(v[2], v[3]);
+                    *reinterpret_cast<u32x2_t*>(lds_c + (row_l + i * 32) * CP + col_l + j * 32 + 8 * g) = p;
+                }
+    };
+
+    if (args.preact != nullptr) {
+        stage_tile(false);
+        __syncthreads();
+        tile_store<BM, BN>(lds_c, reinterpret_cast<uint16_t*>(args.preact), args.ldp, m0, n0, M, N, tid,
+                           args.vec_p != 0);
+        __syncthreads();
+    }
+    stage_tile(true);
+    __syncthreads();
+    tile_store<BM, BN>(lds_c, reinterpret_cast<uint16_t*>(args.C), args.ldc, m0, n0, M, N, tid, vec_c);
+}
+
 template <int BM, int BN, bool TRANS_A, bool TRANS_B, bool GUARD, int EPI>
 __global__ __launch_bounds__(kThreads) void gemm_bf16_kernel(const GemmArgs args) {
     constexpr int WTM = BM / 2, WTN = BN / 2;  // wavefront sub-tile
@@ -333,74 +411,7 @@ __global__ __launch_bounds__(kThreads) void gemm_bf16_kernel(const GemmArgs args
         __syncthreads();
     }
 
-    // ---- epilogue -------------------------------------------------------
-    // acc[i][j][v]: row  m = m0 + wm*WTM + i*32 + (lane & 31)
-    //               col  n = n0 + wn*WTN + j*32 + 8*(v/4) + 4*(lane>>5) + (v%4)
-    constexpr int CP = BN + 4;
-    uint16_t* lds_c = lds;  // the operand stages are dead after the last barrier
-    const int row_l = wm * WTM + (lane & 31);
-    const int col_l = wn * WTN + 4 * (lane >> 5);
-    const bool vec_c = args.vec_c != 0;
-    const uint16_t* bias = reinterpret_cast<const uint16_t*>(args.bias);
-
-    if (args.n_addends > 0 || (EPI != CW_EPI_NONE && bias != nullptr)) {
-#pragma unroll
-        for (int j = 0; j < TN; ++j)
-#pragma unroll
-            for (int g = 0; g < 4; ++g) {
-                const int ncol = n0 + col_l + j * 32 + 8 * g;
-                float bv[4] = {0.0f, 0.0f, 0.0f, 0.0f};
-                if (EPI != CW_EPI_NONE && bias != nullptr && ncol < N)
-                    load4_bf16(bias + ncol, N - ncol, args.vec_bias != 0, bv);
-#pragma unroll
-                for (int i = 0; i < TM; ++i) {
-                    const int mrow = m0 + row_l + i * 32;
-                    float add[4] = {bv[0], bv[1], bv[2], bv[3]};
-                    if (args.n_addends > 0 && mrow < M && ncol < N) {
-                        for (int a = 0; a < args.n_addends; ++a) {
-                            float t[4];
-                            load4_bf16(reinterpret_cast<const uint16_t*>(args.addend[a]) + (int64_t)mrow * args.ldadd + ncol,
-                                       N - ncol, args.vec_add != 0, t);
-#pragma unroll
-                            for (int e = 0; e < 4; ++e) add[e] += t[e];
-                        }
-                    }
-#pragma unroll
-                    for (int e = 0; e < 4; ++e) acc[i][j][4 * g + e] += add[e];
-                }
-            }
-    }
-
-    auto stage_tile = [&](bool activated) {
-#pragma unroll
-        for (int i = 0; i < TM; ++i)
-#pragma unroll
-            for (int j = 0; j < TN; ++j)
-#pragma unroll
-                for (int g = 0; g < 4; ++g) {
-                    float v[4];
-#pragma unroll
-                    for (int e = 0; e < 4; ++e) {
-                        const float x = acc[i][j][4 * g + e];
-                        v[e] = activated ? epi_act<EPI>(x) : x;
-                    }
-                    u32x2_t p;
-                    p.x = pack_bf16x2(v[0], v[1]);
-                    p.y = pack_bf16x2(v[2], v[3]);
-                    *reinterpret_cast<u32x2_t*>(lds_c + (row_l + i * 32) * CP + col_l + j * 32 + 8 * g) = p;
-                }
-    };
-
-    if (args.preact != nullptr) {
-        stage_tile(false);
-        __syncthreads();
-        tile_store<BM, BN>(lds_c, reinterpret_cast<uint16_t*>(args.preact), args.ldp, m0, n0, M, N, tid,
-                           args.vec_p != 0);
-        __syncthreads();
-    }
-    stage_tile(true);
-    __syncthreads();
-    tile_store<BM, BN>(lds_c, reinterpret_cast<uint16_t*>(args.C), args.ldc, m0, n0, M, N, tid, vec_c);
+    gemm_epilogue<BM, BN, TM, TN, EPI>(acc, args, lds, m0, n0, wm, wn, lane, tid);
 }
 
 template <int BM, int BN>
