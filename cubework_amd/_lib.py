@@ -8,7 +8,8 @@ import ctypes
 import os
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(_HERE, "libcubework_hip.so")
+# CUBEWORK_HIP_LIB selects another build of the library (kernel experiments).
+LIB_PATH = os.environ.get("CUBEWORK_HIP_LIB") or os.path.join(_HERE, "libcubework_hip.so")
 
 # enums of include/cubework_hip.h
 CW_BF16, CW_F32 = 0, 1

@@ -37,29 +37,32 @@ def _hipcc():
     raise RuntimeError("hipcc not found")
 
 
-def _compile(src):
-    obj = os.path.join(OBJ_DIR, os.path.splitext(src)[0] + ".o")
-    cmd = [_hipcc(), *HIPCC_FLAGS, "-c", os.path.join(CSRC, src), "-o", obj]
+def _compile(src, extra=(), obj_dir=None):
+    obj = os.path.join(obj_dir or OBJ_DIR, os.path.splitext(src)[0] + ".o")
+    cmd = [_hipcc(), *HIPCC_FLAGS, *extra, "-c", os.path.join(CSRC, src), "-o", obj]
     proc = subprocess.run(cmd, capture_output=True, text=True)
     if proc.returncode != 0:
         raise RuntimeError("hipcc failed for %s:\n%s\n%s" % (src, proc.stdout, proc.stderr))
     return obj
 
 
-def build(verbose=True):
-    """Compile every HIP source for gfx950 and link the shared library."""
-    os.makedirs(OBJ_DIR, exist_ok=True)
+def build(verbose=True, extra_flags=(), lib_path=None, obj_dir=None):
+    """Compile every HIP source for gfx950 and link the shared library.
+    extra_flags / lib_path / obj_dir build a variant beside the default one."""
+    lib_path = lib_path or LIB_PATH
+    obj_dir = obj_dir or OBJ_DIR
+    os.makedirs(obj_dir, exist_ok=True)
     with ThreadPoolExecutor(max_workers=min(8, len(SOURCES))) as pool:
-        objs = list(pool.map(_compile, SOURCES))
-    tmp = LIB_PATH + ".tmp"
+        objs = list(pool.map(lambda src: _compile(src, extra_flags, obj_dir), SOURCES))
+    tmp = lib_path + ".tmp"
     cmd = [_hipcc(), "--offload-arch=gfx950", "-shared", "-fPIC", *objs, "-o", tmp]
     proc = subprocess.run(cmd, capture_output=True, text=True)
     if proc.returncode != 0:
         raise RuntimeError("link failed:\n%s\n%s" % (proc.stdout, proc.stderr))
-    os.replace(tmp, LIB_PATH)
+    os.replace(tmp, lib_path)
     if verbose:
-        print("built", LIB_PATH, os.path.getsize(LIB_PATH), "bytes")
-    return LIB_PATH
+        print("built", lib_path, os.path.getsize(lib_path), "bytes")
+    return lib_path
 
 
 if __name__ == "__main__":

@@ -89,8 +89,8 @@ extern "C" int cw_gemm_ksteps(int layout, int64_t M, int64_t N, int64_t K, int n
     GemmArgs args;
     memset(&args, 0, sizeof(args));
     const int vec = (io_dtype == CW_BF16) ? 8 : 4;       // elements per 16 bytes
-    const uintptr_t out_mask = (io_dtype == CW_BF16) ? 7u : 15u;  // bf16 outputs move 8 bytes at a time
-    const int out_vec = 4;
+    const uintptr_t out_mask = 15u;                      // outputs / addends move 16 bytes at a time
+    const int out_vec = (io_dtype == CW_BF16) ? 8 : 4;   // elements per 16 bytes
     args.vec_a = args.vec_b = 1;
     for (int i = 0; i < n_steps; ++i) {
         if (A_steps[i] == nullptr || B_steps[i] == nullptr)
@@ -110,7 +110,7 @@ extern "C" int cw_gemm_ksteps(int layout, int64_t M, int64_t N, int64_t K, int n
     }
     if (ldadd % out_vec != 0) args.vec_add = 0;
     args.bias = bias;
-    args.vec_bias = (bias == nullptr || (reinterpret_cast<uintptr_t>(bias) & out_mask) == 0) ? 1 : 0;
+    args.vec_bias = (bias == nullptr || (reinterpret_cast<uintptr_t>(bias) & 7u) == 0) ? 1 : 0;
     args.C = C;
     args.vec_c = ((reinterpret_cast<uintptr_t>(C) & out_mask) == 0 && ldc % out_vec == 0) ? 1 : 0;
     args.preact = preact;

@@ -106,9 +106,12 @@ __device__ __forceinline__ float tanh_fast(float x) {
     return 1.0f - 2.0f * __builtin_amdgcn_rcpf(e + 1.0f);
 }
 __device__ __forceinline__ float gelu_tanh(float x) {
-    const float k0 = 0.7978845608028654f, k1 = 0.044715f;
-    const float u = k0 * (x + k1 * x * x * x);
-    return 0.5f * x * (1.0f + tanh_fast(u));
+    // 0.5 x (1 + tanh(u)) = x / (1 + exp(-2u)), u = sqrt(2/pi) (x + 0.044715 x^3):
+    // two multiplies, one fma, one exp2, one add, one reciprocal, one multiply.
+    const float a = -2.0f * 0.7978845608028654f * kLog2e;
+    const float b = a * 0.044715f;
+    const float e = __builtin_amdgcn_exp2f(x * __builtin_fmaf(x * x, b, a));
+    return x * __builtin_amdgcn_rcpf(1.0f + e);
 }
 __device__ __forceinline__ float gelu_tanh_grad(float x) {
     const float k0 = 0.7978845608028654f, k1 = 0.044715f;

@@ -20,6 +20,23 @@ struct GemmArgs {
     int vec_a, vec_b, vec_c, vec_p, vec_add, vec_bias;
 };
 
+// Compact argument block of the LDS-DMA kernel: few enough pointers that they
+// all stay in scalar registers for the whole k loop.
+constexpr int kRingMaxSteps = 4;
+constexpr int kRingMaxAddends = 2;
+struct RingArgs {
+    const void* A[kRingMaxSteps];
+    const void* B[kRingMaxSteps];
+    const void* addend[kRingMaxAddends];
+    const void* bias;
+    void* C;
+    void* preact;
+    int64_t lda, ldb, ldc, ldp, ldadd;
+    int M, N, K;
+    int n_steps, n_addends;
+    int vec_bias, vec_add;  // always 1 on this path; read by the shared epilogue
+};
+
 int gemm_bf16_launch(const GemmArgs& args, int layout, int epilogue, hipStream_t s);
 int gemm_f32_launch(const GemmArgs& args, int layout, int epilogue, hipStream_t s);
 

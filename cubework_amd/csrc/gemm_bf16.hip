@@ -1,6 +1,7 @@
 // bf16 block GEMM: choice of kernel and tile configuration.
 //   - large tile-aligned problems (>= 128 tiles of 256x256, K a multiple of 64,
-//     16-byte aligned rows): the LDS-DMA kernel (gemm_bf16_dma.h);
+//     16-byte aligned rows, at most 4 k-steps and 2 addends): the LDS-DMA
+//     kernel (gemm_bf16_dma.h);
 //   - everything else: the register-staged kernel (gemm_bf16_kernel.h), with
 //     256x256 or 128x128 tiles, guarded when the shape is ragged or unaligned.
 // CW_GEMM_IMPL=staged in the environment forces the register-staged kernel.
@@ -33,7 +34,8 @@ int gemm_bf16_launch(const GemmArgs& args, int layout, int epilogue, hipStream_t
     const bool big = tiles256 >= 128;
     const int tile = big ? 256 : 128;
     const bool exact = all_vec && (args.M % tile) == 0 && (args.N % tile) == 0 && (args.K % gemm_bf16::kBK) == 0;
-    if (big && exact && args.n_steps > 0 && dma_kernel_enabled()) {
+    if (big && exact && args.n_steps > 0 && args.n_steps <= kRingMaxSteps && args.n_addends <= kRingMaxAddends &&
+        dma_kernel_enabled()) {
         switch (layout) {
             case CW_NN: return gemm_bf16_dma_launch_nn(args, epilogue, s);
             case CW_NT: return gemm_bf16_dma_launch_nt(args, epilogue, s);

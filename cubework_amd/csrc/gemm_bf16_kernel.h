@@ -51,6 +51,19 @@ __device__ __forceinline__ void static_for(F&& f) {
     static_for_impl(std::make_integer_sequence<int, N>{}, static_cast<F&&>(f));
 }
 
+// tab[idx] without dynamic indexing: a dynamically indexed member keeps the
+// whole kernel-argument struct in scratch memory, and then every field (the
+// leading dimensions, the operand pointers) is read back through vector
+// loads and counts as lane-varying.
+template <int N>
+__device__ __forceinline__ const void* pick_ptr(const void* const (&tab)[N], int idx) {
+    const void* p = tab[0];
+    static_for<N>([&](auto i) {
+        if (idx == i.value) p = tab[i.value];
+    });
+    return p;
+}
+
 constexpr int kBK = 64;         // k extent of an LDS tile
 constexpr int kPitch = 72;      // elements per LDS row (64 + 8 padding)
 constexpr int kThreads = 256;
@@ -188,114 +201,130 @@ __device__ __forceinline__ void load4_bf16(const uint16_t* __restrict__ p, int n
     }
 }
 
-// Stage a wavefront's sub-tile (values already final, fp32) into the block's
-// LDS C tile as bf16 and write the tile out row by row.
-// LDS C tile: [BM][BN + 4] bf16 (pitch = 8 bytes mod 128: the 8-byte writes of
-// 16 consecutive rows land in 16 different bank pairs).
-template <int BM, int BN>
-__device__ __forceinline__ void tile_store(uint16_t* __restrict__ lds_c, uint16_t* __restrict__ C, int64_t ldc,
-                                           int m0, int n0, int M, int N, int tid, bool vec_ok) {
-    constexpr int CP = BN + 4;
-    constexpr int QUADS_PER_ROW = BN / 4;
-    constexpr int TOTAL = BM * QUADS_PER_ROW;
+// LDS image of the output tile: [BM][BN + 8] bf16. The 528-byte (BN = 256)
+// pitch keeps rows 16-byte aligned for the row-wise readout and spreads the
+// 8-byte writes of 16 consecutive rows over 16 different 16-byte bank groups.
+template <int BN>
+constexpr int c_pitch() { return BN + 8; }
+
+// Write the staged tile out row by row: 16 bytes per lane, a wavefront covers
+// whole 512-byte rows (BN = 256), so global stores are full cache lines.
+template <int BM, int BN, bool FAST>
+__device__ __forceinline__ void tile_store(const uint16_t* __restrict__ lds_c, uint16_t* __restrict__ C, int64_t ldc,
+                                           int m0, int n0, int M, int N, int tid) {
+    constexpr int CP = c_pitch<BN>();
+    constexpr int CHUNKS_PER_ROW = BN / 8;
+    constexpr int TOTAL = BM * CHUNKS_PER_ROW;
+    if constexpr (FAST) {
+        // whole tile in bounds, rows 16-byte aligned: thread -> (row q/32.., chunk q%32), no checks
+        uint16_t* base = C + (int64_t)(m0 + tid / CHUNKS_PER_ROW) * ldc + n0 + (tid % CHUNKS_PER_ROW) * 8;
+        const uint16_t* src = lds_c + (tid / CHUNKS_PER_ROW) * CP + (tid % CHUNKS_PER_ROW) * 8;
+        constexpr int ROWS_PER_PASS = kThreads / CHUNKS_PER_ROW;
+#pragma unroll 8
+        for (int pass = 0; pass < BM / ROWS_PER_PASS; ++pass)
+            *reinterpret_cast<u32x4_t*>(base + (int64_t)pass * ROWS_PER_PASS * ldc) =
+                *reinterpret_cast<const u32x4_t*>(src + pass * ROWS_PER_PASS * CP);
+        return;
+    }
+    const bool vec16 = ((reinterpret_cast<uintptr_t>(C) & 15u) == 0) && ((ldc & 7) == 0);
 #pragma unroll 4
     for (int q = tid; q < TOTAL; q += kThreads) {
-        const int r = q / QUADS_PER_ROW;
-        const int cq = q % QUADS_PER_ROW;
+        const int r = q / CHUNKS_PER_ROW;
+        const int cq = q % CHUNKS_PER_ROW;
         const int row = m0 + r;
-        const int col = n0 + cq * 4;
+        const int col = n0 + cq * 8;
         if (row < M && col < N) {
-            const u32x2_t v = *reinterpret_cast<const u32x2_t*>(lds_c + r * CP + cq * 4);
+            const u32x4_t v = *reinterpret_cast<const u32x4_t*>(lds_c + r * CP + cq * 8);
             uint16_t* dst = C + (int64_t)row * ldc + col;
-            if (vec_ok && col + 4 <= N) {
-                *reinterpret_cast<u32x2_t*>(dst) = v;
+            if (vec16 && col + 8 <= N) {
+                *reinterpret_cast<u32x4_t*>(dst) = v;
             } else {
-                const uint16_t e[4] = {(uint16_t)(v.x & 0xffffu), (uint16_t)(v.x >> 16), (uint16_t)(v.y & 0xffffu),
-                                       (uint16_t)(v.y >> 16)};
+                const uint32_t w[4] = {v.x, v.y, v.z, v.w};
 #pragma unroll
-                for (int i = 0; i < 4; ++i)
-                    if (col + i < N) dst[i] = e[i];
+                for (int i = 0; i < 8; ++i)
+                    if (col + i < N) dst[i] = (uint16_t)(w[i >> 1] >> ((i & 1) * 16));
             }
         }
     }
 }
 
-// Epilogue shared by the block-GEMM kernels: adds the addends and the bias to
-// the fp32 accumulators, optionally stores the pre-activation, applies the
-// activation, packs to bf16, stages the tile in LDS (which must be free: all
-// waves past their last operand read) and writes it out row by row.
+// Epilogue shared by the block-GEMM kernels: value = acc + addends + bias,
+// optionally stored as the pre-activation, then activation, bf16 packing,
+// staging of the tile in LDS (which must be free: all waves past their last
+// operand read) and row-wise stores. The accumulators are only read (one
+// 32x32 MFMA tile at a time), never written back.
 // acc[i][j][v]: row  m = m0 + wm*(BM/2) + i*32 + (lane & 31)
 //               col  n = n0 + wn*(BN/2) + j*32 + 8*(v/4) + 4*(lane>>5) + (v%4)
-template <int BM, int BN, int TM, int TN, int EPI>
-__device__ __forceinline__ void gemm_epilogue(f32x16_t (&acc)[TM][TN], const GemmArgs& args, uint16_t* lds, int m0,
+// FAST: the tile is entirely in bounds and every pointer / leading dimension
+// allows the vector accesses (checked on the host): no per-element guards.
+template <int BM, int BN, int TM, int TN, int EPI, bool FAST, typename Args>
+__device__ __forceinline__ void gemm_epilogue(f32x16_t (&acc)[TM][TN], const Args& args, uint16_t* lds, int m0,
                                               int n0, int wm, int wn, int lane, int tid) {
     constexpr int WTM = BM / 2, WTN = BN / 2;
+    constexpr int CP = c_pitch<BN>();
     const int M = args.M, N = args.N;
-    constexpr int CP = BN + 4;
-    uint16_t* lds_c = lds;  // the operand stages are dead after the last barrier
+    uint16_t* lds_c = lds;
     const int row_l = wm * WTM + (lane & 31);
     const int col_l = wn * WTN + 4 * (lane >> 5);
-    const bool vec_c = args.vec_c != 0;
     const uint16_t* bias = reinterpret_cast<const uint16_t*>(args.bias);
+    const bool use_bias = (EPI != CW_EPI_NONE) && bias != nullptr;
 
-    if (args.n_addends > 0 || (EPI != CW_EPI_NONE && bias != nullptr)) {
+    auto stage_tile = [&](auto activated) {
+        constexpr bool ACT = decltype(activated)::value;
 #pragma unroll
-        for (int j = 0; j < TN; ++j)
+        for (int j = 0; j < TN; ++j) {
+            float bv[4][4];
 #pragma unroll
             for (int g = 0; g < 4; ++g) {
                 const int ncol = n0 + col_l + j * 32 + 8 * g;
-                float bv[4] = {0.0f, 0.0f, 0.0f, 0.0f};
-                if (EPI != CW_EPI_NONE && bias != nullptr && ncol < N)
-                    load4_bf16(bias + ncol, N - ncol, args.vec_bias != 0, bv);
+                if (use_bias && (FAST || ncol < N)) {
+                    load4_bf16(bias + ncol, FAST ? 4 : N - ncol, FAST || args.vec_bias != 0, bv[g]);
+                } else {
 #pragma unroll
-                for (int i = 0; i < TM; ++i) {
-                    const int mrow = m0 + row_l + i * 32;
-                    float add[4] = {bv[0], bv[1], bv[2], bv[3]};
-                    if (args.n_addends > 0 && mrow < M && ncol < N) {
-                        for (int a = 0; a < args.n_addends; ++a) {
-                            float t[4];
-                            load4_bf16(reinterpret_cast<const uint16_t*>(args.addend[a]) + (int64_t)mrow * args.ldadd + ncol,
-                                       N - ncol, args.vec_add != 0, t);
-#pragma unroll
-                            for (int e = 0; e < 4; ++e) add[e] += t[e];
-                        }
-                    }
-#pragma unroll
-                    for (int e = 0; e < 4; ++e) acc[i][j][4 * g + e] += add[e];
+                    for (int e = 0; e < 4; ++e) bv[g][e] = 0.0f;
                 }
             }
-    }
-
-    auto stage_tile = [&](bool activated) {
 #pragma unroll
-        for (int i = 0; i < TM; ++i)
-#pragma unroll
-            for (int j = 0; j < TN; ++j)
+            for (int i = 0; i < TM; ++i) {
+                const int mrow = m0 + row_l + i * 32;
 #pragma unroll
                 for (int g = 0; g < 4; ++g) {
+                    const int ncol = n0 + col_l + j * 32 + 8 * g;
                     float v[4];
 #pragma unroll
-                    for (int e = 0; e < 4; ++e) {
-                        const float x = acc[i][j][4 * g + e];
-                        v[e] = activated ? epi_act<EPI>(x) : x;
+                    for (int e = 0; e < 4; ++e) v[e] = acc[i][j][4 * g + e] + bv[g][e];
+                    if (args.n_addends > 0 && (FAST || (mrow < M && ncol < N))) {
+#pragma unroll 1
+                        for (int a = 0; a < args.n_addends; ++a) {
+                            float t[4];
+                            load4_bf16(reinterpret_cast<const uint16_t*>(pick_ptr(args.addend, a)) + (int64_t)mrow * args.ldadd + ncol,
+                                       FAST ? 4 : N - ncol, FAST || args.vec_add != 0, t);
+#pragma unroll
+                            for (int e = 0; e < 4; ++e) v[e] += t[e];
+                        }
+                    }
+                    if constexpr (ACT) {
+#pragma unroll
+                        for (int e = 0; e < 4; ++e) v[e] = epi_act<EPI>(v[e]);
                     }
                     u32x2_t p;
                     p.x = pack_bf16x2(v[0], v[1]);
                     p.y = pack_bf16x2(v[2], v[3]);
                     *reinterpret_cast<u32x2_t*>(lds_c + (row_l + i * 32) * CP + col_l + j * 32 + 8 * g) = p;
                 }
+            }
+        }
     };
 
     if (args.preact != nullptr) {
-        stage_tile(false);
+        stage_tile(std::false_type{});
         __syncthreads();
-        tile_store<BM, BN>(lds_c, reinterpret_cast<uint16_t*>(args.preact), args.ldp, m0, n0, M, N, tid,
-                           args.vec_p != 0);
+        tile_store<BM, BN, FAST>(lds_c, reinterpret_cast<uint16_t*>(args.preact), args.ldp, m0, n0, M, N, tid);
         __syncthreads();
     }
-    stage_tile(true);
+    stage_tile(std::true_type{});
     __syncthreads();
-    tile_store<BM, BN>(lds_c, reinterpret_cast<uint16_t*>(args.C), args.ldc, m0, n0, M, N, tid, vec_c);
+    tile_store<BM, BN, FAST>(lds_c, reinterpret_cast<uint16_t*>(args.C), args.ldc, m0, n0, M, N, tid);
 }
 
 template <int BM, int BN, bool TRANS_A, bool TRANS_B, bool GUARD, int EPI>
@@ -411,13 +440,13 @@ __global__ __launch_bounds__(kThreads) void gemm_bf16_kernel(const GemmArgs args
         __syncthreads();
     }
 
-    gemm_epilogue<BM, BN, TM, TN, EPI>(acc, args, lds, m0, n0, wm, wn, lane, tid);
+    gemm_epilogue<BM, BN, TM, TN, EPI, !GUARD>(acc, args, lds, m0, n0, wm, wn, lane, tid);
 }
 
 template <int BM, int BN>
 constexpr size_t lds_bytes() {
     const size_t stages = 2u * (BM + BN) * kPitch * sizeof(uint16_t);
-    const size_t ctile = (size_t)BM * (BN + 4) * sizeof(uint16_t);
+    const size_t ctile = (size_t)BM * c_pitch<BN>() * sizeof(uint16_t);
     return stages > ctile ? stages : ctile;
 }
 
