@@ -33,6 +33,21 @@ M, N, K, STEPS_K = 8192, 2048, 2048, 2
 GEMM_FLOP = 2 * M * N * K * STEPS_K
 
 
+def measured_traffic():
+    """Bytes per launch that cross the L2 <-> fabric boundary for the GEMM kernel, from the committed
+    hardware-counter summary (two rocprofv3 --pmc runs of this script, scaled by a plain copy of known
+    size); None when the summary is not there."""
+    import re
+    path = os.path.join(os.path.dirname(os.path.abspath(__file__)), "profiles",
+                        "gemm_bf16_dma_kernel_linear2d_q2_counters.txt")
+    try:
+        with open(path) as f:
+            m = re.search(r"^traffic_bytes_per_launch:\s*(\d+)", f.read(), re.M)
+        return int(m.group(1)) if m else None
+    except OSError:
+        return None
+
+
 def _seeded(shape, seed, std, dtype):
     import torch
     g = torch.Generator().manual_seed(seed)
@@ -52,26 +67,39 @@ def make_gemm_inputs(n_sets, device):
     return sets, bias
 
 
-def event_time_us(fn, iters, warmup):
-    """Average duration of fn() per call from events on the current stream."""
+def graph_time_us(fn, calls, replays=3):
+    """Average duration of one fn() call when `calls` of them are replayed from
+    a HIP graph: the host cost of the Python wrappers (tens of microseconds,
+    more than these kernels run) stays outside the timed region, which is
+    bracketed by events on the replay stream."""
     import torch
-    for _ in range(warmup):
-        fn()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        for _ in range(3):
+            fn()
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        for _ in range(calls):
+            fn()
+    graph.replay()
     torch.cuda.synchronize()
     e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
     e0.record()
-    for _ in range(iters):
-        fn()
+    for _ in range(replays):
+        graph.replay()
     e1.record()
     torch.cuda.synchronize()
-    return e0.elapsed_time(e1) * 1e3 / iters
+    return e0.elapsed_time(e1) * 1e3 / (replays * calls)
 
 
 def bench_bandwidth_kernels(device):
     """LayerNorm2D (config 3) and vocab-parallel CE (config 4) kernels: algorithmic
     bytes per launch / average launch duration. Each call below is one C-ABI
-    entry point; outputs are preallocated by the wrappers per call (torch's
-    caching allocator, no device malloc in the loop after warm-up)."""
+    entry point (cw_ln_bwd_partials launches its partials kernel and a small
+    finalize kernel); the launches are replayed from a HIP graph."""
     import torch
     from cubework_amd import ops
 
@@ -100,7 +128,7 @@ def bench_bandwidth_kernels(device):
         ("ln_bwd_dx", 3 * 33554432 + 2 * 131072 + 2048, lambda: ops.ln_bwd_dx(rot(dys), xs[i[0] % nb], mr, rs, H, gamma)),
     ]
     for name, nbytes, fn in cases:
-        us = event_time_us(fn, 51, 6)
+        us = graph_time_us(fn, 2 * nb)
         out[name] = {"us": round(us, 2), "GBps": round(nbytes / us / 1e3, 1), "frac": round(nbytes / us / 1e3 / HBM_PEAK_GBPS, 3),
                      "bytes": nbytes}
     del xs, dys
@@ -116,7 +144,7 @@ def bench_bandwidth_kernels(device):
          lambda: ops.vpce_bwd(rot(lg), tg, V0, gmax, gsum, None, 1.0 / T, grad_dtype=torch.float32)),
     ]
     for name, nbytes, fn in cases:
-        us = event_time_us(fn, 15, 3)
+        us = graph_time_us(fn, 6)
         out[name] = {"us": round(us, 2), "GBps": round(nbytes / us / 1e3, 1), "frac": round(nbytes / us / 1e3 / HBM_PEAK_GBPS, 3),
                      "bytes": nbytes}
     return out
@@ -182,6 +210,9 @@ def main():
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--no-aux", action="store_true", help="skip the LayerNorm / CE kernels")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="also run a plain 256 MiB device copy three times (the known-size kernel that hardware "
+                         "counter runs of this script are scaled by)")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         sys.stderr.write("bench.py measures one rank's share on ONE GPU; --gpus N with N > 1 is not part of this "
@@ -241,9 +272,16 @@ def main():
                                "2 SUMMA k-steps accumulated in fp32, fused bias+GeLU(tanh), out [8192,2048] bf16",
                    "layout": "NN", "flop_per_step": GEMM_FLOP, "operand_sets_rotated": n_sets, "device_arch": arch},
         "roofline": {"bound": "mfma", "achieved": round(achieved, 2), "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
-                     "frac": round(achieved / MFMA_BF16_PEAK_TFLOPS, 4), "traffic": None,
-                     "kernel": "gemm_bf16_kernel<256,256,NN,bias+gelu_tanh>", "avg_launch_us": round(kernel_us, 2)},
+                     "frac": round(achieved / MFMA_BF16_PEAK_TFLOPS, 4), "traffic": measured_traffic(),
+                     "kernel": "gemm_bf16_dma_kernel<NN, bias+gelu_tanh, 4 stages> (256x256x32 tiles)", "avg_launch_us": round(kernel_us, 2)},
     }
+    if args.calibrate_copy:
+        src = torch.empty(256 << 20, dtype=torch.uint8, device=device).fill_(1)
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        del src, dst
     if not args.no_aux:
         result["aux"] = bench_bandwidth_kernels(device)
         result["aux"]["hbm_peak_GBps"] = HBM_PEAK_GBPS

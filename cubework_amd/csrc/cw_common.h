@@ -81,16 +81,87 @@ __device__ __forceinline__ void store_vec(float* p, const float (&v)[4]) {
     *reinterpret_cast<float4*>(p) = make_float4(v[0], v[1], v[2], v[3]);
 }
 
+// ---- raw 16-byte moves for streaming kernels -----------------------------
+// Data that a kernel touches exactly once goes through non-temporal loads and
+// stores, which do not displace reusable lines from the caches.
+typedef uint32_t raw16_t __attribute__((ext_vector_type(4)));
+
+__device__ __forceinline__ raw16_t load_raw(const void* p) { return *reinterpret_cast<const raw16_t*>(p); }
+__device__ __forceinline__ raw16_t load_raw_stream(const void* p) {
+    return __builtin_nontemporal_load(reinterpret_cast<const raw16_t*>(p));
+}
+__device__ __forceinline__ void store_raw_stream(void* p, raw16_t u) {
+    __builtin_nontemporal_store(u, reinterpret_cast<raw16_t*>(p));
+}
+__device__ __forceinline__ void unpack_raw(raw16_t u, float (&v)[8], const bf16_t*) {
+    v[0] = __uint_as_float(u.x << 16);
+    v[1] = __uint_as_float(u.x & 0xffff0000u);
+    v[2] = __uint_as_float(u.y << 16);
+    v[3] = __uint_as_float(u.y & 0xffff0000u);
+    v[4] = __uint_as_float(u.z << 16);
+    v[5] = __uint_as_float(u.z & 0xffff0000u);
+    v[6] = __uint_as_float(u.w << 16);
+    v[7] = __uint_as_float(u.w & 0xffff0000u);
+}
+__device__ __forceinline__ void unpack_raw(raw16_t u, float (&v)[4], const float*) {
+    v[0] = __uint_as_float(u.x);
+    v[1] = __uint_as_float(u.y);
+    v[2] = __uint_as_float(u.z);
+    v[3] = __uint_as_float(u.w);
+}
+__device__ __forceinline__ raw16_t pack_raw(const float (&v)[8], const bf16_t*) {
+    raw16_t u;
+    u.x = pack_bf16x2(v[0], v[1]);
+    u.y = pack_bf16x2(v[2], v[3]);
+    u.z = pack_bf16x2(v[4], v[5]);
+    u.w = pack_bf16x2(v[6], v[7]);
+    return u;
+}
+__device__ __forceinline__ raw16_t pack_raw(const float (&v)[4], const float*) {
+    raw16_t u;
+    u.x = __float_as_uint(v[0]);
+    u.y = __float_as_uint(v[1]);
+    u.z = __float_as_uint(v[2]);
+    u.w = __float_as_uint(v[3]);
+    return u;
+}
+
 // ---- wavefront (64 lanes) reductions ------------------------------------
+// Within a row of 16 lanes the partner values come through DPP operand
+// modifiers of the adds themselves (no LDS traffic); the four row results are
+// combined through lane reads. Every lane returns the same bits.
+template <int CTRL>
+__device__ __forceinline__ float dpp_move(float v) {
+    return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, 0xF, 0xF, true));
+}
+constexpr int kDppXor1 = 0xB1;         // quad_perm [1,0,3,2]
+constexpr int kDppXor2 = 0x4E;         // quad_perm [2,3,0,1]
+constexpr int kDppHalfMirror = 0x141;  // lane i <-> 7-i of each 8
+constexpr int kDppMirror = 0x140;      // lane i <-> 15-i of each 16
+
 __device__ __forceinline__ float wave_sum(float v) {
-#pragma unroll
-    for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off, 64);
-    return v;
+    v += dpp_move<kDppXor1>(v);
+    v += dpp_move<kDppXor2>(v);
+    v += dpp_move<kDppHalfMirror>(v);
+    v += dpp_move<kDppMirror>(v);
+    const int iv = __float_as_int(v);
+    const float r0 = __int_as_float(__builtin_amdgcn_readlane(iv, 0));
+    const float r1 = __int_as_float(__builtin_amdgcn_readlane(iv, 16));
+    const float r2 = __int_as_float(__builtin_amdgcn_readlane(iv, 32));
+    const float r3 = __int_as_float(__builtin_amdgcn_readlane(iv, 48));
+    return (r0 + r1) + (r2 + r3);
 }
 __device__ __forceinline__ float wave_max(float v) {
-#pragma unroll
-    for (int off = 32; off > 0; off >>= 1) v = fmaxf(v, __shfl_xor(v, off, 64));
-    return v;
+    v = fmaxf(v, dpp_move<kDppXor1>(v));
+    v = fmaxf(v, dpp_move<kDppXor2>(v));
+    v = fmaxf(v, dpp_move<kDppHalfMirror>(v));
+    v = fmaxf(v, dpp_move<kDppMirror>(v));
+    const int iv = __float_as_int(v);
+    const float r0 = __int_as_float(__builtin_amdgcn_readlane(iv, 0));
+    const float r1 = __int_as_float(__builtin_amdgcn_readlane(iv, 16));
+    const float r2 = __int_as_float(__builtin_amdgcn_readlane(iv, 32));
+    const float r3 = __int_as_float(__builtin_amdgcn_readlane(iv, 48));
+    return fmaxf(fmaxf(r0, r1), fmaxf(r2, r3));
 }
 
 constexpr float kLog2e = 1.4426950408889634f;
@@ -114,11 +185,18 @@ __device__ __forceinline__ float gelu_tanh(float x) {
     return x * __builtin_amdgcn_rcpf(1.0f + e);
 }
 __device__ __forceinline__ float gelu_tanh_grad(float x) {
+    // gelu = x s with s = sigmoid(2u), u = k0 (x + k1 x^3):
+    // gelu' = s + x s (1 - s) 2u',  2u' = 2 k0 (1 + 3 k1 x^2).
+    // s (1 - s) is formed as s - s*s so that s = 0 (exp2 overflowed) gives 0.
     const float k0 = 0.7978845608028654f, k1 = 0.044715f;
-    const float u = k0 * (x + k1 * x * x * x);
-    const float t = tanh_fast(u);
-    const float du = k0 * (1.0f + 3.0f * k1 * x * x);
-    return 0.5f * (1.0f + t) + 0.5f * x * (1.0f - t * t) * du;
+    const float a = -2.0f * k0 * kLog2e;
+    const float b = a * k1;
+    const float x2 = x * x;
+    const float e = __builtin_amdgcn_exp2f(x * __builtin_fmaf(x2, b, a));
+    const float s = __builtin_amdgcn_rcpf(1.0f + e);
+    const float ds = __builtin_fmaf(-s, s, s);
+    const float up = __builtin_fmaf(x2, 6.0f * k0 * k1, 2.0f * k0);
+    return __builtin_fmaf(x * ds, up, s);
 }
 __device__ __forceinline__ float gelu_erf(float x) { return 0.5f * x * (1.0f + erff(x * 0.7071067811865476f)); }
 __device__ __forceinline__ float gelu_erf_grad(float x) {
@@ -133,6 +211,13 @@ __device__ __forceinline__ float apply_act(float x) {
     if constexpr (ACT == CW_ACT_GELU_ERF) return gelu_erf(x);
     if constexpr (ACT == CW_ACT_RELU) return x > 0.0f ? x : 0.0f;
     return x;
+}
+template <int ACT>
+__device__ __forceinline__ float act_grad_of(float x) {
+    if constexpr (ACT == CW_ACT_GELU_TANH) return gelu_tanh_grad(x);
+    if constexpr (ACT == CW_ACT_GELU_ERF) return gelu_erf_grad(x);
+    if constexpr (ACT == CW_ACT_RELU) return x > 0.0f ? 1.0f : 0.0f;
+    return 1.0f;
 }
 __device__ __forceinline__ float act_grad(int act, float x) {
     switch (act) {

@@ -3,6 +3,8 @@
 // tile of 64 vectors of columns, lanes keep their columns' sums in registers,
 // wavefronts are combined in a fixed-order LDS tree, slabs by a finalize
 // kernel (no atomics: bit-reproducible).
+#include <type_traits>
+
 #include "cw_common.h"
 #include "reduce_cols.h"
 
@@ -10,13 +12,16 @@ namespace cw {
 
 namespace {
 
-constexpr int kColWaves = 16;  // 1024 threads per block on the vector path
+constexpr int kColWaves = 4;   // wavefronts per block on the vector path, each on its own rows
+constexpr int kColUnroll = 4;  // rows in flight per wavefront
+constexpr int64_t kColBlocks = 1024;  // blocks aimed at (4 resident per compute unit)
 constexpr int64_t kGenericSlabRows = 64;
 
-template <typename T, int MODE>
+// MODE 0: column sums of dY. MODE 1: dPre = dY * ACT'(pre), column sums of dPre.
+template <typename T, int MODE, int ACT>
 __global__ __launch_bounds__(kColWaves * 64) void colsum_vec_kernel(
     int64_t M, int64_t N, const T* __restrict__ dY, int64_t ld_dy, const T* __restrict__ pre, int64_t ld_pre,
-    T* __restrict__ dPre, int64_t ld_dpre, int act, float* __restrict__ ws, int64_t rows_per_slab, int want_sum) {
+    T* __restrict__ dPre, int64_t ld_dpre, float* __restrict__ ws, int64_t rows_per_slab, int want_sum) {
     constexpr int V = elem<T>::kVec;
     extern __shared__ float lds_red[];
     const int lane = threadIdx.x & 63;
@@ -29,18 +34,34 @@ __global__ __launch_bounds__(kColWaves * 64) void colsum_vec_kernel(
 #pragma unroll
     for (int e = 0; e < V; ++e) acc[e] = 0.0f;
     if (valid) {
-        for (int64_t row = r0 + wave; row < r1; row += kColWaves) {
-            float dy[V];
-            load_vec(dY + row * ld_dy + c0, dy);
-            if constexpr (MODE == 1) {
-                float p[V];
-                load_vec(pre + row * ld_pre + c0, p);
+        // kColUnroll rows per wavefront are in flight at a time. The loads are
+        // unconditional (a row past the slab reads the slab's last row and is
+        // then dropped): loads under a branch would wait for one another.
+        for (int64_t row = r0 + wave; row < r1; row += kColWaves * kColUnroll) {
+            raw16_t d_raw[kColUnroll], p_raw[kColUnroll];
 #pragma unroll
-                for (int e = 0; e < V; ++e) dy[e] *= act_grad(act, p[e]);
-                store_vec(dPre + row * ld_dpre + c0, dy);
+            for (int u = 0; u < kColUnroll; ++u) {
+                const int64_t rr = row + u * kColWaves;
+                const int64_t rc = rr < r1 ? rr : r1 - 1;
+                d_raw[u] = load_raw_stream(dY + rc * ld_dy + c0);
+                if constexpr (MODE == 1) p_raw[u] = load_raw_stream(pre + rc * ld_pre + c0);
             }
 #pragma unroll
-            for (int e = 0; e < V; ++e) acc[e] += dy[e];
+            for (int u = 0; u < kColUnroll; ++u) {
+                const int64_t rr = row + u * kColWaves;
+                const bool live = rr < r1;
+                float dy[V];
+                unpack_raw(d_raw[u], dy, (const T*)nullptr);
+                if constexpr (MODE == 1) {
+                    float p[V];
+                    unpack_raw(p_raw[u], p, (const T*)nullptr);
+#pragma unroll
+                    for (int e = 0; e < V; ++e) dy[e] *= act_grad_of<ACT>(p[e]);
+                    if (live) store_raw_stream(dPre + rr * ld_dpre + c0, pack_raw(dy, (const T*)nullptr));
+                }
+#pragma unroll
+                for (int e = 0; e < V; ++e) acc[e] += live ? dy[e] : 0.0f;
+            }
         }
     }
     if (!want_sum) return;
@@ -75,11 +96,14 @@ __global__ __launch_bounds__(256) void colsum_generic_kernel(int64_t M, int64_t 
     if (want_sum) ws[(int64_t)blockIdx.y * N + c] = acc;
 }
 
-// grid (ceil(C/64), nsets); 4 groups of 64 threads split the partials.
-__global__ __launch_bounds__(256) void finalize_cols_kernel(const float* __restrict__ ws, int64_t nparts,
-                                                            int64_t part_stride, int64_t C, float* __restrict__ out0,
-                                                            float* __restrict__ out1) {
-    __shared__ float red[4][64];
+// grid (ceil(C/64), nsets); 16 groups of 64 threads split the partials, each
+// with 16 independent loads in flight, and are combined in a fixed order.
+constexpr int kFinGroups = 16;
+__global__ __launch_bounds__(kFinGroups * 64) void finalize_cols_kernel(const float* __restrict__ ws, int64_t nparts,
+                                                                        int64_t part_stride, int64_t C,
+                                                                        float* __restrict__ out0,
+                                                                        float* __restrict__ out1) {
+    __shared__ float red[kFinGroups][64];
     const int lane = threadIdx.x & 63;
     const int grp = threadIdx.x >> 6;
     const int64_t c = (int64_t)blockIdx.x * 64 + lane;
@@ -87,12 +111,25 @@ __global__ __launch_bounds__(256) void finalize_cols_kernel(const float* __restr
     float acc = 0.0f;
     if (c < C) {
         const float* base = ws + (int64_t)k * C + c;
-        for (int64_t p = grp; p < nparts; p += 4) acc += base[p * part_stride];
+        // 16 loads in flight per batch; indices past the end re-read the last
+        // partial and are dropped, so no load waits behind a branch.
+        for (int64_t p = grp; p < nparts; p += 16 * kFinGroups) {
+            float v[16];
+#pragma unroll
+            for (int u = 0; u < 16; ++u) {
+                const int64_t q = p + u * kFinGroups;
+                v[u] = base[(q < nparts ? q : nparts - 1) * part_stride];
+            }
+#pragma unroll
+            for (int u = 0; u < 16; ++u) acc += (p + u * kFinGroups < nparts) ? v[u] : 0.0f;
+        }
     }
     red[grp][lane] = acc;
     __syncthreads();
     if (grp == 0 && c < C) {
-        const float total = ((red[0][lane] + red[1][lane]) + red[2][lane]) + red[3][lane];
+        float total = red[0][lane];
+#pragma unroll
+        for (int g = 1; g < kFinGroups; ++g) total += red[g][lane];
         float* out = (k == 0) ? out0 : out1;
         if (out != nullptr) out[c] = total;
     }
@@ -108,18 +145,26 @@ int colsum_impl(int64_t M, int64_t N, const void* dY, int64_t ld_dy, const void*
     int64_t slabs, rows_per_slab;
     if (vec) {
         const int64_t coltiles = (N + 64 * V - 1) / (64 * V);
-        slabs = 512 / coltiles;
-        const int64_t max_slabs = (M + kColWaves - 1) / kColWaves;
+        slabs = kColBlocks / coltiles;
+        const int64_t max_slabs = (M + kColWaves * kColUnroll - 1) / (kColWaves * kColUnroll);
         if (slabs > max_slabs) slabs = max_slabs;
+        if (slabs > 512) slabs = 512;  // the bound cw_colsum_workspace_bytes promises
         if (slabs < 1) slabs = 1;
         rows_per_slab = (M + slabs - 1) / slabs;
         slabs = (M + rows_per_slab - 1) / rows_per_slab;
         if (want_sum && workspace_bytes < slabs * N * (int64_t)sizeof(float))
             return fail(CW_ERR_INVALID, "column sum: workspace too small (%lld bytes)", (long long)workspace_bytes);
         const size_t lds = tree_reduce_lds_bytes(V, kColWaves);
-        hipLaunchKernelGGL((colsum_vec_kernel<T, MODE>), dim3((unsigned)coltiles, (unsigned)slabs),
-                           dim3(kColWaves * 64), lds, s, M, N, (const T*)dY, ld_dy, (const T*)pre, ld_pre, (T*)dPre,
-                           ld_dpre, act, (float*)workspace, rows_per_slab, want_sum);
+        const dim3 grid((unsigned)coltiles, (unsigned)slabs), block(kColWaves * 64);
+        auto launch = [&](auto act_c) {
+            constexpr int ACT = decltype(act_c)::value;
+            hipLaunchKernelGGL((colsum_vec_kernel<T, MODE, ACT>), grid, block, lds, s, M, N, (const T*)dY, ld_dy,
+                               (const T*)pre, ld_pre, (T*)dPre, ld_dpre, (float*)workspace, rows_per_slab, want_sum);
+        };
+        if (MODE == 0 || act == CW_ACT_NONE) launch(std::integral_constant<int, CW_ACT_NONE>{});
+        else if (act == CW_ACT_GELU_TANH) launch(std::integral_constant<int, CW_ACT_GELU_TANH>{});
+        else if (act == CW_ACT_GELU_ERF) launch(std::integral_constant<int, CW_ACT_GELU_ERF>{});
+        else launch(std::integral_constant<int, CW_ACT_RELU>{});
     } else {
         rows_per_slab = kGenericSlabRows;
         slabs = (M + rows_per_slab - 1) / rows_per_slab;
@@ -138,7 +183,7 @@ int colsum_impl(int64_t M, int64_t N, const void* dY, int64_t ld_dy, const void*
 
 int finalize_col_partials(const float* ws, int64_t nparts, int64_t part_stride, int nsets, int64_t C, float* out0,
                           float* out1, hipStream_t s) {
-    hipLaunchKernelGGL(finalize_cols_kernel, dim3((unsigned)((C + 63) / 64), (unsigned)nsets), dim3(256), 0, s, ws,
+    hipLaunchKernelGGL(finalize_cols_kernel, dim3((unsigned)((C + 63) / 64), (unsigned)nsets), dim3(kFinGroups * 64), 0, s, ws,
                        nparts, part_stride, C, out0, out1);
     return check_launch("finalize_cols_kernel");
 }

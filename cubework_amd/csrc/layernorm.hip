@@ -5,6 +5,15 @@
 // shuffles, column reductions go through registers -> LDS tree -> a small
 // per-block partial in global memory (no atomics, so results are
 // deterministic).
+//
+// Rows of up to 8 x 64 vectors (bf16: 4096 columns, fp32: 2048) take the
+// "tile" kernels: a wavefront loads NR whole rows into registers with all of
+// its loads in flight at once (non-temporal, each byte is used once), so a
+// row is read from memory exactly once even where two passes over it are
+// needed, and the memory system always sees several KiB outstanding per
+// wavefront. Wider or unaligned rows take the looping kernels below them.
+#include <type_traits>
+
 #include "cw_common.h"
 #include "reduce_cols.h"
 
@@ -13,6 +22,14 @@ namespace cw {
 namespace {
 
 constexpr int kLnBlock = 256;  // 4 wavefronts; one row per wavefront per trip
+
+// Rows a wavefront of the tile kernels holds at a time, by chunks per row, and
+// the resident blocks per compute unit the grid is capped at (measured on
+// 16384 x 1024 bf16: more rows per wavefront cost registers and gained nothing).
+constexpr int kRowsAt1Chunk = 2;
+constexpr int kRowsAt2Chunks = 1;
+constexpr int kRowsAt4Chunks = 1;
+constexpr int kTileBlocksPerCu = 8;
 
 // Sum of (x-mu) and (x-mu)^2 over one row; every lane returns the full sums.
 template <typename T>
@@ -77,7 +94,7 @@ __device__ __forceinline__ void finish_stats(int mode, float s1, float s2, float
         mean = s1;
         var = s2 * inv_h;
     }
-    rstd = 1.0f / sqrtf(var + eps);
+    rstd = __builtin_amdgcn_rsqf(var + eps);  // hardware reciprocal square root, 1 ulp
 }
 
 template <typename T, bool FUSED>
@@ -147,10 +164,244 @@ __global__ __launch_bounds__(kLnBlock) void ln_normalize_kernel(int64_t R, int64
     }
 }
 
+// ---- register-tile kernels ------------------------------------------------
+// Lane l of a wavefront owns columns (j*64 + l)*V .. +V-1, j < NCH, of each of
+// the NR rows the wavefront holds. C % V == 0 and 16-byte aligned rows.
+//
+// Loads are never predicated: a chunk past the end of the row reads column 0
+// and a row past R reads row R-1, then the value is replaced by zero (chunk)
+// or the result is not stored (row). A load under a branch would make the
+// compiler wait for the loads before it, which serialises the memory traffic
+// of the wavefront.
+constexpr int kTileWaves = 4;
+
+template <typename T>
+__device__ __forceinline__ bool chunk_valid(int j, int lane, int64_t C) {
+    return ((int64_t)j * 64 + lane) * elem<T>::kVec < C;
+}
+
+template <typename T, int NCH, int NR>
+struct RowTile {
+    static constexpr int V = elem<T>::kVec;
+    raw16_t raw[NR][NCH];
+
+    __device__ __forceinline__ void load(const T* __restrict__ p, int64_t ld, int64_t row0, int64_t R, int64_t C,
+                                         int lane) {
+#pragma unroll
+        for (int r = 0; r < NR; ++r) {
+            const int64_t row = (row0 + r < R) ? row0 + r : R - 1;
+#pragma unroll
+            for (int j = 0; j < NCH; ++j) {
+                const bool ok = chunk_valid<T>(j, lane, C);
+                const int64_t c0 = ok ? ((int64_t)j * 64 + lane) * V : 0;
+                const raw16_t u = load_raw_stream(p + row * ld + c0);
+                raw[r][j].x = ok ? u.x : 0u;
+                raw[r][j].y = ok ? u.y : 0u;
+                raw[r][j].z = ok ? u.z : 0u;
+                raw[r][j].w = ok ? u.w : 0u;
+            }
+        }
+    }
+
+    // Replaces the rows past R (copies of row R-1) by zeros.
+    __device__ __forceinline__ void zero_dead_rows(int64_t row0, int64_t R) {
+#pragma unroll
+        for (int r = 1; r < NR; ++r) {
+            const bool live = row0 + r < R;
+#pragma unroll
+            for (int j = 0; j < NCH; ++j) {
+                raw[r][j].x = live ? raw[r][j].x : 0u;
+                raw[r][j].y = live ? raw[r][j].y : 0u;
+                raw[r][j].z = live ? raw[r][j].z : 0u;
+                raw[r][j].w = live ? raw[r][j].w : 0u;
+            }
+        }
+    }
+};
+
+// gamma / beta chunks of a lane (zero where absent or past the end).
+template <typename T, int NCH>
+__device__ __forceinline__ void load_param_chunks(const T* __restrict__ p, int64_t C, int lane, raw16_t (&out)[NCH]) {
+#pragma unroll
+    for (int j = 0; j < NCH; ++j) {
+        out[j] = (raw16_t){0u, 0u, 0u, 0u};
+        if (p != nullptr && chunk_valid<T>(j, lane, C)) out[j] = load_raw(p + ((int64_t)j * 64 + lane) * elem<T>::kVec);
+    }
+}
+
+// Sum of (x-mu) and (x-mu)^2 over row r of a tile; every lane gets the sums.
+template <typename T, int NCH, int NR>
+__device__ __forceinline__ void tile_moments(const RowTile<T, NCH, NR>& t, int r, int64_t C, float mu, int lane,
+                                             float& s1, float& s2) {
+    constexpr int V = elem<T>::kVec;
+    float a1 = 0.0f, a2 = 0.0f;
+#pragma unroll
+    for (int j = 0; j < NCH; ++j) {
+        const float mu_j = chunk_valid<T>(j, lane, C) ? mu : 0.0f;  // the zeros of an absent chunk add nothing
+        float v[V];
+        unpack_raw(t.raw[r][j], v, (const T*)nullptr);
+#pragma unroll
+        for (int e = 0; e < V; ++e) {
+            const float d = v[e] - mu_j;
+            a1 += d;
+            a2 += d * d;
+        }
+    }
+    s1 = wave_sum(a1);
+    s2 = wave_sum(a2);
+}
+
+template <typename T, int NCH, int NR>
+__global__ __launch_bounds__(kTileWaves * 64) void ln_stats_tile_kernel(int64_t R, int64_t C,
+                                                                        const T* __restrict__ x, int64_t ld, int mode,
+                                                                        const float* __restrict__ mean,
+                                                                        float* __restrict__ stats) {
+    const int lane = threadIdx.x & 63;
+    const int64_t wave = (int64_t)blockIdx.x * kTileWaves + (threadIdx.x >> 6);
+    const int64_t step = (int64_t)gridDim.x * kTileWaves * NR;
+    const bool centred = mode == CW_LN_TWO_PASS && mean != nullptr;
+    for (int64_t row0 = wave * NR; row0 < R; row0 += step) {
+        RowTile<T, NCH, NR> t;
+        t.load(x, ld, row0, R, C, lane);
+#pragma unroll
+        for (int r = 0; r < NR; ++r) {
+            const int64_t row = row0 + r;
+            const float mu = centred ? mean[row < R ? row : R - 1] : 0.0f;
+            float s1, s2;
+            tile_moments(t, r, C, mu, lane, s1, s2);
+            if (lane == 0 && row < R) {
+                stats[2 * row] = s1;
+                stats[2 * row + 1] = (mode == CW_LN_TWO_PASS && mean == nullptr) ? 0.0f : s2;
+            }
+        }
+    }
+}
+
+template <typename T, int NCH, int NR, bool FUSED>
+__global__ __launch_bounds__(kTileWaves * 64) void ln_normalize_tile_kernel(
+    int64_t R, int64_t C, const T* __restrict__ x, int64_t ld, const float* __restrict__ stats, int mode, float inv_h,
+    float eps, const T* __restrict__ gamma, const T* __restrict__ beta, T* __restrict__ y, int64_t ldy,
+    float* __restrict__ mean_rstd) {
+    constexpr int V = elem<T>::kVec;
+    const int lane = threadIdx.x & 63;
+    const int64_t wave = (int64_t)blockIdx.x * kTileWaves + (threadIdx.x >> 6);
+    const int64_t step = (int64_t)gridDim.x * kTileWaves * NR;
+    raw16_t g_raw[NCH], b_raw[NCH];
+    load_param_chunks<T, NCH>(gamma, C, lane, g_raw);
+    load_param_chunks<T, NCH>(beta, C, lane, b_raw);
+    for (int64_t row0 = wave * NR; row0 < R; row0 += step) {
+        RowTile<T, NCH, NR> t;
+        t.load(x, ld, row0, R, C, lane);
+#pragma unroll
+        for (int r = 0; r < NR; ++r) {
+            const int64_t row = row0 + r;
+            const int64_t row_c = row < R ? row : R - 1;
+            float mean, rstd;
+            if constexpr (FUSED) {
+                float s1, s2;
+                tile_moments(t, r, C, 0.0f, lane, s1, s2);
+                if (mode == CW_LN_TWO_PASS) {
+                    const float mu = s1 * inv_h;
+                    float d1, d2;
+                    tile_moments(t, r, C, mu, lane, d1, d2);
+                    finish_stats(mode, mu, d2, inv_h, eps, mean, rstd);
+                } else {
+                    finish_stats(mode, s1, s2, inv_h, eps, mean, rstd);
+                }
+            } else {
+                finish_stats(mode, stats[2 * row_c], stats[2 * row_c + 1], inv_h, eps, mean, rstd);
+            }
+            if (mean_rstd != nullptr && lane == 0 && row < R) {
+                mean_rstd[2 * row] = mean;
+                mean_rstd[2 * row + 1] = rstd;
+            }
+#pragma unroll
+            for (int j = 0; j < NCH; ++j) {
+                float v[V], g[V], b[V];
+                unpack_raw(t.raw[r][j], v, (const T*)nullptr);
+                unpack_raw(g_raw[j], g, (const T*)nullptr);
+                unpack_raw(b_raw[j], b, (const T*)nullptr);
+#pragma unroll
+                for (int e = 0; e < V; ++e) {
+                    float xh = (v[e] - mean) * rstd;
+                    if (gamma != nullptr) xh *= g[e];
+                    if (beta != nullptr) xh += b[e];
+                    v[e] = xh;
+                }
+                if (row < R && chunk_valid<T>(j, lane, C))
+                    store_raw_stream(y + row * ldy + ((int64_t)j * 64 + lane) * V, pack_raw(v, (const T*)nullptr));
+            }
+        }
+    }
+}
+
+template <typename T, int NCH, int NR>
+__global__ __launch_bounds__(kTileWaves * 64) void ln_bwd_dx_tile_kernel(
+    int64_t R, int64_t C, const T* __restrict__ dY, int64_t ld_dy, const T* __restrict__ x, int64_t ld_x,
+    const float* __restrict__ mean_rstd, const T* __restrict__ gamma, const float* __restrict__ row_sums, float inv_h,
+    T* __restrict__ dx, int64_t ld_dx) {
+    constexpr int V = elem<T>::kVec;
+    const int lane = threadIdx.x & 63;
+    const int64_t wave = (int64_t)blockIdx.x * kTileWaves + (threadIdx.x >> 6);
+    const int64_t step = (int64_t)gridDim.x * kTileWaves * NR;
+    raw16_t g_raw[NCH];
+    load_param_chunks<T, NCH>(gamma, C, lane, g_raw);
+    for (int64_t row0 = wave * NR; row0 < R; row0 += step) {
+        RowTile<T, NCH, NR> tdy, tx;
+        tdy.load(dY, ld_dy, row0, R, C, lane);
+        tx.load(x, ld_x, row0, R, C, lane);
+#pragma unroll
+        for (int r = 0; r < NR; ++r) {
+            const int64_t row = row0 + r;
+            const int64_t row_c = row < R ? row : R - 1;
+            const float mean = mean_rstd[2 * row_c], rstd = mean_rstd[2 * row_c + 1];
+            const float c1 = row_sums[2 * row_c] * inv_h, c2 = row_sums[2 * row_c + 1] * inv_h;
+#pragma unroll
+            for (int j = 0; j < NCH; ++j) {
+                float dy[V], xv[V], g[V];
+                unpack_raw(tdy.raw[r][j], dy, (const T*)nullptr);
+                unpack_raw(tx.raw[r][j], xv, (const T*)nullptr);
+                unpack_raw(g_raw[j], g, (const T*)nullptr);
+#pragma unroll
+                for (int e = 0; e < V; ++e) {
+                    const float xh = (xv[e] - mean) * rstd;
+                    const float gg = gamma != nullptr ? dy[e] * g[e] : dy[e];
+                    dy[e] = (gg - xh * c2 - c1) * rstd;
+                }
+                if (row < R && chunk_valid<T>(j, lane, C))
+                    store_raw_stream(dx + row * ld_dx + ((int64_t)j * 64 + lane) * V, pack_raw(dy, (const T*)nullptr));
+            }
+        }
+    }
+}
+
+// Number of 64-vector chunks a row of C columns spans.
+template <typename T>
+int64_t row_chunks(int64_t C) {
+    return (C + 64 * elem<T>::kVec - 1) / (64 * elem<T>::kVec);
+}
+
+// Calls f(NCH, NR) with compile-time constants chosen for `nch` (<= 8) chunks.
+template <typename F>
+int dispatch_tile(int64_t nch, F&& f) {
+    if (nch <= 1) return f(std::integral_constant<int, 1>{}, std::integral_constant<int, kRowsAt1Chunk>{});
+    if (nch <= 2) return f(std::integral_constant<int, 2>{}, std::integral_constant<int, kRowsAt2Chunks>{});
+    if (nch <= 4) return f(std::integral_constant<int, 4>{}, std::integral_constant<int, kRowsAt4Chunks>{});
+    return f(std::integral_constant<int, 8>{}, std::integral_constant<int, 1>{});
+}
+
+int tile_grid(int64_t R, int nr) {
+    const int64_t rows_per_block = (int64_t)kTileWaves * nr;
+    const int64_t blocks = (R + rows_per_block - 1) / rows_per_block;
+    const int64_t cap = 256 * kTileBlocksPerCu;
+    return (int)(blocks < cap ? (blocks > 0 ? blocks : 1) : cap);
+}
+
 // Backward partials, vector path. Lane `l` owns the columns of chunks
 // (j*64 + l)*V .. +V-1, j < NCH, for every row its wavefront visits, so the
-// dgamma/dbeta accumulators stay in registers for the whole kernel.
-template <typename T, int NCH, int NWAVES>
+// dgamma/dbeta accumulators stay in registers for the whole kernel. A
+// wavefront holds NR rows of dY and x at a time.
+template <typename T, int NCH, int NWAVES, int NR>
 __global__ __launch_bounds__(NWAVES * 64) void ln_bwd_partials_kernel(
     int64_t R, int64_t C, const T* __restrict__ dY, int64_t ld_dy, const T* __restrict__ x, int64_t ld_x,
     const float* __restrict__ mean_rstd, const T* __restrict__ gamma, float* __restrict__ row_sums,
@@ -160,50 +411,48 @@ __global__ __launch_bounds__(NWAVES * 64) void ln_bwd_partials_kernel(
     const int lane = threadIdx.x & 63;
     const int wave = threadIdx.x >> 6;
 
-    float gam[NCH][V];
+    raw16_t g_raw[NCH];
+    load_param_chunks<T, NCH>(gamma, C, lane, g_raw);
     float acc[2 * NCH * V];  // [0, NCH*V): dgamma, [NCH*V, 2*NCH*V): dbeta
-#pragma unroll
-    for (int j = 0; j < NCH; ++j) {
-        const int64_t c0 = ((int64_t)j * 64 + lane) * V;
-        if (gamma != nullptr && c0 < C) {
-            load_vec(gamma + c0, gam[j]);
-        } else {
-#pragma unroll
-            for (int e = 0; e < V; ++e) gam[j][e] = 1.0f;
-        }
-    }
 #pragma unroll
     for (int i = 0; i < 2 * NCH * V; ++i) acc[i] = 0.0f;
 
-    for (int64_t row = (int64_t)blockIdx.x * NWAVES + wave; row < R; row += (int64_t)gridDim.x * NWAVES) {
-        const float mean = mean_rstd[2 * row];
-        const float rstd = mean_rstd[2 * row + 1];
-        const T* dyr = dY + row * ld_dy;
-        const T* xr = x + row * ld_x;
-        float s1 = 0.0f, s2 = 0.0f;
+    const int64_t step = (int64_t)gridDim.x * NWAVES * NR;
+    for (int64_t row0 = ((int64_t)blockIdx.x * NWAVES + wave) * NR; row0 < R; row0 += step) {
+        RowTile<T, NCH, NR> tdy, tx;
+        tdy.load(dY, ld_dy, row0, R, C, lane);
+        tx.load(x, ld_x, row0, R, C, lane);
+        tdy.zero_dead_rows(row0, R);  // a zero dY row adds nothing to the column sums
 #pragma unroll
-        for (int j = 0; j < NCH; ++j) {
-            const int64_t c0 = ((int64_t)j * 64 + lane) * V;
-            if (c0 < C) {
-                float dy[V], xv[V];
-                load_vec(dyr + c0, dy);
-                load_vec(xr + c0, xv);
+        for (int r = 0; r < NR; ++r) {
+            const int64_t row = row0 + r;
+            const int64_t row_c = row < R ? row : R - 1;
+            const float mean = mean_rstd[2 * row_c];
+            const float rstd = mean_rstd[2 * row_c + 1];
+            float s1 = 0.0f, s2 = 0.0f;
+#pragma unroll
+            for (int j = 0; j < NCH; ++j) {
+                float dy[V], xv[V], g[V];
+                unpack_raw(tdy.raw[r][j], dy, (const T*)nullptr);
+                unpack_raw(tx.raw[r][j], xv, (const T*)nullptr);
+                unpack_raw(g_raw[j], g, (const T*)nullptr);
 #pragma unroll
                 for (int e = 0; e < V; ++e) {
+                    const float d = dy[e];
                     const float xh = (xv[e] - mean) * rstd;
-                    const float g = dy[e] * gam[j][e];
-                    s1 += g;
-                    s2 += g * xh;
-                    acc[j * V + e] += dy[e] * xh;
-                    acc[NCH * V + j * V + e] += dy[e];
+                    const float gd = gamma != nullptr ? d * g[e] : d;
+                    s1 += gd;
+                    s2 += gd * xh;
+                    acc[j * V + e] += d * xh;
+                    acc[NCH * V + j * V + e] += d;
                 }
             }
-        }
-        s1 = wave_sum(s1);
-        s2 = wave_sum(s2);
-        if (lane == 0) {
-            row_sums[2 * row] = s1;
-            row_sums[2 * row + 1] = s2;
+            s1 = wave_sum(s1);
+            s2 = wave_sum(s2);
+            if (lane == 0 && row < R) {
+                row_sums[2 * row] = s1;
+                row_sums[2 * row + 1] = s2;
+            }
         }
     }
     if (!want_cols) return;
@@ -327,6 +576,7 @@ __global__ __launch_bounds__(kLnBlock) void ln_bwd_dx_kernel(int64_t R, int64_t 
     }
 }
 
+
 int ln_grid(int64_t R) {
     const int64_t blocks = (R + (kLnBlock / 64) - 1) / (kLnBlock / 64);
     const int64_t cap = 256 * 8;  // 8 resident blocks of 4 wavefronts per CU
@@ -342,6 +592,15 @@ template <typename T>
 int stats_impl(int64_t R, int64_t C, const void* x, int64_t ld, int mode, const float* mean, float* stats,
                hipStream_t s) {
     const int vec_ok = rows_vec_ok<T>(x, ld);
+    const int64_t nch = row_chunks<T>(C);
+    if (vec_ok && (C % elem<T>::kVec) == 0 && nch <= 8) {
+        return dispatch_tile(nch, [&](auto nch_c, auto nr_c) {
+            constexpr int NCH = decltype(nch_c)::value, NR = decltype(nr_c)::value;
+            hipLaunchKernelGGL((ln_stats_tile_kernel<T, NCH, NR>), dim3(tile_grid(R, NR)), dim3(kTileWaves * 64), 0,
+                               s, R, C, (const T*)x, ld, mode, mean, stats);
+            return check_launch("ln_stats_tile_kernel");
+        });
+    }
     hipLaunchKernelGGL(ln_stats_kernel<T>, dim3(ln_grid(R)), dim3(kLnBlock), 0, s, R, C, (const T*)x, ld, mode,
                        mean, stats, vec_ok);
     return check_launch("ln_stats_kernel");
@@ -353,6 +612,16 @@ int normalize_impl(int64_t R, int64_t C, const void* x, int64_t ld, const float*
                    hipStream_t s) {
     const int vec_ok = rows_vec_ok<T>(x, ld) && rows_vec_ok<T>(y, ldy) && (gamma == nullptr || aligned16(gamma)) &&
                        (beta == nullptr || aligned16(beta));
+    const int64_t nch = row_chunks<T>(C);
+    if (vec_ok && (C % elem<T>::kVec) == 0 && nch <= 8) {
+        return dispatch_tile(nch, [&](auto nch_c, auto nr_c) {
+            constexpr int NCH = decltype(nch_c)::value, NR = decltype(nr_c)::value;
+            hipLaunchKernelGGL((ln_normalize_tile_kernel<T, NCH, NR, FUSED>), dim3(tile_grid(R, NR)),
+                               dim3(kTileWaves * 64), 0, s, R, C, (const T*)x, ld, stats, mode, 1.0f / (float)H, eps,
+                               (const T*)gamma, (const T*)beta, (T*)y, ldy, mean_rstd);
+            return check_launch("ln_normalize_tile_kernel");
+        });
+    }
     hipLaunchKernelGGL((ln_normalize_kernel<T, FUSED>), dim3(ln_grid(R)), dim3(kLnBlock), 0, s, R, C, (const T*)x,
                        ld, stats, mode, 1.0f / (float)H, eps, (const T*)gamma, (const T*)beta, (T*)y, ldy,
                        mean_rstd, vec_ok);
@@ -367,14 +636,14 @@ int64_t bwd_blocks(int64_t R, int nwaves) {
     return nb;
 }
 
-template <typename T, int NCH, int NWAVES>
+template <typename T, int NCH, int NWAVES, int NR>
 int bwd_partials_launch(int64_t R, int64_t C, const void* dY, int64_t ld_dy, const void* x, int64_t ld_x,
                         const float* mean_rstd, const void* gamma, float* row_sums, float* ws, int want_cols,
                         hipStream_t s) {
     constexpr int V = elem<T>::kVec;
-    const int64_t nb = bwd_blocks(R, NWAVES);
+    const int64_t nb = bwd_blocks(R, NWAVES * NR);
     const size_t lds = tree_reduce_lds_bytes(2 * NCH * V, NWAVES);
-    auto kern = ln_bwd_partials_kernel<T, NCH, NWAVES>;
+    auto kern = ln_bwd_partials_kernel<T, NCH, NWAVES, NR>;
     if (lds > 48 * 1024) {
         hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
         if (e != hipSuccess) return fail(CW_ERR_LAUNCH, "hipFuncSetAttribute(ln_bwd_partials): %s", hipGetErrorString(e));
@@ -398,19 +667,19 @@ int bwd_partials_impl(int64_t R, int64_t C, const void* dY, int64_t ld_dy, const
     int64_t nparts = 0;
     int rc;
     if (vec && nch <= 8) {
-        int nwaves = nch <= 2 ? 16 : (nch <= 4 ? 8 : 4);
-        nparts = bwd_blocks(R, nwaves);
+        const int rows_per_trip = nch <= 1 ? 16 * 2 : (nch <= 2 ? 16 : (nch <= 4 ? 8 : 4));
+        nparts = bwd_blocks(R, rows_per_trip);
         if (want_cols && workspace_bytes < nparts * 2 * C * (int64_t)sizeof(float))
             return fail(CW_ERR_INVALID, "cw_ln_bwd_partials: workspace too small (%lld bytes)", (long long)workspace_bytes);
         float* ws = (float*)workspace;
         if (nch <= 1)
-            rc = bwd_partials_launch<T, 1, 16>(R, C, dY, ld_dy, x, ld_x, mean_rstd, gamma, row_sums, ws, want_cols, s);
+            rc = bwd_partials_launch<T, 1, 16, 2>(R, C, dY, ld_dy, x, ld_x, mean_rstd, gamma, row_sums, ws, want_cols, s);
         else if (nch <= 2)
-            rc = bwd_partials_launch<T, 2, 16>(R, C, dY, ld_dy, x, ld_x, mean_rstd, gamma, row_sums, ws, want_cols, s);
+            rc = bwd_partials_launch<T, 2, 16, 1>(R, C, dY, ld_dy, x, ld_x, mean_rstd, gamma, row_sums, ws, want_cols, s);
         else if (nch <= 4)
-            rc = bwd_partials_launch<T, 4, 8>(R, C, dY, ld_dy, x, ld_x, mean_rstd, gamma, row_sums, ws, want_cols, s);
+            rc = bwd_partials_launch<T, 4, 8, 1>(R, C, dY, ld_dy, x, ld_x, mean_rstd, gamma, row_sums, ws, want_cols, s);
         else
-            rc = bwd_partials_launch<T, 8, 4>(R, C, dY, ld_dy, x, ld_x, mean_rstd, gamma, row_sums, ws, want_cols, s);
+            rc = bwd_partials_launch<T, 8, 4, 1>(R, C, dY, ld_dy, x, ld_x, mean_rstd, gamma, row_sums, ws, want_cols, s);
         if (rc != CW_OK) return rc;
     } else {
         hipLaunchKernelGGL(ln_bwd_rows_generic_kernel<T>, dim3(ln_grid(R)), dim3(kLnBlock), 0, s, R, C,
@@ -441,6 +710,16 @@ int bwd_dx_impl(int64_t R, int64_t C, const void* dY, int64_t ld_dy, const void*
                 hipStream_t s) {
     const int vec_ok = rows_vec_ok<T>(dY, ld_dy) && rows_vec_ok<T>(x, ld_x) && rows_vec_ok<T>(dx, ld_dx) &&
                        (gamma == nullptr || aligned16(gamma));
+    const int64_t nch = row_chunks<T>(C);
+    if (vec_ok && (C % elem<T>::kVec) == 0 && nch <= 8) {
+        return dispatch_tile(nch, [&](auto nch_c, auto nr_c) {
+            constexpr int NCH = decltype(nch_c)::value, NR = decltype(nr_c)::value;
+            hipLaunchKernelGGL((ln_bwd_dx_tile_kernel<T, NCH, NR>), dim3(tile_grid(R, NR)), dim3(kTileWaves * 64), 0,
+                               s, R, C, (const T*)dY, ld_dy, (const T*)x, ld_x, mean_rstd, (const T*)gamma, row_sums,
+                               1.0f / (float)H, (T*)dx, ld_dx);
+            return check_launch("ln_bwd_dx_tile_kernel");
+        });
+    }
     hipLaunchKernelGGL(ln_bwd_dx_kernel<T>, dim3(ln_grid(R)), dim3(kLnBlock), 0, s, R, C, (const T*)dY, ld_dy,
                        (const T*)x, ld_x, mean_rstd, (const T*)gamma, row_sums, 1.0f / (float)H, (T*)dx, ld_dx,
                        vec_ok);

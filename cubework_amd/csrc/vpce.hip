@@ -11,6 +11,7 @@ namespace cw {
 namespace {
 
 constexpr int kCeBlock = 256;
+constexpr int kCeUnroll = 3;
 constexpr float kNegInf = -__builtin_huge_valf();
 
 // Running (max m, sum s of exp(x - m)) kept in the exp2 domain: m2 = m*log2(e).
@@ -21,10 +22,38 @@ struct OnlineLse {
 };
 
 template <int V>
-__device__ __forceinline__ void lse_add_chunk(OnlineLse& st, const float (&v)[V]) {
+__device__ __forceinline__ float chunk_max(const float (&v)[V]) {
     float cm = v[0];
 #pragma unroll
     for (int e = 1; e < V; ++e) cm = fmaxf(cm, v[e]);
+    return cm;
+}
+
+// Adds U chunks with one rescale of the running sum.
+template <int V, int U>
+__device__ __forceinline__ void lse_add_chunks(OnlineLse& st, const float (&v)[U][V]) {
+    float cm = chunk_max<V>(v[0]);
+#pragma unroll
+    for (int u = 1; u < U; ++u) cm = fmaxf(cm, chunk_max<V>(v[u]));
+    const float m_new = fmaxf(st.m, cm);
+    const float m2_new = (m_new == kNegInf) ? 0.0f : m_new * kLog2e;
+    const float scale = (st.m == kNegInf) ? 0.0f : __builtin_amdgcn_exp2f(st.m2 - m2_new);
+    float s = st.s * scale;
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+        float su = 0.0f;  // per-chunk partial sums keep the add chains short
+#pragma unroll
+        for (int e = 0; e < V; ++e) su += __builtin_amdgcn_exp2f(__builtin_fmaf(v[u][e], kLog2e, -m2_new));
+        s += su;
+    }
+    st.m = m_new;
+    st.m2 = m2_new;
+    st.s = s;
+}
+
+template <int V>
+__device__ __forceinline__ void lse_add_chunk(OnlineLse& st, const float (&v)[V]) {
+    const float cm = chunk_max<V>(v);
     const float m_new = fmaxf(st.m, cm);
     const float m2_new = (m_new == kNegInf) ? 0.0f : m_new * kLog2e;
     // rescale the old sum; an empty state (m == -inf) has s == 0 and stays 0
@@ -70,17 +99,19 @@ __global__ __launch_bounds__(kCeBlock) void vpce_fwd_kernel(int64_t T_rows, int6
         if (vec_ok) {
             const int64_t nvec = V_cols / V;
             int64_t i = tid;
-            // two independent 16-byte loads in flight per trip
-            for (; i + kCeBlock < nvec; i += 2 * kCeBlock) {
-                float v0[V], v1[V];
-                load_vec(xr + i * V, v0);
-                load_vec(xr + (i + kCeBlock) * V, v1);
-                lse_add_chunk<V>(st, v0);
-                lse_add_chunk<V>(st, v1);
+            // kCeUnroll independent 16-byte streaming loads in flight per trip
+            for (; i + (kCeUnroll - 1) * kCeBlock < nvec; i += kCeUnroll * kCeBlock) {
+                raw16_t raw[kCeUnroll];
+#pragma unroll
+                for (int u = 0; u < kCeUnroll; ++u) raw[u] = load_raw_stream(xr + (i + u * kCeBlock) * V);
+                float v[kCeUnroll][V];
+#pragma unroll
+                for (int u = 0; u < kCeUnroll; ++u) unpack_raw(raw[u], v[u], (const T*)nullptr);
+                lse_add_chunks<V, kCeUnroll>(st, v);
             }
             for (; i < nvec; i += kCeBlock) {
                 float v0[V];
-                load_vec(xr + i * V, v0);
+                unpack_raw(load_raw_stream(xr + i * V), v0, (const T*)nullptr);
                 lse_add_chunk<V>(st, v0);
             }
             for (int64_t c = nvec * V + tid; c < V_cols; c += kCeBlock) lse_add_one(st, load_elem(xr + c));
@@ -140,16 +171,36 @@ __global__ __launch_bounds__(256) void vpce_finalize_kernel(int64_t T_rows, int 
     if (gsum != nullptr) gsum[t] = s;
 }
 
+// The gradient is written once and not read again by this kernel: streaming stores.
 template <int V>
 __device__ __forceinline__ void store_grad(bf16_t* p, const float (&v)[V]) {
     static_assert(V == 8, "bf16 gradients are written 8 at a time");
-    store_vec(p, v);
+    store_raw_stream(p, pack_raw(v, (const bf16_t*)nullptr));
 }
 template <int V>
 __device__ __forceinline__ void store_grad(float* p, const float (&v)[V]) {
 #pragma unroll
-    for (int e = 0; e < V; e += 4)
-        *reinterpret_cast<float4*>(p + e) = make_float4(v[e], v[e + 1], v[e + 2], v[e + 3]);
+    for (int e = 0; e < V; e += 4) {
+        const float q[4] = {v[e], v[e + 1], v[e + 2], v[e + 3]};
+        store_raw_stream(p + e, pack_raw(q, (const float*)nullptr));
+    }
+}
+
+// One 16-byte vector of the gradient row: softmax * scale, minus dl at the target column.
+template <typename T, typename G, int V>
+__device__ __forceinline__ void grad_vector(raw16_t raw, int64_t i, int64_t tcol, float m2, float scale, float dl,
+                                            G* __restrict__ gr) {
+    float v[V];
+    unpack_raw(raw, v, (const T*)nullptr);
+#pragma unroll
+    for (int e = 0; e < V; ++e) v[e] = __builtin_amdgcn_exp2f(__builtin_fmaf(v[e], kLog2e, -m2)) * scale;
+    const int64_t rel = tcol - i * V;
+    if (rel >= 0 && rel < V) {
+#pragma unroll
+        for (int e = 0; e < V; ++e)
+            if (e == rel) v[e] -= dl;
+    }
+    store_grad<V>(gr + i * V, v);
 }
 
 template <typename T, typename G>
@@ -173,19 +224,17 @@ __global__ __launch_bounds__(kCeBlock) void vpce_bwd_kernel(int64_t T_rows, int6
         const int64_t tcol = masked ? -1 : (t - vocab_start);
         if (vec_ok) {
             const int64_t nvec = V_cols / V;
-            for (int64_t i = tid; i < nvec; i += kCeBlock) {
-                float v[V];
-                load_vec(xr + i * V, v);
+            int64_t i = tid;
+            for (; i + (kCeUnroll - 1) * kCeBlock < nvec; i += kCeUnroll * kCeBlock) {
+                raw16_t raw[kCeUnroll];
 #pragma unroll
-                for (int e = 0; e < V; ++e) v[e] = __builtin_amdgcn_exp2f(__builtin_fmaf(v[e], kLog2e, -m2)) * scale;
-                const int64_t rel = tcol - i * V;
-                if (rel >= 0 && rel < V) {
+                for (int u = 0; u < kCeUnroll; ++u) raw[u] = load_raw_stream(xr + (i + u * kCeBlock) * V);
 #pragma unroll
-                    for (int e = 0; e < V; ++e)
-                        if (e == rel) v[e] -= dl;
-                }
-                store_grad<V>(gr + i * V, v);
+                for (int u = 0; u < kCeUnroll; ++u)
+                    grad_vector<T, G, V>(raw[u], i + u * kCeBlock, tcol, m2, scale, dl, gr);
             }
+            for (; i < nvec; i += kCeBlock)
+                grad_vector<T, G, V>(load_raw_stream(xr + i * V), i, tcol, m2, scale, dl, gr);
             for (int64_t c = nvec * V + tid; c < V_cols; c += kCeBlock) {
                 float y = __builtin_amdgcn_exp2f(__builtin_fmaf(load_elem(xr + c), kLog2e, -m2)) * scale;
                 if (c == tcol) y -= dl;
