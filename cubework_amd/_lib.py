@@ -32,6 +32,9 @@ SIGNATURES = {
     "cw_last_error": (ctypes.c_char_p, []),
     "cw_gemm_ksteps": (_int, [_int, _i64, _i64, _i64, _int, _pp, _i64, _pp, _i64, _ptr, _int, _ptr, _i64, _ptr, _i64,
                               _pp, _int, _i64, _int, _ptr]),
+    "cw_gemm_workspace_bytes": (_i64, [_int, _i64, _i64, _i64, _int, _int]),
+    "cw_gemm_ksteps_ws": (_int, [_int, _i64, _i64, _i64, _int, _pp, _i64, _pp, _i64, _ptr, _int, _ptr, _i64, _ptr, _i64,
+                                 _pp, _int, _i64, _ptr, _i64, _int, _ptr]),
     "cw_colsum_workspace_bytes": (_i64, [_i64, _i64]),
     "cw_colsum": (_int, [_i64, _i64, _ptr, _i64, _ptr, _ptr, _i64, _int, _ptr]),
     "cw_act_bwd_colsum": (_int, [_int, _i64, _i64, _ptr, _i64, _ptr, _i64, _ptr, _i64, _ptr, _ptr, _i64, _int, _ptr]),

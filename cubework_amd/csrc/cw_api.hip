@@ -53,10 +53,26 @@ extern "C" const char* cw_device_arch(void) {
     return g_arch;
 }
 
+extern "C" int64_t cw_gemm_workspace_bytes(int layout, int64_t M, int64_t N, int64_t K, int n_steps, int io_dtype) {
+    if (layout != CW_NN && layout != CW_NT && layout != CW_TN) return 0;
+    if (io_dtype != CW_BF16) return 0;  // the fp32 GEMM is not split
+    const int slices = gemm_bf16_split_slices(M, N, K, n_steps);
+    return slices > 1 ? (int64_t)slices * M * N * (int64_t)sizeof(float) : 0;
+}
+
 extern "C" int cw_gemm_ksteps(int layout, int64_t M, int64_t N, int64_t K, int n_steps, const void* const* A_steps,
                               int64_t lda, const void* const* B_steps, int64_t ldb, const void* bias, int epilogue,
                               void* C, int64_t ldc, void* preact, int64_t ldp, const void* const* addends,
                               int n_addends, int64_t ldadd, int io_dtype, void* stream) {
+    return cw_gemm_ksteps_ws(layout, M, N, K, n_steps, A_steps, lda, B_steps, ldb, bias, epilogue, C, ldc, preact, ldp,
+                             addends, n_addends, ldadd, nullptr, 0, io_dtype, stream);
+}
+
+extern "C" int cw_gemm_ksteps_ws(int layout, int64_t M, int64_t N, int64_t K, int n_steps,
+                                 const void* const* A_steps, int64_t lda, const void* const* B_steps, int64_t ldb,
+                                 const void* bias, int epilogue, void* C, int64_t ldc, void* preact, int64_t ldp,
+                                 const void* const* addends, int n_addends, int64_t ldadd, void* workspace,
+                                 int64_t workspace_bytes, int io_dtype, void* stream) {
     if (layout != CW_NN && layout != CW_NT && layout != CW_TN)
         return fail(CW_ERR_INVALID, "cw_gemm_ksteps: bad layout %d", layout);
     if (epilogue < CW_EPI_NONE || epilogue > CW_EPI_BIAS_RELU)
@@ -125,6 +141,8 @@ extern "C" int cw_gemm_ksteps(int layout, int64_t M, int64_t N, int64_t K, int n
     args.K = (int)K;
     args.n_steps = n_steps;
     args.n_addends = n_addends;
+    args.workspace = workspace_bytes > 0 ? workspace : nullptr;
+    args.workspace_bytes = workspace != nullptr ? workspace_bytes : 0;
     hipStream_t s = (hipStream_t)stream;
     return io_dtype == CW_BF16 ? gemm_bf16_launch(args, layout, epilogue, s) : gemm_f32_launch(args, layout, epilogue, s);
 }

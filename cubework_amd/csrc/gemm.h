@@ -18,6 +18,9 @@ struct GemmArgs {
     // 1 when the operand's base and leading dimension allow 16-byte (bf16: 8
     // elements, fp32: 4 elements) row accesses; C/preact/addends/bias: 8-byte.
     int vec_a, vec_b, vec_c, vec_p, vec_add, vec_bias;
+    // caller's scratch for split-k partial sums (may be NULL / 0)
+    void* workspace;
+    int64_t workspace_bytes;
 };
 
 // Compact argument block of the LDS-DMA kernel: few enough pointers that they
@@ -35,7 +38,12 @@ struct RingArgs {
     int M, N, K;
     int n_steps, n_addends;
     int vec_bias, vec_add;  // always 1 on this path; read by the shared epilogue
+    float* partial;         // split-k only: [slices][M][N] fp32 partial sums
 };
+
+// Number of k slices the bf16 GEMM would split a problem into (1 = no split)
+// when given scratch; the scratch it then needs is slices * M * N * 4 bytes.
+int gemm_bf16_split_slices(int64_t M, int64_t N, int64_t K, int n_steps);
 
 int gemm_bf16_launch(const GemmArgs& args, int layout, int epilogue, hipStream_t s);
 int gemm_f32_launch(const GemmArgs& args, int layout, int epilogue, hipStream_t s);

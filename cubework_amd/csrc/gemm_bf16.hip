@@ -2,6 +2,11 @@
 //   - large tile-aligned problems (>= 128 tiles of 256x256, K a multiple of 64,
 //     16-byte aligned rows, at most 4 k-steps and 2 addends): the LDS-DMA
 //     kernel (gemm_bf16_dma.h);
+//   - the same kernel split along k when the output has too few 256x256 tiles
+//     to occupy the chip but the reduction is long (the weight-gradient shape
+//     X^T dY), given scratch for the fp32 partial sums: `slices` blocks per
+//     tile, then splitk_reduce_kernel adds them in slice order and applies the
+//     epilogue;
 //   - everything else: the register-staged kernel (gemm_bf16_kernel.h), with
 //     256x256 or 128x128 tiles, guarded when the shape is ragged or unaligned.
 // CW_GEMM_IMPL=staged in the environment forces the register-staged kernel.
@@ -15,6 +20,95 @@ namespace cw {
 int gemm_bf16_dma_launch_nn(const GemmArgs& args, int epilogue, hipStream_t s);
 int gemm_bf16_dma_launch_nt(const GemmArgs& args, int epilogue, hipStream_t s);
 int gemm_bf16_dma_launch_tn(const GemmArgs& args, int epilogue, hipStream_t s);
+
+int gemm_bf16_dma_split_launch_nn(const GemmArgs& args, int slices, hipStream_t s);
+int gemm_bf16_dma_split_launch_nt(const GemmArgs& args, int slices, hipStream_t s);
+int gemm_bf16_dma_split_launch_tn(const GemmArgs& args, int slices, hipStream_t s);
+
+int gemm_bf16_split_slices(int64_t M, int64_t N, int64_t K, int n_steps) {
+    if (M <= 0 || N <= 0 || K <= 0 || n_steps <= 0 || n_steps > kRingMaxSteps) return 1;
+    if ((M % 256) != 0 || (N % 256) != 0 || (K % 64) != 0) return 1;
+    const int64_t tiles = (M / 256) * (N / 256);
+    if (tiles >= 128 || K * n_steps < 2048) return 1;  // enough tiles already, or a short reduction
+    int slices = 8;
+    while (slices > 1 && (tiles * slices > 256 || (K % (64 * slices)) != 0 || K / slices < 256)) slices >>= 1;
+    return slices;
+}
+
+namespace {
+
+// C = epilogue(sum over slices of partial + addends + bias). One thread per 8
+// consecutive columns of a row; slices are added in index order.
+template <int EPI>
+__global__ __launch_bounds__(256) void splitk_reduce_kernel(const float* __restrict__ partial, int slices, int64_t M,
+                                                            int64_t N, const bf16_t* __restrict__ bias,
+                                                            const bf16_t* __restrict__ add0,
+                                                            const bf16_t* __restrict__ add1, int64_t ldadd,
+                                                            bf16_t* __restrict__ C, int64_t ldc,
+                                                            bf16_t* __restrict__ preact, int64_t ldp) {
+    const int64_t vec_per_row = N / 8;
+    const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (idx >= M * vec_per_row) return;
+    const int64_t row = idx / vec_per_row, col = (idx - row * vec_per_row) * 8;
+    const float* p = partial + row * N + col;
+    float v[8];
+#pragma unroll
+    for (int e = 0; e < 8; ++e) v[e] = 0.0f;
+    for (int z = 0; z < slices; ++z) {
+        float lo[4], hi[4];
+        unpack_raw(load_raw_stream(p + (int64_t)z * M * N), lo, (const float*)nullptr);
+        unpack_raw(load_raw_stream(p + (int64_t)z * M * N + 4), hi, (const float*)nullptr);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            v[e] += lo[e];
+            v[4 + e] += hi[e];
+        }
+    }
+    float t[8];
+    if (EPI != CW_EPI_NONE && bias != nullptr) {
+        unpack_raw(load_raw(bias + col), t, (const bf16_t*)nullptr);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) v[e] += t[e];
+    }
+    if (add0 != nullptr) {
+        unpack_raw(load_raw_stream(add0 + row * ldadd + col), t, (const bf16_t*)nullptr);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) v[e] += t[e];
+    }
+    if (add1 != nullptr) {
+        unpack_raw(load_raw_stream(add1 + row * ldadd + col), t, (const bf16_t*)nullptr);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) v[e] += t[e];
+    }
+    if (preact != nullptr) store_raw_stream(preact + row * ldp + col, pack_raw(v, (const bf16_t*)nullptr));
+#pragma unroll
+    for (int e = 0; e < 8; ++e) v[e] = gemm_bf16::epi_act<EPI>(v[e]);
+    store_raw_stream(C + row * ldc + col, pack_raw(v, (const bf16_t*)nullptr));
+}
+
+template <int EPI>
+int launch_splitk_reduce(const GemmArgs& a, int slices, hipStream_t s) {
+    const int64_t threads = (int64_t)a.M * (a.N / 8);
+    hipLaunchKernelGGL(splitk_reduce_kernel<EPI>, dim3((unsigned)((threads + 255) / 256)), dim3(256), 0, s,
+                       (const float*)a.workspace, slices, (int64_t)a.M, (int64_t)a.N, (const bf16_t*)a.bias,
+                       (const bf16_t*)(a.n_addends > 0 ? a.addend[0] : nullptr),
+                       (const bf16_t*)(a.n_addends > 1 ? a.addend[1] : nullptr), a.ldadd, (bf16_t*)a.C, a.ldc,
+                       (bf16_t*)a.preact, a.ldp);
+    return check_launch("splitk_reduce_kernel");
+}
+
+int splitk_reduce(const GemmArgs& a, int slices, int epilogue, hipStream_t s) {
+    switch (epilogue) {
+        case CW_EPI_NONE: return launch_splitk_reduce<CW_EPI_NONE>(a, slices, s);
+        case CW_EPI_BIAS: return launch_splitk_reduce<CW_EPI_BIAS>(a, slices, s);
+        case CW_EPI_BIAS_GELU_TANH: return launch_splitk_reduce<CW_EPI_BIAS_GELU_TANH>(a, slices, s);
+        case CW_EPI_BIAS_GELU_ERF: return launch_splitk_reduce<CW_EPI_BIAS_GELU_ERF>(a, slices, s);
+        case CW_EPI_BIAS_RELU: return launch_splitk_reduce<CW_EPI_BIAS_RELU>(a, slices, s);
+        default: return fail(CW_ERR_INVALID, "cw_gemm_ksteps: bad epilogue %d", epilogue);
+    }
+}
+
+}  // namespace
 
 static bool dma_kernel_enabled() {
     static const bool enabled = [] {
@@ -42,6 +136,20 @@ int gemm_bf16_launch(const GemmArgs& args, int layout, int epilogue, hipStream_t
             case CW_TN: return gemm_bf16_dma_launch_tn(args, epilogue, s);
             default: return fail(CW_ERR_INVALID, "cw_gemm_ksteps: bad layout %d", layout);
         }
+    }
+    const int slices = gemm_bf16_split_slices(args.M, args.N, args.K, args.n_steps);
+    if (slices > 1 && all_vec && args.n_addends <= kRingMaxAddends && dma_kernel_enabled() &&
+        args.workspace != nullptr && aligned16(args.workspace) &&
+        args.workspace_bytes >= (int64_t)slices * args.M * args.N * (int64_t)sizeof(float)) {
+        int rc;
+        switch (layout) {
+            case CW_NN: rc = gemm_bf16_dma_split_launch_nn(args, slices, s); break;
+            case CW_NT: rc = gemm_bf16_dma_split_launch_nt(args, slices, s); break;
+            case CW_TN: rc = gemm_bf16_dma_split_launch_tn(args, slices, s); break;
+            default: return fail(CW_ERR_INVALID, "cw_gemm_ksteps: bad layout %d", layout);
+        }
+        if (rc != CW_OK) return rc;
+        return splitk_reduce(args, slices, epilogue, s);
     }
     switch (layout) {
         case CW_NN: return gemm_bf16_launch_nn(args, epilogue, big, exact, s);

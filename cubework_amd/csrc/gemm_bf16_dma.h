@@ -120,7 +120,10 @@ struct FragReader {
 
 #define CW_PIN() __builtin_amdgcn_sched_barrier(0)
 
-template <bool TRANS_A, bool TRANS_B, int EPI, int NS>
+// SPLIT: blockIdx.y selects one of gridDim.y equal slices of every step's k
+// range; the block writes its fp32 partial tile to args.partial and
+// splitk_reduce_kernel finishes the sum and the epilogue.
+template <bool TRANS_A, bool TRANS_B, int EPI, int NS, bool SPLIT>
 __global__ __launch_bounds__(kThreads) void gemm_bf16_dma_kernel(const RingArgs args) {
     extern __shared__ __attribute__((aligned(16))) uint16_t lds[];
     lds_char* lds_base = (lds_char*)lds;
@@ -149,7 +152,10 @@ __global__ __launch_bounds__(kThreads) void gemm_bf16_dma_kernel(const RingArgs 
     const int m0 = (first_m + in_group % gsz) * kTile;
     const int n0 = (in_group / gsz) * kTile;
 
-    const int kt_per_step = K / kBK;
+    const int k_len = SPLIT ? K / (int)gridDim.y : K;  // k extent of this block within each step
+    const int k_beg = SPLIT ? (int)blockIdx.y * k_len : 0;
+    const int k_end = k_beg + k_len;
+    const int kt_per_step = k_len / kBK;
     const int KT = kt_per_step * args.n_steps;
 
     uint32_t a_even, a_odd, b_even, b_odd;
@@ -174,15 +180,15 @@ __global__ __launch_bounds__(kThreads) void gemm_bf16_dma_kernel(const RingArgs 
     // issue position stays on it: the loop keeps issuing (harmless duplicate
     // loads into a free stage) so that its body has no branches and the load
     // counter arithmetic is the same in every iteration.
-    int is_kt = 0, is_step = 0, is_k0 = 0, is_stage = 0;
+    int is_kt = 0, is_step = 0, is_k0 = k_beg, is_stage = 0;
     const char* is_a = reinterpret_cast<const char*>(args.A[0]);
     const char* is_b = reinterpret_cast<const char*>(args.B[0]);
     auto issue_advance = [&]() {
         if (is_kt + 1 < KT) {
             ++is_kt;
             is_k0 += kBK;
-            if (is_k0 >= K) {
-                is_k0 = 0;
+            if (is_k0 >= k_end) {
+                is_k0 = k_beg;
                 ++is_step;
                 is_a = reinterpret_cast<const char*>(gemm_bf16::pick_ptr(args.A, is_step));
                 is_b = reinterpret_cast<const char*>(gemm_bf16::pick_ptr(args.B, is_step));
@@ -266,7 +272,26 @@ __global__ __launch_bounds__(kThreads) void gemm_bf16_dma_kernel(const RingArgs 
     }
     dma_wait<0>();
     __syncthreads();
-    gemm_bf16::gemm_epilogue<kTile, kTile, 4, 4, EPI, true>(acc, args, lds, m0, n0, wm, wn, lane, tid);
+    if constexpr (SPLIT) {
+        // accumulator element 4g+e of tile (i, j): row (lane & 31) + 32 i, column 4 (lane >> 5) + 32 j + 8 g + e
+        float* part = args.partial + (int64_t)blockIdx.y * M * N + (int64_t)(m0 + wm * 128 + (lane & 31)) * N + n0 +
+                      wn * 128 + 4 * (lane >> 5);
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+#pragma unroll
+            for (int j = 0; j < 4; ++j)
+#pragma unroll
+                for (int g = 0; g < 4; ++g) {
+                    raw16_t u;
+                    u.x = __float_as_uint(acc[i][j][4 * g]);
+                    u.y = __float_as_uint(acc[i][j][4 * g + 1]);
+                    u.z = __float_as_uint(acc[i][j][4 * g + 2]);
+                    u.w = __float_as_uint(acc[i][j][4 * g + 3]);
+                    *reinterpret_cast<raw16_t*>(part + (int64_t)i * 32 * N + j * 32 + 8 * g) = u;
+                }
+    } else {
+        gemm_bf16::gemm_epilogue<kTile, kTile, 4, 4, EPI, true>(acc, args, lds, m0, n0, wm, wn, lane, tid);
+    }
 }
 
 template <int NS>
@@ -284,13 +309,14 @@ inline RingArgs to_ring_args(const GemmArgs& g) {
     r.lda = g.lda; r.ldb = g.ldb; r.ldc = g.ldc; r.ldp = g.ldp; r.ldadd = g.ldadd;
     r.M = g.M; r.N = g.N; r.K = g.K; r.n_steps = g.n_steps; r.n_addends = g.n_addends;
     r.vec_bias = 1; r.vec_add = 1;
+    r.partial = nullptr;
     return r;
 }
 
 template <bool TA, bool TB, int EPI, int NS>
 int launch_dma_cfg(const GemmArgs& gargs, hipStream_t s) {
     const RingArgs args = to_ring_args(gargs);
-    auto kern = gemm_bf16_dma_kernel<TA, TB, EPI, NS>;
+    auto kern = gemm_bf16_dma_kernel<TA, TB, EPI, NS, false>;
     constexpr size_t lds = lds_bytes_dma<NS>();
     static_assert(lds <= 160 * 1024, "LDS image does not fit the CU");
     hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
@@ -302,6 +328,22 @@ int launch_dma_cfg(const GemmArgs& gargs, hipStream_t s) {
 }
 
 constexpr int kStages = 4;
+
+// Split-k launch: `slices` blocks per output tile, partial sums to the
+// caller's scratch. The epilogue is left to splitk_reduce.
+template <bool TA, bool TB>
+int launch_dma_split(const GemmArgs& gargs, int slices, hipStream_t s) {
+    RingArgs args = to_ring_args(gargs);
+    args.partial = reinterpret_cast<float*>(gargs.workspace);
+    auto kern = gemm_bf16_dma_kernel<TA, TB, CW_EPI_NONE, kStages, true>;
+    constexpr size_t lds = lds_bytes_dma<kStages>();
+    hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    if (e != hipSuccess) return fail(CW_ERR_LAUNCH, "hipFuncSetAttribute(gemm_bf16_ring, split): %s", hipGetErrorString(e));
+    const int tiles = (args.M / kTile) * (args.N / kTile);
+    const int grid = ((tiles + 7) / 8) * 8;
+    hipLaunchKernelGGL(kern, dim3(grid, slices), dim3(kThreads), lds, s, args);
+    return check_launch("gemm_bf16_dma_kernel (split k)");
+}
 
 template <bool TA, bool TB>
 int launch_dma(const GemmArgs& args, int epilogue, hipStream_t s) {

@@ -7,4 +7,8 @@ int gemm_bf16_dma_launch_nt(const GemmArgs& args, int epilogue, hipStream_t s) {
     return gemm_dma::launch_dma<false, false>(args, epilogue, s);
 }
 
+int gemm_bf16_dma_split_launch_nt(const GemmArgs& args, int slices, hipStream_t s) {
+    return gemm_dma::launch_dma_split<false, false>(args, slices, s);
+}
+
 }  // namespace cw

@@ -7,4 +7,8 @@ int gemm_bf16_dma_launch_tn(const GemmArgs& args, int epilogue, hipStream_t s) {
     return gemm_dma::launch_dma<true, true>(args, epilogue, s);
 }
 
+int gemm_bf16_dma_split_launch_tn(const GemmArgs& args, int slices, hipStream_t s) {
+    return gemm_dma::launch_dma_split<true, true>(args, slices, s);
+}
+
 }  // namespace cw

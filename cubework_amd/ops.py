@@ -128,10 +128,13 @@ def gemm_ksteps(layout: str, A_steps: Sequence[torch.Tensor], B_steps: Sequence[
     preact = torch.empty((M, N), dtype=a0.dtype, device=a0.device) if want_preact else None
     epi = epilogue_code(bias is not None, activation)
     ta, tb, tadd = _ptr_table(A_steps), _ptr_table(B_steps), _ptr_table(addends)
-    rc = lib.cw_gemm_ksteps(LAYOUTS[layout], M, N, K, len(A_steps), ta, lda, tb, ldb, _p(bias), epi, _p(out),
-                            _ld(out), _p(preact), _ld(preact) if preact is not None else 0, tadd, len(addends),
-                            ldadd, dt, _stream())
-    _lib.check(rc, "cw_gemm_ksteps")
+    # scratch for the split-k path (few output tiles, long reduction: the weight-gradient shape)
+    ws_bytes = lib.cw_gemm_workspace_bytes(LAYOUTS[layout], M, N, K, len(A_steps), dt)
+    ws = torch.empty(ws_bytes, dtype=torch.uint8, device=a0.device) if ws_bytes > 0 else None
+    rc = lib.cw_gemm_ksteps_ws(LAYOUTS[layout], M, N, K, len(A_steps), ta, lda, tb, ldb, _p(bias), epi, _p(out),
+                               _ld(out), _p(preact), _ld(preact) if preact is not None else 0, tadd, len(addends),
+                               ldadd, _p(ws), ws_bytes, dt, _stream())
+    _lib.check(rc, "cw_gemm_ksteps_ws")
     return (out, preact) if want_preact else out
 
 

@@ -105,6 +105,32 @@ int cw_gemm_ksteps(int layout, int64_t M, int64_t N, int64_t K, int n_steps,
                    const void* const* addends, int n_addends, int64_t ldadd,
                    int io_dtype, void* stream);
 
+/*
+ * cw_gemm_ksteps with caller-provided scratch. When the output has too few
+ * tiles to occupy the chip and the reduction is long -- the weight-gradient
+ * products X^T dY of _SUMMA_AB.backward / _SUMMA_ABT.backward
+ * (parallel_2d/_operation.py:63-66, 141-144, through _SUMMA_ATB.forward
+ * :197-204), of F.linear's backward (parallel_1d/module.py:147,209,269,338) and
+ * of _Linear3D.backward (parallel_3d/_operation.py:53) -- the k range of every
+ * step is split over several workgroups per tile, whose fp32 partial sums go
+ * through `workspace` and are added in a fixed order (bit-reproducible; the
+ * reference leaves this choice, and its scratch, to the BLAS library inside
+ * torch.matmul). cw_gemm_workspace_bytes gives the size that enables it (0 when
+ * the shape is not split); with workspace NULL or smaller the call behaves
+ * exactly like cw_gemm_ksteps. The scratch must not be shared by calls that
+ * may overlap on the device.
+ */
+int64_t cw_gemm_workspace_bytes(int layout, int64_t M, int64_t N, int64_t K, int n_steps, int io_dtype);
+int cw_gemm_ksteps_ws(int layout, int64_t M, int64_t N, int64_t K, int n_steps,
+                      const void* const* A_steps, int64_t lda,
+                      const void* const* B_steps, int64_t ldb,
+                      const void* bias, int epilogue,
+                      void* C, int64_t ldc,
+                      void* preact, int64_t ldp,
+                      const void* const* addends, int n_addends, int64_t ldadd,
+                      void* workspace, int64_t workspace_bytes,
+                      int io_dtype, void* stream);
+
 /* ---- bias / activation backward ---------------------------------------- */
 /*
  * Number of bytes of scratch cw_colsum / cw_act_bwd_colsum / cw_ln_bwd_partials

@@ -142,6 +142,40 @@ def test_kstep_sum_equals_concatenated_gemm():
     assert_parity(two[rows.to(dev)], want, torch.bfloat16, "config-2 sampled rows")
 
 
+@pytest.mark.parametrize("layout", LAYOUTS)
+def test_bf16_split_k_long_reduction(layout):
+    # 2 x 3 output tiles of 256x256 and k = 2 x 1024: few tiles, long reduction -> the k range of every
+    # step is split over several workgroups per tile (cw_gemm_workspace_bytes > 0)
+    from cubework_amd import _lib
+    from cubework_amd.ops import LAYOUTS as CODES
+
+    assert _lib.load().cw_gemm_workspace_bytes(CODES[layout], 512, 768, 1024, 2, 0) > 0
+    _run(layout, 512, 768, 1024, 2, torch.bfloat16, act="gelu_tanh", n_add=1, preact=True, seed=5)
+    _run(layout, 512, 768, 1024, 2, torch.bfloat16, act=None, bias=False, seed=6)
+
+
+def test_split_k_matches_unsplit_call():
+    """The same product through cw_gemm_ksteps (no scratch: one workgroup per tile) and through
+    cw_gemm_ksteps_ws (split k): both round one fp32 sum to bf16, so they agree to the parity bar, and the
+    split result is bit-reproducible from call to call."""
+    from cubework_amd import _lib, ops
+
+    dev = "cuda:0"
+    M, N, K, steps = 256, 512, 4096, 2
+    A = [randn((K, M), torch.bfloat16, 40 + i).to(dev) for i in range(steps)]
+    B = [randn((K, N), torch.bfloat16, 50 + i, std=0.05).to(dev) for i in range(steps)]
+    lib = _lib.load()
+    split1 = ops.gemm_ksteps("TN", A, B)
+    split2 = ops.gemm_ksteps("TN", A, B)
+    plain = torch.empty((M, N), dtype=torch.bfloat16, device=dev)
+    rc = lib.cw_gemm_ksteps(ops.LAYOUTS["TN"], M, N, K, steps, ops._ptr_table(A), M, ops._ptr_table(B), N, None, 0,
+                            plain.data_ptr(), N, None, 0, None, 0, 0, 0, torch.cuda.current_stream().cuda_stream)
+    assert rc == 0, lib.cw_last_error()
+    torch.cuda.synchronize()
+    assert torch.equal(split1, split2)
+    assert_parity(split1, plain.float().cpu(), torch.bfloat16, "split k vs one workgroup per tile")
+
+
 def test_rejects_bad_arguments():
     from cubework_amd import ops, _lib
 
