@@ -150,6 +150,79 @@ def bench_bandwidth_kernels(device):
     return out
 
 
+def event_time_us(fn, iters, warmup):
+    """Average duration of fn() per call from events on the current stream."""
+    import torch
+    for _ in range(warmup):
+        fn()
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for _ in range(iters):
+        fn()
+    e1.record()
+    torch.cuda.synchronize()
+    return e0.elapsed_time(e1) * 1e3 / iters
+
+
+def bench_other_configs(device, sets):
+    """The other GEMM orientations at config 2's FLOP count (the backward products of the same layer),
+    config 1's fp32 forward GEMM, and one OPT-1.3B-shaped block (config 5) forward+backward."""
+    import torch
+    from cubework_amd import ops
+    from cubework_amd.distributed import initialize
+    from cubework_amd.opt_block import OPTBlock
+
+    out = {}
+    n_sets = len(sets)
+    i = [0]
+
+    def rot():
+        i[0] += 1
+        return sets[i[0] % n_sets]
+
+    # dX = sum_i dY_i W_i^T (NT): A_i [8192,2048], B_i [2048,2048] read as [N,K]
+    dx = torch.empty((M, N), dtype=torch.bfloat16, device=device)
+    us = event_time_us(lambda: ops.gemm_ksteps("NT", *rot(), out=dx), 50, 10)
+    out["gemm_nt_dX"] = {"us": round(us, 2), "TFLOPs": round(GEMM_FLOP / us / 1e6, 1),
+                         "frac": round(GEMM_FLOP / us / 1e6 / MFMA_BF16_PEAK_TFLOPS, 4)}
+    # dW = sum_i X_i^T dY_i (TN): A_i [8192,2048] read as [K,M], B_i [8192,2048] -> [2048,2048], k = 2 x 8192
+    dw = torch.empty((K, N), dtype=torch.bfloat16, device=device)
+
+    def tn():
+        a, _ = rot()
+        b, _ = rot()
+        ops.gemm_ksteps("TN", a, b, out=dw)
+    us = event_time_us(tn, 50, 10)
+    out["gemm_tn_dW_splitk"] = {"us": round(us, 2), "TFLOPs": round(GEMM_FLOP / us / 1e6, 1),
+                                "frac": round(GEMM_FLOP / us / 1e6 / MFMA_BF16_PEAK_TFLOPS, 4)}
+    # config 1 forward: x [4096,1024] fp32, W [4096,1024] fp32 (NT), fp32 MFMA
+    x1 = _seeded((4096, 1024), 1, 1.0, torch.float32).to(device)
+    w1 = ((torch.rand((4096, 1024), generator=torch.Generator().manual_seed(2)) * 2 - 1) * (6.0 / 5120) ** 0.5).to(device)
+    b1 = torch.zeros(4096, dtype=torch.float32, device=device)
+    o1 = torch.empty((4096, 4096), dtype=torch.float32, device=device)
+    us = event_time_us(lambda: ops.gemm_ksteps("NT", [x1], [w1], b1, None, out=o1), 30, 5)
+    flop1 = 2.0 * 4096 * 1024 * 4096
+    out["linear1d_fp32_fwd"] = {"us": round(us, 2), "TFLOPs": round(flop1 / us / 1e6, 1),
+                                "frac_fp32_mfma": round(flop1 / us / 1e6 / 157.3, 4)}
+    # config 5: OPT-1.3B-shaped block, batch 4 x seq 2048, bf16, forward + backward
+    initialize("2d", 1)
+    torch.manual_seed(0)
+    blk = OPTBlock(hidden=2048, heads=32, ffn=8192, dtype=torch.bfloat16, activation="relu").to(device)
+    xb = _seeded((4, 2048, 2048), 11, 1.0, torch.bfloat16).to(device).requires_grad_(True)
+    dyb = _seeded((4, 2048, 2048), 12, 1.0, torch.bfloat16).to(device)
+
+    def block_step():
+        y = blk(xb)
+        y.backward(dyb)
+    us = event_time_us(block_step, 10, 3)
+    lin_flop = 3 * 2.0 * 8192 * 2048 * (6144 + 2048 + 8192 + 8192)
+    out["opt_block_fwd_bwd"] = {"ms": round(us / 1e3, 3), "linear_flop": lin_flop,
+                                "linear_TFLOPs_if_all_time_were_linears": round(lin_flop / us / 1e6, 1),
+                                "note": "attention core is torch scaled_dot_product_attention (model code in the reference)"}
+    return out
+
+
 def cpu_baseline():
     """The reference's CPU path (torch on gloo, world size 1) for the same
     workload, through the oracle's restatement of _SUMMA_AB.forward +
@@ -285,6 +358,8 @@ def main():
     if not args.no_aux:
         result["aux"] = bench_bandwidth_kernels(device)
         result["aux"]["hbm_peak_GBps"] = HBM_PEAK_GBPS
+    if not args.no_aux:
+        result["other_configs"] = bench_other_configs(device, sets)
     if not args.no_cpu:
         result["cpu_baseline"] = cpu_baseline()
     print(json.dumps(result))

@@ -176,6 +176,21 @@ __global__ __launch_bounds__(kThreads) void gemm_bf16_dma_kernel(const RingArgs 
 #pragma unroll
             for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.0f;
 
+    // the lane's bias values, fetched ahead of every operand load so that the
+    // epilogue finds them in registers
+    gemm_bf16::u32x2_t bias_raw[4][4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+#pragma unroll
+        for (int g = 0; g < 4; ++g) bias_raw[j][g] = gemm_bf16::u32x2_t{0u, 0u};
+    if (!SPLIT && EPI != CW_EPI_NONE && args.bias != nullptr) {
+        const uint16_t* bp = reinterpret_cast<const uint16_t*>(args.bias) + n0 + wn * 128 + 4 * (lane >> 5);
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+#pragma unroll
+            for (int g = 0; g < 4; ++g) bias_raw[j][g] = *reinterpret_cast<const gemm_bf16::u32x2_t*>(bp + j * 32 + 8 * g);
+    }
+
     // state of the tile whose loads are issued next. Past the last tile the
     // issue position stays on it: the loop keeps issuing (harmless duplicate
     // loads into a free stage) so that its body has no branches and the load
@@ -290,7 +305,7 @@ __global__ __launch_bounds__(kThreads) void gemm_bf16_dma_kernel(const RingArgs 
                     *reinterpret_cast<raw16_t*>(part + (int64_t)i * 32 * N + j * 32 + 8 * g) = u;
                 }
     } else {
-        gemm_bf16::gemm_epilogue<kTile, kTile, 4, 4, EPI, true>(acc, args, lds, m0, n0, wm, wn, lane, tid);
+        gemm_bf16::gemm_epilogue_slabs<EPI>(acc, args, bias_raw, lds, m0, n0, wm, wn, lane, tid);
     }
 }
 

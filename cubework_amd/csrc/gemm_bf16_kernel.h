@@ -327,6 +327,86 @@ __device__ __forceinline__ void gemm_epilogue(f32x16_t (&acc)[TM][TN], const Arg
     tile_store<BM, BN, FAST>(lds_c, reinterpret_cast<uint16_t*>(args.C), args.ldc, m0, n0, M, N, tid);
 }
 
+// Epilogue of the 256x256 LDS-DMA kernel (whole tile in bounds, aligned): the
+// tile goes out in four slabs of 2 x 32 rows (accumulator row index i of both
+// wavefront rows), staged through two alternating LDS buffers. The global
+// stores of slab i drain while slab i+1 is computed, and one barrier per slab
+// is enough: a buffer is rewritten two slabs after it was read.
+// bias_raw[j][g]: the lane's 4 bias values (bf16 pairs) for accumulator
+// columns j*32 + 8g .. +3, loaded by the caller ahead of the k loop.
+template <int EPI, typename Args>
+__device__ __forceinline__ void gemm_epilogue_slabs(f32x16_t (&acc)[4][4], const Args& args,
+                                                    const u32x2_t (&bias_raw)[4][4], uint16_t* lds, int m0, int n0,
+                                                    int wm, int wn, int lane, int tid) {
+    constexpr int CP = c_pitch<256>();
+    constexpr int BUF = 64 * CP;  // elements per staging buffer
+    const int lrow = wm * 32 + (lane & 31);
+    const int col_l = wn * 128 + 4 * (lane >> 5);
+    int buf = 0;
+
+    auto stage = [&](auto slab, auto activated) {
+        constexpr int I = decltype(slab)::value;
+        constexpr bool ACT = decltype(activated)::value;
+        const int mrow = m0 + wm * 128 + I * 32 + (lane & 31);
+        uint16_t* dst = lds + buf * BUF + lrow * CP + col_l;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+#pragma unroll
+            for (int g = 0; g < 4; ++g) {
+                const u32x2_t b = bias_raw[j][g];
+                float v[4];
+                v[0] = acc[I][j][4 * g] + __uint_as_float(b.x << 16);
+                v[1] = acc[I][j][4 * g + 1] + __uint_as_float(b.x & 0xffff0000u);
+                v[2] = acc[I][j][4 * g + 2] + __uint_as_float(b.y << 16);
+                v[3] = acc[I][j][4 * g + 3] + __uint_as_float(b.y & 0xffff0000u);
+                if (args.n_addends > 0) {
+                    const int ncol = n0 + col_l + j * 32 + 8 * g;
+#pragma unroll 1
+                    for (int a = 0; a < args.n_addends; ++a) {
+                        float t[4];
+                        load4_bf16(reinterpret_cast<const uint16_t*>(pick_ptr(args.addend, a)) + (int64_t)mrow * args.ldadd + ncol,
+                                   4, true, t);
+#pragma unroll
+                        for (int e = 0; e < 4; ++e) v[e] += t[e];
+                    }
+                }
+                if constexpr (ACT) {
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) v[e] = epi_act<EPI>(v[e]);
+                }
+                u32x2_t p;
+                p.x = pack_bf16x2(v[0], v[1]);
+                p.y = pack_bf16x2(v[2], v[3]);
+                *reinterpret_cast<u32x2_t*>(dst + j * 32 + 8 * g) = p;
+            }
+        }
+    };
+    // 64 staged rows x 32 chunks of 16 bytes: 8 per thread, whole 512-byte rows per wavefront pass
+    auto store = [&](int slab, uint16_t* out, int64_t ld) {
+        const int r = tid >> 5, cq = tid & 31;
+        const uint16_t* src = lds + buf * BUF + r * CP + cq * 8;
+#pragma unroll
+        for (int pass = 0; pass < 8; ++pass) {
+            const int lr = r + 8 * pass;
+            const int grow = m0 + (lr >= 32 ? 128 : 0) + slab * 32 + (lr & 31);
+            *reinterpret_cast<u32x4_t*>(out + (int64_t)grow * ld + n0 + cq * 8) =
+                *reinterpret_cast<const u32x4_t*>(src + pass * 8 * CP);
+        }
+    };
+    static_for<4>([&](auto slab) {
+        if (args.preact != nullptr) {
+            stage(slab, std::false_type{});
+            __syncthreads();
+            store(decltype(slab)::value, reinterpret_cast<uint16_t*>(args.preact), args.ldp);
+            buf ^= 1;
+        }
+        stage(slab, std::true_type{});
+        __syncthreads();
+        store(decltype(slab)::value, reinterpret_cast<uint16_t*>(args.C), args.ldc);
+        buf ^= 1;
+    });
+}
+
 template <int BM, int BN, bool TRANS_A, bool TRANS_B, bool GUARD, int EPI>
 __global__ __launch_bounds__(kThreads) void gemm_bf16_kernel(const GemmArgs args) {
     constexpr int WTM = BM / 2, WTN = BN / 2;  // wavefront sub-tile
