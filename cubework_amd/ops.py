@@ -350,3 +350,35 @@ def vpce_bwd(logits: torch.Tensor, targets: torch.Tensor, vocab_start: int, gmax
                          dloss_scale, _p(grad), _ld(grad), _dtype_code(logits), _dtype_code(grad), _stream())
     _lib.check(rc, "cw_vpce_bwd")
     return grad.reshape(shape)
+
+
+# --------------------------------------------------------------------------
+# attention core
+# --------------------------------------------------------------------------
+def _bshd_strides(t: torch.Tensor):
+    """(batch, token, head) strides of a [b, s, h, d] view with unit stride in d."""
+    if t.dim() != 4 or t.stride(3) != 1:
+        raise ValueError("expected a [batch, tokens, heads, head_dim] view with unit stride in head_dim")
+    return t.stride(0), t.stride(1), t.stride(2)
+
+
+def attn_fwd(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, scale: Optional[float] = None, causal: bool = True,
+             want_lse: bool = False):
+    """softmax(scale q k^T + causal mask) v for [b, s, h, d] views (e.g. slices of the qkv projection's
+    output); returns [b, s, h*d] (and the [b, h, s] log-sum-exp). See cw_attn_fwd."""
+    lib = _lib.load()
+    _require_device(q, k, v)
+    if q.shape != k.shape or q.shape != v.shape or q.dtype != k.dtype or q.dtype != v.dtype:
+        raise ValueError("q, k, v must agree in shape and dtype")
+    strides = _bshd_strides(q)
+    if _bshd_strides(k) != strides or _bshd_strides(v) != strides:
+        raise ValueError("q, k, v must share their strides (views of one projection output)")
+    B, S, H, D = q.shape
+    scale = D ** -0.5 if scale is None else float(scale)
+    out = torch.empty((B, S, H, D), dtype=q.dtype, device=q.device)
+    lse = torch.empty((B, H, S), dtype=torch.float32, device=q.device) if want_lse else None
+    rc = lib.cw_attn_fwd(B, H, S, D, _p(q), _p(k), _p(v), strides[0], strides[1], strides[2], scale, 1 if causal else 0,
+                         _p(out), out.stride(0), out.stride(1), out.stride(2), _p(lse), _dtype_code(q), _stream())
+    _lib.check(rc, "cw_attn_fwd")
+    out = out.view(B, S, H * D)
+    return (out, lse) if want_lse else out

@@ -258,6 +258,25 @@ int cw_vpce_bwd(int64_t T, int64_t V, const void* logits, int64_t ld,
                 const float* dloss_rows, float dloss_scale,
                 void* grad, int64_t ld_grad, int io_dtype, int grad_dtype, void* stream);
 
+/* ---- attention core ------------------------------------------------------ */
+/*
+ * out[b, s, h, :] = softmax_j(scale * q[b,s,h,:] . k[b,j,h,:] + causal mask) . v[b,j,h,:]
+ * Replaces OPTAttention.forward's scaled bmm / mask / softmax / bmm
+ * (benchmark/opt/opt.py:84-117) in one pass; the probabilities are never
+ * written. q, k, v are views into the qkv projection's output: element
+ * (b, s, h, c) at b*stride_b + s*stride_s + h*stride_h + c (elements, unit
+ * stride in c; opt.py:72-76 makes them [b, s, heads, 3*d] slices), out
+ * likewise with its own strides ([b, s, heads*d] as opt.py:123-128 leaves it).
+ * lse (optional, [B,H,S] fp32) receives log sum_j exp(scale * q.k_j) for the
+ * backward. D = 64 and CW_BF16 only in this build (CW_ERR_UNSUPPORTED else).
+ */
+int cw_attn_fwd(int64_t B, int64_t H, int64_t S, int64_t D,
+                const void* q, const void* k, const void* v,
+                int64_t stride_b, int64_t stride_s, int64_t stride_h,
+                float scale, int causal,
+                void* out, int64_t out_stride_b, int64_t out_stride_s, int64_t out_stride_h,
+                float* lse, int io_dtype, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

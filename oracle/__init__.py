@@ -14,6 +14,7 @@ line by line in torch, and is pinned by
   * brute-force float64 golden vectors (tests/golden/, pure-Python loops),
   * torch library routines the reference's tests use as their own oracle
     (A @ W + b, nn.LayerNorm, F.cross_entropy),
+  * for the attention core: pure-Python float64 loops, F.scaled_dot_product_attention and its autograd,
   * invariants (split-invariance of statistics, sum of softmax gradient = 0,
     k-step sum == concatenated GEMM, grid composition == master result).
 Parity status: every function below is pinned by at least one such check in
@@ -28,4 +29,5 @@ from .summa import (gemm_ksteps, summa_ab_rank, summa_abt_rank, summa_atb_rank, 
 from .layernorm import (ln2d_partial_stats, ln2d_mean_rstd, ln2d_normalize, ln2d_backward_partials, ln2d_backward_dx,  # noqa: F401
                         ln3d_forward, ln3d_backward, ln_forward_full, ln_backward_full)
 from .vpce import vpce_fwd_local, vpce_finalize, vpce_bwd, vpce_reference_full  # noqa: F401
+from .attention import split_qkv, attention_core, attention_core_backward, attention_brute_force  # noqa: F401
 from . import grid  # noqa: F401

@@ -1,0 +1,84 @@
+"""GPU parity of the attention core (cw_attn_fwd through the C ABI) against the CPU oracle.
+Bar: <= 1e-2 relative (bf16 I/O, fp32 accumulation and softmax)."""
+import pytest
+import torch
+
+from tests.util import assert_parity, randn
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+
+
+def _qkv(b, s, h, d, seed, std=1.0):
+    """One projection output [b, s, h*3*d] as the reference lays it out (benchmark/opt/opt.py:72-76)."""
+    return randn((b, s, h * 3 * d), torch.bfloat16, seed, std=std)
+
+
+def _views(qkv, h, d):
+    b, s, _ = qkv.shape
+    t = qkv.view(b, s, h, 3 * d)
+    return t[..., :d], t[..., d:2 * d], t[..., 2 * d:]
+
+
+@pytest.mark.parametrize("shape", [(1, 64, 1), (2, 256, 3), (1, 100, 2), (2, 257, 2), (1, 1, 1), (1, 33, 1),
+                                   (1, 640, 2), (1, 1000, 1)])
+@pytest.mark.parametrize("causal", [True, False])
+def test_attention_forward_parity(shape, causal):
+    import oracle
+    from cubework_amd import ops
+
+    b, s, h = shape
+    d = 64
+    qkv = _qkv(b, s, h, d, seed=s + h, std=1.5)
+    want, want_lse = oracle.attention_core(*oracle.split_qkv(qkv, h), causal=causal, return_lse=True)
+    q, k, v = _views(qkv.to(DEV), h, d)
+    got, lse = ops.attn_fwd(q, k, v, causal=causal, want_lse=True)
+    torch.cuda.synchronize()
+    assert_parity(got, want, torch.bfloat16, "attention out %s causal=%s" % (shape, causal))
+    assert_parity(lse, want_lse, torch.float32, "attention lse %s" % (shape,), scale=100)
+
+
+def test_attention_rows_are_convex_combinations():
+    """With V = 1 every output is exactly 1 (the probabilities of a row sum to one), and the first query of
+    a causal row attends to key 0 only, so its output is V[0]."""
+    from cubework_amd import ops
+
+    b, s, h, d = 1, 512, 2, 64
+    qkv = _qkv(b, s, h, d, seed=3).to(DEV)
+    q, k, v = _views(qkv, h, d)
+    with_ones = qkv.clone()
+    q1, k1, v1 = _views(with_ones, h, d)
+    v1.fill_(1.0)
+    out = ops.attn_fwd(q1, k1, v1)
+    assert (out.float() - 1.0).abs().max().item() <= 2 ** -7
+    out = ops.attn_fwd(q, k, v)
+    assert torch.equal(out[0, 0].view(h, d), v[0, 0])
+
+
+def test_attention_full_size_sampled_rows():
+    """The OPT-1.3B-shaped workload (batch 4, 2048 tokens, 32 heads of 64): sampled (batch, head) pairs
+    against the float32 oracle."""
+    import oracle
+    from cubework_amd import ops
+
+    b, s, h, d = 4, 2048, 32, 64
+    g = torch.Generator(device="cpu").manual_seed(0)
+    qkv = (torch.randn((b, s, h * 3 * d), generator=g)).to(torch.bfloat16)
+    q, k, v = _views(qkv.to(DEV), h, d)
+    got = ops.attn_fwd(q, k, v).view(b, s, h, d)
+    torch.cuda.synchronize()
+    qc, kc, vc = oracle.split_qkv(qkv, h)
+    for bi, hi in [(0, 0), (3, 31), (1, 17)]:
+        want = oracle.attention_core(qc[bi:bi + 1, hi:hi + 1], kc[bi:bi + 1, hi:hi + 1], vc[bi:bi + 1, hi:hi + 1])
+        assert_parity(got[bi, :, hi, :], want[0], torch.bfloat16, "full-size attention (b=%d, h=%d)" % (bi, hi))
+
+
+def test_attention_rejects_unsupported():
+    from cubework_amd import ops
+
+    q = torch.zeros((1, 8, 1, 32), dtype=torch.bfloat16, device=DEV)
+    with pytest.raises(RuntimeError):
+        ops.attn_fwd(q, q, q)
+    q = torch.zeros((1, 8, 1, 64), dtype=torch.float32, device=DEV)
+    with pytest.raises(RuntimeError):
+        ops.attn_fwd(q, q, q)
