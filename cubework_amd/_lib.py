@@ -37,6 +37,9 @@ SIGNATURES = {
                                  _pp, _int, _i64, _ptr, _i64, _int, _ptr]),
     "cw_attn_fwd": (_int, [_i64, _i64, _i64, _i64, _ptr, _ptr, _ptr, _i64, _i64, _i64, _f32, _int, _ptr, _i64, _i64, _i64,
                            _ptr, _int, _ptr]),
+    "cw_attn_bwd_workspace_bytes": (_i64, [_i64, _i64, _i64]),
+    "cw_attn_bwd": (_int, [_i64, _i64, _i64, _i64, _ptr, _ptr, _ptr, _i64, _i64, _i64, _ptr, _ptr, _i64, _i64, _i64, _ptr,
+                           _f32, _int, _ptr, _ptr, _ptr, _i64, _i64, _i64, _ptr, _i64, _int, _ptr]),
     "cw_colsum_workspace_bytes": (_i64, [_i64, _i64]),
     "cw_colsum": (_int, [_i64, _i64, _ptr, _i64, _ptr, _ptr, _i64, _int, _ptr]),
     "cw_act_bwd_colsum": (_int, [_int, _i64, _i64, _ptr, _i64, _ptr, _i64, _ptr, _i64, _ptr, _ptr, _i64, _int, _ptr]),

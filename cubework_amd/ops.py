@@ -382,3 +382,62 @@ def attn_fwd(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, scale: Optional[
     _lib.check(rc, "cw_attn_fwd")
     out = out.view(B, S, H * D)
     return (out, lse) if want_lse else out
+
+
+def attn_bwd(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, out: torch.Tensor, d_out: torch.Tensor,
+             lse: torch.Tensor, dq: torch.Tensor, dk: torch.Tensor, dv: torch.Tensor,
+             scale: Optional[float] = None, causal: bool = True) -> None:
+    """Gradients of attn_fwd into the [b, s, h, d] views dq, dk, dv (e.g. slices of one buffer shaped like
+    the qkv projection's output). out / d_out: [b, s, h*d] or [b, s, h, d]. See cw_attn_bwd."""
+    lib = _lib.load()
+    _require_device(q, k, v, out, d_out, lse, dq, dk, dv)
+    B, S, H, D = q.shape
+    strides = _bshd_strides(q)
+    if _bshd_strides(k) != strides or _bshd_strides(v) != strides:
+        raise ValueError("q, k, v must share their strides")
+    gstrides = _bshd_strides(dq)
+    if _bshd_strides(dk) != gstrides or _bshd_strides(dv) != gstrides or dq.shape != q.shape:
+        raise ValueError("dq, dk, dv must be [b, s, h, d] views sharing their strides")
+    out4 = out.reshape(B, S, H, D)
+    dout4 = d_out.reshape(B, S, H, D)
+    if dout4.stride(3) != 1 or _bshd_strides(dout4) != _bshd_strides(out4):
+        out4, dout4 = out4.contiguous(), dout4.contiguous()
+    ostr = _bshd_strides(out4)
+    scale = D ** -0.5 if scale is None else float(scale)
+    ws_bytes = lib.cw_attn_bwd_workspace_bytes(B, H, S)
+    ws = torch.empty(max(ws_bytes, 16), dtype=torch.uint8, device=q.device)
+    rc = lib.cw_attn_bwd(B, H, S, D, _p(q), _p(k), _p(v), strides[0], strides[1], strides[2], _p(out4), _p(dout4),
+                         ostr[0], ostr[1], ostr[2], _p(lse), scale, 1 if causal else 0, _p(dq), _p(dk), _p(dv),
+                         gstrides[0], gstrides[1], gstrides[2], _p(ws), ws.numel(), _dtype_code(q), _stream())
+    _lib.check(rc, "cw_attn_bwd")
+
+
+class _AttentionCore(torch.autograd.Function):
+    """qkv [b, s, heads*3*d] (per head: q, k, v side by side, benchmark/opt/opt.py:72-76) -> [b, s, heads*d]."""
+
+    @staticmethod
+    def forward(ctx, qkv: torch.Tensor, heads: int, scale: Optional[float], causal: bool):
+        b, s, w = qkv.shape
+        d = w // (3 * heads)
+        qkv = qkv if qkv.stride(-1) == 1 else qkv.contiguous()
+        t = qkv.view(b, s, heads, 3 * d) if qkv.is_contiguous() else qkv.reshape(b, s, heads, 3 * d)
+        q, k, v = t[..., :d], t[..., d:2 * d], t[..., 2 * d:]
+        out, lse = attn_fwd(q, k, v, scale, causal, want_lse=True)
+        ctx.save_for_backward(t, out, lse)
+        ctx.meta = (heads, d, scale, causal)
+        return out
+
+    @staticmethod
+    def backward(ctx, d_out: torch.Tensor):
+        t, out, lse = ctx.saved_tensors
+        heads, d, scale, causal = ctx.meta
+        b, s = t.shape[0], t.shape[1]
+        q, k, v = t[..., :d], t[..., d:2 * d], t[..., 2 * d:]
+        g = torch.empty((b, s, heads, 3 * d), dtype=t.dtype, device=t.device)
+        attn_bwd(q, k, v, out, d_out.contiguous(), lse, g[..., :d], g[..., d:2 * d], g[..., 2 * d:], scale, causal)
+        return g.view(b, s, heads * 3 * d), None, None, None
+
+
+def attention_core(qkv: torch.Tensor, heads: int, scale: Optional[float] = None, causal: bool = True) -> torch.Tensor:
+    """Differentiable fused attention core on the qkv projection's output."""
+    return _AttentionCore.apply(qkv, heads, scale, causal)

@@ -6,8 +6,11 @@ Structure of benchmark/opt/opt.py:45-211 of the reference (OPTAttention +
 OPTDecoderLayer, pre-LayerNorm variant, dropout 0): LayerNorm -> qkv Linear ->
 causal attention -> out Linear -> residual -> LayerNorm -> fc1 -> activation ->
 fc2 -> residual. The four Linears and two LayerNorms are cubework_amd.module
-layers (HIP path); the attention core (scaled QK^T, causal mask, softmax, PV)
-is model code in the reference and stays a torch call here.
+layers (HIP path). The attention core (scaled QK^T, causal mask, softmax, PV:
+benchmark/opt/opt.py:84-117) is the fused HIP kernel pair cw_attn_fwd /
+cw_attn_bwd for the shapes it provides (bf16, head size 64, which is OPT-1.3B's);
+other head sizes or dtypes use torch's scaled_dot_product_attention, as model
+code would.
 """
 from typing import Dict, Optional, Tuple
 
@@ -16,6 +19,7 @@ import torch.nn as nn
 import torch.nn.functional as F
 
 from . import module as cube_nn
+from . import ops
 
 
 class OPTBlock(nn.Module):
@@ -35,6 +39,8 @@ class OPTBlock(nn.Module):
         self.fc2 = cube_nn.Linear(ffn, hidden, dtype=dtype)
 
     def _attention_core(self, qkv: torch.Tensor) -> torch.Tensor:
+        if self.head_dim == 64 and qkv.dtype == torch.bfloat16 and qkv.is_cuda:
+            return ops.attention_core(qkv, self.heads)
         b, s, _ = qkv.shape
         qkv = qkv.view(b, s, self.heads, 3 * self.head_dim).permute(0, 2, 1, 3)
         q, k, v = torch.chunk(qkv, 3, dim=-1)

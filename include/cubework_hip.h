@@ -277,6 +277,25 @@ int cw_attn_fwd(int64_t B, int64_t H, int64_t S, int64_t D,
                 void* out, int64_t out_stride_b, int64_t out_stride_s, int64_t out_stride_h,
                 float* lse, int io_dtype, void* stream);
 
+/*
+ * Backward of cw_attn_fwd: dq, dk, dv from q, k, v, out, d_out and the forward's lse; what
+ * autograd derives for benchmark/opt/opt.py:84-117 (bmm, mask, softmax, bmm), with the
+ * probabilities recomputed instead of saved. out / d_out share one set of strides, dq / dk /
+ * dv another (e.g. the three slices of one [b, s, heads, 3*d] gradient buffer, so that the
+ * gradient of the qkv projection's output needs no concatenation). workspace:
+ * cw_attn_bwd_workspace_bytes(B, H, S) bytes. No atomics: bit-reproducible.
+ */
+int64_t cw_attn_bwd_workspace_bytes(int64_t B, int64_t H, int64_t S);
+int cw_attn_bwd(int64_t B, int64_t H, int64_t S, int64_t D,
+                const void* q, const void* k, const void* v,
+                int64_t stride_b, int64_t stride_s, int64_t stride_h,
+                const void* out, const void* d_out,
+                int64_t out_stride_b, int64_t out_stride_s, int64_t out_stride_h,
+                const float* lse, float scale, int causal,
+                void* dq, void* dk, void* dv,
+                int64_t grad_stride_b, int64_t grad_stride_s, int64_t grad_stride_h,
+                void* workspace, int64_t workspace_bytes, int io_dtype, void* stream);
+
 #ifdef __cplusplus
 }
 #endif
