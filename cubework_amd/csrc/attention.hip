@@ -15,30 +15,25 @@
 // as the A operand uses the same permutation, which the transposing LDS
 // read of V provides).
 //
-// Block = 4 wavefronts x 64 query rows; K/V tiles of 64 rows are staged in
+// Block = 8 wavefronts x 32 query rows; K/V tiles of 64 rows are staged in
 // LDS (two stages, register prefetch of the next tile), K as [kv][d] read with
 // ds_read_b128, V as [kv][d] read with ds_read_b64_tr_b16. Two blocks are
-// resident per compute unit so that one wavefront's softmax arithmetic
-// overlaps another's MFMAs.
-#include "cw_common.h"
+// resident per compute unit (four wavefronts per SIMD): the kernel is bound by
+// the softmax arithmetic (one v_exp_f32 per score), which the other
+// wavefronts' MFMAs and LDS reads hide behind.
+#include "attention_common.h"
 
 namespace cw {
 
 namespace {
 
-typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
-typedef float f32x16_t __attribute__((ext_vector_type(16)));
-typedef short s16x4_t __attribute__((ext_vector_type(4)));
-typedef short s16x8_t __attribute__((ext_vector_type(8)));
-typedef __attribute__((address_space(3))) char lds_char;
+using namespace attn;
 
-constexpr int kHead = 64;            // head size
-constexpr int kAttnThreads = 256;    // 4 wavefronts
-constexpr int kQPerWave = 64;        // two 32-row query tiles per wavefront
-constexpr int kQPerBlock = 4 * kQPerWave;
-constexpr int kKvTile = 64;          // K/V rows per LDS stage
-constexpr int kTileBytes = kKvTile * kHead * 2;  // 8 KB per operand per stage
-constexpr float kNegBig = -__builtin_huge_valf();
+constexpr int kQT = 1;                    // 32-row query tiles per wavefront
+constexpr int kWaves = 8;                 // wavefronts per block
+constexpr int kThreads = kWaves * 64;
+constexpr int kQPerWave = 32 * kQT;
+constexpr int kQPerBlock = kWaves * kQPerWave;
 
 struct AttnArgs {
     const uint16_t* q;
@@ -53,17 +48,8 @@ struct AttnArgs {
     int causal;
 };
 
-// K tile in LDS: row r (128 B) holds its 16-byte chunk c at position c ^ ((r >> 1) & 7).
-__device__ __forceinline__ int k_lds_offset(int r, int c) { return r * 128 + ((c ^ ((r >> 1) & 7)) << 4); }
-// V tile in LDS: row r holds its 16-byte chunk c inside 32-byte unit (c >> 1) ^ (r & 3).
-__device__ __forceinline__ int v_lds_offset(int r, int c) { return r * 128 + ((((c >> 1) ^ (r & 3)) << 5) | ((c & 1) << 4)); }
-
-__device__ __forceinline__ float xchg32(float v) {
-    return __int_as_float(__builtin_amdgcn_ds_bpermute((int)(((threadIdx.x & 63) ^ 32) << 2), __float_as_int(v)));
-}
-
-__global__ __launch_bounds__(kAttnThreads, 2) void attn_fwd_kernel(const AttnArgs a) {
-    __shared__ __attribute__((aligned(16))) char lds_raw[2 * 2 * kTileBytes];
+__global__ __launch_bounds__(kThreads, 2) void attn_fwd_kernel(const AttnArgs a) {
+    __shared__ __attribute__((aligned(16))) char lds_raw[2 * 2 * kImage];
     lds_char* lds = (lds_char*)lds_raw;
 
     const int tid = threadIdx.x;
@@ -85,9 +71,9 @@ __global__ __launch_bounds__(kAttnThreads, 2) void attn_fwd_kernel(const AttnArg
     const uint16_t* vp = a.v + b * a.sb + h * a.sh;
 
     // Q fragments (B operand): lane = query row l32 of tile qt, 8 d-values at 16 kb + 8 half
-    bf16x8_t qf[2][4];
+    bf16x8_t qf[kQT][4];
 #pragma unroll
-    for (int qt = 0; qt < 2; ++qt) {
+    for (int qt = 0; qt < kQT; ++qt) {
         int row = qw0 + 32 * qt + l32;
         row = row < S ? row : S - 1;
         const uint16_t* p = qp + (int64_t)row * a.ss + 8 * half;
@@ -95,92 +81,77 @@ __global__ __launch_bounds__(kAttnThreads, 2) void attn_fwd_kernel(const AttnArg
         for (int kb = 0; kb < 4; ++kb) qf[qt][kb] = __builtin_bit_cast(bf16x8_t, load_raw(p + 16 * kb));
     }
 
-    f32x16_t oacc[2][2];
+    f32x16_t oacc[kQT][2];
 #pragma unroll
-    for (int qt = 0; qt < 2; ++qt)
+    for (int qt = 0; qt < kQT; ++qt)
 #pragma unroll
         for (int dt = 0; dt < 2; ++dt)
 #pragma unroll
             for (int e = 0; e < 16; ++e) oacc[qt][dt][e] = 0.0f;
-    float m_run[2] = {kNegBig, kNegBig};  // running maximum of scale*log2e*s
-    float l_run[2] = {0.0f, 0.0f};        // this lane's share of the running sum
+    float m_run[kQT], l_run[kQT];  // running maximum of scale*log2e*s; this lane's share of the running sum
+#pragma unroll
+    for (int qt = 0; qt < kQT; ++qt) {
+        m_run[qt] = kNegBig;
+        l_run[qt] = 0.0f;
+    }
 
     int q_hi = q0 + kQPerBlock;
     q_hi = q_hi < S ? q_hi : S;
     const int kv_end = a.causal ? q_hi : S;
-    const int n_tiles = (kv_end + kKvTile - 1) / kKvTile;
+    const int n_tiles = (kv_end + kTile - 1) / kTile;
 
-    // K/V tile loader: 512 chunks of 16 bytes per operand, two per thread
-    raw16_t kreg[2], vreg[2];
-    auto g2r = [&](int tile) {
-#pragma unroll
-        for (int u = 0; u < 2; ++u) {
-            const int id = tid + u * kAttnThreads;
-            int row = tile * kKvTile + (id >> 3);
-            row = row < S ? row : S - 1;
-            const int64_t off = (int64_t)row * a.ss + (id & 7) * 8;
-            kreg[u] = load_raw(kp + off);
-            vreg[u] = load_raw(vp + off);
-        }
-    };
-    auto r2s = [&](int stage) {
-        lds_char* ks = lds + stage * 2 * kTileBytes;
-        lds_char* vs = ks + kTileBytes;
-#pragma unroll
-        for (int u = 0; u < 2; ++u) {
-            const int id = tid + u * kAttnThreads;
-            const int r = id >> 3, c = id & 7;
-            *(__attribute__((address_space(3))) raw16_t*)(ks + k_lds_offset(r, c)) = kreg[u];
-            *(__attribute__((address_space(3))) raw16_t*)(vs + v_lds_offset(r, c)) = vreg[u];
-        }
-    };
-
-    // per-lane LDS read offsets
-    // K fragment (kt, kb): row 32 kt + l32, chunk 2 kb + half
-    // V^T fragment (dt, kvb): rows 16 kvb + 4 hh + {0..3} and + 8, columns 32 dt + 16 (grp & 1) + ...
-    const int grp = lane >> 4, i16 = lane & 15;
-    const int v_hh = grp >> 1;  // which half of the k slots this lane feeds (= lane >> 5)
-
-    g2r(0);
-    r2s(0);
+    TileRegs<kThreads> kreg, vreg;
+    ReadOffsets ro;
+    ro.init(lane);
+    // stage = K row image, V transpose image
+    tile_g2r(kreg, kp, a.ss, 0, S, tid);
+    tile_g2r(vreg, vp, a.ss, 0, S, tid);
+    tile_r2s<true, false>(kreg, lds, nullptr, tid);
+    tile_r2s<false, true>(vreg, nullptr, lds + kImage, tid);
     __syncthreads();
 
     for (int t = 0; t < n_tiles; ++t) {
-        const int stage = t & 1;
-        const int kv0 = t * kKvTile;
-        if (t + 1 < n_tiles) g2r(t + 1);
+        lds_char* ks = lds + (t & 1) * 2 * kImage;
+        lds_char* vs = ks + kImage;
+        const int kv0 = t * kTile;
+        if (t + 1 < n_tiles) {
+            tile_g2r(kreg, kp, a.ss, kv0 + kTile, S, tid);
+            tile_g2r(vreg, vp, a.ss, kv0 + kTile, S, tid);
+        }
 
         const bool active = !a.causal || kv0 <= qw0 + kQPerWave - 1;
         if (active) {
-            lds_char* ks = lds + stage * 2 * kTileBytes;
-            lds_char* vs = ks + kTileBytes;
-            const bool need_mask = (a.causal && kv0 + kKvTile - 1 > qw0) || kv0 + kKvTile > S;
-#pragma unroll
-            for (int kt = 0; kt < 2; ++kt) {
+            const bool need_mask = (a.causal && kv0 + kTile - 1 > qw0) || kv0 + kTile > S;
+            // Only tiles on the diagonal or past the end of the sequence need the mask: a scalar branch
+            // around the compare/select work, which interior tiles skip.
+            const bool masked = __builtin_amdgcn_readfirstlane((int)need_mask) != 0;
+            auto half_tile = [&](auto kt_c) {
+                constexpr int kt = decltype(kt_c)::value;
                 // S^T tiles for both query tiles against kv rows 32 kt .. +31
-                f32x16_t st[2];
+                f32x16_t st[kQT];
 #pragma unroll
-                for (int qt = 0; qt < 2; ++qt)
+                for (int qt = 0; qt < kQT; ++qt)
 #pragma unroll
                     for (int e = 0; e < 16; ++e) st[qt][e] = 0.0f;
 #pragma unroll
                 for (int kb = 0; kb < 4; ++kb) {
-                    const bf16x8_t kf = *(__attribute__((address_space(3))) const bf16x8_t*)(ks + k_lds_offset(32 * kt + l32, 2 * kb + half));
-                    st[0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf, qf[0][kb], st[0], 0, 0, 0);
-                    st[1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf, qf[1][kb], st[1], 0, 0, 0);
+                    const bf16x8_t kf = read_rows<32 * kt>(ks, ro, kb);
+#pragma unroll
+                    for (int qt = 0; qt < kQT; ++qt)
+                        st[qt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf, qf[qt][kb], st[qt], 0, 0, 0);
                 }
-                bf16x8_t pb[2][2];
+                bf16x8_t pb[kQT][2];
 #pragma unroll
-                for (int qt = 0; qt < 2; ++qt) {
+                for (int qt = 0; qt < kQT; ++qt) {
                     // element e: kv = kv0 + 32 kt + 8 (e / 4) + 4 half + e % 4, query = qw0 + 32 qt + l32
-                    if (need_mask) {
+                    if (masked) {
+                        // live <=> kv <= min(query, S-1) <=> 32 kt + 8 (e/4) + e%4 <= lim
                         const int qi = qw0 + 32 * qt + l32;
+                        const int last = a.causal ? (qi < S - 1 ? qi : S - 1) : S - 1;
+                        const int lim = last - kv0 - 4 * half;
 #pragma unroll
-                        for (int e = 0; e < 16; ++e) {
-                            const int kvi = kv0 + 32 * kt + 8 * (e >> 2) + 4 * half + (e & 3);
-                            const bool dead = (a.causal && kvi > qi) || kvi >= S;
-                            st[qt][e] = dead ? kNegBig : st[qt][e];
-                        }
+                        for (int e = 0; e < 16; ++e)
+                            st[qt][e] = (32 * kt + 8 * (e >> 2) + (e & 3) > lim) ? kNegBig : st[qt][e];
                     }
                     float mx = st[qt][0];
 #pragma unroll
@@ -188,70 +159,57 @@ __global__ __launch_bounds__(kAttnThreads, 2) void attn_fwd_kernel(const AttnArg
                     mx = fmaxf(mx, xchg32(mx));
                     const float m_new = fmaxf(m_run[qt], mx * a.scale_log2e);
                     const float m_use = (m_new == kNegBig) ? 0.0f : m_new;  // a row with no live key yet
-                    const float alpha = __builtin_amdgcn_exp2f(m_run[qt] - m_use);
-                    float psum = 0.0f;
+                    // rescale the running sum and O^T only when some row's maximum moved
+                    if (__builtin_amdgcn_ballot_w64(m_new != m_run[qt]) != 0) {
+                        const float alpha = __builtin_amdgcn_exp2f(m_run[qt] - m_use);
+                        l_run[qt] *= alpha;
+#pragma unroll
+                        for (int dt = 0; dt < 2; ++dt)
+#pragma unroll
+                            for (int e = 0; e < 16; ++e) oacc[qt][dt][e] *= alpha;
+                        m_run[qt] = m_new;
+                    }
                     float p[16];
 #pragma unroll
-                    for (int e = 0; e < 16; ++e) {
+                    for (int e = 0; e < 16; ++e)
                         p[e] = __builtin_amdgcn_exp2f(__builtin_fmaf(st[qt][e], a.scale_log2e, -m_use));
-                        psum += p[e];
-                    }
-                    m_run[qt] = m_new;
-                    l_run[qt] = l_run[qt] * alpha + psum;
-#pragma unroll
-                    for (int dt = 0; dt < 2; ++dt)
-#pragma unroll
-                        for (int e = 0; e < 16; ++e) oacc[qt][dt][e] *= alpha;
-                    // k slot j of 16-block kvb: e = 8 kvb + j  (kv = 16 kvb + 4 half + j for j < 4, + 8 + 4 half + j - 4 above)
-#pragma unroll
-                    for (int kvb = 0; kvb < 2; ++kvb) {
-                        bf16x8_t v8;
-#pragma unroll
-                        for (int j = 0; j < 8; ++j) v8[j] = (__bf16)p[8 * kvb + j];
-                        pb[qt][kvb] = v8;
-                    }
+                    // k slot j of 16-block kvb <-> e = 8 kvb + j. The row sum is taken over the rounded
+                    // probabilities, the values the second product uses.
+                    pb[qt][0] = pack_slots(p, 0);
+                    pb[qt][1] = pack_slots(p, 1);
+                    l_run[qt] += sum_slots(pb[qt][1], sum_slots(pb[qt][0], 0.0f));
                 }
                 // O^T += V^T P^T over the 32 kv rows of this half tile
 #pragma unroll
-                for (int kvb = 0; kvb < 2; ++kvb) {
+                for (int dt = 0; dt < 2; ++dt) {
+                    const bf16x8_t vf0 = read_transposed<32 * kt>(vs, ro, dt);
+                    const bf16x8_t vf1 = read_transposed<32 * kt + 16>(vs, ro, dt);
 #pragma unroll
-                    for (int dt = 0; dt < 2; ++dt) {
-                        const int r0 = 32 * kt + 16 * kvb + 4 * v_hh + (i16 >> 2);
-                        const int unit = 2 * dt + (grp & 1);  // 32-byte unit = 16 columns
-                        const int off_lo = r0 * 128 + ((unit ^ (r0 & 3)) << 5) + 8 * (i16 & 3);
-                        const int r1 = r0 + 8;
-                        const int off_hi = r1 * 128 + ((unit ^ (r1 & 3)) << 5) + 8 * (i16 & 3);
-                        const s16x4_t lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4_t*)(vs + off_lo));
-                        const s16x4_t hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4_t*)(vs + off_hi));
-                        const bf16x8_t vf = __builtin_bit_cast(bf16x8_t, (s16x8_t)__builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
-                        oacc[0][dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf, pb[0][kvb], oacc[0][dt], 0, 0, 0);
-                        oacc[1][dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf, pb[1][kvb], oacc[1][dt], 0, 0, 0);
+                    for (int qt = 0; qt < kQT; ++qt) {
+                        oacc[qt][dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf0, pb[qt][0], oacc[qt][dt], 0, 0, 0);
+                        oacc[qt][dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf1, pb[qt][1], oacc[qt][dt], 0, 0, 0);
                     }
                 }
-            }
+            };
+            half_tile(std::integral_constant<int, 0>{});
+            half_tile(std::integral_constant<int, 1>{});
         }
-        if (t + 1 < n_tiles) r2s(stage ^ 1);
+        if (t + 1 < n_tiles) {
+            lds_char* nx = lds + ((t + 1) & 1) * 2 * kImage;
+            tile_r2s<true, false>(kreg, nx, nullptr, tid);
+            tile_r2s<false, true>(vreg, nullptr, nx + kImage, tid);
+        }
         __syncthreads();
     }
 
-    // finish: combine the two halves' sums, normalise, store. Lane holds
-    // O^T[d = 32 dt + 8 (e / 4) + 4 half + e % 4][q = l32] of query tile qt.
+    // finish: combine the two halves' sums, normalise, store
 #pragma unroll
-    for (int qt = 0; qt < 2; ++qt) {
+    for (int qt = 0; qt < kQT; ++qt) {
         const int qi = qw0 + 32 * qt + l32;
         const float l_tot = l_run[qt] + xchg32(l_run[qt]);
         const float inv = l_tot > 0.0f ? __builtin_amdgcn_rcpf(l_tot) : 0.0f;
         if (qi < S) {
-            uint16_t* op = a.o + b * a.ob + (int64_t)qi * a.os + h * a.oh;
-#pragma unroll
-            for (int dt = 0; dt < 2; ++dt)
-#pragma unroll
-                for (int g = 0; g < 4; ++g) {
-                    uint32_t w0 = pack_bf16x2(oacc[qt][dt][4 * g] * inv, oacc[qt][dt][4 * g + 1] * inv);
-                    uint32_t w1 = pack_bf16x2(oacc[qt][dt][4 * g + 2] * inv, oacc[qt][dt][4 * g + 3] * inv);
-                    uint2 w = make_uint2(w0, w1);
-                    *reinterpret_cast<uint2*>(op + 32 * dt + 8 * g + 4 * half) = w;
-                }
+            store_row_pieces(a.o + b * a.ob + (int64_t)qi * a.os + h * a.oh, oacc[qt], inv, half);
             if (half == 0 && a.lse != nullptr)
                 a.lse[(int64_t)bh * S + qi] = (m_run[qt] + __builtin_amdgcn_logf(l_tot)) * kLn2;  // natural-log LSE of scale*s
         }
@@ -290,7 +248,7 @@ extern "C" int cw_attn_fwd(int64_t B, int64_t H, int64_t S, int64_t D, const voi
     a.scale_log2e = scale * kLog2e;
     a.causal = causal ? 1 : 0;
     a.n_qblocks = (int)((S + kQPerBlock - 1) / kQPerBlock);
-    hipLaunchKernelGGL(attn_fwd_kernel, dim3((unsigned)(a.n_qblocks * B * H)), dim3(kAttnThreads), 0,
+    hipLaunchKernelGGL(attn_fwd_kernel, dim3((unsigned)(a.n_qblocks * B * H)), dim3(kThreads), 0,
                        (hipStream_t)stream, a);
     return check_launch("attn_fwd_kernel");
 }

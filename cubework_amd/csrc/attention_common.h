@@ -1,0 +1,129 @@
+// Pieces shared by the attention forward and backward kernels (gfx950, head
+// size 64, bf16): LDS tile images, MFMA operand reads, tile loader.
+#pragma once
+
+#include <type_traits>
+
+#include "cw_common.h"
+
+namespace cw {
+namespace attn {
+
+typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
+typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+typedef float f32x16_t __attribute__((ext_vector_type(16)));
+typedef float f32x4_t __attribute__((ext_vector_type(4)));
+typedef short s16x4_t __attribute__((ext_vector_type(4)));
+typedef short s16x8_t __attribute__((ext_vector_type(8)));
+typedef __attribute__((address_space(3))) char lds_char;
+
+constexpr int kHead = 64;                  // head size
+constexpr int kTile = 64;                  // rows of a streamed tile
+constexpr int kImage = kTile * kHead * 2;  // 8 KB: one LDS image of a tile
+constexpr float kNegBig = -__builtin_huge_valf();
+
+// A 64-row tile ([row][64 bf16], 128 bytes per row) is kept in LDS in one or
+// both of two images:
+//   row image       : 16-byte chunk c of row r at position c ^ ((r >> 1) & 7); read with ds_read_b128 as
+//                     the MFMA operand "row = r0 + lane % 32, k = 8 values at 16 kb + 8 (lane / 32)";
+//   transpose image : chunk c of row r inside 32-byte unit (c >> 1) ^ (r & 3); read with
+//                     ds_read_b64_tr_b16 as the operand "row = column 32 dt + lane % 32 of the tile,
+//                     k slots = tile rows r0 + 4 (lane / 32) + {0..3} and + 8 + {0..3}".
+// Both read patterns are free of bank conflicts (SQ_LDS_BANK_CONFLICT = 0).
+__device__ __forceinline__ int row_image_offset(int r, int c) { return r * 128 + ((c ^ ((r >> 1) & 7)) << 4); }
+__device__ __forceinline__ int tr_image_offset(int r, int c) { return r * 128 + ((((c >> 1) ^ (r & 3)) << 5) | ((c & 1) << 4)); }
+
+// Per-lane byte offsets of the two read patterns, computed once. A read adds a
+// compile-time row offset (a multiple of 16 rows, which leaves the swizzle
+// terms unchanged) as the instruction's immediate.
+struct ReadOffsets {
+    int rows[4];  // [kb]
+    int tr[2];    // [dt]
+    __device__ __forceinline__ void init(int lane) {
+        const int l32 = lane & 31, half = lane >> 5, grp = lane >> 4, i16 = lane & 15;
+#pragma unroll
+        for (int kb = 0; kb < 4; ++kb) rows[kb] = row_image_offset(l32, 2 * kb + half);
+        const int ra = 4 * (grp >> 1) + (i16 >> 2);
+#pragma unroll
+        for (int dt = 0; dt < 2; ++dt) tr[dt] = ra * 128 + (((2 * dt + (grp & 1)) ^ (ra & 3)) << 5) + 8 * (i16 & 3);
+    }
+};
+
+template <int R0>
+__device__ __forceinline__ bf16x8_t read_rows(lds_char* img, const ReadOffsets& ro, int kb) {
+    static_assert(R0 % 16 == 0, "row offset must keep the swizzle");
+    return *(__attribute__((address_space(3))) const bf16x8_t*)(img + ro.rows[kb] + R0 * 128);
+}
+template <int R0>
+__device__ __forceinline__ bf16x8_t read_transposed(lds_char* img, const ReadOffsets& ro, int dt) {
+    static_assert(R0 % 16 == 0, "row offset must keep the swizzle");
+    lds_char* p = img + ro.tr[dt] + R0 * 128;
+    const s16x4_t lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4_t*)p);
+    const s16x4_t hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4_t*)(p + 8 * 128));
+    return __builtin_bit_cast(bf16x8_t, (s16x8_t)__builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
+}
+
+// bf16 B operand from 8 consecutive accumulator elements (k slot j <-> element 8 blk + j).
+__device__ __forceinline__ bf16x8_t pack_slots(const float (&x)[16], int blk) {
+    bf16x8_t r;
+#pragma unroll
+    for (int j = 0; j < 8; ++j) r[j] = (__bf16)x[8 * blk + j];
+    return r;
+}
+// Sum of the 8 bf16 values of an operand, in fp32 (v_dot2 with ones).
+__device__ __forceinline__ float sum_slots(bf16x8_t v, float acc) {
+    const bf16x2_t ones = {(__bf16)1.0f, (__bf16)1.0f};
+    acc = __builtin_amdgcn_fdot2_f32_bf16(__builtin_shufflevector(v, v, 0, 1), ones, acc, false);
+    acc = __builtin_amdgcn_fdot2_f32_bf16(__builtin_shufflevector(v, v, 2, 3), ones, acc, false);
+    acc = __builtin_amdgcn_fdot2_f32_bf16(__builtin_shufflevector(v, v, 4, 5), ones, acc, false);
+    acc = __builtin_amdgcn_fdot2_f32_bf16(__builtin_shufflevector(v, v, 6, 7), ones, acc, false);
+    return acc;
+}
+
+// Lane (row = lane % 32, half = lane / 32) holds, of a transposed 64 x 32 result, the values
+// d = 32 dt + 8 (e / 4) + 4 half + e % 4 of its row: write them, times `mul`, as bf16.
+__device__ __forceinline__ void store_row_pieces(uint16_t* rowp, const f32x16_t (&acc)[2], float mul, int half) {
+#pragma unroll
+    for (int dt = 0; dt < 2; ++dt)
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+            const uint2 w = make_uint2(pack_bf16x2(acc[dt][4 * g] * mul, acc[dt][4 * g + 1] * mul),
+                                       pack_bf16x2(acc[dt][4 * g + 2] * mul, acc[dt][4 * g + 3] * mul));
+            *reinterpret_cast<uint2*>(rowp + 32 * dt + 8 * g + 4 * half) = w;
+        }
+}
+
+// The value of lane ^ 32.
+__device__ __forceinline__ float xchg32(float v) {
+    return __int_as_float(__builtin_amdgcn_ds_bpermute((int)(((threadIdx.x & 63) ^ 32) << 2), __float_as_int(v)));
+}
+
+// Loader of one 64-row tile: 512 chunks of 16 bytes spread over NT threads; rows past S read row S-1.
+template <int NT>
+struct TileRegs {
+    static constexpr int kPer = 512 / NT;
+    raw16_t r[kPer];
+};
+template <int NT>
+__device__ __forceinline__ void tile_g2r(TileRegs<NT>& t, const uint16_t* base, int64_t row_stride, int row0, int S, int tid) {
+#pragma unroll
+    for (int u = 0; u < TileRegs<NT>::kPer; ++u) {
+        const int id = tid + u * NT;
+        int row = row0 + (id >> 3);
+        row = row < S ? row : S - 1;
+        t.r[u] = load_raw(base + (int64_t)row * row_stride + (id & 7) * 8);
+    }
+}
+template <bool ROW_IMAGE, bool TR_IMAGE, int NT>
+__device__ __forceinline__ void tile_r2s(const TileRegs<NT>& t, lds_char* row_img, lds_char* tr_img, int tid) {
+#pragma unroll
+    for (int u = 0; u < TileRegs<NT>::kPer; ++u) {
+        const int id = tid + u * NT;
+        const int r = id >> 3, c = id & 7;
+        if (ROW_IMAGE) *(__attribute__((address_space(3))) raw16_t*)(row_img + row_image_offset(r, c)) = t.r[u];
+        if (TR_IMAGE) *(__attribute__((address_space(3))) raw16_t*)(tr_img + tr_image_offset(r, c)) = t.r[u];
+    }
+}
+
+}  // namespace attn
+}  // namespace cw
