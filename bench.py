@@ -205,6 +205,23 @@ def bench_other_configs(device, sets):
     flop1 = 2.0 * 4096 * 1024 * 4096
     out["linear1d_fp32_fwd"] = {"us": round(us, 2), "TFLOPs": round(flop1 / us / 1e6, 1),
                                 "frac_fp32_mfma": round(flop1 / us / 1e6 / 157.3, 4)}
+    # attention core of config 5: batch 4, 32 heads of 64, 2048 tokens, causal; FLOP counted on the
+    # unmasked half only (4 b h s^2 d / 2 forward, 2.5 x that backward)
+    b_, s_, h_, d_ = 4, 2048, 32, 64
+    qkv = _seeded((b_, s_, h_ * 3 * d_), 21, 1.0, torch.bfloat16).to(device)
+    t4 = qkv.view(b_, s_, h_, 3 * d_)
+    q_, k_, v_ = t4[..., :d_], t4[..., d_:2 * d_], t4[..., 2 * d_:]
+    attn_flop = 4.0 * b_ * h_ * s_ * s_ * d_ / 2
+    us = event_time_us(lambda: ops.attn_fwd(q_, k_, v_), 30, 5)
+    out["attention_fwd_causal"] = {"us": round(us, 2), "TFLOPs": round(attn_flop / us / 1e6, 1),
+                                   "frac": round(attn_flop / us / 1e6 / MFMA_BF16_PEAK_TFLOPS, 4)}
+    o_, lse_ = ops.attn_fwd(q_, k_, v_, want_lse=True)
+    do_ = _seeded((b_, s_, h_ * d_), 22, 1.0, torch.bfloat16).to(device)
+    g_ = torch.empty_like(t4)
+    us = event_time_us(lambda: ops.attn_bwd(q_, k_, v_, o_, do_, lse_, g_[..., :d_], g_[..., d_:2 * d_], g_[..., 2 * d_:]), 30, 5)
+    out["attention_bwd_causal"] = {"us": round(us, 2), "TFLOPs": round(2.5 * attn_flop / us / 1e6, 1),
+                                   "frac": round(2.5 * attn_flop / us / 1e6 / MFMA_BF16_PEAK_TFLOPS, 4)}
+    del qkv, t4, o_, do_, g_
     # config 5: OPT-1.3B-shaped block, batch 4 x seq 2048, bf16, forward + backward
     initialize("2d", 1)
     torch.manual_seed(0)
