@@ -205,6 +205,28 @@ def bench_other_configs(device, sets):
     flop1 = 2.0 * 4096 * 1024 * 4096
     out["linear1d_fp32_fwd"] = {"us": round(us, 2), "TFLOPs": round(flop1 / us / 1e6, 1),
                                 "frac_fp32_mfma": round(flop1 / us / 1e6 / 157.3, 4)}
+    # vocab-parallel embedding (rank 1 of 4 of OPT's 50272 x 2048 table, 8192 tokens): bytes = ids + the rows
+    # actually read (about a quarter of the tokens are live) + the output written
+    e_tok, e_dim, e_vloc = 8192, 2048, 12568
+    ids = torch.randint(0, 50272, (e_tok,), generator=torch.Generator().manual_seed(31)).to(device)
+    tabs = [_seeded((e_vloc, e_dim), 32 + j, 0.02, torch.bfloat16).to(device) for j in range(6)]  # 6 x 49 MiB
+    live = int(((ids >= e_vloc) & (ids < 2 * e_vloc)).sum().item())
+    j = [0]
+
+    def emb_fwd():
+        j[0] += 1
+        ops.embedding_fwd(ids, tabs[j[0] % 6], e_vloc)
+    us = event_time_us(emb_fwd, 30, 5)
+    nbytes = e_tok * 8 + live * e_dim * 2 + e_tok * e_dim * 2
+    out["vocab_embedding_fwd"] = {"us": round(us, 2), "GBps": round(nbytes / us / 1e3, 1), "bytes": nbytes,
+                                  "frac": round(nbytes / us / 1e3 / HBM_PEAK_GBPS, 3)}
+    dys_e = [_seeded((e_tok, e_dim), 40 + j_, 1.0, torch.bfloat16).to(device) for j_ in range(4)]
+    us = event_time_us(lambda: ops.embedding_bwd(ids, dys_e[j[0] % 4], e_vloc, e_vloc), 20, 3)
+    nbytes = 3 * e_tok * 8 + live * e_dim * 2 + e_vloc * e_dim * 2
+    out["vocab_embedding_bwd"] = {"us": round(us, 2), "GBps": round(nbytes / us / 1e3, 1), "bytes": nbytes,
+                                  "frac": round(nbytes / us / 1e3 / HBM_PEAK_GBPS, 3),
+                                  "note": "includes the caller-side stable sort of the ids and the zero fill"}
+    del tabs, dys_e
     # attention core of config 5: batch 4, 32 heads of 64, 2048 tokens, causal; FLOP counted on the
     # unmasked half only (4 b h s^2 d / 2 forward, 2.5 x that backward)
     b_, s_, h_, d_ = 4, 2048, 32, 64

@@ -1,0 +1,221 @@
+// Vocab-parallel embedding, one rank's vocabulary slice, for gfx950.
+// forward : out[t, :] = (start <= id[t] < start + V_loc) ? weight[id[t] - start, :] : 0
+//           (cubework/module/parallel_1d/module.py:441-455, parallel_2d/module.py:345-355 of the
+//           reference: mask, shifted index, F.embedding, zeroed masked rows) in one pass: a masked
+//           row is never read, only written as zeros.
+// backward: d_weight[r, :] = sum over tokens with id - start == r of d_out[t, :]
+//           (autograd of F.embedding), deterministic: the caller supplies the token order sorted
+//           by id, one block owns one run of equal ids, its wavefronts split the run and are
+//           combined in a fixed order. No atomics.
+// Both are HBM-streaming kernels: 16-byte accesses, one wavefront per row.
+#include "cw_common.h"
+
+namespace cw {
+
+namespace {
+
+constexpr int kEmbWaves = 4;
+
+template <typename T>
+__global__ __launch_bounds__(kEmbWaves * 64) void embed_fwd_kernel(int64_t T_rows, int64_t E, const int64_t* __restrict__ ids,
+                                                                   int64_t vocab_start, int64_t V_loc,
+                                                                   const T* __restrict__ weight, int64_t ldw,
+                                                                   T* __restrict__ out, int64_t ldo, int vec_ok) {
+    constexpr int V = elem<T>::kVec;
+    const int lane = threadIdx.x & 63;
+    const int64_t wave = (int64_t)blockIdx.x * kEmbWaves + (threadIdx.x >> 6);
+    const int64_t nwaves = (int64_t)gridDim.x * kEmbWaves;
+    for (int64_t t = wave; t < T_rows; t += nwaves) {
+        const int64_t local = ids[t] - vocab_start;
+        const bool masked = local < 0 || local >= V_loc;  // same for the whole wavefront
+        const T* src = weight + (masked ? 0 : local) * ldw;
+        T* dst = out + t * ldo;
+        if (vec_ok) {
+            const int64_t nvec = E / V;
+            for (int64_t c = lane; c < nvec; c += 64) {
+                raw16_t v = (raw16_t){0u, 0u, 0u, 0u};
+                if (!masked) v = load_raw(src + c * V);
+                store_raw_stream(dst + c * V, v);
+            }
+            for (int64_t c = nvec * V + lane; c < E; c += 64) store_elem(dst + c, masked ? 0.0f : load_elem(src + c));
+        } else {
+            for (int64_t c = lane; c < E; c += 64) store_elem(dst + c, masked ? 0.0f : load_elem(src + c));
+        }
+    }
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void zero_rows_kernel(int64_t R, int64_t E, T* __restrict__ p, int64_t ld, int vec_ok) {
+    constexpr int V = elem<T>::kVec;
+    const int lane = threadIdx.x & 63;
+    const int64_t wave = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+    const int64_t nwaves = (int64_t)gridDim.x * 4;
+    for (int64_t r = wave; r < R; r += nwaves) {
+        T* dst = p + r * ld;
+        if (vec_ok) {
+            const int64_t nvec = E / V;
+            for (int64_t c = lane; c < nvec; c += 64) store_raw_stream(dst + c * V, (raw16_t){0u, 0u, 0u, 0u});
+            for (int64_t c = nvec * V + lane; c < E; c += 64) store_elem(dst + c, 0.0f);
+        } else {
+            for (int64_t c = lane; c < E; c += 64) store_elem(dst + c, 0.0f);
+        }
+    }
+}
+
+// One block per position i of the sorted order; only the first position of a run of equal ids works.
+// Wavefront w sums tokens i + w, i + w + 4, ... of the run for a slab of 64 x V x NCH columns at a time.
+template <typename T, int NCH>
+__global__ __launch_bounds__(kEmbWaves * 64) void embed_bwd_kernel(int64_t T_rows, int64_t E,
+                                                                   const int64_t* __restrict__ sorted_ids,
+                                                                   const int64_t* __restrict__ order, int64_t vocab_start,
+                                                                   int64_t V_loc, int64_t skip_row,
+                                                                   const T* __restrict__ d_out, int64_t ldo,
+                                                                   T* __restrict__ d_weight, int64_t ldw) {
+    constexpr int V = elem<T>::kVec;
+    __shared__ float red[kEmbWaves - 1][NCH * V][64];
+    const int64_t i = blockIdx.x;
+    const int64_t id = sorted_ids[i];
+    if (i > 0 && sorted_ids[i - 1] == id) return;
+    const int64_t local = id - vocab_start;
+    if (local < 0 || local >= V_loc || local == skip_row) return;
+    int64_t run = 1;
+    while (i + run < T_rows && sorted_ids[i + run] == id) ++run;
+
+    const int lane = threadIdx.x & 63;
+    const int wave = threadIdx.x >> 6;
+    T* dst = d_weight + local * ldw;
+    for (int64_t col0 = 0; col0 < E; col0 += (int64_t)64 * V * NCH) {
+        float acc[NCH][V];
+#pragma unroll
+        for (int j = 0; j < NCH; ++j)
+#pragma unroll
+            for (int e = 0; e < V; ++e) acc[j][e] = 0.0f;
+        for (int64_t r = wave; r < run; r += kEmbWaves) {
+            const T* src = d_out + order[i + r] * ldo + col0;
+#pragma unroll
+            for (int j = 0; j < NCH; ++j) {
+                const int64_t c = ((int64_t)j * 64 + lane) * V;
+                if (col0 + c < E) {
+                    float v[V];
+                    unpack_raw(load_raw_stream(src + c), v, (const T*)nullptr);
+#pragma unroll
+                    for (int e = 0; e < V; ++e) acc[j][e] += v[e];
+                }
+            }
+        }
+        if (wave > 0) {
+#pragma unroll
+            for (int j = 0; j < NCH; ++j)
+#pragma unroll
+                for (int e = 0; e < V; ++e) red[wave - 1][j * V + e][lane] = acc[j][e];
+        }
+        __syncthreads();
+        if (wave == 0) {
+#pragma unroll
+            for (int j = 0; j < NCH; ++j) {
+                const int64_t c = ((int64_t)j * 64 + lane) * V;
+                if (col0 + c < E) {
+#pragma unroll
+                    for (int w = 0; w < kEmbWaves - 1; ++w)
+#pragma unroll
+                        for (int e = 0; e < V; ++e) acc[j][e] += red[w][j * V + e][lane];
+                    store_raw_stream(dst + col0 + c, pack_raw(acc[j], (const T*)nullptr));
+                }
+            }
+        }
+        __syncthreads();
+    }
+}
+
+// Element-wise variant for rows that are not 16-byte aligned / E not a multiple of the vector.
+template <typename T>
+__global__ __launch_bounds__(256) void embed_bwd_generic_kernel(int64_t T_rows, int64_t E,
+                                                                const int64_t* __restrict__ sorted_ids,
+                                                                const int64_t* __restrict__ order, int64_t vocab_start,
+                                                                int64_t V_loc, int64_t skip_row,
+                                                                const T* __restrict__ d_out, int64_t ldo,
+                                                                T* __restrict__ d_weight, int64_t ldw) {
+    const int64_t i = blockIdx.x;
+    const int64_t id = sorted_ids[i];
+    if (i > 0 && sorted_ids[i - 1] == id) return;
+    const int64_t local = id - vocab_start;
+    if (local < 0 || local >= V_loc || local == skip_row) return;
+    int64_t run = 1;
+    while (i + run < T_rows && sorted_ids[i + run] == id) ++run;
+    for (int64_t c = threadIdx.x; c < E; c += 256) {
+        float acc = 0.0f;
+        for (int64_t r = 0; r < run; ++r) acc += load_elem(d_out + order[i + r] * ldo + c);
+        store_elem(d_weight + local * ldw + c, acc);
+    }
+}
+
+int rows_grid(int64_t rows, int waves_per_block) {
+    int64_t blocks = (rows + waves_per_block - 1) / waves_per_block;
+    const int64_t cap = 256 * 8;
+    blocks = blocks < cap ? blocks : cap;
+    return (int)(blocks > 0 ? blocks : 1);
+}
+
+template <typename T>
+int fwd_impl(int64_t T_rows, int64_t E, const int64_t* ids, int64_t vocab_start, int64_t V_loc, const void* weight,
+             int64_t ldw, void* out, int64_t ldo, hipStream_t s) {
+    const int vec_ok = aligned16(weight) && aligned16(out) && ldw % elem<T>::kVec == 0 && ldo % elem<T>::kVec == 0;
+    hipLaunchKernelGGL(embed_fwd_kernel<T>, dim3(rows_grid(T_rows, kEmbWaves)), dim3(kEmbWaves * 64), 0, s, T_rows, E, ids,
+                       vocab_start, V_loc, (const T*)weight, ldw, (T*)out, ldo, vec_ok);
+    return check_launch("embed_fwd_kernel");
+}
+
+template <typename T>
+int bwd_impl(int64_t T_rows, int64_t E, const int64_t* sorted_ids, const int64_t* order, int64_t vocab_start,
+             int64_t V_loc, int64_t skip_row, const void* d_out, int64_t ldo, void* d_weight, int64_t ldw, hipStream_t s) {
+    constexpr int V = elem<T>::kVec;
+    const int w_vec = aligned16(d_weight) && ldw % V == 0;
+    hipLaunchKernelGGL(zero_rows_kernel<T>, dim3(rows_grid(V_loc, 4)), dim3(256), 0, s, V_loc, E, (T*)d_weight, ldw, w_vec);
+    int rc = check_launch("zero_rows_kernel");
+    if (rc != CW_OK || T_rows == 0) return rc;
+    const bool vec = w_vec && aligned16(d_out) && ldo % V == 0 && E % V == 0;
+    if (vec) {
+        if (E <= 64 * V)
+            hipLaunchKernelGGL((embed_bwd_kernel<T, 1>), dim3((unsigned)T_rows), dim3(kEmbWaves * 64), 0, s, T_rows, E, sorted_ids,
+                               order, vocab_start, V_loc, skip_row, (const T*)d_out, ldo, (T*)d_weight, ldw);
+        else
+            hipLaunchKernelGGL((embed_bwd_kernel<T, 4>), dim3((unsigned)T_rows), dim3(kEmbWaves * 64), 0, s, T_rows, E, sorted_ids,
+                               order, vocab_start, V_loc, skip_row, (const T*)d_out, ldo, (T*)d_weight, ldw);
+    } else {
+        hipLaunchKernelGGL(embed_bwd_generic_kernel<T>, dim3((unsigned)T_rows), dim3(256), 0, s, T_rows, E, sorted_ids, order,
+                           vocab_start, V_loc, skip_row, (const T*)d_out, ldo, (T*)d_weight, ldw);
+    }
+    return check_launch("embed_bwd_kernel");
+}
+
+}  // namespace
+}  // namespace cw
+
+using namespace cw;
+
+extern "C" int cw_embed_fwd(int64_t T, int64_t E, const int64_t* ids, int64_t vocab_start, int64_t V_loc,
+                            const void* weight, int64_t ldw, void* out, int64_t ldo, int io_dtype, void* stream) {
+    if (T < 0 || E <= 0 || V_loc <= 0) return fail(CW_ERR_INVALID, "cw_embed_fwd: bad shape T=%lld E=%lld V_loc=%lld", (long long)T, (long long)E, (long long)V_loc);
+    if (io_dtype != CW_BF16 && io_dtype != CW_F32) return fail(CW_ERR_INVALID, "cw_embed_fwd: bad io_dtype %d", io_dtype);
+    if (T == 0) return CW_OK;
+    if (ids == nullptr || weight == nullptr || out == nullptr || ldw < E || ldo < E)
+        return fail(CW_ERR_INVALID, "cw_embed_fwd: null pointer or leading dimension < E");
+    hipStream_t s = (hipStream_t)stream;
+    return io_dtype == CW_BF16 ? fwd_impl<bf16_t>(T, E, ids, vocab_start, V_loc, weight, ldw, out, ldo, s)
+                               : fwd_impl<float>(T, E, ids, vocab_start, V_loc, weight, ldw, out, ldo, s);
+}
+
+extern "C" int cw_embed_bwd(int64_t T, int64_t E, const int64_t* sorted_ids, const int64_t* order, int64_t vocab_start,
+                            int64_t V_loc, int64_t skip_row, const void* d_out, int64_t ldo, void* d_weight,
+                            int64_t ldw, int io_dtype, void* stream) {
+    if (T < 0 || E <= 0 || V_loc <= 0) return fail(CW_ERR_INVALID, "cw_embed_bwd: bad shape T=%lld E=%lld V_loc=%lld", (long long)T, (long long)E, (long long)V_loc);
+    if (io_dtype != CW_BF16 && io_dtype != CW_F32) return fail(CW_ERR_INVALID, "cw_embed_bwd: bad io_dtype %d", io_dtype);
+    if (T > INT32_MAX) return fail(CW_ERR_INVALID, "cw_embed_bwd: too many tokens");
+    if (d_weight == nullptr || ldw < E) return fail(CW_ERR_INVALID, "cw_embed_bwd: d_weight is NULL or ldw < E");
+    if (T > 0 && (sorted_ids == nullptr || order == nullptr || d_out == nullptr || ldo < E))
+        return fail(CW_ERR_INVALID, "cw_embed_bwd: null pointer or leading dimension < E");
+    hipStream_t s = (hipStream_t)stream;
+    return io_dtype == CW_BF16
+               ? bwd_impl<bf16_t>(T, E, sorted_ids, order, vocab_start, V_loc, skip_row, d_out, ldo, d_weight, ldw, s)
+               : bwd_impl<float>(T, E, sorted_ids, order, vocab_start, V_loc, skip_row, d_out, ldo, d_weight, ldw, s);
+}

@@ -441,3 +441,61 @@ class _AttentionCore(torch.autograd.Function):
 def attention_core(qkv: torch.Tensor, heads: int, scale: Optional[float] = None, causal: bool = True) -> torch.Tensor:
     """Differentiable fused attention core on the qkv projection's output."""
     return _AttentionCore.apply(qkv, heads, scale, causal)
+
+
+# --------------------------------------------------------------------------
+# vocab-parallel embedding
+# --------------------------------------------------------------------------
+def embedding_fwd(ids: torch.Tensor, weight: torch.Tensor, vocab_start: int = 0) -> torch.Tensor:
+    """Rows of `weight` ([V_loc, E]) for the ids inside [vocab_start, vocab_start + V_loc), zeros for the
+    others; ids of any shape, result ids.shape + (E,). See cw_embed_fwd."""
+    lib = _lib.load()
+    _require_device(ids, weight)
+    if ids.dtype != torch.int64:
+        raise TypeError("ids must be int64")
+    w = _rows(weight)
+    flat = ids.reshape(-1).contiguous()
+    T, (V_loc, E) = flat.numel(), w.shape
+    out = torch.empty((T, E), dtype=w.dtype, device=w.device)
+    rc = lib.cw_embed_fwd(T, E, _p(flat), int(vocab_start), V_loc, _p(w), _ld(w), _p(out), _ld(out), _dtype_code(w),
+                          _stream())
+    _lib.check(rc, "cw_embed_fwd")
+    return out.view(tuple(ids.shape) + (E,))
+
+
+def embedding_bwd(ids: torch.Tensor, d_out: torch.Tensor, num_rows: int, vocab_start: int = 0,
+                  skip_row: int = -1) -> torch.Tensor:
+    """Gradient of embedding_fwd with respect to the [num_rows, E] weight slice. See cw_embed_bwd."""
+    lib = _lib.load()
+    _require_device(ids, d_out)
+    g = _rows(d_out.reshape(-1, d_out.shape[-1]))
+    flat = ids.reshape(-1)
+    T, E = g.shape
+    sorted_ids, order = torch.sort(flat, stable=True)
+    dw = torch.empty((num_rows, E), dtype=g.dtype, device=g.device)
+    rc = lib.cw_embed_bwd(T, E, _p(sorted_ids), _p(order), int(vocab_start), num_rows, int(skip_row), _p(g), _ld(g),
+                          _p(dw), _ld(dw), _dtype_code(g), _stream())
+    _lib.check(rc, "cw_embed_bwd")
+    return dw
+
+
+class _VocabEmbedding(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, ids, weight, vocab_start, skip_row):
+        ctx.save_for_backward(ids)
+        ctx.meta = (weight.shape[0], vocab_start, skip_row)
+        return embedding_fwd(ids, weight, vocab_start)
+
+    @staticmethod
+    def backward(ctx, d_out):
+        (ids,) = ctx.saved_tensors
+        rows, vocab_start, skip_row = ctx.meta
+        return None, embedding_bwd(ids, d_out, rows, vocab_start, skip_row), None, None
+
+
+def vocab_embedding(ids: torch.Tensor, weight: torch.Tensor, vocab_start: int = 0,
+                    padding_idx: Optional[int] = None) -> torch.Tensor:
+    """Differentiable masked embedding lookup of one vocabulary slice. padding_idx is the row of `weight`
+    that receives no gradient (what F.embedding's padding_idx means for the tensor it is handed)."""
+    skip = -1 if padding_idx is None else int(padding_idx)
+    return _VocabEmbedding.apply(ids, weight, int(vocab_start), skip)

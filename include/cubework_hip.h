@@ -258,6 +258,31 @@ int cw_vpce_bwd(int64_t T, int64_t V, const void* logits, int64_t ld,
                 const float* dloss_rows, float dloss_scale,
                 void* grad, int64_t ld_grad, int io_dtype, int grad_dtype, void* stream);
 
+/* ---- vocab-parallel embedding -------------------------------------------- */
+/*
+ * out[t, :] = (vocab_start <= ids[t] < vocab_start + V_loc) ? weight[ids[t] - vocab_start, :] : 0
+ * Replaces the mask / shifted index / F.embedding / zeroing of masked rows in
+ * VocabParallelEmbedding1D.forward (cubework/module/parallel_1d/module.py:441-452),
+ * VocabParallelEmbedding2D.forward (parallel_2d/module.py:345-353),
+ * VocabParallelEmbedding3D.forward (parallel_3d/module.py:455-466), and, with
+ * vocab_start = 0 and V_loc = num_embeddings, F.embedding in Embedding1D/2D/3D
+ * (parallel_1d/module.py:390, parallel_2d/module.py:290, parallel_3d/module.py:396).
+ * The index arithmetic is integer-exact; the copy is bit-exact.
+ */
+int cw_embed_fwd(int64_t T, int64_t E, const int64_t* ids, int64_t vocab_start, int64_t V_loc,
+                 const void* weight, int64_t ldw, void* out, int64_t ldo, int io_dtype, void* stream);
+
+/*
+ * d_weight[r, :] = sum over tokens t with ids[t] - vocab_start == r of d_out[t, :] (fp32 sum, rounded
+ * once); rows without tokens, and row skip_row (F.embedding's padding_idx, -1 for none), are zero.
+ * Autograd of the F.embedding call above. sorted_ids / order: the ids in ascending order and the
+ * token position of each (a stable sort by the caller); runs of equal ids are summed in that order,
+ * without atomics, so the result is bit-reproducible.
+ */
+int cw_embed_bwd(int64_t T, int64_t E, const int64_t* sorted_ids, const int64_t* order,
+                 int64_t vocab_start, int64_t V_loc, int64_t skip_row,
+                 const void* d_out, int64_t ldo, void* d_weight, int64_t ldw, int io_dtype, void* stream);
+
 /* ---- attention core ------------------------------------------------------ */
 /*
  * out[b, s, h, :] = softmax_j(scale * q[b,s,h,:] . k[b,j,h,:] + causal mask) . v[b,j,h,:]

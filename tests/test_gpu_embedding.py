@@ -1,0 +1,109 @@
+"""GPU parity of the vocab-parallel embedding (cw_embed_fwd / cw_embed_bwd through the C ABI): the lookup
+is a bit-exact copy with integer-exact masking; the gradient is an fp32 sum rounded once."""
+import pytest
+import torch
+
+from tests.util import assert_parity, randn
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+
+
+def _ids(shape, vocab, seed, hot=None):
+    g = torch.Generator().manual_seed(seed)
+    ids = torch.randint(0, vocab, shape, generator=g)
+    if hot is not None:  # a frequent token: long runs in the sorted order
+        ids.view(-1)[::3] = hot
+    return ids
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("case", [(4, 37, 1000, 256, 250, 64), (2, 128, 50272, 12568, 12568, 2048),
+                                  (1, 5, 64, 64, 0, 8), (3, 11, 300, 100, 100, 52), (1, 1, 16, 4, 12, 520)])
+def test_embedding_forward_backward_parity(case, dtype):
+    import oracle
+    from cubework_amd import ops
+
+    b, s, vocab, v_loc, start, e = case
+    ids = _ids((b, s), vocab, seed=b * s, hot=start + 1 if v_loc > 1 else None)
+    edges = torch.tensor([start - 1, start, start + v_loc - 1, start + v_loc, 0, vocab - 1]).clamp(0, vocab - 1)
+    n = min(6, ids.numel())
+    ids.view(-1)[:n] = edges[:n]
+    w = randn((v_loc, e), dtype, 5)
+    want = oracle.vocab_embedding_fwd(ids, w, start)
+    got = ops.embedding_fwd(ids.to(DEV), w.to(DEV), start)
+    torch.cuda.synchronize()
+    assert got.shape == (b, s, e)
+    assert torch.equal(got.cpu(), want), "the lookup must be a bit-exact copy / exact zeros"
+
+    d_out = randn((b, s, e), dtype, 6)
+    for pad in (None, 1 if v_loc > 1 else 0):
+        want_dw = oracle.vocab_embedding_bwd(ids, d_out, v_loc, start, pad)
+        got_dw = ops.embedding_bwd(ids.to(DEV), d_out.to(DEV), v_loc, start, -1 if pad is None else pad)
+        again = ops.embedding_bwd(ids.to(DEV), d_out.to(DEV), v_loc, start, -1 if pad is None else pad)
+        torch.cuda.synchronize()
+        assert torch.equal(got_dw, again), "no atomics: bit-reproducible"
+        assert_parity(got_dw, want_dw, dtype, "embedding d_weight %s pad=%s" % (case, pad))
+        untouched = torch.ones(v_loc, dtype=torch.bool)
+        local = ids.view(-1) - start
+        live = (local >= 0) & (local < v_loc)
+        untouched[local[live]] = False
+        assert (got_dw.cpu()[untouched] == 0).all(), "rows without tokens are exactly zero"
+
+
+def test_vocab_slices_sum_to_the_full_lookup():
+    """Four vocabulary slices: every token is live in exactly one, so the slices' outputs sum (the
+    all-reduce of parallel_1d/module.py:454) to F.embedding on the whole table, bit for bit."""
+    from cubework_amd import ops
+
+    vocab, e, p = 1024, 128, 4
+    ids = _ids((2, 77), vocab, 3).to(DEV)
+    table = randn((vocab, e), torch.bfloat16, 4).to(DEV)
+    total = torch.zeros((2, 77, e), dtype=torch.float32, device=DEV)
+    for r in range(p):
+        total += ops.embedding_fwd(ids, table[r * vocab // p:(r + 1) * vocab // p], r * vocab // p).float()
+    assert torch.equal(total.to(torch.bfloat16), torch.nn.functional.embedding(ids, table))
+
+
+@pytest.mark.parametrize("mode", [None, "1d", "2d", "3d"])
+@pytest.mark.parametrize("vocab_parallel", [False, True])
+def test_facade_embedding_size1(mode, vocab_parallel):
+    import cubework_amd.module as cube_nn
+    from cubework_amd.distributed import initialize
+
+    initialize(mode, 1)
+    torch.manual_seed(0)
+    emb = cube_nn.Embedding(200, 64, vocab_parallel=vocab_parallel and mode is not None, padding_idx=3,
+                            dtype=torch.bfloat16).to(DEV)
+    assert emb.weight.shape == (200, 64) and (emb.weight[3] == 0).all()
+    ids = _ids((8, 16), 200, 9).to(DEV)   # 8 rows: divisible by every batch split at size 1
+    ids[0, :4] = 3
+    out = emb(ids)
+    ref_w = emb.weight.detach().clone().requires_grad_(True)
+    ref = torch.nn.functional.embedding(ids, ref_w, padding_idx=3)
+    assert torch.equal(out, ref)
+    d = randn((8, 16, 64), torch.bfloat16, 10).to(DEV)
+    out.backward(d)
+    ref.backward(d)
+    assert_parity(emb.weight.grad, ref_w.grad.float().cpu(), torch.bfloat16, "embedding weight grad (%s)" % mode)
+    assert (emb.weight.grad[3] == 0).all()
+
+
+def test_vocab_parallel_embedding_one_rank_of_four():
+    """Rank 1 of a 1D group of 4: the layer's own slice through the kernel, the peers' contribution staged
+    where the all-reduce would deliver it."""
+    import cubework_amd.module as cube_nn
+    from cubework_amd.distributed import ParallelManager as pm
+    from cubework_amd.distributed import initialize
+
+    initialize("1d", 4, rank=1)
+    torch.manual_seed(0)
+    emb = cube_nn.VocabParallelEmbedding1D(400, 32).to(torch.bfloat16).to(DEV)
+    assert emb.weight.shape == (100, 32) and emb.vocab_start_index == 100
+    ids = _ids((4, 9), 400, 2).to(DEV)
+    peers = randn((4, 9, 32), torch.bfloat16, 7).to(DEV)
+    pm.PARALLEL_1D.stage("all_reduce", [peers])
+    out = emb(ids)
+    local = torch.nn.functional.embedding((ids - 100).clamp(0, 99), emb.weight.detach())
+    local[(ids < 100) | (ids >= 200)] = 0
+    assert torch.equal(out, local + peers)
