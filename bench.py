@@ -257,6 +257,15 @@ def bench_other_configs(device, sets):
         y = blk(xb)
         y.backward(dyb)
     us = event_time_us(block_step, 10, 3)
+    # gradient-norm clipping over the block's 12 parameter gradients (one read for the norm, read + write
+    # for the scaling)
+    from cubework_amd.clip_grad import clip_grad_norm
+    params = [p for p in blk.parameters() if p.grad is not None]
+    grad_bytes = sum(p.grad.numel() * p.grad.element_size() for p in params)
+    us_clip = event_time_us(lambda: clip_grad_norm(params, 1.0), 20, 3)
+    out["clip_grad_norm_block"] = {"us": round(us_clip, 2), "bytes": 3 * grad_bytes, "tensors": len(params),
+                                   "GBps": round(3 * grad_bytes / us_clip / 1e3, 1),
+                                   "frac": round(3 * grad_bytes / us_clip / 1e3 / HBM_PEAK_GBPS, 3)}
     lin_flop = 3 * 2.0 * 8192 * 2048 * (6144 + 2048 + 8192 + 8192)
     out["opt_block_fwd_bwd"] = {"ms": round(us / 1e3, 3), "linear_flop": lin_flop,
                                 "linear_TFLOPs_if_all_time_were_linears": round(lin_flop / us / 1e6, 1),

@@ -283,6 +283,29 @@ int cw_embed_bwd(int64_t T, int64_t E, const int64_t* sorted_ids, const int64_t*
                  int64_t vocab_start, int64_t V_loc, int64_t skip_row,
                  const void* d_out, int64_t ldo, void* d_weight, int64_t ldw, int io_dtype, void* stream);
 
+/* ---- gradient-norm clipping ---------------------------------------------- */
+/*
+ * out2[0] = sum over tensors with groups[i] == 0 of |g|^p, out2[1] = sum over tensors with
+ * groups[i] == 1 of factors[i] * |g|^p (p = norm_type; for norm_type = +inf both are maxima of |g|
+ * and factors are not used). Replaces the per-tensor torch.norm(...) ** norm_type, the
+ * num_partitions weighting and the two torch.stack / torch.sum of clip_grad_norm
+ * (cubework/utils/clip_grad.py:31-46); group 1 = parameters tagged with NUM_PARTITIONS, whose sum
+ * the caller all-reduces and divides by the tensor-parallel size (:48-49) before taking the root.
+ * grads / numels / factors / groups are HOST arrays; all tensors share io_dtype and are contiguous.
+ * Two deterministic stages through `workspace` (cw_multi_norm_workspace_bytes), no atomics.
+ */
+int64_t cw_multi_norm_workspace_bytes(int n_tensors, const int64_t* numels);
+int cw_multi_norm_partials(int n_tensors, const void* const* grads, const int64_t* numels,
+                           const float* factors, const unsigned char* groups, float norm_type,
+                           float* out2, void* workspace, int64_t workspace_bytes,
+                           int io_dtype, void* stream);
+/*
+ * g *= coef[0] for every tensor, coef in device memory (clip_grad.py:64-68: the clamped
+ * coefficient is applied without a host round trip).
+ */
+int cw_multi_scale(int n_tensors, void* const* grads, const int64_t* numels, const float* coef,
+                   int io_dtype, void* stream);
+
 /* ---- attention core ------------------------------------------------------ */
 /*
  * out[b, s, h, :] = softmax_j(scale * q[b,s,h,:] . k[b,j,h,:] + causal mask) . v[b,j,h,:]

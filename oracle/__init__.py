@@ -31,4 +31,5 @@ from .layernorm import (ln2d_partial_stats, ln2d_mean_rstd, ln2d_normalize, ln2d
 from .vpce import vpce_fwd_local, vpce_finalize, vpce_bwd, vpce_reference_full  # noqa: F401
 from .attention import split_qkv, attention_core, attention_core_backward, attention_brute_force  # noqa: F401
 from .embedding import vocab_embedding_fwd, vocab_embedding_bwd  # noqa: F401
+from .clip_grad import clip_grad_norm  # noqa: F401
 from . import grid  # noqa: F401

@@ -1,0 +1,79 @@
+"""GPU parity of clip_grad_norm (cw_multi_norm_partials / cw_multi_scale through the C ABI) against
+torch.nn.utils.clip_grad_norm_, which the reference's function is adapted from and equals at
+tensor-parallel size 1 (cubework/utils/clip_grad.py:1-4)."""
+import pytest
+import torch
+
+from tests.util import assert_parity, randn
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+
+
+def _params(shapes, dtype, seed, tp_every=2):
+    from cubework_amd.global_vars import NUM_PARTITIONS
+    ps = []
+    for i, shp in enumerate(shapes):
+        p = torch.nn.Parameter(torch.zeros(shp, dtype=dtype, device=DEV))
+        p.grad = randn(shp, dtype, seed + i, std=0.5 + 0.1 * i).to(DEV)
+        if i % tp_every == 0:
+            setattr(p, NUM_PARTITIONS, 1)
+        ps.append(p)
+    return ps
+
+
+SHAPES = [(1000, 33), (7,), (70000,), (256, 256), (1,), (65536,), (65537,), (3, 5, 11)] + [(129, 17)] * 60
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("norm_type", [2.0, float("inf"), 1.0, 3.0])
+@pytest.mark.parametrize("max_norm", [0.5, 1e9])
+def test_clip_grad_norm_matches_torch(dtype, norm_type, max_norm):
+    from cubework_amd.clip_grad import clip_grad_norm
+    from cubework_amd.distributed import initialize
+
+    initialize("2d", 1)
+    ours = _params(SHAPES, dtype, 1)
+    ref = [torch.nn.Parameter(torch.zeros_like(p, dtype=torch.float32, device="cpu")) for p in ours]
+    for r, p in zip(ref, ours):
+        r.grad = p.grad.detach().float().cpu()
+    want = torch.nn.utils.clip_grad_norm_(ref, max_norm, norm_type)
+    got = clip_grad_norm(ours, max_norm, norm_type)
+    torch.cuda.synchronize()
+    assert abs(got.item() - want.item()) <= 1e-4 * abs(want.item()), (got.item(), want.item())
+    for r, p in zip(ref, ours):
+        assert_parity(p.grad, r.grad, dtype, "clipped gradient")
+
+
+def test_tensor_parallel_weighting_and_mixed_dtypes():
+    """Parameters tagged with NUM_PARTITIONS = n enter the norm n times (clip_grad.py:41-43); gradients of
+    two dtypes are clipped with one common coefficient; parameters without a gradient are skipped."""
+    from cubework_amd.clip_grad import clip_grad_norm
+    from cubework_amd.distributed import initialize
+    from cubework_amd.global_vars import NUM_PARTITIONS
+
+    initialize(None, 1)
+    a = torch.nn.Parameter(torch.zeros(300, device=DEV))
+    b = torch.nn.Parameter(torch.zeros((40, 8), dtype=torch.bfloat16, device=DEV))
+    c = torch.nn.Parameter(torch.zeros(5, device=DEV))
+    a.grad = randn((300,), torch.float32, 1).to(DEV)
+    b.grad = randn((40, 8), torch.bfloat16, 2).to(DEV)
+    setattr(b, NUM_PARTITIONS, 4)
+    ga, gb = a.grad.clone(), b.grad.clone()
+    import oracle
+    want, clipped = oracle.clip_grad_norm([ga, gb], [0, 4], 1.0)
+    got = clip_grad_norm([a, b, c], 1.0)
+    assert abs(got.item() - want.item()) <= 1e-5 * want.item()
+    assert_parity(a.grad, clipped[0].float(), torch.float32, "fp32 gradient", scale=10)
+    assert_parity(b.grad, clipped[1].float(), torch.bfloat16, "bf16 gradient")
+    assert c.grad is None
+
+
+def test_clip_grad_norm_empty_and_reproducible():
+    from cubework_amd.clip_grad import clip_grad_norm
+
+    assert clip_grad_norm([], 1.0).item() == 0.0
+    ps = _params([(50000,), (123, 45)], torch.bfloat16, 9)
+    n1 = clip_grad_norm(ps, 1e9)
+    n2 = clip_grad_norm(ps, 1e9)
+    assert n1.item() == n2.item()

@@ -39,3 +39,23 @@ def test_edge_ids_and_padding_row():
     live = ((ids >= 10) & (ids < 14)).float().unsqueeze(-1)
     (ref,) = torch.autograd.grad(F.embedding(shifted, ref_w, padding_idx=1) * live, ref_w, d_out)
     assert torch.equal(oracle.vocab_embedding_bwd(ids, d_out, 4, 10, padding_idx=1), ref)
+
+
+def test_clip_grad_oracle_against_torch_and_by_hand():
+    """oracle.clip_grad_norm equals torch.nn.utils.clip_grad_norm_ for untagged parameters (the function the
+    reference adapts, cubework/utils/clip_grad.py:1-4), and a parameter tagged with n partitions counts n times."""
+    shapes = [(13, 5), (7,), (1,), (4, 4, 4)]
+    for norm_type in (2.0, 1.0, 3.0, float("inf")):
+        for max_norm in (0.3, 1e6):
+            ps = [torch.nn.Parameter(torch.zeros(s)) for s in shapes]
+            for i, p in enumerate(ps):
+                p.grad = randn(s if False else shapes[i], torch.float32, 20 + i)
+            grads = [p.grad.clone() for p in ps]
+            want = torch.nn.utils.clip_grad_norm_(ps, max_norm, norm_type)
+            total, clipped = oracle.clip_grad_norm(grads, [0] * len(ps), max_norm, norm_type)
+            assert torch.allclose(total.float(), want, rtol=1e-5)
+            for c, p in zip(clipped, ps):
+                assert torch.allclose(c.float(), p.grad, rtol=1e-5, atol=1e-7)
+    g = [torch.tensor([3.0]), torch.tensor([2.0, 2.0])]
+    total, clipped = oracle.clip_grad_norm(g, [0, 2], 1.0)  # sqrt(9 + 2 * 8) = 5
+    assert abs(total.item() - 5.0) < 1e-12 and torch.allclose(clipped[0], torch.tensor([3.0 / (5 + 1e-6)], dtype=torch.float64))
