@@ -315,7 +315,7 @@ def cpu_baseline():
         rows = M
     else:
         rows = max(256, min(M, int(15.0 / (3 * per_row)) // 256 * 256))
-    iters = max(2, min(10, int(12.0 / max(per_row * rows, 1e-6))))
+    iters = max(2, min(300, int(10.0 / max(per_row * rows, 1e-6))))  # about 10 s of CPU work
     t = run(rows, iters)
     if inited:
         dist.destroy_process_group()
