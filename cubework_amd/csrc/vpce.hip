@@ -11,7 +11,8 @@ namespace cw {
 namespace {
 
 constexpr int kCeBlock = 256;
-constexpr int kCeUnroll = 3;
+constexpr int kCeUnroll = 3;     // 16-byte loads in flight per thread, forward
+constexpr int kCeBwdUnroll = 6;  // backward (no dependent chain between the vectors)
 constexpr float kNegInf = -__builtin_huge_valf();
 
 // Running (max m, sum s of exp(x - m)) kept in the exp2 domain: m2 = m*log2(e).
@@ -225,12 +226,12 @@ __global__ __launch_bounds__(kCeBlock) void vpce_bwd_kernel(int64_t T_rows, int6
         if (vec_ok) {
             const int64_t nvec = V_cols / V;
             int64_t i = tid;
-            for (; i + (kCeUnroll - 1) * kCeBlock < nvec; i += kCeUnroll * kCeBlock) {
-                raw16_t raw[kCeUnroll];
+            for (; i + (kCeBwdUnroll - 1) * kCeBlock < nvec; i += kCeBwdUnroll * kCeBlock) {
+                raw16_t raw[kCeBwdUnroll];
 #pragma unroll
-                for (int u = 0; u < kCeUnroll; ++u) raw[u] = load_raw_stream(xr + (i + u * kCeBlock) * V);
+                for (int u = 0; u < kCeBwdUnroll; ++u) raw[u] = load_raw_stream(xr + (i + u * kCeBlock) * V);
 #pragma unroll
-                for (int u = 0; u < kCeUnroll; ++u)
+                for (int u = 0; u < kCeBwdUnroll; ++u)
                     grad_vector<T, G, V>(raw[u], i + u * kCeBlock, tcol, m2, scale, dl, gr);
             }
             for (; i < nvec; i += kCeBlock)
@@ -251,7 +252,7 @@ __global__ __launch_bounds__(kCeBlock) void vpce_bwd_kernel(int64_t T_rows, int6
 }
 
 int ce_grid(int64_t T_rows) {
-    const int64_t cap = 256 * 16;
+    const int64_t cap = (int64_t)1 << 20;  // one block per row: finished blocks are replaced one by one
     return (int)(T_rows < cap ? T_rows : cap);
 }
 
