@@ -10,7 +10,7 @@ from tests.util import assert_parity, rand_uniform, randn
 pytestmark = pytest.mark.gpu
 
 DEV = "cuda:0"
-SHAPES = [(64, 1024), (33, 520), (16, 100), (5, 7), (300, 2048), (9, 4096), (3, 8200)]
+SHAPES = [(64, 1024), (33, 520), (16, 100), (5, 7), (300, 2048), (9, 4096), (3, 8200), (7, 512), (1, 256), (2050, 264)]
 
 
 def _inputs(R, C, dtype, seed):
