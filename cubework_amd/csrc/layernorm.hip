@@ -457,24 +457,13 @@ __global__ __launch_bounds__(NWAVES * 64) void ln_bwd_partials_kernel(
     }
     if (!want_cols) return;
 
-    block_tree_reduce<2 * NCH * V, NWAVES>(acc, lds_red, wave, lane);
-    if (wave == 0) {
-        float* out = col_ws + (int64_t)blockIdx.x * 2 * C;
-#pragma unroll
-        for (int j = 0; j < NCH; ++j) {
-            const int64_t c0 = ((int64_t)j * 64 + lane) * V;
-            if (c0 < C) {
-#pragma unroll
-                for (int e = 0; e < V; e += 4) {
-                    *reinterpret_cast<float4*>(out + c0 + e) =
-                        make_float4(acc[j * V + e], acc[j * V + e + 1], acc[j * V + e + 2], acc[j * V + e + 3]);
-                    *reinterpret_cast<float4*>(out + C + c0 + e) =
-                        make_float4(acc[NCH * V + j * V + e], acc[NCH * V + j * V + e + 1],
-                                    acc[NCH * V + j * V + e + 2], acc[NCH * V + j * V + e + 3]);
-                }
-            }
-        }
-    }
+    // accumulator i: set i / (NCH*V) (0 = dgamma, 1 = dbeta), chunk j = (i % (NCH*V)) / V, element e = i % V
+    float* out = col_ws + (int64_t)blockIdx.x * 2 * C;
+    block_flat_reduce<2 * NCH * V, NWAVES>(acc, lds_red, wave, lane, [&](int i, int l, float total) {
+        const int set = i / (NCH * V), rem = i - set * (NCH * V);
+        const int64_t c = ((int64_t)(rem / V) * 64 + l) * V + (rem % V);
+        if (c < C) out[(int64_t)set * C + c] = total;
+    });
 }
 
 // Backward partials for shapes the vector kernel does not take (ragged C,
@@ -642,7 +631,7 @@ int bwd_partials_launch(int64_t R, int64_t C, const void* dY, int64_t ld_dy, con
                         hipStream_t s) {
     constexpr int V = elem<T>::kVec;
     const int64_t nb = bwd_blocks(R, NWAVES * NR);
-    const size_t lds = tree_reduce_lds_bytes(2 * NCH * V, NWAVES);
+    const size_t lds = flat_reduce_lds_bytes(2 * NCH * V, NWAVES);
     auto kern = ln_bwd_partials_kernel<T, NCH, NWAVES, NR>;
     if (lds > 48 * 1024) {
         hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);

@@ -32,6 +32,26 @@ __device__ __forceinline__ void block_tree_reduce(float (&acc)[NREG], float* lds
     }
 }
 
+// Flat variant for wide accumulator sets: every wavefront writes its NREG x 64 accumulators to LDS once
+// ([wave][reg][lane], NWAVES * NREG * 256 bytes), one barrier, then thread t adds the NWAVES values of
+// accumulator slots t, t + NWAVES*64, ... in wavefront order and hands each total to sink(reg, lane, total).
+inline size_t flat_reduce_lds_bytes(int nreg, int nwaves) { return (size_t)nwaves * nreg * 64 * sizeof(float); }
+
+template <int NREG, int NWAVES, typename Sink>
+__device__ __forceinline__ void block_flat_reduce(const float (&acc)[NREG], float* lds, int wave, int lane, Sink&& sink) {
+    float* mine = lds + (size_t)wave * NREG * 64;
+#pragma unroll
+    for (int i = 0; i < NREG; ++i) mine[i * 64 + lane] = acc[i];
+    __syncthreads();
+    const int tid = wave * 64 + lane;
+    for (int o = tid; o < NREG * 64; o += NWAVES * 64) {
+        float total = lds[o];
+#pragma unroll
+        for (int w = 1; w < NWAVES; ++w) total += lds[(size_t)w * NREG * 64 + o];
+        sink(o >> 6, o & 63, total);
+    }
+}
+
 // out_k[c] = sum_p ws[p*part_stride + k*C + c], k < nsets (nsets is 1 or 2;
 // out1 is ignored when nsets == 1). Enqueued on `s`.
 int finalize_col_partials(const float* ws, int64_t nparts, int64_t part_stride, int nsets, int64_t C, float* out0,
