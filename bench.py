@@ -290,7 +290,16 @@ def cpu_baseline():
             s.bind(("127.0.0.1", 0))
             port = s.getsockname()[1]
             s.close()
-            dist.init_process_group("gloo", init_method="tcp://127.0.0.1:%d" % port, rank=0, world_size=1)
+            # gloo announces its connections on stdout; keep stdout for the one JSON line
+            sys.stdout.flush()
+            saved = os.dup(1)
+            os.dup2(2, 1)
+            try:
+                dist.init_process_group("gloo", init_method="tcp://127.0.0.1:%d" % port, rank=0, world_size=1)
+            finally:
+                sys.stdout.flush()
+                os.dup2(saved, 1)
+                os.close(saved)
             inited = True
     except Exception:  # the baseline still runs without the (unused at world size 1) group
         inited = False
