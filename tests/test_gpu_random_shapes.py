@@ -1,0 +1,104 @@
+"""Seeded random shapes through the C ABI against the CPU oracle: the block GEMM across its three code
+paths (register-staged, LDS-DMA, split-k), the attention core, LayerNorm and the cross-entropy slice.
+Shapes are drawn once from fixed seeds, so the cases are the same in every run."""
+import random
+
+import pytest
+import torch
+
+from tests.util import assert_parity, randn
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+
+
+def _gemm_cases():
+    rng = random.Random(1234)
+    cases = []
+    for _ in range(10):  # ragged: register-staged kernel with guards
+        cases.append((rng.choice(["NN", "NT", "TN"]), rng.randint(1, 700), rng.randint(1, 700), rng.randint(1, 300),
+                      rng.randint(1, 3)))
+    for _ in range(6):   # tile-aligned with many tiles: LDS-DMA kernel
+        cases.append((rng.choice(["NN", "NT", "TN"]), 256 * rng.randint(8, 12), 256 * rng.randint(8, 16),
+                      64 * rng.randint(1, 5), rng.randint(1, 4)))
+    for _ in range(6):   # few tiles, long reduction: split-k
+        cases.append((rng.choice(["NN", "NT", "TN"]), 256 * rng.randint(1, 3), 256 * rng.randint(1, 4),
+                      512 * rng.randint(2, 5), rng.randint(1, 4)))
+    return cases
+
+
+@pytest.mark.parametrize("case", _gemm_cases())
+def test_random_gemm(case):
+    import oracle
+    from cubework_amd import ops
+
+    layout, M, N, K, steps = case
+    a_shape = (K, M) if layout == "TN" else (M, K)
+    b_shape = (N, K) if layout == "NT" else (K, N)
+    A = [randn(a_shape, torch.bfloat16, 7 * s + M) for s in range(steps)]
+    B = [randn(b_shape, torch.bfloat16, 7 * s + N + 1, std=0.05) for s in range(steps)]
+    bias = randn((N,), torch.bfloat16, K, std=0.3)
+    act = ["relu", "gelu_tanh", None][(M + N + K) % 3]
+    want = oracle.gemm_ksteps(layout, A, B, bias, act)
+    got = ops.gemm_ksteps(layout, [a.to(DEV) for a in A], [b.to(DEV) for b in B], bias.to(DEV), act)
+    torch.cuda.synchronize()
+    assert_parity(got, want, torch.bfloat16, "gemm %s" % (case,))
+
+
+def _attn_cases():
+    rng = random.Random(99)
+    return [(rng.randint(1, 3), rng.randint(1, 900), rng.randint(1, 5), rng.random() < 0.7) for _ in range(12)]
+
+
+@pytest.mark.parametrize("case", _attn_cases())
+def test_random_attention(case):
+    import oracle
+    from cubework_amd import ops
+
+    b, s, h, causal = case
+    d = 64
+    qkv = randn((b, s, h * 3 * d), torch.bfloat16, s + 3 * h, std=1.3)
+    d_out = randn((b, s, h * d), torch.bfloat16, s + 5)
+    qc, kc, vc = oracle.split_qkv(qkv, h)
+    want = oracle.attention_core(qc, kc, vc, causal=causal)
+    dq, dk, dv = oracle.attention_core_backward(qc, kc, vc, d_out, causal=causal)
+    t = qkv.to(DEV).view(b, s, h, 3 * d)
+    q, k, v = t[..., :d], t[..., d:2 * d], t[..., 2 * d:]
+    out, lse = ops.attn_fwd(q, k, v, causal=causal, want_lse=True)
+    g = torch.empty_like(t)
+    ops.attn_bwd(q, k, v, out, d_out.to(DEV), lse, g[..., :d], g[..., d:2 * d], g[..., 2 * d:], causal=causal)
+    torch.cuda.synchronize()
+    assert_parity(out, want, torch.bfloat16, "attention out %s" % (case,))
+    if s == 1:
+        assert_parity(g.permute(0, 2, 1, 3), torch.cat([dq, dk, dv], dim=-1), torch.bfloat16, "attention grads %s" % (case,))
+        return
+    for name, got, ref in (("dq", g[..., :d], dq), ("dk", g[..., d:2 * d], dk), ("dv", g[..., 2 * d:], dv)):
+        assert_parity(got.permute(0, 2, 1, 3), ref, torch.bfloat16, "attention %s %s" % (name, case), scale=2)
+
+
+def _ln_cases():
+    rng = random.Random(5)
+    return [(rng.randint(1, 600), 8 * rng.randint(1, 520)) for _ in range(8)] + [(rng.randint(1, 50), rng.randint(1, 3000)) for _ in range(4)]
+
+
+@pytest.mark.parametrize("shape", _ln_cases())
+def test_random_layernorm(shape):
+    import oracle
+    from cubework_amd import ops
+
+    R, C = shape
+    x = randn((R, C), torch.bfloat16, R + C)
+    dy = randn((R, C), torch.bfloat16, R + C + 1)
+    gamma = (1 + 0.1 * randn((C,), torch.float32, 3)).to(torch.bfloat16)
+    beta = randn((C,), torch.bfloat16, 4, std=0.05)
+    y_ref, mr_ref = oracle.ln_forward_full(x, gamma, beta, 1e-5)
+    dx_ref, dg_ref, db_ref = oracle.ln_backward_full(dy, x, mr_ref, gamma)
+    xd, dyd, gd, bd = (t.to(DEV) for t in (x, dy, gamma, beta))
+    y, mr = ops.ln_forward_fused(xd, 1e-5, gd, bd)
+    rs, dgam, dbet = ops.ln_bwd_partials(dyd, xd, mr, gd)
+    dx = ops.ln_bwd_dx(dyd, xd, mr, rs, C, gd)
+    torch.cuda.synchronize()
+    assert_parity(y, y_ref, torch.bfloat16, "ln y %s" % (shape,))
+    assert_parity(dx, dx_ref, torch.bfloat16, "ln dx %s" % (shape,), scale=2)
+    assert_parity(dgam, dg_ref, torch.float32, "ln dgamma %s" % (shape,), scale=100)
+    assert_parity(dbet, db_ref, torch.float32, "ln dbeta %s" % (shape,), scale=100)
