@@ -37,8 +37,11 @@ SIGNATURES = {
                                  _pp, _int, _i64, _ptr, _i64, _int, _ptr]),
     "cw_multi_norm_workspace_bytes": (_i64, [_int, _ptr]),
     "cw_multi_norm_partials": (_int, [_int, _pp, _ptr, _ptr, _ptr, _f32, _ptr, _ptr, _i64, _int, _ptr]),
+    "cw_clip_coef": (_int, [_int, _ptr, _f32, _f32, _f32, _ptr, _ptr]),
     "cw_multi_scale": (_int, [_int, _pp, _ptr, _ptr, _int, _ptr]),
     "cw_embed_fwd": (_int, [_i64, _i64, _ptr, _i64, _i64, _ptr, _i64, _ptr, _i64, _int, _ptr]),
+    "cw_embed_sort_workspace_bytes": (_i64, [_i64]),
+    "cw_embed_sort_ids": (_int, [_i64, _ptr, _i64, _i64, _ptr, _ptr, _ptr, _i64, _ptr]),
     "cw_embed_bwd": (_int, [_i64, _i64, _ptr, _ptr, _i64, _i64, _i64, _ptr, _i64, _ptr, _i64, _int, _ptr]),
     "cw_attn_fwd": (_int, [_i64, _i64, _i64, _i64, _ptr, _ptr, _ptr, _i64, _i64, _i64, _f32, _int, _ptr, _i64, _i64, _i64,
                            _ptr, _int, _ptr]),

@@ -32,22 +32,19 @@ def _tables(grads):
     return ptrs, numels
 
 
-def _norm_partials(grads, factors, groups, norm_type):
-    """(standard, tensor-parallel) partial results of the gradients of one dtype, as a [2] fp32 tensor."""
+def _norm_partials(grads, factors, groups, norm_type, out):
+    """(standard, tensor-parallel) partial results of the gradients of one dtype into the [2] fp32 view `out`."""
     lib = _lib.load()
     ptrs, numels = _tables(grads)
     n = len(grads)
     fac = (ctypes.c_float * max(n, 1))(*factors)
     grp = (ctypes.c_ubyte * max(n, 1))(*groups)
-    dev = grads[0].device
-    out = torch.empty(2, dtype=torch.float32, device=dev)
     ws_bytes = lib.cw_multi_norm_workspace_bytes(n, ctypes.cast(numels, ctypes.c_void_p))
-    ws = torch.empty(ws_bytes, dtype=torch.uint8, device=dev)
+    ws = torch.empty(ws_bytes, dtype=torch.uint8, device=out.device)
     rc = lib.cw_multi_norm_partials(n, ptrs, ctypes.cast(numels, ctypes.c_void_p), ctypes.cast(fac, ctypes.c_void_p),
                                     ctypes.cast(grp, ctypes.c_void_p), norm_type, out.data_ptr(), ws.data_ptr(),
                                     ws_bytes, ops._dtype_code(grads[0]), ops._stream())
     _lib.check(rc, "cw_multi_norm_partials")
-    return out
 
 
 def _scale(grads, coef):
@@ -77,28 +74,28 @@ def clip_grad_norm(parameters: Union[Tensor, Iterable[Tensor]], max_norm: float,
             raise RuntimeError("clip_grad_norm: gradients must be contiguous")
         parts = getattr(p, NUM_PARTITIONS, 0)
         by_dtype.setdefault(g.dtype, []).append((g, float(parts) if parts > 0 else 1.0, 1 if parts > 0 else 0))
-    std = tp = None
-    for items in by_dtype.values():
-        out = _norm_partials([g for g, _, _ in items], [f for _, f, _ in items], [k for _, _, k in items], norm_type)
+    sets = torch.empty((len(by_dtype), 2), dtype=torch.float32, device=device)
+    for i, items in enumerate(by_dtype.values()):
+        _norm_partials([g for g, _, _ in items], [f for _, f, _ in items], [k for _, _, k in items], norm_type, sets[i])
+    tp_scale = 1.0
+    if pm.TENSOR.is_initialized() and pm.TENSOR.world_size > 1:
+        # the peers' share: maximum of everything, or sum of the tensor-parallel column divided by the group size
         if norm_type == inf:
-            std = out[0] if std is None else torch.maximum(std, out[0])
-            tp = out[1] if tp is None else torch.maximum(tp, out[1])
+            sets = all_reduce(sets.amax().reshape(1), pm.TENSOR, op="max").expand(2).reshape(1, 2).contiguous()
         else:
-            std = out[0] if std is None else std + out[0]
-            tp = out[1] if tp is None else tp + out[1]
-    if norm_type == inf:
-        total_norm = torch.maximum(std, tp)
-        if pm.TENSOR.is_initialized() and pm.TENSOR.world_size > 1:
-            total_norm = all_reduce(total_norm, pm.TENSOR, op="max")
-    else:
-        if pm.TENSOR.is_initialized() and pm.TENSOR.world_size > 1:
-            tp = all_reduce(tp, pm.TENSOR) / pm.TENSOR.world_size
-        total_norm = (std + tp) ** (1.0 / norm_type)
+            sets = sets.sum(0, keepdim=True)
+            sets[0, 1] = all_reduce(sets[0, 1].clone(), pm.TENSOR)
+            tp_scale = 1.0 / pm.TENSOR.world_size
+    norm_coef = torch.empty(2, dtype=torch.float32, device=device)
+    lib = _lib.load()
+    rc = lib.cw_clip_coef(sets.shape[0], sets.data_ptr(), tp_scale, norm_type, max_norm, norm_coef.data_ptr(), ops._stream())
+    _lib.check(rc, "cw_clip_coef")
+    total_norm = norm_coef[0]
     if error_if_nonfinite and torch.logical_or(total_norm.isnan(), total_norm.isinf()):
         raise RuntimeError(f"The total norm of order {norm_type} for gradients from `parameters` is non-finite, so it "
                            "cannot be clipped. To disable this error and scale the gradients by the non-finite norm "
                            "anyway, set `error_if_nonfinite=False`")
-    clip_coef_clamped = torch.clamp(max_norm / (total_norm + 1e-6), max=1.0).to(torch.float32).reshape(1).contiguous()
+    clip_coef_clamped = norm_coef[1:]
     for items in by_dtype.values():
         _scale([g for g, _, _ in items], clip_coef_clamped)
-    return total_norm.to(device)
+    return total_norm

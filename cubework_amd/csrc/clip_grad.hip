@@ -131,6 +131,32 @@ __global__ __launch_bounds__(kClipThreads) void multi_scale_kernel(const TensorB
     }
 }
 
+// One thread: combines the (standard, tensor-parallel) results of n_sets calls of the norm stage into
+// the total norm and the clamped scaling coefficient.
+__global__ void clip_coef_kernel(const float* __restrict__ sets, int n_sets, float tp_scale, float norm_type,
+                                 float max_norm, float* __restrict__ out2) {
+    if (threadIdx.x != 0 || blockIdx.x != 0) return;
+    float norm;
+    if (__builtin_isinf(norm_type)) {
+        norm = 0.0f;
+        for (int i = 0; i < 2 * n_sets; ++i) {
+            const float v = sets[i];
+            norm = (v != v) ? v : fmaxf(norm, v);  // a NaN gradient makes the norm NaN, as torch.max does
+        }
+    } else {
+        float std_sum = 0.0f, tp_sum = 0.0f;
+        for (int i = 0; i < n_sets; ++i) {
+            std_sum += sets[2 * i];
+            tp_sum += sets[2 * i + 1];
+        }
+        const float total = std_sum + tp_sum * tp_scale;
+        norm = norm_type == 2.0f ? sqrtf(total) : (norm_type == 1.0f ? total : powf(total, 1.0f / norm_type));
+    }
+    const float coef = max_norm / (norm + 1e-6f);
+    out2[0] = norm;
+    out2[1] = coef > 1.0f ? 1.0f : coef;  // NaN stays NaN, as torch.clamp(max=1) leaves it
+}
+
 int64_t blocks_of(int64_t numel) { return (numel + kChunk - 1) / kChunk; }
 
 // Fills `b` with tensors [first, ...) until it is full; returns the index of the next tensor.
@@ -202,6 +228,16 @@ extern "C" int cw_multi_norm_partials(int n_tensors, const void* const* grads, c
     if (kind == 0) hipLaunchKernelGGL(norm_finalize_kernel<0>, dim3(1), dim3(256), 0, s, ws, offset, out2);
     else hipLaunchKernelGGL(norm_finalize_kernel<2>, dim3(1), dim3(256), 0, s, ws, offset, out2);
     return check_launch("norm_finalize_kernel");
+}
+
+extern "C" int cw_clip_coef(int n_sets, const float* sets, float tp_scale, float norm_type, float max_norm,
+                            float* out2, void* stream) {
+    if (n_sets < 1 || n_sets > 64) return fail(CW_ERR_INVALID, "cw_clip_coef: n_sets %d outside [1, 64]", n_sets);
+    if (sets == nullptr || out2 == nullptr) return fail(CW_ERR_INVALID, "cw_clip_coef: null argument");
+    if (!(norm_type > 0.0f)) return fail(CW_ERR_INVALID, "cw_clip_coef: norm_type must be positive (inf for the maximum norm)");
+    hipLaunchKernelGGL(clip_coef_kernel, dim3(1), dim3(64), 0, (hipStream_t)stream, sets, n_sets, tp_scale, norm_type,
+                       max_norm, out2);
+    return check_launch("clip_coef_kernel");
 }
 
 extern "C" int cw_multi_scale(int n_tensors, void* const* grads, const int64_t* numels, const float* coef,

@@ -463,6 +463,25 @@ def embedding_fwd(ids: torch.Tensor, weight: torch.Tensor, vocab_start: int = 0)
     return out.view(tuple(ids.shape) + (E,))
 
 
+def embedding_token_order(ids: torch.Tensor, num_rows: int, vocab_start: int = 0):
+    """(sorted_ids, order) of the flat int64 ids by the row of the slice they select, ties in token order;
+    ids outside the slice come last as vocab_start + num_rows. See cw_embed_sort_ids."""
+    lib = _lib.load()
+    _require_device(ids)
+    if ids.dtype != torch.int64:
+        raise TypeError("ids must be int64, got %s" % ids.dtype)
+    flat = ids.reshape(-1).contiguous()
+    T = flat.numel()
+    sorted_ids = torch.empty_like(flat)
+    order = torch.empty_like(flat)
+    ws_bytes = lib.cw_embed_sort_workspace_bytes(T)
+    ws = torch.empty(ws_bytes, dtype=torch.uint8, device=flat.device) if ws_bytes > 0 else None
+    rc = lib.cw_embed_sort_ids(T, _p(flat), int(vocab_start), int(num_rows), _p(sorted_ids), _p(order),
+                               _p(ws), ws_bytes, _stream())
+    _lib.check(rc, "cw_embed_sort_ids")
+    return sorted_ids, order
+
+
 def embedding_bwd(ids: torch.Tensor, d_out: torch.Tensor, num_rows: int, vocab_start: int = 0,
                   skip_row: int = -1) -> torch.Tensor:
     """Gradient of embedding_fwd with respect to the [num_rows, E] weight slice. See cw_embed_bwd."""
@@ -471,7 +490,7 @@ def embedding_bwd(ids: torch.Tensor, d_out: torch.Tensor, num_rows: int, vocab_s
     g = _rows(d_out.reshape(-1, d_out.shape[-1]))
     flat = ids.reshape(-1)
     T, E = g.shape
-    sorted_ids, order = torch.sort(flat, stable=True)
+    sorted_ids, order = embedding_token_order(flat, num_rows, vocab_start)
     dw = torch.empty((num_rows, E), dtype=g.dtype, device=g.device)
     rc = lib.cw_embed_bwd(T, E, _p(sorted_ids), _p(order), int(vocab_start), num_rows, int(skip_row), _p(g), _ld(g),
                           _p(dw), _ld(dw), _dtype_code(g), _stream())

@@ -283,6 +283,22 @@ int cw_embed_bwd(int64_t T, int64_t E, const int64_t* sorted_ids, const int64_t*
                  int64_t vocab_start, int64_t V_loc, int64_t skip_row,
                  const void* d_out, int64_t ldo, void* d_weight, int64_t ldw, int io_dtype, void* stream);
 
+/*
+ * The token order cw_embed_bwd takes, made on the device: sorted_ids[i] / order[i] = id and position of
+ * the i-th token in ascending order of the selected row, ties in token order (a stable sort by id for
+ * the ids in range). Ids outside [vocab_start, vocab_start + V_loc) are written as
+ * vocab_start + V_loc and come last, so cw_embed_bwd skips them. Replaces the sort inside the
+ * autograd of F.embedding (the reference's backward of parallel_1d/module.py:390,452 and its 2D / 3D
+ * counterparts sorts the indices through torch's embedding_dense_backward). Integer-exact.
+ * T <= 16384 needs no workspace (one launch places every token by counting the tokens ahead of it);
+ * above that a sorting network runs over `workspace` of cw_embed_sort_workspace_bytes(T) bytes.
+ * T <= 2^30, V_loc < 2^32 - 1.
+ */
+int64_t cw_embed_sort_workspace_bytes(int64_t T);
+int cw_embed_sort_ids(int64_t T, const int64_t* ids, int64_t vocab_start, int64_t V_loc,
+                      int64_t* sorted_ids, int64_t* order, void* workspace, int64_t workspace_bytes,
+                      void* stream);
+
 /* ---- gradient-norm clipping ---------------------------------------------- */
 /*
  * out2[0] = sum over tensors with groups[i] == 0 of |g|^p, out2[1] = sum over tensors with
@@ -299,6 +315,17 @@ int cw_multi_norm_partials(int n_tensors, const void* const* grads, const int64_
                            const float* factors, const unsigned char* groups, float norm_type,
                            float* out2, void* workspace, int64_t workspace_bytes,
                            int io_dtype, void* stream);
+/*
+ * Total norm and clamped coefficient from the results of n_sets cw_multi_norm_partials calls (one per
+ * dtype), `sets` = [n_sets][2] fp32 in device memory: out2[0] = (sum_i sets[i][0] + tp_scale *
+ * sum_i sets[i][1]) ^ (1 / norm_type) (for +inf: the maximum of all entries), out2[1] =
+ * min(max_norm / (out2[0] + 1e-6), 1). Replaces clip_grad.py:46-50,57-61 (tensor-parallel sum divided
+ * by the group size, the root, clip_coef and its clamp) with one launch; a caller with a
+ * tensor-parallel group larger than 1 all-reduces the second column first and passes
+ * tp_scale = 1 / size.
+ */
+int cw_clip_coef(int n_sets, const float* sets, float tp_scale, float norm_type, float max_norm,
+                 float* out2, void* stream);
 /*
  * g *= coef[0] for every tensor, coef in device memory (clip_grad.py:64-68: the clamped
  * coefficient is applied without a host round trip).

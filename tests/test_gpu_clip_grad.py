@@ -77,3 +77,35 @@ def test_clip_grad_norm_empty_and_reproducible():
     n1 = clip_grad_norm(ps, 1e9)
     n2 = clip_grad_norm(ps, 1e9)
     assert n1.item() == n2.item()
+
+
+@pytest.mark.parametrize("norm_type", [2.0, float("inf")])
+def test_clip_grad_norm_with_peer_sums(norm_type):
+    """A tensor-parallel group of 4 with the peers' results pre-staged: the tensor-parallel sum is
+    all-reduced and divided by the group size (clip_grad.py:48-49), the maximum norm is the maximum over
+    the group (:34-35)."""
+    from cubework_amd.clip_grad import clip_grad_norm
+    from cubework_amd.distributed import ParallelManager as pm
+    from cubework_amd.distributed import initialize
+    from cubework_amd.global_vars import NUM_PARTITIONS
+
+    initialize("1d", 4)
+    a = torch.nn.Parameter(torch.zeros(500, device=DEV))
+    b = torch.nn.Parameter(torch.zeros((64, 9), device=DEV))
+    a.grad = randn((500,), torch.float32, 5).to(DEV)
+    b.grad = randn((64, 9), torch.float32, 6).to(DEV)
+    setattr(b, NUM_PARTITIONS, 4)
+    ga, gb = a.grad.double().cpu(), b.grad.double().cpu()
+    if norm_type == 2.0:
+        peers = [torch.tensor(v, dtype=torch.float32, device=DEV) for v in (1000.0, 2000.0, 3000.0)]
+        want = ((ga ** 2).sum() + (4 * (gb ** 2).sum() + 6000.0) / 4) ** 0.5
+    else:
+        peers = [torch.tensor([v], dtype=torch.float32, device=DEV) for v in (0.5, 7.25, 1.0)]
+        want = torch.tensor(7.25, dtype=torch.float64)
+    pm.TENSOR.stage("all_reduce", peers)
+    got = clip_grad_norm([a, b], 2.0, norm_type)
+    assert abs(got.item() - want.item()) <= 1e-5 * want.item(), (got.item(), want.item())
+    coef = min(2.0 / (want.item() + 1e-6), 1.0)
+    assert_parity(a.grad, (ga * coef).float(), torch.float32, "gradient a", scale=10)
+    assert_parity(b.grad, (gb * coef).float(), torch.float32, "gradient b", scale=10)
+    initialize(None, 1)

@@ -107,3 +107,35 @@ def test_vocab_parallel_embedding_one_rank_of_four():
     local = torch.nn.functional.embedding((ids - 100).clamp(0, 99), emb.weight.detach())
     local[(ids < 100) | (ids >= 200)] = 0
     assert torch.equal(out, local + peers)
+
+
+@pytest.mark.parametrize("T", [1, 2, 3, 100, 1023, 8192, 16384, 16385, 50000, 140000])
+def test_token_order_is_the_stable_sort(T):
+    """cw_embed_sort_ids against Python's sorted() on (row, position) pairs: bit-exact, including ids
+    below, inside and above the slice, negative ids and the extremes of int64. Sizes cover one workgroup
+    in LDS (<= 16384) and the multi-launch network with 4 and 16 chunks."""
+    from cubework_amd import ops
+
+    start, rows = 1000, 777
+    g = torch.Generator().manual_seed(T)
+    ids = torch.randint(start - 300, start + rows + 300, (T,), generator=g, dtype=torch.int64)
+    edges = torch.tensor([start - 1, start, start + rows - 1, start + rows, 0, -5, 2 ** 63 - 1, -2 ** 63], dtype=torch.int64)
+    n = min(T, edges.numel())
+    ids[:n] = edges[:n]
+    keyed = sorted((((v - start) if start <= v < start + rows else rows), i) for i, v in enumerate(ids.tolist()))
+    want_ids = torch.tensor([start + r for r, _ in keyed], dtype=torch.int64)
+    want_order = torch.tensor([i for _, i in keyed], dtype=torch.int64)
+    got_ids, got_order = ops.embedding_token_order(ids.to(DEV), rows, start)
+    torch.cuda.synchronize()
+    assert torch.equal(got_ids.cpu(), want_ids)
+    assert torch.equal(got_order.cpu(), want_order)
+
+
+def test_token_order_repeated_id():
+    """Every token selects the same row: the order is the identity."""
+    from cubework_amd import ops
+
+    ids = torch.full((5000,), 42, dtype=torch.int64, device=DEV)
+    got_ids, got_order = ops.embedding_token_order(ids, 100, 0)
+    assert torch.equal(got_ids, ids)
+    assert torch.equal(got_order.cpu(), torch.arange(5000))
