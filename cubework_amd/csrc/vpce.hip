@@ -4,6 +4,8 @@
 // the bit-exact target mask / shifted index / gather. backward: recomputes the
 // softmax from the logits and the global (max, sum) and writes the gradient;
 // the logits are never modified.
+#include <type_traits>
+
 #include "cw_common.h"
 
 namespace cw {
@@ -204,6 +206,25 @@ __device__ __forceinline__ void grad_vector(raw16_t raw, int64_t i, int64_t tcol
     store_grad<V>(gr + i * V, v);
 }
 
+// fp32 gradient of bf16 logits: four logits (8 bytes) in, four floats (16 bytes) out per lane, so that the
+// stores of one instruction cover one contiguous 1 KB span. With 16-byte loads a lane would write 32
+// bytes in two stores that each leave every other 16 bytes to the next instruction.
+typedef uint32_t raw8_t __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ void grad_quad(raw8_t raw, int64_t i, int64_t tcol, float m2, float scale, float dl,
+                                          float* __restrict__ gr) {
+    float v[4] = {__uint_as_float(raw.x << 16), __uint_as_float(raw.x & 0xffff0000u), __uint_as_float(raw.y << 16),
+                  __uint_as_float(raw.y & 0xffff0000u)};
+#pragma unroll
+    for (int e = 0; e < 4; ++e) v[e] = __builtin_amdgcn_exp2f(__builtin_fmaf(v[e], kLog2e, -m2)) * scale;
+    const int64_t rel = tcol - i * 4;
+    if (rel >= 0 && rel < 4) {
+#pragma unroll
+        for (int e = 0; e < 4; ++e)
+            if (e == rel) v[e] -= dl;
+    }
+    store_raw_stream(gr + i * 4, pack_raw(v, (const float*)nullptr));
+}
+
 template <typename T, typename G>
 __global__ __launch_bounds__(kCeBlock) void vpce_bwd_kernel(int64_t T_rows, int64_t V_cols,
                                                             const T* __restrict__ logits, int64_t ld,
@@ -223,7 +244,28 @@ __global__ __launch_bounds__(kCeBlock) void vpce_bwd_kernel(int64_t T_rows, int6
         const int64_t t = targets[row];
         const bool masked = (t < vocab_start) || (t >= vocab_start + V_cols);
         const int64_t tcol = masked ? -1 : (t - vocab_start);
-        if (vec_ok) {
+        if (vec_ok && std::is_same<T, bf16_t>::value && std::is_same<G, float>::value) {
+            constexpr int U = 2 * kCeBwdUnroll;
+            const int64_t nq = V_cols / 4;
+            const bf16_t* xb = reinterpret_cast<const bf16_t*>(xr);
+            float* gf = reinterpret_cast<float*>(gr);
+            int64_t i = tid;
+            for (; i + (U - 1) * kCeBlock < nq; i += U * kCeBlock) {
+                raw8_t raw[U];
+#pragma unroll
+                for (int u = 0; u < U; ++u)
+                    raw[u] = __builtin_nontemporal_load(reinterpret_cast<const raw8_t*>(xb + (i + u * kCeBlock) * 4));
+#pragma unroll
+                for (int u = 0; u < U; ++u) grad_quad(raw[u], i + u * kCeBlock, tcol, m2, scale, dl, gf);
+            }
+            for (; i < nq; i += kCeBlock)
+                grad_quad(__builtin_nontemporal_load(reinterpret_cast<const raw8_t*>(xb + i * 4)), i, tcol, m2, scale, dl, gf);
+            for (int64_t c = nq * 4 + tid; c < V_cols; c += kCeBlock) {
+                float y = __builtin_amdgcn_exp2f(__builtin_fmaf(load_elem(xr + c), kLog2e, -m2)) * scale;
+                if (c == tcol) y -= dl;
+                store_elem(gr + c, y);
+            }
+        } else if (vec_ok) {
             const int64_t nvec = V_cols / V;
             int64_t i = tid;
             for (; i + (kCeBwdUnroll - 1) * kCeBlock < nvec; i += kCeBwdUnroll * kCeBlock) {
