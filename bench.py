@@ -115,6 +115,7 @@ def bench_bandwidth_kernels(device):
     stats = ops.ln_partial_stats(xs[0]) + ops.ln_partial_stats(peer)
     _, mr = ops.ln_normalize(xs[0], stats, H, 1e-5, gamma, beta)
     rs = ops.ln_bwd_partials(dys[0], xs[0], mr, gamma)[0] * 2
+    mr_whole = ops.ln_forward_fused(xs[0], 1e-5, gamma, beta)[1]  # the same rows taken as whole (H = 1024)
     i = [0]
 
     def rot(lst):
@@ -126,6 +127,9 @@ def bench_bandwidth_kernels(device):
         ("ln_normalize", 2 * 33554432 + 2 * 131072 + 4096, lambda: ops.ln_normalize(rot(xs), stats, H, 1e-5, gamma, beta)),
         ("ln_bwd_partials", 2 * 33554432 + 2 * 131072 + 8192, lambda: ops.ln_bwd_partials(rot(dys), xs[i[0] % nb], mr, gamma)),
         ("ln_bwd_dx", 3 * 33554432 + 2 * 131072 + 2048, lambda: ops.ln_bwd_dx(rot(dys), xs[i[0] % nb], mr, rs, H, gamma)),
+        # rows complete on the rank (tensor-parallel size 1): partials + dx in one pass, dy and x read once
+        ("ln_backward_fused", 3 * 33554432 + 2 * 131072 + 8192,
+         lambda: ops.ln_backward_fused(rot(dys), xs[i[0] % nb], mr_whole, gamma)),
     ]
     for name, nbytes, fn in cases:
         us = graph_time_us(fn, 2 * nb)

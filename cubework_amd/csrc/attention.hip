@@ -156,7 +156,7 @@ __global__ __launch_bounds__(kThreads, 2) void attn_fwd_kernel(const AttnArgs a)
                     float mx = st[qt][0];
 #pragma unroll
                     for (int e = 1; e < 16; ++e) mx = fmaxf(mx, st[qt][e]);
-                    mx = fmaxf(mx, xchg32(mx));
+                    mx = max_halves(mx);
                     const float m_new = fmaxf(m_run[qt], mx * a.scale_log2e);
                     const float m_use = (m_new == kNegBig) ? 0.0f : m_new;  // a row with no live key yet
                     // rescale the running sum and O^T only when some row's maximum moved
@@ -206,7 +206,7 @@ __global__ __launch_bounds__(kThreads, 2) void attn_fwd_kernel(const AttnArgs a)
 #pragma unroll
     for (int qt = 0; qt < kQT; ++qt) {
         const int qi = qw0 + 32 * qt + l32;
-        const float l_tot = l_run[qt] + xchg32(l_run[qt]);
+        const float l_tot = sum_halves(l_run[qt]);
         const float inv = l_tot > 0.0f ? __builtin_amdgcn_rcpf(l_tot) : 0.0f;
         if (qi < S) {
             store_row_pieces(a.o + b * a.ob + (int64_t)qi * a.os + h * a.oh, oacc[qt], inv, half);

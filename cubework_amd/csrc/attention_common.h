@@ -93,9 +93,16 @@ __device__ __forceinline__ void store_row_pieces(uint16_t* rowp, const f32x16_t 
         }
 }
 
-// The value of lane ^ 32.
-__device__ __forceinline__ float xchg32(float v) {
-    return __int_as_float(__builtin_amdgcn_ds_bpermute((int)(((threadIdx.x & 63) ^ 32) << 2), __float_as_int(v)));
+// Lane l and lane l ^ 32 combined, the same result in both: v_permlane32_swap exchanges the upper half of
+// its first operand with the lower half of its second, so with v in both the first comes back as the
+// lower half's values in all lanes and the second as the upper half's. One VALU instruction, no LDS trip.
+__device__ __forceinline__ float max_halves(float v) {
+    const auto r = __builtin_amdgcn_permlane32_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+    return fmaxf(__uint_as_float(r[0]), __uint_as_float(r[1]));
+}
+__device__ __forceinline__ float sum_halves(float v) {
+    const auto r = __builtin_amdgcn_permlane32_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+    return __uint_as_float(r[0]) + __uint_as_float(r[1]);
 }
 
 // Loader of one 64-row tile: 512 chunks of 16 bytes spread over NT threads; rows past S read row S-1.

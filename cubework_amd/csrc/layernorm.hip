@@ -401,11 +401,13 @@ int tile_grid(int64_t R, int nr) {
 // (j*64 + l)*V .. +V-1, j < NCH, for every row its wavefront visits, so the
 // dgamma/dbeta accumulators stay in registers for the whole kernel. A
 // wavefront holds NR rows of dY and x at a time.
-template <typename T, int NCH, int NWAVES, int NR>
+// FUSE_DX: the rows are complete on this rank (C is the whole hidden size), so the row sums are final and
+// dx is written from the registers that hold the row, in the same pass.
+template <typename T, int NCH, int NWAVES, int NR, bool FUSE_DX>
 __global__ __launch_bounds__(NWAVES * 64) void ln_bwd_partials_kernel(
     int64_t R, int64_t C, const T* __restrict__ dY, int64_t ld_dy, const T* __restrict__ x, int64_t ld_x,
     const float* __restrict__ mean_rstd, const T* __restrict__ gamma, float* __restrict__ row_sums,
-    float* __restrict__ col_ws, int want_cols) {
+    float* __restrict__ col_ws, int want_cols, T* __restrict__ dx, int64_t ld_dx, float inv_h) {
     constexpr int V = elem<T>::kVec;
     extern __shared__ float lds_red[];
     const int lane = threadIdx.x & 63;
@@ -452,6 +454,24 @@ __global__ __launch_bounds__(NWAVES * 64) void ln_bwd_partials_kernel(
             if (lane == 0 && row < R) {
                 row_sums[2 * row] = s1;
                 row_sums[2 * row + 1] = s2;
+            }
+            if (FUSE_DX) {
+                const float c1 = s1 * inv_h, c2 = s2 * inv_h;
+#pragma unroll
+                for (int j = 0; j < NCH; ++j) {
+                    float dy[V], xv[V], g[V];
+                    unpack_raw(tdy.raw[r][j], dy, (const T*)nullptr);
+                    unpack_raw(tx.raw[r][j], xv, (const T*)nullptr);
+                    unpack_raw(g_raw[j], g, (const T*)nullptr);
+#pragma unroll
+                    for (int e = 0; e < V; ++e) {
+                        const float xh = (xv[e] - mean) * rstd;
+                        const float gg = gamma != nullptr ? dy[e] * g[e] : dy[e];
+                        dy[e] = (gg - xh * c2 - c1) * rstd;
+                    }
+                    if (row < R && chunk_valid<T>(j, lane, C))
+                        store_raw_stream(dx + row * ld_dx + ((int64_t)j * 64 + lane) * V, pack_raw(dy, (const T*)nullptr));
+                }
             }
         }
     }
@@ -625,30 +645,45 @@ int64_t bwd_blocks(int64_t R, int nwaves) {
     return nb;
 }
 
-template <typename T, int NCH, int NWAVES, int NR>
-int bwd_partials_launch(int64_t R, int64_t C, const void* dY, int64_t ld_dy, const void* x, int64_t ld_x,
-                        const float* mean_rstd, const void* gamma, float* row_sums, float* ws, int want_cols,
-                        hipStream_t s) {
+template <typename T, int NCH, int NWAVES, int NR, bool FUSE_DX>
+int bwd_partials_launch_as(int64_t R, int64_t C, const void* dY, int64_t ld_dy, const void* x, int64_t ld_x,
+                           const float* mean_rstd, const void* gamma, float* row_sums, float* ws, int want_cols,
+                           void* dx, int64_t ld_dx, hipStream_t s) {
     constexpr int V = elem<T>::kVec;
     const int64_t nb = bwd_blocks(R, NWAVES * NR);
     const size_t lds = flat_reduce_lds_bytes(2 * NCH * V, NWAVES);
-    auto kern = ln_bwd_partials_kernel<T, NCH, NWAVES, NR>;
+    auto kern = ln_bwd_partials_kernel<T, NCH, NWAVES, NR, FUSE_DX>;
     if (lds > 48 * 1024) {
         hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
         if (e != hipSuccess) return fail(CW_ERR_LAUNCH, "hipFuncSetAttribute(ln_bwd_partials): %s", hipGetErrorString(e));
     }
     hipLaunchKernelGGL(kern, dim3((unsigned)nb), dim3(NWAVES * 64), lds, s, R, C, (const T*)dY, ld_dy, (const T*)x,
-                       ld_x, mean_rstd, (const T*)gamma, row_sums, ws, want_cols);
+                       ld_x, mean_rstd, (const T*)gamma, row_sums, ws, want_cols, (T*)dx, ld_dx, 1.0f / (float)C);
     return check_launch("ln_bwd_partials_kernel");
+}
+
+template <typename T, int NCH, int NWAVES, int NR>
+int bwd_partials_launch(int64_t R, int64_t C, const void* dY, int64_t ld_dy, const void* x, int64_t ld_x,
+                        const float* mean_rstd, const void* gamma, float* row_sums, float* ws, int want_cols,
+                        void* dx, int64_t ld_dx, hipStream_t s) {
+    if (dx != nullptr)
+        return bwd_partials_launch_as<T, NCH, NWAVES, NR, true>(R, C, dY, ld_dy, x, ld_x, mean_rstd, gamma, row_sums, ws,
+                                                                want_cols, dx, ld_dx, s);
+    return bwd_partials_launch_as<T, NCH, NWAVES, NR, false>(R, C, dY, ld_dy, x, ld_x, mean_rstd, gamma, row_sums, ws,
+                                                             want_cols, nullptr, 0, s);
 }
 
 constexpr int64_t kGenericSlabRows = 64;
 
+// dx != nullptr asks for the fused backward (C is the whole hidden size); *dx_done tells whether the
+// kernel chosen wrote dx or the caller still has to run the dx kernel.
 template <typename T>
 int bwd_partials_impl(int64_t R, int64_t C, const void* dY, int64_t ld_dy, const void* x, int64_t ld_x,
                       const float* mean_rstd, const void* gamma, float* row_sums, float* dgamma, float* dbeta,
-                      void* workspace, int64_t workspace_bytes, hipStream_t s) {
+                      void* workspace, int64_t workspace_bytes, hipStream_t s, void* dx = nullptr, int64_t ld_dx = 0,
+                      bool* dx_done = nullptr) {
     constexpr int V = elem<T>::kVec;
+    if (dx_done != nullptr) *dx_done = false;
     const int want_cols = (dgamma != nullptr || dbeta != nullptr) ? 1 : 0;
     const bool vec = rows_vec_ok<T>(dY, ld_dy) && rows_vec_ok<T>(x, ld_x) && (gamma == nullptr || aligned16(gamma)) &&
                      (C % V) == 0;
@@ -661,15 +696,17 @@ int bwd_partials_impl(int64_t R, int64_t C, const void* dY, int64_t ld_dy, const
         if (want_cols && workspace_bytes < nparts * 2 * C * (int64_t)sizeof(float))
             return fail(CW_ERR_INVALID, "cw_ln_bwd_partials: workspace too small (%lld bytes)", (long long)workspace_bytes);
         float* ws = (float*)workspace;
+        void* fdx = (dx != nullptr && rows_vec_ok<T>(dx, ld_dx)) ? dx : nullptr;
         if (nch <= 1)
-            rc = bwd_partials_launch<T, 1, 16, 2>(R, C, dY, ld_dy, x, ld_x, mean_rstd, gamma, row_sums, ws, want_cols, s);
+            rc = bwd_partials_launch<T, 1, 16, 2>(R, C, dY, ld_dy, x, ld_x, mean_rstd, gamma, row_sums, ws, want_cols, fdx, ld_dx, s);
         else if (nch <= 2)
-            rc = bwd_partials_launch<T, 2, 16, 1>(R, C, dY, ld_dy, x, ld_x, mean_rstd, gamma, row_sums, ws, want_cols, s);
+            rc = bwd_partials_launch<T, 2, 16, 1>(R, C, dY, ld_dy, x, ld_x, mean_rstd, gamma, row_sums, ws, want_cols, fdx, ld_dx, s);
         else if (nch <= 4)
-            rc = bwd_partials_launch<T, 4, 8, 1>(R, C, dY, ld_dy, x, ld_x, mean_rstd, gamma, row_sums, ws, want_cols, s);
+            rc = bwd_partials_launch<T, 4, 8, 1>(R, C, dY, ld_dy, x, ld_x, mean_rstd, gamma, row_sums, ws, want_cols, fdx, ld_dx, s);
         else
-            rc = bwd_partials_launch<T, 8, 4, 1>(R, C, dY, ld_dy, x, ld_x, mean_rstd, gamma, row_sums, ws, want_cols, s);
+            rc = bwd_partials_launch<T, 8, 4, 1>(R, C, dY, ld_dy, x, ld_x, mean_rstd, gamma, row_sums, ws, want_cols, fdx, ld_dx, s);
         if (rc != CW_OK) return rc;
+        if (dx_done != nullptr) *dx_done = fdx != nullptr;
     } else {
         hipLaunchKernelGGL(ln_bwd_rows_generic_kernel<T>, dim3(ln_grid(R)), dim3(kLnBlock), 0, s, R, C,
                            (const T*)dY, ld_dy, (const T*)x, ld_x, mean_rstd, (const T*)gamma, row_sums);
@@ -794,6 +831,42 @@ extern "C" int cw_ln_bwd_partials(int64_t R, int64_t C, const void* dY, int64_t 
                                                            dbeta, workspace, workspace_bytes, s)
                                : bwd_partials_impl<float>(R, C, dY, ld_dy, x, ld_x, mean_rstd, gamma, row_sums, dgamma,
                                                           dbeta, workspace, workspace_bytes, s);
+}
+
+namespace cw {
+namespace {
+template <typename T>
+int backward_fused_impl(int64_t R, int64_t C, const void* dY, int64_t ld_dy, const void* x, int64_t ld_x,
+                        const float* mean_rstd, const void* gamma, float* row_sums, void* dx, int64_t ld_dx,
+                        float* dgamma, float* dbeta, void* workspace, int64_t workspace_bytes, hipStream_t s) {
+    bool dx_done = false;
+    int rc = bwd_partials_impl<T>(R, C, dY, ld_dy, x, ld_x, mean_rstd, gamma, row_sums, dgamma, dbeta, workspace,
+                                  workspace_bytes, s, dx, ld_dx, &dx_done);
+    if (rc != CW_OK || dx_done) return rc;
+    return bwd_dx_impl<T>(R, C, dY, ld_dy, x, ld_x, mean_rstd, gamma, row_sums, C, dx, ld_dx, s);
+}
+}  // namespace
+}  // namespace cw
+
+extern "C" int cw_ln_backward_fused(int64_t R, int64_t C, const void* dY, int64_t ld_dy, const void* x, int64_t ld_x,
+                                    const float* mean_rstd, const void* gamma, float* row_sums, void* dx,
+                                    int64_t ld_dx, float* dgamma, float* dbeta, void* workspace,
+                                    int64_t workspace_bytes, int io_dtype, void* stream) {
+    int rc = check_rc("cw_ln_backward_fused", R, C, io_dtype);
+    if (rc != CW_OK) return rc;
+    if ((dgamma == nullptr) != (dbeta == nullptr))
+        return fail(CW_ERR_INVALID, "cw_ln_backward_fused: dgamma and dbeta must both be given or both be NULL");
+    if (R == 0) return CW_OK;
+    if (dY == nullptr || x == nullptr || mean_rstd == nullptr || row_sums == nullptr || dx == nullptr || ld_dy < C ||
+        ld_x < C || ld_dx < C)
+        return fail(CW_ERR_INVALID, "cw_ln_backward_fused: null pointer or leading dimension < C");
+    if (dgamma != nullptr && workspace == nullptr) return fail(CW_ERR_INVALID, "cw_ln_backward_fused: workspace is NULL");
+    hipStream_t s = (hipStream_t)stream;
+    return io_dtype == CW_BF16
+               ? backward_fused_impl<bf16_t>(R, C, dY, ld_dy, x, ld_x, mean_rstd, gamma, row_sums, dx, ld_dx, dgamma, dbeta,
+                                             workspace, workspace_bytes, s)
+               : backward_fused_impl<float>(R, C, dY, ld_dy, x, ld_x, mean_rstd, gamma, row_sums, dx, ld_dx, dgamma, dbeta,
+                                            workspace, workspace_bytes, s);
 }
 
 extern "C" int cw_ln_bwd_dx(int64_t R, int64_t C, const void* dY, int64_t ld_dy, const void* x, int64_t ld_x,

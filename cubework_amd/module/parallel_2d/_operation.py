@@ -212,9 +212,12 @@ class _Layernorm2D(torch.autograd.Function):
         x, gamma, mean_rstd = ctx.saved_tensors
         hidden_size, row_mode, col_mode, w_dtype, b_dtype = ctx.meta
         with torch.no_grad():
-            row_sums, dgamma, dbeta = ops.ln_bwd_partials(output_grad, x, mean_rstd, gamma)
-            row_sums = all_reduce(row_sums, row_mode)
-            input_grad = ops.ln_bwd_dx(output_grad, x, mean_rstd, row_sums, hidden_size, gamma)
+            if row_mode.world_size == 1:
+                input_grad, dgamma, dbeta = ops.ln_backward_fused(output_grad, x, mean_rstd, gamma)
+            else:
+                row_sums, dgamma, dbeta = ops.ln_bwd_partials(output_grad, x, mean_rstd, gamma)
+                row_sums = all_reduce(row_sums, row_mode)
+                input_grad = ops.ln_bwd_dx(output_grad, x, mean_rstd, row_sums, hidden_size, gamma)
             weight_grad = reduce_scatter(dgamma, -1, col_mode).to(w_dtype)
             bias_grad = reduce_scatter(dbeta, -1, col_mode).to(b_dtype)
         return input_grad, weight_grad, bias_grad, None, None, None, None

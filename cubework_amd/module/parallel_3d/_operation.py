@@ -195,9 +195,12 @@ class _Layernorm3D(torch.autograd.Function):
         x, weight, mean_rstd = ctx.saved_tensors
         hidden, out_mode, ixw_mode, w_dtype, b_dtype = ctx.meta
         with torch.no_grad():
-            row_sums, dgamma, dbeta = ops.ln_bwd_partials(output_grad, x, mean_rstd, weight)
-            row_sums = all_reduce(row_sums, out_mode)
-            input_grad = ops.ln_bwd_dx(output_grad, x, mean_rstd, row_sums, hidden, weight)
+            if out_mode.world_size == 1:
+                input_grad, dgamma, dbeta = ops.ln_backward_fused(output_grad, x, mean_rstd, weight)
+            else:
+                row_sums, dgamma, dbeta = ops.ln_bwd_partials(output_grad, x, mean_rstd, weight)
+                row_sums = all_reduce(row_sums, out_mode)
+                input_grad = ops.ln_bwd_dx(output_grad, x, mean_rstd, row_sums, hidden, weight)
             weight_grad = all_reduce(dgamma, ixw_mode).to(w_dtype)
             bias_grad = all_reduce(dbeta, ixw_mode).to(b_dtype)
         return input_grad, weight_grad, bias_grad, None, None, None, None, None, None

@@ -293,6 +293,32 @@ def ln_bwd_dx(dy: torch.Tensor, x: torch.Tensor, mean_rstd: torch.Tensor, row_su
     return dx.reshape(shape)
 
 
+def ln_backward_fused(dy: torch.Tensor, x: torch.Tensor, mean_rstd: torch.Tensor,
+                      gamma: Optional[torch.Tensor] = None, want_param_grads: bool = True):
+    """Backward of LayerNorm over rows this rank holds whole: (dx, dgamma [C] fp32 or None, dbeta [C] fp32
+    or None) in one pass over dy and x. See cw_ln_backward_fused."""
+    lib = _lib.load()
+    shape = x.shape
+    dy, x = _rows(dy), _rows(x)
+    _require_device(dy, x, mean_rstd, gamma)
+    if dy.shape != x.shape or dy.dtype != x.dtype:
+        raise ValueError("dy and x must agree in shape and dtype")
+    R, C = x.shape
+    gamma = None if gamma is None else gamma.to(x.dtype).contiguous()
+    row_sums = torch.empty((R, 2), dtype=torch.float32, device=x.device)
+    dx = torch.empty((R, C), dtype=x.dtype, device=x.device)
+    dgamma = dbeta = ws = None
+    if want_param_grads:
+        dgamma = torch.empty(C, dtype=torch.float32, device=x.device)
+        dbeta = torch.empty(C, dtype=torch.float32, device=x.device)
+        ws = _workspace(R, C, x.device)
+    rc = lib.cw_ln_backward_fused(R, C, _p(dy), _ld(dy), _p(x), _ld(x), _p(mean_rstd), _p(gamma), _p(row_sums), _p(dx),
+                                  _ld(dx), _p(dgamma), _p(dbeta), _p(ws), ws.numel() if ws is not None else 0,
+                                  _dtype_code(x), _stream())
+    _lib.check(rc, "cw_ln_backward_fused")
+    return dx.reshape(shape), dgamma, dbeta
+
+
 # --------------------------------------------------------------------------
 # vocab-parallel cross-entropy
 # --------------------------------------------------------------------------

@@ -219,6 +219,18 @@ int cw_ln_bwd_dx(int64_t R, int64_t C, const void* dY, int64_t ld_dy,
                  const float* row_sums, int64_t H, void* dx, int64_t ld_dx,
                  int io_dtype, void* stream);
 
+/*
+ * cw_ln_bwd_partials + cw_ln_bwd_dx with H = C in one pass over dY and x, for rows that are complete on
+ * this rank: what _Layernorm_2D.backward (parallel_2d/_operation.py:330-347) and
+ * _Layernorm3D.backward (parallel_3d/_operation.py:294-311) compute when the group their sums are
+ * all-reduced over has one member. The counterpart of cw_ln_forward_fused. row_sums ([R,2] fp32) is
+ * written as by cw_ln_bwd_partials; shapes the one-pass kernel does not take run the two kernels.
+ */
+int cw_ln_backward_fused(int64_t R, int64_t C, const void* dY, int64_t ld_dy,
+                         const void* x, int64_t ld_x, const float* mean_rstd, const void* gamma,
+                         float* row_sums, void* dx, int64_t ld_dx, float* dgamma, float* dbeta,
+                         void* workspace, int64_t workspace_bytes, int io_dtype, void* stream);
+
 /* ---- vocab-parallel cross-entropy -------------------------------------- */
 /*
  * One online pass over this rank's vocabulary slice logits[T,V] (columns

@@ -85,6 +85,37 @@ def test_ln_fused_matches_nn_layernorm(shape, mode, dtype):
     assert_parity(db, br.grad, torch.float32, "dbeta vs autograd", scale=50)
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("affine", [True, False])
+@pytest.mark.parametrize("shape", [(64, 1024), (17, 200), (4, 2048), (1000, 512), (33, 4096), (5, 1001), (3, 5000), (300, 64)])
+def test_ln_backward_fused_matches_autograd(shape, affine, dtype):
+    """Rows complete on this rank: one pass gives dx, dgamma, dbeta. Against F.layer_norm's autograd, and
+    bit-identical to the two-kernel path (partials, then dx with H = C) that it replaces. Shapes cover
+    every chunk count of the one-pass kernel, ragged widths and the generic fallback."""
+    from cubework_amd import ops
+
+    R, C = shape
+    eps = 1e-5
+    x, dy, gamma, beta = _inputs(R, C, dtype, 11)
+    xr = x.float().requires_grad_(True)
+    gr = gamma.float().requires_grad_(True)
+    br = beta.float().requires_grad_(True)
+    y_ref = torch.nn.functional.layer_norm(xr, (C,), gr if affine else None, br if affine else None, eps)
+    y_ref.backward(dy.float())
+    g_dev = gamma.to(DEV) if affine else None
+    _, mr = ops.ln_forward_fused(x.to(DEV), eps, g_dev, beta.to(DEV) if affine else None)
+    dx, dg, db = ops.ln_backward_fused(dy.to(DEV), x.to(DEV), mr, g_dev)
+    s = 10 if dtype == torch.float32 else 1
+    assert_parity(dx, xr.grad.to(dtype), dtype, "fused dx vs autograd", scale=s)
+    if affine:
+        assert_parity(dg, gr.grad, torch.float32, "fused dgamma vs autograd", scale=50)
+        assert_parity(db, br.grad, torch.float32, "fused dbeta vs autograd", scale=50)
+    rs, dg2, db2 = ops.ln_bwd_partials(dy.to(DEV), x.to(DEV), mr, g_dev)
+    dx2 = ops.ln_bwd_dx(dy.to(DEV), x.to(DEV), mr, rs, C, g_dev)
+    assert torch.equal(dx, dx2)
+    assert torch.equal(dg, dg2) and torch.equal(db, db2)
+
+
 def test_ln3d_two_pass_with_peer():
     """3D flavour on one rank of a depth-2 output group: mean exchange, then
     the centred second moment (parallel_3d/_operation.py:273-276)."""
