@@ -109,6 +109,13 @@ __global__ __launch_bounds__(kThreads, 2) void attn_fwd_kernel(const AttnArgs a)
     tile_r2s<true, false>(kreg, lds, nullptr, tid);
     tile_r2s<false, true>(vreg, nullptr, lds + kImage, tid);
     __syncthreads();
+    // The Q fragments must have arrived before the loop. Left pending, the compiler waits for them
+    // inside the loop in every trip, and such a wait also covers the younger loads in flight: the next
+    // tile's prefetch, whose latency the trip is there to hide.
+#pragma unroll
+    for (int qt = 0; qt < kQT; ++qt)
+#pragma unroll
+        for (int kb = 0; kb < 4; ++kb) asm volatile("" : "+v"(qf[qt][kb]));
 
     for (int t = 0; t < n_tiles; ++t) {
         lds_char* ks = lds + (t & 1) * 2 * kImage;

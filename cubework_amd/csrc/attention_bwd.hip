@@ -105,8 +105,8 @@ __global__ __launch_bounds__(kThreads, 1) void attn_dq_kernel(const BwdArgs a) {
             dof[kb] = __builtin_bit_cast(bf16x8_t, load_raw(g + 16 * kb));
         }
     }
-    const float lse2 = a.lse[(int64_t)bh * S + qrow] * kLog2e;
-    const float dlt = a.delta[(int64_t)bh * S + qrow];
+    const float lse2_ld = a.lse[(int64_t)bh * S + qrow] * kLog2e;
+    const float dlt_ld = a.delta[(int64_t)bh * S + qrow];
     f32x16_t dq[2];
 #pragma unroll
     for (int dt = 0; dt < 2; ++dt)
@@ -126,6 +126,12 @@ __global__ __launch_bounds__(kThreads, 1) void attn_dq_kernel(const BwdArgs a) {
     tile_r2s<true, true>(kr, lds, lds + kImage, tid);
     tile_r2s<true, false>(vr, lds + 2 * kImage, nullptr, tid);
     __syncthreads();
+    // Everything loaded so far must have arrived before the loop: a wait for it inside the loop would
+    // also cover the younger loads in flight there, the next tile's prefetch.
+    float lse2 = lse2_ld, dlt = dlt_ld;
+    asm volatile("" : "+v"(lse2), "+v"(dlt));
+#pragma unroll
+    for (int kb = 0; kb < 4; ++kb) asm volatile("" : "+v"(qf[kb]), "+v"(dof[kb]));
 
     for (int t = 0; t < n_tiles; ++t) {
         lds_char* k_rows = lds + (t & 1) * 3 * kImage;
@@ -235,16 +241,19 @@ __global__ __launch_bounds__(kThreads, 1) void attn_dkdv_kernel(const BwdArgs a)
     ReadOffsets ro;
     ro.init(lane);
     TileRegs<kThreads> qr, gr;
-    float stat = 0.0f;  // threads 0..63: L*log2e of tile row tid; 64..127: D of tile row tid - 64
+    // threads 0..63: L of tile row tid (stored times log2e); 64..127: D of tile row tid - 64. Every thread
+    // loads (no branch around the load: the value is not needed before the tile it belongs to is stored,
+    // and a wait inside a branch would cover the tile prefetch issued just before); the rest discard.
+    float stat = 0.0f;
+    const float* statp = tid < kTile ? lsep : dltp;
+    const float stat_mul = tid < kTile ? kLog2e : 1.0f;
     auto load_stats = [&](int q0) {
-        if (tid < 2 * kTile) {
-            int row = q0 + (tid & (kTile - 1));
-            row = row < S ? row : S - 1;
-            stat = tid < kTile ? lsep[row] * kLog2e : dltp[row];
-        }
+        int row = q0 + (tid & (kTile - 1));
+        row = row < S ? row : S - 1;
+        stat = statp[row];
     };
     auto store_stats = [&](lds_char* stage) {
-        if (tid < 2 * kTile) *(__attribute__((address_space(3))) float*)(stage + 4 * kImage + tid * 4) = stat;
+        if (tid < 2 * kTile) *(__attribute__((address_space(3))) float*)(stage + 4 * kImage + tid * 4) = stat * stat_mul;
     };
     tile_g2r(qr, qp, a.ss, first_tile * kTile, S, tid);
     tile_g2r(gr, gp, a.os, first_tile * kTile, S, tid);
@@ -253,6 +262,8 @@ __global__ __launch_bounds__(kThreads, 1) void attn_dkdv_kernel(const BwdArgs a)
     tile_r2s<true, true>(gr, lds + 2 * kImage, lds + 3 * kImage, tid);
     store_stats(lds);
     __syncthreads();
+#pragma unroll
+    for (int kb = 0; kb < 4; ++kb) asm volatile("" : "+v"(kf[kb]), "+v"(vf[kb]));  // arrived before the loop
 
     for (int t = first_tile; t < n_tiles; ++t) {
         lds_char* stg = lds + ((t - first_tile) & 1) * kDkdvStage;
