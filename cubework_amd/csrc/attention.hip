@@ -100,14 +100,15 @@ __global__ __launch_bounds__(kThreads, 2) void attn_fwd_kernel(const AttnArgs a)
     const int kv_end = a.causal ? q_hi : S;
     const int n_tiles = (kv_end + kTile - 1) / kTile;
 
-    TileRegs<kThreads> kreg, vreg;
+    TileDma<kThreads> dma;
+    dma.init(tid);
+    const uint32_t lds_addr = (uint32_t)(uintptr_t)lds;
     ReadOffsets ro;
     ro.init(lane);
-    // stage = K row image, V transpose image
-    tile_g2r(kreg, kp, a.ss, 0, S, tid);
-    tile_g2r(vreg, vp, a.ss, 0, S, tid);
-    tile_r2s<true, false>(kreg, lds, nullptr, tid);
-    tile_r2s<false, true>(vreg, nullptr, lds + kImage, tid);
+    // stage = K row image, V transpose image, filled by the load unit
+    dma.load<true, false>(kp, a.ss, 0, S, lds_addr, 0);
+    dma.load<false, true>(vp, a.ss, 0, S, 0, lds_addr + kImage);
+    dma_wait<0>();
     __syncthreads();
     // The Q fragments must have arrived before the loop. Left pending, the compiler waits for them
     // inside the loop in every trip, and such a wait also covers the younger loads in flight: the next
@@ -122,8 +123,10 @@ __global__ __launch_bounds__(kThreads, 2) void attn_fwd_kernel(const AttnArgs a)
         lds_char* vs = ks + kImage;
         const int kv0 = t * kTile;
         if (t + 1 < n_tiles) {
-            tile_g2r(kreg, kp, a.ss, kv0 + kTile, S, tid);
-            tile_g2r(vreg, vp, a.ss, kv0 + kTile, S, tid);
+            // the other stage was last read in the previous trip, which ended with a barrier
+            const uint32_t nx = lds_addr + ((t + 1) & 1) * 2 * kImage;
+            dma.load<true, false>(kp, a.ss, kv0 + kTile, S, nx, 0);
+            dma.load<false, true>(vp, a.ss, kv0 + kTile, S, 0, nx + kImage);
         }
 
         const bool active = !a.causal || kv0 <= qw0 + kQPerWave - 1;
@@ -201,11 +204,7 @@ __global__ __launch_bounds__(kThreads, 2) void attn_fwd_kernel(const AttnArgs a)
             half_tile(std::integral_constant<int, 0>{});
             half_tile(std::integral_constant<int, 1>{});
         }
-        if (t + 1 < n_tiles) {
-            lds_char* nx = lds + ((t + 1) & 1) * 2 * kImage;
-            tile_r2s<true, false>(kreg, nx, nullptr, tid);
-            tile_r2s<false, true>(vreg, nullptr, nx + kImage, tid);
-        }
+        dma_wait<0>();  // the next tile has landed (a third stage and loads two tiles ahead gained nothing)
         __syncthreads();
     }
 
@@ -243,6 +242,8 @@ extern "C" int cw_attn_fwd(int64_t B, int64_t H, int64_t S, int64_t D, const voi
                          stride_b % 8 == 0 && stride_s % 8 == 0 && stride_h % 8 == 0 && out_stride_b % 4 == 0 &&
                          out_stride_s % 4 == 0 && out_stride_h % 4 == 0;
     if (!aligned) return fail(CW_ERR_ALIGNMENT, "cw_attn_fwd: q/k/v need 16-byte aligned rows, out 8-byte aligned rows");
+    if (stride_s <= 0 || stride_s >= (1 << 23))
+        return fail(CW_ERR_INVALID, "cw_attn_fwd: token stride %lld outside (0, 2^23) elements", (long long)stride_s);
     AttnArgs a;
     a.q = (const uint16_t*)q;
     a.k = (const uint16_t*)k;

@@ -120,11 +120,13 @@ __global__ __launch_bounds__(kThreads, 1) void attn_dq_kernel(const BwdArgs a) {
 
     ReadOffsets ro;
     ro.init(lane);
-    TileRegs<kThreads> kr, vr;
-    tile_g2r(kr, kp, a.ss, 0, S, tid);
-    tile_g2r(vr, vp, a.ss, 0, S, tid);
-    tile_r2s<true, true>(kr, lds, lds + kImage, tid);
-    tile_r2s<true, false>(vr, lds + 2 * kImage, nullptr, tid);
+    TileDma<kThreads> dma;
+    dma.init(tid);
+    const uint32_t lds_addr = (uint32_t)(uintptr_t)lds;
+    // stage = K row image, K transpose image, V row image, filled by the load unit
+    dma.load<true, true>(kp, a.ss, 0, S, lds_addr, lds_addr + kImage);
+    dma.load<true, false>(vp, a.ss, 0, S, lds_addr + 2 * kImage, 0);
+    dma_wait<0>();
     __syncthreads();
     // Everything loaded so far must have arrived before the loop: a wait for it inside the loop would
     // also cover the younger loads in flight there, the next tile's prefetch.
@@ -139,8 +141,10 @@ __global__ __launch_bounds__(kThreads, 1) void attn_dq_kernel(const BwdArgs a) {
         lds_char* v_rows = k_rows + 2 * kImage;
         const int kv0 = t * kTile;
         if (t + 1 < n_tiles) {
-            tile_g2r(kr, kp, a.ss, kv0 + kTile, S, tid);
-            tile_g2r(vr, vp, a.ss, kv0 + kTile, S, tid);
+            // the other stage was last read in the previous trip, which ended with a barrier
+            const uint32_t nx = lds_addr + ((t + 1) & 1) * 3 * kImage;
+            dma.load<true, true>(kp, a.ss, kv0 + kTile, S, nx, nx + kImage);
+            dma.load<true, false>(vp, a.ss, kv0 + kTile, S, nx + 2 * kImage, 0);
         }
         const bool active = !a.causal || kv0 <= qw0 + kRowsPerWave - 1;
         if (active) {
@@ -182,11 +186,7 @@ __global__ __launch_bounds__(kThreads, 1) void attn_dq_kernel(const BwdArgs a) {
             half_tile(std::integral_constant<int, 0>{});
             half_tile(std::integral_constant<int, 1>{});
         }
-        if (t + 1 < n_tiles) {
-            lds_char* nx = lds + ((t + 1) & 1) * 3 * kImage;
-            tile_r2s<true, true>(kr, nx, nx + kImage, tid);
-            tile_r2s<true, false>(vr, nx + 2 * kImage, nullptr, tid);
-        }
+        dma_wait<0>();
         __syncthreads();
     }
     if (qi < S) store_row_pieces(a.dq + b * a.gb + (int64_t)qi * a.gs + h * a.gh, dq, a.scale, half);
@@ -240,7 +240,9 @@ __global__ __launch_bounds__(kThreads, 1) void attn_dkdv_kernel(const BwdArgs a)
 
     ReadOffsets ro;
     ro.init(lane);
-    TileRegs<kThreads> qr, gr;
+    TileDma<kThreads> dma;
+    dma.init(tid);
+    const uint32_t lds_addr = (uint32_t)(uintptr_t)lds;
     // threads 0..63: L of tile row tid (stored times log2e); 64..127: D of tile row tid - 64. Every thread
     // loads (no branch around the load: the value is not needed before the tile it belongs to is stored,
     // and a wait inside a branch would cover the tile prefetch issued just before); the rest discard.
@@ -255,12 +257,12 @@ __global__ __launch_bounds__(kThreads, 1) void attn_dkdv_kernel(const BwdArgs a)
     auto store_stats = [&](lds_char* stage) {
         if (tid < 2 * kTile) *(__attribute__((address_space(3))) float*)(stage + 4 * kImage + tid * 4) = stat * stat_mul;
     };
-    tile_g2r(qr, qp, a.ss, first_tile * kTile, S, tid);
-    tile_g2r(gr, gp, a.os, first_tile * kTile, S, tid);
+    // stage = Q row and transpose images, dO row and transpose images (filled by the load unit), row statistics
+    dma.load<true, true>(qp, a.ss, first_tile * kTile, S, lds_addr, lds_addr + kImage);
+    dma.load<true, true>(gp, a.os, first_tile * kTile, S, lds_addr + 2 * kImage, lds_addr + 3 * kImage);
     load_stats(first_tile * kTile);
-    tile_r2s<true, true>(qr, lds, lds + kImage, tid);
-    tile_r2s<true, true>(gr, lds + 2 * kImage, lds + 3 * kImage, tid);
     store_stats(lds);
+    dma_wait<0>();
     __syncthreads();
 #pragma unroll
     for (int kb = 0; kb < 4; ++kb) asm volatile("" : "+v"(kf[kb]), "+v"(vf[kb]));  // arrived before the loop
@@ -274,8 +276,10 @@ __global__ __launch_bounds__(kThreads, 1) void attn_dkdv_kernel(const BwdArgs a)
         lds_char* stats = stg + 4 * kImage + 16 * half;  // + 4 bytes x (4 half): the lane's rows start at 8 g + 4 half
         const int q0 = t * kTile;
         if (t + 1 < n_tiles) {
-            tile_g2r(qr, qp, a.ss, q0 + kTile, S, tid);
-            tile_g2r(gr, gp, a.os, q0 + kTile, S, tid);
+            // the other stage was last read in the previous trip, which ended with a barrier
+            const uint32_t nx = lds_addr + ((t + 1 - first_tile) & 1) * kDkdvStage;
+            dma.load<true, true>(qp, a.ss, q0 + kTile, S, nx, nx + kImage);
+            dma.load<true, true>(gp, a.os, q0 + kTile, S, nx + 2 * kImage, nx + 3 * kImage);
             load_stats(q0 + kTile);
         }
         // the wavefront's keys kw0 .. kw0+31 see queries >= kw0 only
@@ -338,12 +342,8 @@ __global__ __launch_bounds__(kThreads, 1) void attn_dkdv_kernel(const BwdArgs a)
             q_tile(std::integral_constant<int, 0>{});
             q_tile(std::integral_constant<int, 1>{});
         }
-        if (t + 1 < n_tiles) {
-            lds_char* nx = lds + ((t + 1 - first_tile) & 1) * kDkdvStage;
-            tile_r2s<true, true>(qr, nx, nx + kImage, tid);
-            tile_r2s<true, true>(gr, nx + 2 * kImage, nx + 3 * kImage, tid);
-            store_stats(nx);
-        }
+        if (t + 1 < n_tiles) store_stats(lds + ((t + 1 - first_tile) & 1) * kDkdvStage);
+        dma_wait<0>();
         __syncthreads();
     }
     if (kvi < S) {
@@ -388,6 +388,9 @@ extern "C" int cw_attn_bwd(int64_t B, int64_t H, int64_t S, int64_t D, const voi
                          grad_stride_b % 4 == 0 && grad_stride_s % 4 == 0 && grad_stride_h % 4 == 0 &&
                          (reinterpret_cast<uintptr_t>(workspace) & 3u) == 0;
     if (!aligned) return fail(CW_ERR_ALIGNMENT, "cw_attn_bwd: inputs need 16-byte aligned rows, gradients 8-byte aligned rows");
+    if (stride_s <= 0 || stride_s >= (1 << 23) || out_stride_s <= 0 || out_stride_s >= (1 << 23))
+        return fail(CW_ERR_INVALID, "cw_attn_bwd: token strides %lld / %lld outside (0, 2^23) elements", (long long)stride_s,
+                    (long long)out_stride_s);
     BwdArgs a;
     a.q = (const uint16_t*)q; a.k = (const uint16_t*)k; a.v = (const uint16_t*)v;
     a.o = (const uint16_t*)out; a.d_o = (const uint16_t*)d_out;

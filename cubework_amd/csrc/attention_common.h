@@ -105,32 +105,68 @@ __device__ __forceinline__ float sum_halves(float v) {
     return __uint_as_float(r[0]) + __uint_as_float(r[1]);
 }
 
-// Loader of one 64-row tile: 512 chunks of 16 bytes spread over NT threads; rows past S read row S-1.
+// ---- tile loads straight into LDS ------------------------------------------------------------------
+// global_load_lds_dwordx4: lane l of the issuing wavefront writes its 16 bytes at LDS address
+// M0 + 16 l, so one instruction fills 64 consecutive chunk positions of an image and the image's swizzle
+// is applied on the global side: the lane fetches the chunk that belongs at its position. No staging
+// registers, no LDS write instructions. The compiler does not see these loads (inline asm); the kernel
+// waits for them itself (dma_wait) before the barrier that publishes the tile.
+__device__ __forceinline__ void dma16(const char* gbase, uint32_t voff, uint32_t lds_addr) {
+    asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, %2" : : "s"(lds_addr), "v"(voff), "s"(gbase) : "memory", "m0");
+}
+// Waits until at most N of this thread's loads are in flight (loads complete in issue order).
+template <int N>
+__device__ __forceinline__ void dma_wait() {
+    asm volatile("s_waitcnt vmcnt(%0)" : : "n"(N) : "memory");
+}
+
+// Which chunk (row, 16-byte column) of a 64-row tile lives at chunk position p of an image.
+__device__ __forceinline__ void row_image_source(int p, int& r, int& c) {
+    r = p >> 3;
+    c = (p & 7) ^ ((r >> 1) & 7);
+}
+__device__ __forceinline__ void tr_image_source(int p, int& r, int& c) {
+    r = p >> 3;
+    c = ((((p & 7) >> 1) ^ (r & 3)) << 1) | (p & 1);
+}
+
+// Per-thread state of the loader of one tensor: with NT threads each thread owns 512 / NT chunk
+// positions of every image; `row` / `col` say which chunk of the tile belongs there.
 template <int NT>
-struct TileRegs {
+struct TileDma {
     static constexpr int kPer = 512 / NT;
-    raw16_t r[kPer];
+    int row_r[kPer], row_c[kPer], tr_r[kPer], tr_c[kPer];
+    uint32_t wave_off[kPer];  // LDS byte offset of the wavefront's 64 positions inside an image
+    __device__ __forceinline__ void init(int tid) {
+#pragma unroll
+        for (int u = 0; u < kPer; ++u) {
+            const int p = tid + u * NT;
+            row_image_source(p, row_r[u], row_c[u]);
+            tr_image_source(p, tr_r[u], tr_c[u]);
+            wave_off[u] = (uint32_t)__builtin_amdgcn_readfirstlane((p >> 6) * 1024);
+        }
+    }
+    // Tile rows row0 .. row0+63 of the [S, 64] bf16 matrix at `base` (row stride in elements); rows past
+    // S read row S-1. row_img / tr_img: LDS byte addresses of the images to fill (ROW_IMAGE / TR_IMAGE
+    // say which are wanted).
+    template <bool ROW_IMAGE, bool TR_IMAGE>
+    __device__ __forceinline__ void load(const uint16_t* base, int64_t row_stride, int row0, int S, uint32_t row_img,
+                                         uint32_t tr_img) const {
+        const char* g = reinterpret_cast<const char*>(base + (int64_t)row0 * row_stride);
+        const int last = S - 1 - row0;
+#pragma unroll
+        for (int u = 0; u < kPer; ++u) {
+            if (ROW_IMAGE) {
+                const int r = row_r[u] < last ? row_r[u] : last;
+                dma16(g, (uint32_t)((r * (int)row_stride + row_c[u] * 8) * 2), row_img + wave_off[u]);
+            }
+            if (TR_IMAGE) {
+                const int r = tr_r[u] < last ? tr_r[u] : last;
+                dma16(g, (uint32_t)((r * (int)row_stride + tr_c[u] * 8) * 2), tr_img + wave_off[u]);
+            }
+        }
+    }
 };
-template <int NT>
-__device__ __forceinline__ void tile_g2r(TileRegs<NT>& t, const uint16_t* base, int64_t row_stride, int row0, int S, int tid) {
-#pragma unroll
-    for (int u = 0; u < TileRegs<NT>::kPer; ++u) {
-        const int id = tid + u * NT;
-        int row = row0 + (id >> 3);
-        row = row < S ? row : S - 1;
-        t.r[u] = load_raw(base + (int64_t)row * row_stride + (id & 7) * 8);
-    }
-}
-template <bool ROW_IMAGE, bool TR_IMAGE, int NT>
-__device__ __forceinline__ void tile_r2s(const TileRegs<NT>& t, lds_char* row_img, lds_char* tr_img, int tid) {
-#pragma unroll
-    for (int u = 0; u < TileRegs<NT>::kPer; ++u) {
-        const int id = tid + u * NT;
-        const int r = id >> 3, c = id & 7;
-        if (ROW_IMAGE) *(__attribute__((address_space(3))) raw16_t*)(row_img + row_image_offset(r, c)) = t.r[u];
-        if (TR_IMAGE) *(__attribute__((address_space(3))) raw16_t*)(tr_img + tr_image_offset(r, c)) = t.r[u];
-    }
-}
 
 }  // namespace attn
 }  // namespace cw
