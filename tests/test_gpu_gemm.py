@@ -106,6 +106,14 @@ def test_fp32_exact_and_ragged(layout):
     _run(layout, 7, 5, 3, 1, torch.float32, act="relu", seed=15)
 
 
+@pytest.mark.parametrize("layout", LAYOUTS)
+def test_fp32_tall_tiles(layout):
+    """Outputs large enough for the 256-row tiles: exact tiles with addend and pre-activation copy, and a
+    ragged shape through the guarded instantiation."""
+    _run(layout, 4096, 4096, 32, 2, torch.float32, act="gelu_tanh", n_add=1, preact=True, seed=16)
+    _run(layout, 4100, 4104, 40, 1, torch.float32, act="relu", n_add=1, preact=True, seed=17)
+
+
 def test_fp32_linear1d_col_shape():
     # BASELINE config 1: x [8,512,1024] fp32, W [4096,1024], b zeros -> F.linear
     import oracle
