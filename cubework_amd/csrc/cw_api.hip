@@ -57,7 +57,8 @@ extern "C" int64_t cw_gemm_workspace_bytes(int layout, int64_t M, int64_t N, int
     if (layout != CW_NN && layout != CW_NT && layout != CW_TN) return 0;
     if (io_dtype != CW_BF16) return 0;  // the fp32 GEMM is not split
     const int slices = gemm_bf16_split_slices(M, N, K, n_steps);
-    return slices > 1 ? (int64_t)slices * M * N * (int64_t)sizeof(float) : 0;
+    if (slices > 1) return (int64_t)slices * M * N * (int64_t)sizeof(float);
+    return gemm_bf16_ktail_workspace_bytes(layout, M, N, K, n_steps);
 }
 
 extern "C" int cw_gemm_ksteps(int layout, int64_t M, int64_t N, int64_t K, int n_steps, const void* const* A_steps,

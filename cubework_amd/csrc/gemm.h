@@ -38,12 +38,17 @@ struct RingArgs {
     int M, N, K;
     int n_steps, n_addends;
     int vec_bias, vec_add;  // always 1 on this path; read by the shared epilogue
+    // > 0: one more step follows the n_steps regular ones, with k extent k_tail and the operands
+    // A[n_steps], B[n_steps] (how a reduction length that is not a multiple of the k tile is finished)
+    int k_tail;
     float* partial;         // split-k only: [slices][M][N] fp32 partial sums
 };
 
 // Number of k slices the bf16 GEMM would split a problem into (1 = no split)
 // when given scratch; the scratch it then needs is slices * M * N * 4 bytes.
 int gemm_bf16_split_slices(int64_t M, int64_t N, int64_t K, int n_steps);
+// Scratch for finishing a reduction length that is not a multiple of 32 on the LDS-DMA kernel (0: not used).
+int64_t gemm_bf16_ktail_workspace_bytes(int layout, int64_t M, int64_t N, int64_t K, int n_steps);
 
 int gemm_bf16_launch(const GemmArgs& args, int layout, int epilogue, hipStream_t s);
 int gemm_f32_launch(const GemmArgs& args, int layout, int epilogue, hipStream_t s);

@@ -17,9 +17,9 @@
 
 namespace cw {
 
-int gemm_bf16_dma_launch_nn(const GemmArgs& args, int epilogue, hipStream_t s);
-int gemm_bf16_dma_launch_nt(const GemmArgs& args, int epilogue, hipStream_t s);
-int gemm_bf16_dma_launch_tn(const GemmArgs& args, int epilogue, hipStream_t s);
+int gemm_bf16_dma_launch_nn(const GemmArgs& args, int epilogue, hipStream_t s, const void* tail_a, const void* tail_b);
+int gemm_bf16_dma_launch_nt(const GemmArgs& args, int epilogue, hipStream_t s, const void* tail_a, const void* tail_b);
+int gemm_bf16_dma_launch_tn(const GemmArgs& args, int epilogue, hipStream_t s, const void* tail_a, const void* tail_b);
 
 int gemm_bf16_dma_split_launch_nn(const GemmArgs& args, int slices, hipStream_t s);
 int gemm_bf16_dma_split_launch_nt(const GemmArgs& args, int slices, hipStream_t s);
@@ -110,12 +110,53 @@ int splitk_reduce(const GemmArgs& a, int slices, int epilogue, hipStream_t s) {
 
 }  // namespace
 
+// Rows K-32 .. K-1 of a [K, N] operand (row pitch ld) into `out` (same pitch), the first `zero_rows` of
+// them as zeros: the k-slow operand of the short extra step that finishes a reduction length K which is
+// not a multiple of 32. The step covers k in [K-32, K); the part that overlaps the regular steps
+// (zero_rows = 32 - K % 32 rows) must not count twice, and a zero row of this operand takes it out.
+__global__ __launch_bounds__(256) void ktail_rows_kernel(const uint16_t* __restrict__ src, int64_t ld, int64_t K, int N,
+                                                         int zero_rows, uint16_t* __restrict__ out) {
+    const int vec_per_row = N / 8;
+    const int idx = blockIdx.x * 256 + threadIdx.x;
+    if (idx >= 32 * vec_per_row) return;
+    const int r = idx / vec_per_row, c = (idx - r * vec_per_row) * 8;
+    raw16_t v = (raw16_t){0u, 0u, 0u, 0u};
+    if (r >= zero_rows) v = load_raw(src + (K - 32 + r) * ld + c);
+    *reinterpret_cast<raw16_t*>(out + (int64_t)r * ld + c) = v;
+}
+
+int64_t gemm_bf16_ktail_workspace_bytes(int layout, int64_t M, int64_t N, int64_t K, int n_steps) {
+    if (layout == CW_NT || n_steps != 1 || K < 64 || (K % 32) == 0 || (K % 8) != 0) return 0;
+    const int64_t tiles = ((M + 255) / 256) * ((N + 255) / 256);
+    if (tiles < 128 || M < 256 || N < 256 || (N % 8) != 0) return 0;
+    return 32 * N * (int64_t)sizeof(uint16_t);
+}
+
 static bool dma_kernel_enabled() {
     static const bool enabled = [] {
         const char* v = std::getenv("CW_GEMM_IMPL");
         return !(v != nullptr && std::strcmp(v, "staged") == 0);
     }();
     return enabled;
+}
+
+static int staged_launch(const GemmArgs& a, int layout, int epilogue, bool big, bool exact, hipStream_t s) {
+    switch (layout) {
+        case CW_NN: return gemm_bf16_launch_nn(a, epilogue, big, exact, s);
+        case CW_NT: return gemm_bf16_launch_nt(a, epilogue, big, exact, s);
+        case CW_TN: return gemm_bf16_launch_tn(a, epilogue, big, exact, s);
+        default: return fail(CW_ERR_INVALID, "cw_gemm_ksteps: bad layout %d", layout);
+    }
+}
+
+static int dma_launch(const GemmArgs& a, int layout, int epilogue, hipStream_t s, const void* tail_a = nullptr,
+                      const void* tail_b = nullptr) {
+    switch (layout) {
+        case CW_NN: return gemm_bf16_dma_launch_nn(a, epilogue, s, tail_a, tail_b);
+        case CW_NT: return gemm_bf16_dma_launch_nt(a, epilogue, s, tail_a, tail_b);
+        case CW_TN: return gemm_bf16_dma_launch_tn(a, epilogue, s, tail_a, tail_b);
+        default: return fail(CW_ERR_INVALID, "cw_gemm_ksteps: bad layout %d", layout);
+    }
 }
 
 int gemm_bf16_launch(const GemmArgs& args, int layout, int epilogue, hipStream_t s) {
@@ -128,14 +169,34 @@ int gemm_bf16_launch(const GemmArgs& args, int layout, int epilogue, hipStream_t
     const bool big = tiles256 >= 128;
     const int tile = big ? 256 : 128;
     const bool exact = all_vec && (args.M % tile) == 0 && (args.N % tile) == 0 && (args.K % gemm_bf16::kBK) == 0;
-    if (big && exact && args.n_steps > 0 && args.n_steps <= kRingMaxSteps && args.n_addends <= kRingMaxAddends &&
-        dma_kernel_enabled()) {
-        switch (layout) {
-            case CW_NN: return gemm_bf16_dma_launch_nn(args, epilogue, s);
-            case CW_NT: return gemm_bf16_dma_launch_nt(args, epilogue, s);
-            case CW_TN: return gemm_bf16_dma_launch_tn(args, epilogue, s);
-            default: return fail(CW_ERR_INVALID, "cw_gemm_ksteps: bad layout %d", layout);
-        }
+    const bool ring_ok = args.n_steps > 0 && args.n_steps <= kRingMaxSteps && args.n_addends <= kRingMaxAddends &&
+                         dma_kernel_enabled();
+    // The LDS-DMA kernel takes M and N that are not tile multiples (its last tiles overlap their
+    // neighbours): a vocabulary slice of 12568 columns is 50 tiles instead of 49.1. What it needs is one
+    // full tile in each direction and 16-byte steps wherever a tile origin moves along a contiguous
+    // dimension (N always: the output and a [K, N] operand; M for a [K, M] operand).
+    const bool edges_ok = args.M >= 256 && args.N >= 256 && (args.N % 8) == 0 && (layout != CW_TN || (args.M % 8) == 0);
+    if (big && all_vec && ring_ok && edges_ok && (args.K % gemm_bf16::kBK) == 0) return dma_launch(args, layout, epilogue, s);
+    // A reduction length that is not a multiple of the k tile (a vocabulary slice as K: 12568 = 392 x 32 +
+    // 24), with B stored [K, N]: the regular step covers the first K - K % 32 columns, one more step of 32
+    // covers [K-32, K) with a copy of B's last 32 rows whose overlapping rows are zero. The copy (64 bytes
+    // per column) lives in the caller's scratch and has B's row pitch, which the steps share.
+    if (big && all_vec && ring_ok && edges_ok && layout != CW_NT && args.n_steps == 1 && args.K >= 64 &&
+        (args.K % 32) != 0 && (args.K % 8) == 0 && args.workspace != nullptr && aligned16(args.workspace) &&
+        args.workspace_bytes >= 32 * args.ldb * (int64_t)sizeof(uint16_t)) {
+        const int kr = args.K % 32;
+        uint16_t* tail_b = reinterpret_cast<uint16_t*>(args.workspace);
+        const int vecs = 32 * (args.N / 8);
+        hipLaunchKernelGGL(ktail_rows_kernel, dim3((vecs + 255) / 256), dim3(256), 0, s,
+                           reinterpret_cast<const uint16_t*>(args.B[0]), args.ldb, (int64_t)args.K, args.N, 32 - kr, tail_b);
+        int rc = check_launch("ktail_rows_kernel");
+        if (rc != CW_OK) return rc;
+        // A's part of the step: columns (NN, A is [M, K]) or rows (TN, A is [K, M]) K-32 .. K-1, in place
+        const uint16_t* a0 = reinterpret_cast<const uint16_t*>(args.A[0]);
+        const void* tail_a = layout == CW_TN ? a0 + (int64_t)(args.K - 32) * args.lda : a0 + (args.K - 32);
+        GemmArgs main_part = args;
+        main_part.K = args.K - kr;
+        return dma_launch(main_part, layout, epilogue, s, tail_a, tail_b);
     }
     const int slices = gemm_bf16_split_slices(args.M, args.N, args.K, args.n_steps);
     if (slices > 1 && all_vec && args.n_addends <= kRingMaxAddends && dma_kernel_enabled() &&
@@ -151,12 +212,7 @@ int gemm_bf16_launch(const GemmArgs& args, int layout, int epilogue, hipStream_t
         if (rc != CW_OK) return rc;
         return splitk_reduce(args, slices, epilogue, s);
     }
-    switch (layout) {
-        case CW_NN: return gemm_bf16_launch_nn(args, epilogue, big, exact, s);
-        case CW_NT: return gemm_bf16_launch_nt(args, epilogue, big, exact, s);
-        case CW_TN: return gemm_bf16_launch_tn(args, epilogue, big, exact, s);
-        default: return fail(CW_ERR_INVALID, "cw_gemm_ksteps: bad layout %d", layout);
-    }
+    return staged_launch(args, layout, epilogue, big, exact, s);
 }
 
 }  // namespace cw

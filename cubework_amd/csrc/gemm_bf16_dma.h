@@ -135,7 +135,10 @@ __global__ __launch_bounds__(kThreads) void gemm_bf16_dma_kernel(const RingArgs 
     const int wm = wave >> 1, wn = wave & 1;
 
     const int M = args.M, N = args.N, K = args.K;
-    const int tiles_m = M / kTile, tiles_n = N / kTile;
+    // M and N need not be tile multiples (but are at least one tile): the last tile of a row or column of
+    // tiles is moved back to end at the edge. It overlaps its neighbour, and both compute the shared
+    // elements from the same operands in the same order, so the duplicate stores write identical bits.
+    const int tiles_m = (M + kTile - 1) / kTile, tiles_n = (N + kTile - 1) / kTile;
     const int total = tiles_m * tiles_n;
     int tile;
     {
@@ -149,14 +152,17 @@ __global__ __launch_bounds__(kThreads) void gemm_bf16_dma_kernel(const RingArgs 
     const int first_m = group * GROUP_M;
     const int gsz = (tiles_m - first_m) < GROUP_M ? (tiles_m - first_m) : GROUP_M;
     const int in_group = tile - group * GROUP_M * tiles_n;
-    const int m0 = (first_m + in_group % gsz) * kTile;
-    const int n0 = (in_group / gsz) * kTile;
+    int m0 = (first_m + in_group % gsz) * kTile;
+    int n0 = (in_group / gsz) * kTile;
+    m0 = m0 + kTile > M ? M - kTile : m0;
+    n0 = n0 + kTile > N ? N - kTile : n0;
 
     const int k_len = SPLIT ? K / (int)gridDim.y : K;  // k extent of this block within each step
     const int k_beg = SPLIT ? (int)blockIdx.y * k_len : 0;
     const int k_end = k_beg + k_len;
     const int kt_per_step = k_len / kBK;
-    const int KT = kt_per_step * args.n_steps;
+    const int k_tail = SPLIT ? 0 : args.k_tail;
+    const int KT = kt_per_step * args.n_steps + k_tail / kBK;
 
     uint32_t a_even, a_odd, b_even, b_odd;
     dma_lane_offsets<TRANS_A>(lane, args.lda, m0, a_even, a_odd);
@@ -195,18 +201,19 @@ __global__ __launch_bounds__(kThreads) void gemm_bf16_dma_kernel(const RingArgs 
     // issue position stays on it: the loop keeps issuing (harmless duplicate
     // loads into a free stage) so that its body has no branches and the load
     // counter arithmetic is the same in every iteration.
-    int is_kt = 0, is_step = 0, is_k0 = k_beg, is_stage = 0;
+    int is_kt = 0, is_step = 0, is_k0 = k_beg, is_stage = 0, is_k_end = k_end;
     const char* is_a = reinterpret_cast<const char*>(args.A[0]);
     const char* is_b = reinterpret_cast<const char*>(args.B[0]);
     auto issue_advance = [&]() {
         if (is_kt + 1 < KT) {
             ++is_kt;
             is_k0 += kBK;
-            if (is_k0 >= k_end) {
+            if (is_k0 >= is_k_end) {
                 is_k0 = k_beg;
                 ++is_step;
                 is_a = reinterpret_cast<const char*>(gemm_bf16::pick_ptr(args.A, is_step));
                 is_b = reinterpret_cast<const char*>(gemm_bf16::pick_ptr(args.B, is_step));
+                if (is_step == args.n_steps) is_k_end = k_beg + k_tail;  // the short extra step
             }
         }
         is_stage = (is_stage + 1 == NS) ? 0 : is_stage + 1;
@@ -319,6 +326,7 @@ constexpr size_t lds_bytes_dma() {
 inline RingArgs to_ring_args(const GemmArgs& g) {
     RingArgs r = {};
     for (int i = 0; i < g.n_steps && i < kRingMaxSteps; ++i) { r.A[i] = g.A[i]; r.B[i] = g.B[i]; }
+    r.k_tail = 0;
     for (int i = 0; i < g.n_addends && i < kRingMaxAddends; ++i) r.addend[i] = g.addend[i];
     r.bias = g.bias; r.C = g.C; r.preact = g.preact;
     r.lda = g.lda; r.ldb = g.ldb; r.ldc = g.ldc; r.ldp = g.ldp; r.ldadd = g.ldadd;
@@ -328,15 +336,22 @@ inline RingArgs to_ring_args(const GemmArgs& g) {
     return r;
 }
 
+// tail_a / tail_b != nullptr: the extra short step (k extent kBK) that finishes a reduction length which is
+// not a multiple of the k tile; gargs.K is then the part covered by the regular steps.
 template <bool TA, bool TB, int EPI, int NS>
-int launch_dma_cfg(const GemmArgs& gargs, hipStream_t s) {
-    const RingArgs args = to_ring_args(gargs);
+int launch_dma_cfg(const GemmArgs& gargs, hipStream_t s, const void* tail_a = nullptr, const void* tail_b = nullptr) {
+    RingArgs args = to_ring_args(gargs);
+    if (tail_a != nullptr && tail_b != nullptr && gargs.n_steps < kRingMaxSteps) {
+        args.A[gargs.n_steps] = tail_a;
+        args.B[gargs.n_steps] = tail_b;
+        args.k_tail = kBK;
+    }
     auto kern = gemm_bf16_dma_kernel<TA, TB, EPI, NS, false>;
     constexpr size_t lds = lds_bytes_dma<NS>();
     static_assert(lds <= 160 * 1024, "LDS image does not fit the CU");
     hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
     if (e != hipSuccess) return fail(CW_ERR_LAUNCH, "hipFuncSetAttribute(gemm_bf16_ring): %s", hipGetErrorString(e));
-    const int tiles = (args.M / kTile) * (args.N / kTile);
+    const int tiles = ((args.M + kTile - 1) / kTile) * ((args.N + kTile - 1) / kTile);
     const int grid = ((tiles + 7) / 8) * 8;
     hipLaunchKernelGGL(kern, dim3(grid), dim3(kThreads), lds, s, args);
     return check_launch("gemm_bf16_dma_kernel");
@@ -354,20 +369,20 @@ int launch_dma_split(const GemmArgs& gargs, int slices, hipStream_t s) {
     constexpr size_t lds = lds_bytes_dma<kStages>();
     hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
     if (e != hipSuccess) return fail(CW_ERR_LAUNCH, "hipFuncSetAttribute(gemm_bf16_ring, split): %s", hipGetErrorString(e));
-    const int tiles = (args.M / kTile) * (args.N / kTile);
+    const int tiles = ((args.M + kTile - 1) / kTile) * ((args.N + kTile - 1) / kTile);
     const int grid = ((tiles + 7) / 8) * 8;
     hipLaunchKernelGGL(kern, dim3(grid, slices), dim3(kThreads), lds, s, args);
     return check_launch("gemm_bf16_dma_kernel (split k)");
 }
 
 template <bool TA, bool TB>
-int launch_dma(const GemmArgs& args, int epilogue, hipStream_t s) {
+int launch_dma(const GemmArgs& args, int epilogue, hipStream_t s, const void* tail_a = nullptr, const void* tail_b = nullptr) {
     switch (epilogue) {
-        case CW_EPI_NONE: return launch_dma_cfg<TA, TB, CW_EPI_NONE, kStages>(args, s);
-        case CW_EPI_BIAS: return launch_dma_cfg<TA, TB, CW_EPI_BIAS, kStages>(args, s);
-        case CW_EPI_BIAS_GELU_TANH: return launch_dma_cfg<TA, TB, CW_EPI_BIAS_GELU_TANH, kStages>(args, s);
-        case CW_EPI_BIAS_GELU_ERF: return launch_dma_cfg<TA, TB, CW_EPI_BIAS_GELU_ERF, kStages>(args, s);
-        case CW_EPI_BIAS_RELU: return launch_dma_cfg<TA, TB, CW_EPI_BIAS_RELU, kStages>(args, s);
+        case CW_EPI_NONE: return launch_dma_cfg<TA, TB, CW_EPI_NONE, kStages>(args, s, tail_a, tail_b);
+        case CW_EPI_BIAS: return launch_dma_cfg<TA, TB, CW_EPI_BIAS, kStages>(args, s, tail_a, tail_b);
+        case CW_EPI_BIAS_GELU_TANH: return launch_dma_cfg<TA, TB, CW_EPI_BIAS_GELU_TANH, kStages>(args, s, tail_a, tail_b);
+        case CW_EPI_BIAS_GELU_ERF: return launch_dma_cfg<TA, TB, CW_EPI_BIAS_GELU_ERF, kStages>(args, s, tail_a, tail_b);
+        case CW_EPI_BIAS_RELU: return launch_dma_cfg<TA, TB, CW_EPI_BIAS_RELU, kStages>(args, s, tail_a, tail_b);
         default: return fail(CW_ERR_INVALID, "cw_gemm_ksteps: bad epilogue %d", epilogue);
     }
 }

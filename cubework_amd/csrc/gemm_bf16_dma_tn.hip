@@ -3,8 +3,8 @@
 
 namespace cw {
 
-int gemm_bf16_dma_launch_tn(const GemmArgs& args, int epilogue, hipStream_t s) {
-    return gemm_dma::launch_dma<true, true>(args, epilogue, s);
+int gemm_bf16_dma_launch_tn(const GemmArgs& args, int epilogue, hipStream_t s, const void* tail_a, const void* tail_b) {
+    return gemm_dma::launch_dma<true, true>(args, epilogue, s, tail_a, tail_b);
 }
 
 int gemm_bf16_dma_split_launch_tn(const GemmArgs& args, int slices, hipStream_t s) {

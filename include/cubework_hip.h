@@ -115,10 +115,15 @@ int cw_gemm_ksteps(int layout, int64_t M, int64_t N, int64_t K, int n_steps,
  * step is split over several workgroups per tile, whose fp32 partial sums go
  * through `workspace` and are added in a fixed order (bit-reproducible; the
  * reference leaves this choice, and its scratch, to the BLAS library inside
- * torch.matmul). cw_gemm_workspace_bytes gives the size that enables it (0 when
- * the shape is not split); with workspace NULL or smaller the call behaves
- * exactly like cw_gemm_ksteps. The scratch must not be shared by calls that
- * may overlap on the device.
+ * torch.matmul). The scratch also serves a large product whose reduction
+ * length is not a multiple of the kernel's k tile and whose B is stored [K, N]
+ * (the input gradient dC W of the vocabulary-slice classifiers,
+ * parallel_2d/_operation.py:408, parallel_1d/module.py:209: K = 12568): 32 rows
+ * of B are copied there, zero-padded, for one short extra k step.
+ * cw_gemm_workspace_bytes gives the size that enables either (0 when the shape
+ * uses neither); with workspace NULL or smaller the call behaves exactly like
+ * cw_gemm_ksteps (same results, a slower kernel). The scratch must not be
+ * shared by calls that may overlap on the device.
  */
 int64_t cw_gemm_workspace_bytes(int layout, int64_t M, int64_t N, int64_t K, int n_steps, int io_dtype);
 int cw_gemm_ksteps_ws(int layout, int64_t M, int64_t N, int64_t K, int n_steps,

@@ -72,6 +72,35 @@ def test_bf16_exact_tiles_big_config(layout):
 
 
 @pytest.mark.parametrize("layout", LAYOUTS)
+@pytest.mark.parametrize("shape", [(4104, 8200, 64), (4096, 8216, 128), (8200, 4096, 64)])
+def test_bf16_ragged_around_aligned_core(layout, shape):
+    """Large outputs whose M and / or N are not tile multiples (a vocabulary slice: 12568 = 49 x 256 + 24):
+    aligned core on the LDS-DMA kernel, strips on the guarded kernel, every part with bias, addend,
+    pre-activation copy and activation."""
+    M, N, K = shape
+    _run(layout, M, N, K, 2, torch.bfloat16, act="gelu_tanh", n_add=1, preact=True, seed=5)
+
+
+@pytest.mark.parametrize("layout", ["NN", "TN"])
+@pytest.mark.parametrize("K", [72, 344, 1000, 1048])
+def test_bf16_ragged_reduction_length(layout, K):
+    """K = 32 n + 8 / 16 / 24 on a large output with B stored [K, N]: regular steps over the first K - K % 32
+    columns plus one short step over [K-32, K) whose overlap is zeroed in a scratch copy of B's last rows.
+    Inputs are kept large in the overlap so that counting it twice would show."""
+    _run(layout, 4096, 8192, K, 1, torch.bfloat16, act="relu", n_add=1, preact=True, seed=7)
+
+
+def test_bf16_vocab_slice_as_reduction_length():
+    # input gradient of a vocabulary-slice classifier, reduced M: dC [2048, 12568] x W [12568, 8192]
+    _run("NN", 2048, 8192, 12568, 1, torch.bfloat16, act=None, bias=False, seed=8)
+
+
+def test_bf16_vocab_slice_classifier_shape():
+    # logits of one vocabulary slice: [8192, 2048] x [12568, 2048]^T (reduced K keeps the CPU oracle quick)
+    _run("NT", 8192, 12568, 256, 1, torch.bfloat16, act=None, seed=6)
+
+
+@pytest.mark.parametrize("layout", LAYOUTS)
 @pytest.mark.parametrize("shape", [(300, 200, 100), (257, 264, 72), (1, 8, 8), (129, 1, 3), (64, 130, 520)])
 def test_bf16_ragged(layout, shape):
     M, N, K = shape
