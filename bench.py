@@ -200,6 +200,19 @@ def bench_other_configs(device, sets):
     us = event_time_us(tn, 50, 10)
     out["gemm_tn_dW_splitk"] = {"us": round(us, 2), "TFLOPs": round(GEMM_FLOP / us / 1e6, 1),
                                 "frac": round(GEMM_FLOP / us / 1e6 / MFMA_BF16_PEAK_TFLOPS, 4)}
+    # vocabulary-slice classifier of the OPT-1.3B-shaped model (one rank of four: 12568 of 50272 classes):
+    # logits = x W^T, and the two gradients. 12568 is not a tile multiple: it is N, M and K in turn.
+    xc = _seeded((8192, 2048), 51, 1.0, torch.bfloat16).to(device)
+    wc = _seeded((12568, 2048), 52, 0.02, torch.bfloat16).to(device)
+    dcl = _seeded((8192, 12568), 53, 1.0, torch.bfloat16).to(device)
+    cls_flop = 2.0 * 8192 * 12568 * 2048
+    for name, fn in (("classifier_logits_nt", lambda: ops.gemm_ksteps("NT", [xc], [wc])),
+                     ("classifier_dW_tn", lambda: ops.gemm_ksteps("TN", [dcl], [xc])),
+                     ("classifier_dX_nn", lambda: ops.gemm_ksteps("NN", [dcl], [wc]))):
+        us = event_time_us(fn, 10, 3)
+        out[name] = {"us": round(us, 2), "TFLOPs": round(cls_flop / us / 1e6, 1),
+                     "frac": round(cls_flop / us / 1e6 / MFMA_BF16_PEAK_TFLOPS, 4)}
+    del xc, wc, dcl
     # config 1 forward: x [4096,1024] fp32, W [4096,1024] fp32 (NT), fp32 MFMA
     x1 = _seeded((4096, 1024), 1, 1.0, torch.float32).to(device)
     w1 = ((torch.rand((4096, 1024), generator=torch.Generator().manual_seed(2)) * 2 - 1) * (6.0 / 5120) ** 0.5).to(device)
