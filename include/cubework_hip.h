@@ -94,7 +94,9 @@ const char* cw_last_error(void);
  * K is the reduction length of ONE step. bias (length N, io_dtype) may be
  * NULL for any epilogue. preact (optional, [M,N], ld = ldp) receives the value
  * before the activation, for the backward of a fused activation. Accumulation
- * across k and across steps is fp32; the result is rounded once.
+ * across k and across steps is fp32; the result is rounded once. C and preact
+ * must not overlap the operands, the addends or each other (an element may be
+ * computed and stored by two workgroups, with identical bits).
  */
 int cw_gemm_ksteps(int layout, int64_t M, int64_t N, int64_t K, int n_steps,
                    const void* const* A_steps, int64_t lda,
