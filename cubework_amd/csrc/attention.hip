@@ -1,4 +1,4 @@
-// Fused causal attention core for gfx950, head size 64, bf16:
+// Fused causal attention core for gfx950, head sizes 64 and 128, bf16:
 //   O = softmax(scale * Q K^T + causal mask) V        per (batch, head)
 // (benchmark/opt/opt.py:81-117 of the reference: scaled bmm, additive mask,
 // softmax, bmm). One pass over K/V per block of queries with a running
@@ -16,11 +16,11 @@
 // read of V provides).
 //
 // Block = 8 wavefronts x 32 query rows; K/V tiles of 64 rows are staged in
-// LDS (two stages, register prefetch of the next tile), K as [kv][d] read with
-// ds_read_b128, V as [kv][d] read with ds_read_b64_tr_b16. Two blocks are
-// resident per compute unit (four wavefronts per SIMD): the kernel is bound by
-// the softmax arithmetic (one v_exp_f32 per score), which the other
-// wavefronts' MFMAs and LDS reads hide behind.
+// LDS (two stages, the next tile loaded straight into LDS while this one is
+// used), K as [kv][d] read with ds_read_b128, V as [kv][d] read with
+// ds_read_b64_tr_b16. At head size 64 two blocks are resident per compute
+// unit (four wavefronts per SIMD); the softmax arithmetic (one v_exp_f32 per
+// score) weighs about as much as the matrix products there.
 #include "attention_common.h"
 
 namespace cw {
@@ -48,8 +48,13 @@ struct AttnArgs {
     int causal;
 };
 
-__global__ __launch_bounds__(kThreads, 2) void attn_fwd_kernel(const AttnArgs a) {
-    __shared__ __attribute__((aligned(16))) char lds_raw[2 * 2 * kImage];
+// NP: head size / 64. A tile of NP x 64 columns is NP images side by side ("panels"); everything that
+// runs over the head dimension runs over NP times as many 16-wide k blocks (scores) or 32-wide output
+// blocks (O^T). Head size 64 keeps two blocks per compute unit, 128 has the registers and LDS of one.
+template <int NP>
+__global__ __launch_bounds__(kThreads, NP == 1 ? 2 : 1) void attn_fwd_kernel(const AttnArgs a) {
+    constexpr int kStage = 2 * NP * kImage;  // K panels (row images), then V panels (transpose images)
+    __shared__ __attribute__((aligned(16))) char lds_raw[2 * kStage];
     lds_char* lds = (lds_char*)lds_raw;
 
     const int tid = threadIdx.x;
@@ -71,21 +76,21 @@ __global__ __launch_bounds__(kThreads, 2) void attn_fwd_kernel(const AttnArgs a)
     const uint16_t* vp = a.v + b * a.sb + h * a.sh;
 
     // Q fragments (B operand): lane = query row l32 of tile qt, 8 d-values at 16 kb + 8 half
-    bf16x8_t qf[kQT][4];
+    bf16x8_t qf[kQT][4 * NP];
 #pragma unroll
     for (int qt = 0; qt < kQT; ++qt) {
         int row = qw0 + 32 * qt + l32;
         row = row < S ? row : S - 1;
         const uint16_t* p = qp + (int64_t)row * a.ss + 8 * half;
 #pragma unroll
-        for (int kb = 0; kb < 4; ++kb) qf[qt][kb] = __builtin_bit_cast(bf16x8_t, load_raw(p + 16 * kb));
+        for (int kb = 0; kb < 4 * NP; ++kb) qf[qt][kb] = __builtin_bit_cast(bf16x8_t, load_raw(p + 16 * kb));
     }
 
-    f32x16_t oacc[kQT][2];
+    f32x16_t oacc[kQT][2 * NP];
 #pragma unroll
     for (int qt = 0; qt < kQT; ++qt)
 #pragma unroll
-        for (int dt = 0; dt < 2; ++dt)
+        for (int dt = 0; dt < 2 * NP; ++dt)
 #pragma unroll
             for (int e = 0; e < 16; ++e) oacc[qt][dt][e] = 0.0f;
     float m_run[kQT], l_run[kQT];  // running maximum of scale*log2e*s; this lane's share of the running sum
@@ -106,8 +111,14 @@ __global__ __launch_bounds__(kThreads, 2) void attn_fwd_kernel(const AttnArgs a)
     ReadOffsets ro;
     ro.init(lane);
     // stage = K row image, V transpose image, filled by the load unit
-    dma.load<true, false>(kp, a.ss, 0, S, lds_addr, 0);
-    dma.load<false, true>(vp, a.ss, 0, S, 0, lds_addr + kImage);
+    auto load_stage = [&](int row0, uint32_t stage_addr) {
+#pragma unroll
+        for (int p = 0; p < NP; ++p) {
+            dma.template load<true, false>(kp + 64 * p, a.ss, row0, S, stage_addr + p * kImage, 0);
+            dma.template load<false, true>(vp + 64 * p, a.ss, row0, S, 0, stage_addr + (NP + p) * kImage);
+        }
+    };
+    load_stage(0, lds_addr);
     dma_wait<0>();
     __syncthreads();
     // The Q fragments must have arrived before the loop. Left pending, the compiler waits for them
@@ -116,17 +127,15 @@ __global__ __launch_bounds__(kThreads, 2) void attn_fwd_kernel(const AttnArgs a)
 #pragma unroll
     for (int qt = 0; qt < kQT; ++qt)
 #pragma unroll
-        for (int kb = 0; kb < 4; ++kb) asm volatile("" : "+v"(qf[qt][kb]));
+        for (int kb = 0; kb < 4 * NP; ++kb) asm volatile("" : "+v"(qf[qt][kb]));
 
     for (int t = 0; t < n_tiles; ++t) {
-        lds_char* ks = lds + (t & 1) * 2 * kImage;
-        lds_char* vs = ks + kImage;
+        lds_char* ks = lds + (t & 1) * kStage;
+        lds_char* vs = ks + NP * kImage;
         const int kv0 = t * kTile;
         if (t + 1 < n_tiles) {
             // the other stage was last read in the previous trip, which ended with a barrier
-            const uint32_t nx = lds_addr + ((t + 1) & 1) * 2 * kImage;
-            dma.load<true, false>(kp, a.ss, kv0 + kTile, S, nx, 0);
-            dma.load<false, true>(vp, a.ss, kv0 + kTile, S, 0, nx + kImage);
+            load_stage(kv0 + kTile, lds_addr + ((t + 1) & 1) * kStage);
         }
 
         const bool active = !a.causal || kv0 <= qw0 + kQPerWave - 1;
@@ -144,8 +153,8 @@ __global__ __launch_bounds__(kThreads, 2) void attn_fwd_kernel(const AttnArgs a)
 #pragma unroll
                     for (int e = 0; e < 16; ++e) st[qt][e] = 0.0f;
 #pragma unroll
-                for (int kb = 0; kb < 4; ++kb) {
-                    const bf16x8_t kf = read_rows<32 * kt>(ks, ro, kb);
+                for (int kb = 0; kb < 4 * NP; ++kb) {
+                    const bf16x8_t kf = read_rows<32 * kt>(ks + (kb >> 2) * kImage, ro, kb & 3);
 #pragma unroll
                     for (int qt = 0; qt < kQT; ++qt)
                         st[qt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf, qf[qt][kb], st[qt], 0, 0, 0);
@@ -174,7 +183,7 @@ __global__ __launch_bounds__(kThreads, 2) void attn_fwd_kernel(const AttnArgs a)
                         const float alpha = __builtin_amdgcn_exp2f(m_run[qt] - m_use);
                         l_run[qt] *= alpha;
 #pragma unroll
-                        for (int dt = 0; dt < 2; ++dt)
+                        for (int dt = 0; dt < 2 * NP; ++dt)
 #pragma unroll
                             for (int e = 0; e < 16; ++e) oacc[qt][dt][e] *= alpha;
                         m_run[qt] = m_new;
@@ -191,9 +200,9 @@ __global__ __launch_bounds__(kThreads, 2) void attn_fwd_kernel(const AttnArgs a)
                 }
                 // O^T += V^T P^T over the 32 kv rows of this half tile
 #pragma unroll
-                for (int dt = 0; dt < 2; ++dt) {
-                    const bf16x8_t vf0 = read_transposed<32 * kt>(vs, ro, dt);
-                    const bf16x8_t vf1 = read_transposed<32 * kt + 16>(vs, ro, dt);
+                for (int dt = 0; dt < 2 * NP; ++dt) {
+                    const bf16x8_t vf0 = read_transposed<32 * kt>(vs + (dt >> 1) * kImage, ro, dt & 1);
+                    const bf16x8_t vf1 = read_transposed<32 * kt + 16>(vs + (dt >> 1) * kImage, ro, dt & 1);
 #pragma unroll
                     for (int qt = 0; qt < kQT; ++qt) {
                         oacc[qt][dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf0, pb[qt][0], oacc[qt][dt], 0, 0, 0);
@@ -215,7 +224,9 @@ __global__ __launch_bounds__(kThreads, 2) void attn_fwd_kernel(const AttnArgs a)
         const float l_tot = sum_halves(l_run[qt]);
         const float inv = l_tot > 0.0f ? __builtin_amdgcn_rcpf(l_tot) : 0.0f;
         if (qi < S) {
-            store_row_pieces(a.o + b * a.ob + (int64_t)qi * a.os + h * a.oh, oacc[qt], inv, half);
+            uint16_t* orow = a.o + b * a.ob + (int64_t)qi * a.os + h * a.oh;
+#pragma unroll
+            for (int p = 0; p < NP; ++p) store_row_pieces(orow + 64 * p, oacc[qt] + 2 * p, inv, half);
             if (half == 0 && a.lse != nullptr)
                 a.lse[(int64_t)bh * S + qi] = (m_run[qt] + __builtin_amdgcn_logf(l_tot)) * kLn2;  // natural-log LSE of scale*s
         }
@@ -233,7 +244,7 @@ extern "C" int cw_attn_fwd(int64_t B, int64_t H, int64_t S, int64_t D, const voi
                            int io_dtype, void* stream) {
     if (B < 0 || H < 0 || S < 0 || D <= 0) return fail(CW_ERR_INVALID, "cw_attn_fwd: bad shape B=%lld H=%lld S=%lld D=%lld", (long long)B, (long long)H, (long long)S, (long long)D);
     if (io_dtype != CW_BF16) return fail(CW_ERR_UNSUPPORTED, "cw_attn_fwd: only bf16 is provided");
-    if (D != kHead) return fail(CW_ERR_UNSUPPORTED, "cw_attn_fwd: head size %lld is not provided (64 only)", (long long)D);
+    if (D != 64 && D != 128) return fail(CW_ERR_UNSUPPORTED, "cw_attn_fwd: head size %lld is not provided (64 and 128)", (long long)D);
     if (B == 0 || H == 0 || S == 0) return CW_OK;
     if (q == nullptr || k == nullptr || v == nullptr || out == nullptr) return fail(CW_ERR_INVALID, "cw_attn_fwd: null pointer");
     if (S > INT32_MAX / 2 || B * H > (1 << 20) || ((S + kQPerBlock - 1) / kQPerBlock) * B * H > INT32_MAX)
@@ -256,7 +267,8 @@ extern "C" int cw_attn_fwd(int64_t B, int64_t H, int64_t S, int64_t D, const voi
     a.scale_log2e = scale * kLog2e;
     a.causal = causal ? 1 : 0;
     a.n_qblocks = (int)((S + kQPerBlock - 1) / kQPerBlock);
-    hipLaunchKernelGGL(attn_fwd_kernel, dim3((unsigned)(a.n_qblocks * B * H)), dim3(kThreads), 0,
-                       (hipStream_t)stream, a);
+    const dim3 grid((unsigned)(a.n_qblocks * B * H));
+    if (D == 64) hipLaunchKernelGGL(attn_fwd_kernel<1>, grid, dim3(kThreads), 0, (hipStream_t)stream, a);
+    else hipLaunchKernelGGL(attn_fwd_kernel<2>, grid, dim3(kThreads), 0, (hipStream_t)stream, a);
     return check_launch("attn_fwd_kernel");
 }

@@ -1,4 +1,4 @@
-// Backward of the fused attention core for gfx950 (head size 64, bf16):
+// Backward of the fused attention core for gfx950 (head sizes 64 and 128, bf16):
 // given Q, K, V, O, dO and the forward's log-sum-exp L (natural log),
 //   P_ij  = exp(scale q_i.k_j - L_i)              (recomputed, never stored)
 //   D_i   = sum_d dO_id O_id
@@ -49,15 +49,18 @@ struct BwdArgs {
     int64_t sb, ss, sh;  // q/k/v strides (elements): batch, token, head
     int64_t ob, os, oh;  // o / dO strides
     int64_t gb, gs, gh;  // dq/dk/dv strides
-    int S, H, BH, n_blocks;
+    int S, H, BH, n_blocks;  // n_blocks: query blocks of the dQ kernel
+    int D;                   // head size (64 or 128)
     float scale, scale_log2e;
     int causal;
 };
 
-// ---- D_i = sum_d dO_id O_id : one 8-lane group per (b, h, i) row ------------
+// ---- D_i = sum_d dO_id O_id : one group of LPR = head size / 8 lanes per (b, h, i) row -------------
+template <int LPR>
 __global__ __launch_bounds__(256) void attn_delta_kernel(const BwdArgs a) {
-    const int64_t row = (int64_t)blockIdx.x * 32 + (threadIdx.x >> 3);  // (bh, i) flattened
-    const int sub = threadIdx.x & 7;
+    constexpr int kRows = 256 / LPR;
+    const int64_t row = (int64_t)blockIdx.x * kRows + (threadIdx.x / LPR);  // (bh, i) flattened
+    const int sub = threadIdx.x % LPR;
     const int64_t total = (int64_t)a.BH * a.S;
     const int64_t rc = row < total ? row : total - 1;
     const int bh = (int)(rc / a.S);
@@ -72,14 +75,17 @@ __global__ __launch_bounds__(256) void attn_delta_kernel(const BwdArgs a) {
     for (int e = 0; e < 8; ++e) s += x[e] * y[e];
     s += dpp_move<kDppXor1>(s);
     s += dpp_move<kDppXor2>(s);
-    s += dpp_move<kDppHalfMirror>(s);
+    s += dpp_move<kDppHalfMirror>(s);  // lanes 0..7 of a row of 16 lanes hold the sum of their 8
+    if (LPR == 16) s += dpp_move<kDppMirror>(s);  // lane l + lane 15 - l: both halves of the 16
     if (sub == 0 && row < total) a.delta[row] = s;
 }
 
 // ---- dQ ---------------------------------------------------------------------
-// LDS per stage: K row image, K transpose image, V row image.
+// LDS per stage: K row images, K transpose images, V row images (NP = head size / 64 panels of each).
+template <int NP>
 __global__ __launch_bounds__(kThreads, 1) void attn_dq_kernel(const BwdArgs a) {
-    __shared__ __attribute__((aligned(16))) char lds_raw[2 * 3 * kImage];
+    constexpr int kStage = 3 * NP * kImage;
+    __shared__ __attribute__((aligned(16))) char lds_raw[2 * kStage];
     lds_char* lds = (lds_char*)lds_raw;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, half = lane >> 5, l32 = lane & 31;
     const int S = a.S;
@@ -95,21 +101,21 @@ __global__ __launch_bounds__(kThreads, 1) void attn_dq_kernel(const BwdArgs a) {
     // the lane's query row: Q and dO fragments (B operands), L*log2e and D
     const int qi = qw0 + l32;
     const int qrow = qi < S ? qi : S - 1;
-    bf16x8_t qf[4], dof[4];
+    bf16x8_t qf[4 * NP], dof[4 * NP];
     {
         const uint16_t* p = a.q + b * a.sb + (int64_t)qrow * a.ss + h * a.sh + 8 * half;
         const uint16_t* g = a.d_o + b * a.ob + (int64_t)qrow * a.os + h * a.oh + 8 * half;
 #pragma unroll
-        for (int kb = 0; kb < 4; ++kb) {
+        for (int kb = 0; kb < 4 * NP; ++kb) {
             qf[kb] = __builtin_bit_cast(bf16x8_t, load_raw(p + 16 * kb));
             dof[kb] = __builtin_bit_cast(bf16x8_t, load_raw(g + 16 * kb));
         }
     }
     const float lse2_ld = a.lse[(int64_t)bh * S + qrow] * kLog2e;
     const float dlt_ld = a.delta[(int64_t)bh * S + qrow];
-    f32x16_t dq[2];
+    f32x16_t dq[2 * NP];
 #pragma unroll
-    for (int dt = 0; dt < 2; ++dt)
+    for (int dt = 0; dt < 2 * NP; ++dt)
 #pragma unroll
         for (int e = 0; e < 16; ++e) dq[dt][e] = 0.0f;
 
@@ -123,9 +129,15 @@ __global__ __launch_bounds__(kThreads, 1) void attn_dq_kernel(const BwdArgs a) {
     TileDma<kThreads> dma;
     dma.init(tid);
     const uint32_t lds_addr = (uint32_t)(uintptr_t)lds;
-    // stage = K row image, K transpose image, V row image, filled by the load unit
-    dma.load<true, true>(kp, a.ss, 0, S, lds_addr, lds_addr + kImage);
-    dma.load<true, false>(vp, a.ss, 0, S, lds_addr + 2 * kImage, 0);
+    // stage = K row images, K transpose images, V row images, filled by the load unit
+    auto load_stage = [&](int row0, uint32_t st) {
+#pragma unroll
+        for (int p = 0; p < NP; ++p) {
+            dma.template load<true, true>(kp + 64 * p, a.ss, row0, S, st + p * kImage, st + (NP + p) * kImage);
+            dma.template load<true, false>(vp + 64 * p, a.ss, row0, S, st + (2 * NP + p) * kImage, 0);
+        }
+    };
+    load_stage(0, lds_addr);
     dma_wait<0>();
     __syncthreads();
     // Everything loaded so far must have arrived before the loop: a wait for it inside the loop would
@@ -133,18 +145,16 @@ __global__ __launch_bounds__(kThreads, 1) void attn_dq_kernel(const BwdArgs a) {
     float lse2 = lse2_ld, dlt = dlt_ld;
     asm volatile("" : "+v"(lse2), "+v"(dlt));
 #pragma unroll
-    for (int kb = 0; kb < 4; ++kb) asm volatile("" : "+v"(qf[kb]), "+v"(dof[kb]));
+    for (int kb = 0; kb < 4 * NP; ++kb) asm volatile("" : "+v"(qf[kb]), "+v"(dof[kb]));
 
     for (int t = 0; t < n_tiles; ++t) {
-        lds_char* k_rows = lds + (t & 1) * 3 * kImage;
-        lds_char* k_tr = k_rows + kImage;
-        lds_char* v_rows = k_rows + 2 * kImage;
+        lds_char* k_rows = lds + (t & 1) * kStage;
+        lds_char* k_tr = k_rows + NP * kImage;
+        lds_char* v_rows = k_rows + 2 * NP * kImage;
         const int kv0 = t * kTile;
         if (t + 1 < n_tiles) {
             // the other stage was last read in the previous trip, which ended with a barrier
-            const uint32_t nx = lds_addr + ((t + 1) & 1) * 3 * kImage;
-            dma.load<true, true>(kp, a.ss, kv0 + kTile, S, nx, nx + kImage);
-            dma.load<true, false>(vp, a.ss, kv0 + kTile, S, nx + 2 * kImage, 0);
+            load_stage(kv0 + kTile, lds_addr + ((t + 1) & 1) * kStage);
         }
         const bool active = !a.causal || kv0 <= qw0 + kRowsPerWave - 1;
         if (active) {
@@ -161,9 +171,9 @@ __global__ __launch_bounds__(kThreads, 1) void attn_dq_kernel(const BwdArgs a) {
                     dpt[e] = 0.0f;
                 }
 #pragma unroll
-                for (int kb = 0; kb < 4; ++kb) {
-                    st = __builtin_amdgcn_mfma_f32_32x32x16_bf16(read_rows<32 * kt>(k_rows, ro, kb), qf[kb], st, 0, 0, 0);
-                    dpt = __builtin_amdgcn_mfma_f32_32x32x16_bf16(read_rows<32 * kt>(v_rows, ro, kb), dof[kb], dpt, 0, 0, 0);
+                for (int kb = 0; kb < 4 * NP; ++kb) {
+                    st = __builtin_amdgcn_mfma_f32_32x32x16_bf16(read_rows<32 * kt>(k_rows + (kb >> 2) * kImage, ro, kb & 3), qf[kb], st, 0, 0, 0);
+                    dpt = __builtin_amdgcn_mfma_f32_32x32x16_bf16(read_rows<32 * kt>(v_rows + (kb >> 2) * kImage, ro, kb & 3), dof[kb], dpt, 0, 0, 0);
                 }
                 // element e: key kv0 + 32 kt + 8 (e / 4) + 4 half + e % 4, query qi
                 float ds[16];
@@ -178,9 +188,10 @@ __global__ __launch_bounds__(kThreads, 1) void attn_dq_kernel(const BwdArgs a) {
                 }
                 const bf16x8_t dsb0 = pack_slots(ds, 0), dsb1 = pack_slots(ds, 1);
 #pragma unroll
-                for (int dt = 0; dt < 2; ++dt) {
-                    dq[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(read_transposed<32 * kt>(k_tr, ro, dt), dsb0, dq[dt], 0, 0, 0);
-                    dq[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(read_transposed<32 * kt + 16>(k_tr, ro, dt), dsb1, dq[dt], 0, 0, 0);
+                for (int dt = 0; dt < 2 * NP; ++dt) {
+                    lds_char* kt_img = k_tr + (dt >> 1) * kImage;
+                    dq[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(read_transposed<32 * kt>(kt_img, ro, dt & 1), dsb0, dq[dt], 0, 0, 0);
+                    dq[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(read_transposed<32 * kt + 16>(kt_img, ro, dt & 1), dsb1, dq[dt], 0, 0, 0);
                 }
             };
             half_tile(std::integral_constant<int, 0>{});
@@ -189,14 +200,24 @@ __global__ __launch_bounds__(kThreads, 1) void attn_dq_kernel(const BwdArgs a) {
         dma_wait<0>();
         __syncthreads();
     }
-    if (qi < S) store_row_pieces(a.dq + b * a.gb + (int64_t)qi * a.gs + h * a.gh, dq, a.scale, half);
+    if (qi < S) {
+        uint16_t* grow = a.dq + b * a.gb + (int64_t)qi * a.gs + h * a.gh;
+#pragma unroll
+        for (int p = 0; p < NP; ++p) store_row_pieces(grow + 64 * p, dq + 2 * p, a.scale, half);
+    }
 }
 
 // ---- dK, dV -----------------------------------------------------------------
-// LDS per stage: Q row image, Q transpose image, dO row image, dO transpose image, L*log2e and D of the 64 rows.
-constexpr int kDkdvStage = 4 * kImage + 2 * kTile * 4;
+// LDS per stage: Q row images, Q transpose images, dO row images, dO transpose images (NP = head size / 64
+// panels of each), L*log2e and D of the 64 rows. NW wavefronts of 32 key rows: 8 at head size 64; 4 at 128,
+// where a wavefront's accumulators and fragments need more than the 256 registers that 8 would leave it.
+template <int NP>
+constexpr int dkdv_stage_bytes() { return 4 * NP * kImage + 2 * kTile * 4; }
 
-__global__ __launch_bounds__(kThreads, 1) void attn_dkdv_kernel(const BwdArgs a) {
+template <int NP, int NW>
+__global__ __launch_bounds__(NW * 64, 1) void attn_dkdv_kernel(const BwdArgs a) {
+    constexpr int kDkdvStage = dkdv_stage_bytes<NP>();
+    constexpr int kStatsAt = 4 * NP * kImage;
     extern __shared__ __attribute__((aligned(16))) char lds_dyn[];
     lds_char* lds = (lds_char*)lds_dyn;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, half = lane >> 5, l32 = lane & 31;
@@ -204,7 +225,7 @@ __global__ __launch_bounds__(kThreads, 1) void attn_dkdv_kernel(const BwdArgs a)
     const int bh = (int)(blockIdx.x % (unsigned)a.BH);
     const int b = bh / a.H, h = bh - b * a.H;
     const int kvblk = (int)(blockIdx.x / (unsigned)a.BH);  // under the causal mask the first key block is the longest
-    const int kvb0 = kvblk * kRowsPerBlock;
+    const int kvb0 = kvblk * (NW * kRowsPerWave);
     const int kw0 = kvb0 + wave * kRowsPerWave;
 
     const uint16_t* qp = a.q + b * a.sb + h * a.sh;
@@ -215,19 +236,19 @@ __global__ __launch_bounds__(kThreads, 1) void attn_dkdv_kernel(const BwdArgs a)
     // the lane's key row: K and V fragments (B operands)
     const int kvi = kw0 + l32;
     const int kvrow = kvi < S ? kvi : S - 1;
-    bf16x8_t kf[4], vf[4];
+    bf16x8_t kf[4 * NP], vf[4 * NP];
     {
         const uint16_t* pk = a.k + b * a.sb + (int64_t)kvrow * a.ss + h * a.sh + 8 * half;
         const uint16_t* pv = a.v + b * a.sb + (int64_t)kvrow * a.ss + h * a.sh + 8 * half;
 #pragma unroll
-        for (int kb = 0; kb < 4; ++kb) {
+        for (int kb = 0; kb < 4 * NP; ++kb) {
             kf[kb] = __builtin_bit_cast(bf16x8_t, load_raw(pk + 16 * kb));
             vf[kb] = __builtin_bit_cast(bf16x8_t, load_raw(pv + 16 * kb));
         }
     }
-    f32x16_t dk[2], dv[2];
+    f32x16_t dk[2 * NP], dv[2 * NP];
 #pragma unroll
-    for (int dt = 0; dt < 2; ++dt)
+    for (int dt = 0; dt < 2 * NP; ++dt)
 #pragma unroll
         for (int e = 0; e < 16; ++e) {
             dk[dt][e] = 0.0f;
@@ -240,7 +261,7 @@ __global__ __launch_bounds__(kThreads, 1) void attn_dkdv_kernel(const BwdArgs a)
 
     ReadOffsets ro;
     ro.init(lane);
-    TileDma<kThreads> dma;
+    TileDma<NW * 64> dma;
     dma.init(tid);
     const uint32_t lds_addr = (uint32_t)(uintptr_t)lds;
     // threads 0..63: L of tile row tid (stored times log2e); 64..127: D of tile row tid - 64. Every thread
@@ -255,31 +276,35 @@ __global__ __launch_bounds__(kThreads, 1) void attn_dkdv_kernel(const BwdArgs a)
         stat = statp[row];
     };
     auto store_stats = [&](lds_char* stage) {
-        if (tid < 2 * kTile) *(__attribute__((address_space(3))) float*)(stage + 4 * kImage + tid * 4) = stat * stat_mul;
+        if (tid < 2 * kTile) *(__attribute__((address_space(3))) float*)(stage + kStatsAt + tid * 4) = stat * stat_mul;
     };
     // stage = Q row and transpose images, dO row and transpose images (filled by the load unit), row statistics
-    dma.load<true, true>(qp, a.ss, first_tile * kTile, S, lds_addr, lds_addr + kImage);
-    dma.load<true, true>(gp, a.os, first_tile * kTile, S, lds_addr + 2 * kImage, lds_addr + 3 * kImage);
+    auto load_stage = [&](int row0, uint32_t st) {
+#pragma unroll
+        for (int p = 0; p < NP; ++p) {
+            dma.template load<true, true>(qp + 64 * p, a.ss, row0, S, st + p * kImage, st + (NP + p) * kImage);
+            dma.template load<true, true>(gp + 64 * p, a.os, row0, S, st + (2 * NP + p) * kImage, st + (3 * NP + p) * kImage);
+        }
+    };
+    load_stage(first_tile * kTile, lds_addr);
     load_stats(first_tile * kTile);
     store_stats(lds);
     dma_wait<0>();
     __syncthreads();
 #pragma unroll
-    for (int kb = 0; kb < 4; ++kb) asm volatile("" : "+v"(kf[kb]), "+v"(vf[kb]));  // arrived before the loop
+    for (int kb = 0; kb < 4 * NP; ++kb) asm volatile("" : "+v"(kf[kb]), "+v"(vf[kb]));  // arrived before the loop
 
     for (int t = first_tile; t < n_tiles; ++t) {
         lds_char* stg = lds + ((t - first_tile) & 1) * kDkdvStage;
         lds_char* q_rows = stg;
-        lds_char* q_tr = stg + kImage;
-        lds_char* g_rows = stg + 2 * kImage;
-        lds_char* g_tr = stg + 3 * kImage;
-        lds_char* stats = stg + 4 * kImage + 16 * half;  // + 4 bytes x (4 half): the lane's rows start at 8 g + 4 half
+        lds_char* q_tr = stg + NP * kImage;
+        lds_char* g_rows = stg + 2 * NP * kImage;
+        lds_char* g_tr = stg + 3 * NP * kImage;
+        lds_char* stats = stg + kStatsAt + 16 * half;  // + 4 bytes x (4 half): the lane's rows start at 8 g + 4 half
         const int q0 = t * kTile;
         if (t + 1 < n_tiles) {
             // the other stage was last read in the previous trip, which ended with a barrier
-            const uint32_t nx = lds_addr + ((t + 1 - first_tile) & 1) * kDkdvStage;
-            dma.load<true, true>(qp, a.ss, q0 + kTile, S, nx, nx + kImage);
-            dma.load<true, true>(gp, a.os, q0 + kTile, S, nx + 2 * kImage, nx + 3 * kImage);
+            load_stage(q0 + kTile, lds_addr + ((t + 1 - first_tile) & 1) * kDkdvStage);
             load_stats(q0 + kTile);
         }
         // the wavefront's keys kw0 .. kw0+31 see queries >= kw0 only
@@ -300,9 +325,9 @@ __global__ __launch_bounds__(kThreads, 1) void attn_dkdv_kernel(const BwdArgs a)
                     dp_acc[e] = 0.0f;
                 }
 #pragma unroll
-                for (int kb = 0; kb < 4; ++kb) {
-                    s_acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(read_rows<32 * qt>(q_rows, ro, kb), kf[kb], s_acc, 0, 0, 0);
-                    dp_acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(read_rows<32 * qt>(g_rows, ro, kb), vf[kb], dp_acc, 0, 0, 0);
+                for (int kb = 0; kb < 4 * NP; ++kb) {
+                    s_acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(read_rows<32 * qt>(q_rows + (kb >> 2) * kImage, ro, kb & 3), kf[kb], s_acc, 0, 0, 0);
+                    dp_acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(read_rows<32 * qt>(g_rows + (kb >> 2) * kImage, ro, kb & 3), vf[kb], dp_acc, 0, 0, 0);
                 }
                 float p[16], ds[16];
 #pragma unroll
@@ -331,9 +356,11 @@ __global__ __launch_bounds__(kThreads, 1) void attn_dkdv_kernel(const BwdArgs a)
                     const bf16x8_t pb = pack_slots(p, sl);
                     const bf16x8_t dsb = pack_slots(ds, sl);
 #pragma unroll
-                    for (int dt = 0; dt < 2; ++dt) {
-                        const bf16x8_t gt = sl == 0 ? read_transposed<32 * qt>(g_tr, ro, dt) : read_transposed<32 * qt + 16>(g_tr, ro, dt);
-                        const bf16x8_t qtr = sl == 0 ? read_transposed<32 * qt>(q_tr, ro, dt) : read_transposed<32 * qt + 16>(q_tr, ro, dt);
+                    for (int dt = 0; dt < 2 * NP; ++dt) {
+                        lds_char* gi = g_tr + (dt >> 1) * kImage;
+                        lds_char* qi_img = q_tr + (dt >> 1) * kImage;
+                        const bf16x8_t gt = sl == 0 ? read_transposed<32 * qt>(gi, ro, dt & 1) : read_transposed<32 * qt + 16>(gi, ro, dt & 1);
+                        const bf16x8_t qtr = sl == 0 ? read_transposed<32 * qt>(qi_img, ro, dt & 1) : read_transposed<32 * qt + 16>(qi_img, ro, dt & 1);
                         dv[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(gt, pb, dv[dt], 0, 0, 0);
                         dk[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(qtr, dsb, dk[dt], 0, 0, 0);
                     }
@@ -347,8 +374,13 @@ __global__ __launch_bounds__(kThreads, 1) void attn_dkdv_kernel(const BwdArgs a)
         __syncthreads();
     }
     if (kvi < S) {
-        store_row_pieces(a.dk + b * a.gb + (int64_t)kvi * a.gs + h * a.gh, dk, a.scale, half);
-        store_row_pieces(a.dv + b * a.gb + (int64_t)kvi * a.gs + h * a.gh, dv, 1.0f, half);
+        uint16_t* dkrow = a.dk + b * a.gb + (int64_t)kvi * a.gs + h * a.gh;
+        uint16_t* dvrow = a.dv + b * a.gb + (int64_t)kvi * a.gs + h * a.gh;
+#pragma unroll
+        for (int p = 0; p < NP; ++p) {
+            store_row_pieces(dkrow + 64 * p, dk + 2 * p, a.scale, half);
+            store_row_pieces(dvrow + 64 * p, dv + 2 * p, 1.0f, half);
+        }
     }
 }
 
@@ -371,7 +403,7 @@ extern "C" int cw_attn_bwd(int64_t B, int64_t H, int64_t S, int64_t D, const voi
     if (B < 0 || H < 0 || S < 0 || D <= 0)
         return fail(CW_ERR_INVALID, "cw_attn_bwd: bad shape B=%lld H=%lld S=%lld D=%lld", (long long)B, (long long)H, (long long)S, (long long)D);
     if (io_dtype != CW_BF16) return fail(CW_ERR_UNSUPPORTED, "cw_attn_bwd: only bf16 is provided");
-    if (D != kHead) return fail(CW_ERR_UNSUPPORTED, "cw_attn_bwd: head size %lld is not provided (64 only)", (long long)D);
+    if (D != 64 && D != 128) return fail(CW_ERR_UNSUPPORTED, "cw_attn_bwd: head size %lld is not provided (64 and 128)", (long long)D);
     if (B == 0 || H == 0 || S == 0) return CW_OK;
     if (q == nullptr || k == nullptr || v == nullptr || out == nullptr || d_out == nullptr || lse == nullptr ||
         dq == nullptr || dk == nullptr || dv == nullptr || workspace == nullptr)
@@ -402,17 +434,31 @@ extern "C" int cw_attn_bwd(int64_t B, int64_t H, int64_t S, int64_t D, const voi
     a.S = (int)S; a.H = (int)H; a.BH = (int)(B * H); a.n_blocks = (int)nblk;
     a.scale = scale; a.scale_log2e = scale * kLog2e;
     a.causal = causal ? 1 : 0;
+    a.D = (int)D;
     hipStream_t s = (hipStream_t)stream;
     const int64_t rows = B * H * S;
-    hipLaunchKernelGGL(attn_delta_kernel, dim3((unsigned)((rows + 31) / 32)), dim3(256), 0, s, a);
+    if (D == 64) hipLaunchKernelGGL(attn_delta_kernel<8>, dim3((unsigned)((rows + 31) / 32)), dim3(256), 0, s, a);
+    else hipLaunchKernelGGL(attn_delta_kernel<16>, dim3((unsigned)((rows + 15) / 16)), dim3(256), 0, s, a);
     int rc = check_launch("attn_delta_kernel");
     if (rc != CW_OK) return rc;
-    hipLaunchKernelGGL(attn_dq_kernel, dim3((unsigned)(nblk * B * H)), dim3(kThreads), 0, s, a);
+    if (D == 64) hipLaunchKernelGGL(attn_dq_kernel<1>, dim3((unsigned)(nblk * B * H)), dim3(kThreads), 0, s, a);
+    else hipLaunchKernelGGL(attn_dq_kernel<2>, dim3((unsigned)(nblk * B * H)), dim3(kThreads), 0, s, a);
     rc = check_launch("attn_dq_kernel");
     if (rc != CW_OK) return rc;
-    constexpr int lds_bytes = 2 * kDkdvStage;
-    hipError_t e = hipFuncSetAttribute((const void*)attn_dkdv_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes);
-    if (e != hipSuccess) return fail(CW_ERR_LAUNCH, "hipFuncSetAttribute(attn_dkdv_kernel): %s", hipGetErrorString(e));
-    hipLaunchKernelGGL(attn_dkdv_kernel, dim3((unsigned)(nblk * B * H)), dim3(kThreads), lds_bytes, s, a);
+    if (D == 64) {
+        constexpr int lds_bytes = 2 * dkdv_stage_bytes<1>();
+        auto kern = attn_dkdv_kernel<1, 8>;
+        hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes);
+        if (e != hipSuccess) return fail(CW_ERR_LAUNCH, "hipFuncSetAttribute(attn_dkdv_kernel): %s", hipGetErrorString(e));
+        hipLaunchKernelGGL(kern, dim3((unsigned)(nblk * B * H)), dim3(8 * 64), lds_bytes, s, a);
+    } else {
+        constexpr int lds_bytes = 2 * dkdv_stage_bytes<2>();
+        auto kern = attn_dkdv_kernel<2, 4>;
+        const int64_t nkv = (S + 4 * kRowsPerWave - 1) / (4 * kRowsPerWave);
+        if (nkv * B * H > INT32_MAX) return fail(CW_ERR_INVALID, "cw_attn_bwd: S or B*H too large");
+        hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes);
+        if (e != hipSuccess) return fail(CW_ERR_LAUNCH, "hipFuncSetAttribute(attn_dkdv_kernel): %s", hipGetErrorString(e));
+        hipLaunchKernelGGL(kern, dim3((unsigned)(nkv * B * H)), dim3(4 * 64), lds_bytes, s, a);
+    }
     return check_launch("attn_dkdv_kernel");
 }

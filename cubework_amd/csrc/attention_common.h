@@ -17,7 +17,7 @@ typedef short s16x4_t __attribute__((ext_vector_type(4)));
 typedef short s16x8_t __attribute__((ext_vector_type(8)));
 typedef __attribute__((address_space(3))) char lds_char;
 
-constexpr int kHead = 64;                  // head size
+constexpr int kHead = 64;                  // columns of one LDS image (a head of 128 is two images side by side)
 constexpr int kTile = 64;                  // rows of a streamed tile
 constexpr int kImage = kTile * kHead * 2;  // 8 KB: one LDS image of a tile
 constexpr float kNegBig = -__builtin_huge_valf();
@@ -82,7 +82,7 @@ __device__ __forceinline__ float sum_slots(bf16x8_t v, float acc) {
 
 // Lane (row = lane % 32, half = lane / 32) holds, of a transposed 64 x 32 result, the values
 // d = 32 dt + 8 (e / 4) + 4 half + e % 4 of its row: write them, times `mul`, as bf16.
-__device__ __forceinline__ void store_row_pieces(uint16_t* rowp, const f32x16_t (&acc)[2], float mul, int half) {
+__device__ __forceinline__ void store_row_pieces(uint16_t* rowp, const f32x16_t* acc, float mul, int half) {
 #pragma unroll
     for (int dt = 0; dt < 2; ++dt)
 #pragma unroll

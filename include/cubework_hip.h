@@ -362,7 +362,8 @@ int cw_multi_scale(int n_tensors, void* const* grads, const int64_t* numels, con
  * stride in c; opt.py:72-76 makes them [b, s, heads, 3*d] slices), out
  * likewise with its own strides ([b, s, heads*d] as opt.py:123-128 leaves it).
  * lse (optional, [B,H,S] fp32) receives log sum_j exp(scale * q.k_j) for the
- * backward. D = 64 and CW_BF16 only in this build (CW_ERR_UNSUPPORTED else).
+ * backward. D = 64 or 128 and CW_BF16 only in this build (CW_ERR_UNSUPPORTED
+ * else); token strides below 2^23 elements.
  */
 int cw_attn_fwd(int64_t B, int64_t H, int64_t S, int64_t D,
                 const void* q, const void* k, const void* v,

@@ -76,7 +76,7 @@ def test_attention_full_size_sampled_rows():
 def test_attention_rejects_unsupported():
     from cubework_amd import ops
 
-    q = torch.zeros((1, 8, 1, 32), dtype=torch.bfloat16, device=DEV)
+    q = torch.zeros((1, 8, 1, 96), dtype=torch.bfloat16, device=DEV)
     with pytest.raises(RuntimeError):
         ops.attn_fwd(q, q, q)
     q = torch.zeros((1, 8, 1, 64), dtype=torch.float32, device=DEV)
@@ -133,3 +133,55 @@ def test_attention_core_autograd_and_reproducibility():
     want = torch.cat([dq, dk, dv], dim=-1).permute(0, 2, 1, 3).reshape(b, s, h * 3 * d)
     assert_parity(g1, want, torch.bfloat16, "d qkv", scale=2)
     assert_parity(y, oracle.attention_core(qc, kc, vc), torch.bfloat16, "attention_core forward")
+
+
+@pytest.mark.parametrize("shape", [(1, 64, 1), (2, 256, 2), (1, 100, 2), (1, 257, 1), (1, 1, 1), (1, 33, 2), (1, 700, 2),
+                                   (1, 129, 3)])
+@pytest.mark.parametrize("causal", [True, False])
+def test_attention_head_size_128(shape, causal):
+    """Head size 128 (OPT-6.7B and larger): two 64-column panels per tile; forward, log-sum-exp and the
+    three gradients against the oracle. 129 and 257 tokens cross the key-block size of the dK/dV kernel
+    (128 keys at this head size)."""
+    import oracle
+    from cubework_amd import ops
+
+    b, s, h = shape
+    d = 128
+    qkv = _qkv(b, s, h, d, seed=3 * s + h, std=1.2)
+    d_out = randn((b, s, h * d), torch.bfloat16, seed=s + 17)
+    qc, kc, vc = oracle.split_qkv(qkv, h)
+    want, want_lse = oracle.attention_core(qc, kc, vc, causal=causal, return_lse=True)
+    want_g = oracle.attention_core_backward(qc, kc, vc, d_out, causal=causal)
+    dev = qkv.to(DEV)
+    q, k, v = _views(dev, h, d)
+    out, lse = ops.attn_fwd(q, k, v, causal=causal, want_lse=True)
+    g = torch.full((b, s, h, 3 * d), float("nan"), dtype=torch.bfloat16, device=DEV)
+    ops.attn_bwd(q, k, v, out, d_out.to(DEV), lse, g[..., :d], g[..., d:2 * d], g[..., 2 * d:], causal=causal)
+    torch.cuda.synchronize()
+    assert_parity(out, want, torch.bfloat16, "attention out d=128 %s" % (shape,))
+    assert_parity(lse, want_lse, torch.float32, "attention lse d=128 %s" % (shape,), scale=100)
+    if s == 1:
+        assert_parity(g.permute(0, 2, 1, 3), torch.cat(want_g, dim=-1), torch.bfloat16, "attention grads d=128 %s" % (shape,))
+        return
+    for name, got, ref in (("dq", g[..., :d], want_g[0]), ("dk", g[..., d:2 * d], want_g[1]), ("dv", g[..., 2 * d:], want_g[2])):
+        assert_parity(got.permute(0, 2, 1, 3), ref, torch.bfloat16, "attention %s d=128 %s causal=%s" % (name, shape, causal),
+                      scale=2)
+
+
+def test_attention_head_size_128_autograd():
+    import oracle
+    from cubework_amd import ops
+
+    b, s, h, d = 2, 320, 3, 128
+    qkv = _qkv(b, s, h, d, seed=31)
+    d_out = randn((b, s, h * d), torch.bfloat16, seed=32)
+    x = qkv.to(DEV).requires_grad_(True)
+    ops.attention_core(x, h).backward(d_out.to(DEV))
+    g1 = x.grad.clone()
+    x.grad = None
+    ops.attention_core(x, h).backward(d_out.to(DEV))
+    assert torch.equal(g1, x.grad)
+    qc, kc, vc = oracle.split_qkv(qkv, h)
+    dq, dk, dv = oracle.attention_core_backward(qc, kc, vc, d_out)
+    want = torch.cat([dq, dk, dv], dim=-1).permute(0, 2, 1, 3).reshape(b, s, h * 3 * d)
+    assert_parity(g1, want, torch.bfloat16, "d qkv, head size 128", scale=2)
