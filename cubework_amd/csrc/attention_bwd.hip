@@ -34,6 +34,11 @@ constexpr int kWaves = 8;
 constexpr int kThreads = kWaves * 64;
 constexpr int kRowsPerWave = 32;
 constexpr int kRowsPerBlock = kWaves * kRowsPerWave;
+// dK/dV kernel at head size 64: wavefronts per block and groups of 32 keys per wavefront. 4 x 2 (every LDS
+// operand read feeding two MFMAs, but one wavefront per SIMD: 510 registers) ran the kernel in 278 us against
+// 190 us for 8 x 1.
+constexpr int kDkdvWaves = 8, kDkdvGroups = 1;
+static_assert(kDkdvWaves * kDkdvGroups * kRowsPerWave == kRowsPerBlock, "the dK/dV kernel's key block equals the dQ kernel's query block");
 
 struct BwdArgs {
     const uint16_t* q;
@@ -214,8 +219,11 @@ __global__ __launch_bounds__(kThreads, 1) void attn_dq_kernel(const BwdArgs a) {
 template <int NP>
 constexpr int dkdv_stage_bytes() { return 4 * NP * kImage + 2 * kTile * 4; }
 
-template <int NP, int NW>
+// KG: groups of 32 key rows per wavefront. With two, every A operand read from LDS (Q, dO, their
+// transposes) feeds two MFMAs instead of one.
+template <int NP, int NW, int KG>
 __global__ __launch_bounds__(NW * 64, 1) void attn_dkdv_kernel(const BwdArgs a) {
+    constexpr int kKeysPerWave = KG * kRowsPerWave;
     constexpr int kDkdvStage = dkdv_stage_bytes<NP>();
     constexpr int kStatsAt = 4 * NP * kImage;
     extern __shared__ __attribute__((aligned(16))) char lds_dyn[];
@@ -225,35 +233,38 @@ __global__ __launch_bounds__(NW * 64, 1) void attn_dkdv_kernel(const BwdArgs a) 
     const int bh = (int)(blockIdx.x % (unsigned)a.BH);
     const int b = bh / a.H, h = bh - b * a.H;
     const int kvblk = (int)(blockIdx.x / (unsigned)a.BH);  // under the causal mask the first key block is the longest
-    const int kvb0 = kvblk * (NW * kRowsPerWave);
-    const int kw0 = kvb0 + wave * kRowsPerWave;
+    const int kvb0 = kvblk * (NW * kKeysPerWave);
+    const int kw0 = kvb0 + wave * kKeysPerWave;
 
     const uint16_t* qp = a.q + b * a.sb + h * a.sh;
     const uint16_t* gp = a.d_o + b * a.ob + h * a.oh;
     const float* lsep = a.lse + (int64_t)bh * S;
     const float* dltp = a.delta + (int64_t)bh * S;
 
-    // the lane's key row: K and V fragments (B operands)
-    const int kvi = kw0 + l32;
-    const int kvrow = kvi < S ? kvi : S - 1;
-    bf16x8_t kf[4 * NP], vf[4 * NP];
-    {
+    // the lane's key rows (one per group): K and V fragments (B operands)
+    bf16x8_t kf[KG][4 * NP], vf[KG][4 * NP];
+#pragma unroll
+    for (int kg = 0; kg < KG; ++kg) {
+        const int kvi = kw0 + 32 * kg + l32;
+        const int kvrow = kvi < S ? kvi : S - 1;
         const uint16_t* pk = a.k + b * a.sb + (int64_t)kvrow * a.ss + h * a.sh + 8 * half;
         const uint16_t* pv = a.v + b * a.sb + (int64_t)kvrow * a.ss + h * a.sh + 8 * half;
 #pragma unroll
         for (int kb = 0; kb < 4 * NP; ++kb) {
-            kf[kb] = __builtin_bit_cast(bf16x8_t, load_raw(pk + 16 * kb));
-            vf[kb] = __builtin_bit_cast(bf16x8_t, load_raw(pv + 16 * kb));
+            kf[kg][kb] = __builtin_bit_cast(bf16x8_t, load_raw(pk + 16 * kb));
+            vf[kg][kb] = __builtin_bit_cast(bf16x8_t, load_raw(pv + 16 * kb));
         }
     }
-    f32x16_t dk[2 * NP], dv[2 * NP];
+    f32x16_t dk[KG][2 * NP], dv[KG][2 * NP];
 #pragma unroll
-    for (int dt = 0; dt < 2 * NP; ++dt)
+    for (int kg = 0; kg < KG; ++kg)
 #pragma unroll
-        for (int e = 0; e < 16; ++e) {
-            dk[dt][e] = 0.0f;
-            dv[dt][e] = 0.0f;
-        }
+        for (int dt = 0; dt < 2 * NP; ++dt)
+#pragma unroll
+            for (int e = 0; e < 16; ++e) {
+                dk[kg][dt][e] = 0.0f;
+                dv[kg][dt][e] = 0.0f;
+            }
 
     // query tiles: under the causal mask only queries >= the block's first key take part
     const int first_tile = a.causal ? kvb0 / kTile : 0;
@@ -292,7 +303,9 @@ __global__ __launch_bounds__(NW * 64, 1) void attn_dkdv_kernel(const BwdArgs a) 
     dma_wait<0>();
     __syncthreads();
 #pragma unroll
-    for (int kb = 0; kb < 4 * NP; ++kb) asm volatile("" : "+v"(kf[kb]), "+v"(vf[kb]));  // arrived before the loop
+    for (int kg = 0; kg < KG; ++kg)
+#pragma unroll
+        for (int kb = 0; kb < 4 * NP; ++kb) asm volatile("" : "+v"(kf[kg][kb]), "+v"(vf[kg][kb]));  // arrived before the loop
 
     for (int t = first_tile; t < n_tiles; ++t) {
         lds_char* stg = lds + ((t - first_tile) & 1) * kDkdvStage;
@@ -307,62 +320,79 @@ __global__ __launch_bounds__(NW * 64, 1) void attn_dkdv_kernel(const BwdArgs a) 
             load_stage(q0 + kTile, lds_addr + ((t + 1 - first_tile) & 1) * kDkdvStage);
             load_stats(q0 + kTile);
         }
-        // the wavefront's keys kw0 .. kw0+31 see queries >= kw0 only
+        // the wavefront's keys kw0 .. kw0 + kKeysPerWave - 1 see queries >= kw0 only
         const bool active = !a.causal || q0 + kTile - 1 >= kw0;
         if (active) {
-            const bool need_mask = (a.causal && q0 < kw0 + kRowsPerWave - 1) || q0 + kTile > S;
+            const bool need_mask = (a.causal && q0 < kw0 + kKeysPerWave - 1) || q0 + kTile > S;
             const bool masked = __builtin_amdgcn_readfirstlane((int)need_mask) != 0;  // scalar branch
-            // query element e of query tile qt (row q0 + 32 qt + 8 (e/4) + 4 half + e%4) is live
-            // <=> row >= key (causal) and row < S  <=>  lo <= 32 qt + 8 (e/4) + e%4 < hi
-            const int lo = a.causal ? kvi - q0 - 4 * half : -(1 << 30);
+            // query element e of query tile qt (row q0 + 32 qt + 8 (e/4) + 4 half + e%4) is live for the
+            // key of group kg <=> row >= key (causal) and row < S  <=>  lo + 32 kg <= 32 qt + 8 (e/4) + e%4 < hi
+            const int lo = a.causal ? kw0 + l32 - q0 - 4 * half : -(1 << 30);
             const int hi = S - q0 - 4 * half;
             auto q_tile = [&](auto qt_c) {
                 constexpr int qt = decltype(qt_c)::value;
-                f32x16_t s_acc, dp_acc;
+                f32x16_t s_acc[KG], dp_acc[KG];
 #pragma unroll
-                for (int e = 0; e < 16; ++e) {
-                    s_acc[e] = 0.0f;
-                    dp_acc[e] = 0.0f;
-                }
-#pragma unroll
-                for (int kb = 0; kb < 4 * NP; ++kb) {
-                    s_acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(read_rows<32 * qt>(q_rows + (kb >> 2) * kImage, ro, kb & 3), kf[kb], s_acc, 0, 0, 0);
-                    dp_acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(read_rows<32 * qt>(g_rows + (kb >> 2) * kImage, ro, kb & 3), vf[kb], dp_acc, 0, 0, 0);
-                }
-                float p[16], ds[16];
-#pragma unroll
-                for (int g = 0; g < 4; ++g) {
-                    // L*log2e and D of query rows 32 qt + 8 g + 4 half + {0..3}
-                    const f32x4_t l2 = *(__attribute__((address_space(3))) const f32x4_t*)(stats + (32 * qt + 8 * g) * 4);
-                    const f32x4_t dl = *(__attribute__((address_space(3))) const f32x4_t*)(stats + (kTile + 32 * qt + 8 * g) * 4);
-#pragma unroll
-                    for (int i = 0; i < 4; ++i) {
-                        const int e = 4 * g + i;
-                        p[e] = __builtin_amdgcn_exp2f(__builtin_fmaf(s_acc[e], a.scale_log2e, -l2[i]));
-                        ds[e] = p[e] * (dp_acc[e] - dl[i]);
-                    }
-                }
-                if (masked) {
+                for (int kg = 0; kg < KG; ++kg)
 #pragma unroll
                     for (int e = 0; e < 16; ++e) {
-                        const int r = 32 * qt + 8 * (e >> 2) + (e & 3);
-                        const bool dead = r < lo || r >= hi;
-                        p[e] = dead ? 0.0f : p[e];
-                        ds[e] = dead ? 0.0f : ds[e];
+                        s_acc[kg][e] = 0.0f;
+                        dp_acc[kg][e] = 0.0f;
+                    }
+#pragma unroll
+                for (int kb = 0; kb < 4 * NP; ++kb) {
+                    const bf16x8_t qa = read_rows<32 * qt>(q_rows + (kb >> 2) * kImage, ro, kb & 3);
+                    const bf16x8_t ga = read_rows<32 * qt>(g_rows + (kb >> 2) * kImage, ro, kb & 3);
+#pragma unroll
+                    for (int kg = 0; kg < KG; ++kg) {
+                        s_acc[kg] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(qa, kf[kg][kb], s_acc[kg], 0, 0, 0);
+                        dp_acc[kg] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ga, vf[kg][kb], dp_acc[kg], 0, 0, 0);
+                    }
+                }
+                bf16x8_t pb[KG][2], dsb[KG][2];
+#pragma unroll
+                for (int kg = 0; kg < KG; ++kg) {
+                    float p[16], ds[16];
+#pragma unroll
+                    for (int g = 0; g < 4; ++g) {
+                        // L*log2e and D of query rows 32 qt + 8 g + 4 half + {0..3}
+                        const f32x4_t l2 = *(__attribute__((address_space(3))) const f32x4_t*)(stats + (32 * qt + 8 * g) * 4);
+                        const f32x4_t dl = *(__attribute__((address_space(3))) const f32x4_t*)(stats + (kTile + 32 * qt + 8 * g) * 4);
+#pragma unroll
+                        for (int i = 0; i < 4; ++i) {
+                            const int e = 4 * g + i;
+                            p[e] = __builtin_amdgcn_exp2f(__builtin_fmaf(s_acc[kg][e], a.scale_log2e, -l2[i]));
+                            ds[e] = p[e] * (dp_acc[kg][e] - dl[i]);
+                        }
+                    }
+                    if (masked) {
+#pragma unroll
+                        for (int e = 0; e < 16; ++e) {
+                            const int r = 32 * qt + 8 * (e >> 2) + (e & 3);
+                            const bool dead = r < lo + 32 * kg || r >= hi;
+                            p[e] = dead ? 0.0f : p[e];
+                            ds[e] = dead ? 0.0f : ds[e];
+                        }
+                    }
+#pragma unroll
+                    for (int sl = 0; sl < 2; ++sl) {
+                        pb[kg][sl] = pack_slots(p, sl);
+                        dsb[kg][sl] = pack_slots(ds, sl);
                     }
                 }
 #pragma unroll
                 for (int sl = 0; sl < 2; ++sl) {
-                    const bf16x8_t pb = pack_slots(p, sl);
-                    const bf16x8_t dsb = pack_slots(ds, sl);
 #pragma unroll
                     for (int dt = 0; dt < 2 * NP; ++dt) {
                         lds_char* gi = g_tr + (dt >> 1) * kImage;
                         lds_char* qi_img = q_tr + (dt >> 1) * kImage;
                         const bf16x8_t gt = sl == 0 ? read_transposed<32 * qt>(gi, ro, dt & 1) : read_transposed<32 * qt + 16>(gi, ro, dt & 1);
                         const bf16x8_t qtr = sl == 0 ? read_transposed<32 * qt>(qi_img, ro, dt & 1) : read_transposed<32 * qt + 16>(qi_img, ro, dt & 1);
-                        dv[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(gt, pb, dv[dt], 0, 0, 0);
-                        dk[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(qtr, dsb, dk[dt], 0, 0, 0);
+#pragma unroll
+                        for (int kg = 0; kg < KG; ++kg) {
+                            dv[kg][dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(gt, pb[kg][sl], dv[kg][dt], 0, 0, 0);
+                            dk[kg][dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(qtr, dsb[kg][sl], dk[kg][dt], 0, 0, 0);
+                        }
                     }
                 }
             };
@@ -373,13 +403,17 @@ __global__ __launch_bounds__(NW * 64, 1) void attn_dkdv_kernel(const BwdArgs a) 
         dma_wait<0>();
         __syncthreads();
     }
-    if (kvi < S) {
-        uint16_t* dkrow = a.dk + b * a.gb + (int64_t)kvi * a.gs + h * a.gh;
-        uint16_t* dvrow = a.dv + b * a.gb + (int64_t)kvi * a.gs + h * a.gh;
 #pragma unroll
-        for (int p = 0; p < NP; ++p) {
-            store_row_pieces(dkrow + 64 * p, dk + 2 * p, a.scale, half);
-            store_row_pieces(dvrow + 64 * p, dv + 2 * p, 1.0f, half);
+    for (int kg = 0; kg < KG; ++kg) {
+        const int kvi = kw0 + 32 * kg + l32;
+        if (kvi < S) {
+            uint16_t* dkrow = a.dk + b * a.gb + (int64_t)kvi * a.gs + h * a.gh;
+            uint16_t* dvrow = a.dv + b * a.gb + (int64_t)kvi * a.gs + h * a.gh;
+#pragma unroll
+            for (int p = 0; p < NP; ++p) {
+                store_row_pieces(dkrow + 64 * p, dk[kg] + 2 * p, a.scale, half);
+                store_row_pieces(dvrow + 64 * p, dv[kg] + 2 * p, 1.0f, half);
+            }
         }
     }
 }
@@ -447,13 +481,13 @@ extern "C" int cw_attn_bwd(int64_t B, int64_t H, int64_t S, int64_t D, const voi
     if (rc != CW_OK) return rc;
     if (D == 64) {
         constexpr int lds_bytes = 2 * dkdv_stage_bytes<1>();
-        auto kern = attn_dkdv_kernel<1, 8>;
+        auto kern = attn_dkdv_kernel<1, kDkdvWaves, kDkdvGroups>;
         hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes);
         if (e != hipSuccess) return fail(CW_ERR_LAUNCH, "hipFuncSetAttribute(attn_dkdv_kernel): %s", hipGetErrorString(e));
-        hipLaunchKernelGGL(kern, dim3((unsigned)(nblk * B * H)), dim3(8 * 64), lds_bytes, s, a);
+        hipLaunchKernelGGL(kern, dim3((unsigned)(nblk * B * H)), dim3(kDkdvWaves * 64), lds_bytes, s, a);
     } else {
         constexpr int lds_bytes = 2 * dkdv_stage_bytes<2>();
-        auto kern = attn_dkdv_kernel<2, 4>;
+        auto kern = attn_dkdv_kernel<2, 4, 1>;
         const int64_t nkv = (S + 4 * kRowsPerWave - 1) / (4 * kRowsPerWave);
         if (nkv * B * H > INT32_MAX) return fail(CW_ERR_INVALID, "cw_attn_bwd: S or B*H too large");
         hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes);
