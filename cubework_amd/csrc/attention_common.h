@@ -1,5 +1,6 @@
-// Pieces shared by the attention forward and backward kernels (gfx950, head
-// size 64, bf16): LDS tile images, MFMA operand reads, tile loader.
+// Pieces shared by the attention forward and backward kernels (gfx950, bf16):
+// LDS tile images of 64 columns (a head of 128 is two of them side by side),
+// MFMA operand reads, tile loader.
 #pragma once
 
 #include <type_traits>
