@@ -51,3 +51,47 @@ def test_argument_validation_without_a_device():
     assert lib.cw_colsum_workspace_bytes(8192, 2048) >= 512 * 2048 * 4
     with pytest.raises(_lib.CubeworkHipError):
         _lib.check(-1, "example")
+
+
+def test_scratch_sizes_and_refusals_of_the_later_entry_points():
+    """Host-only parts of the entry points added after the first set: scratch sizing and the argument checks
+    that come before any device work."""
+    import ctypes as C
+    from cubework_amd import _lib
+    if not os.path.exists(_lib.LIB_PATH):
+        pytest.skip("libcubework_hip.so not built yet")
+    lib = _lib.load()
+    NN, NT, TN, BF16, F32 = 0, 1, 2, 0, 1
+    # split-k: few tiles, long reduction (config-2 weight gradient: 64 tiles x 4 slices of fp32 partials)
+    assert lib.cw_gemm_workspace_bytes(TN, 2048, 2048, 8192, 2, BF16) == 4 * 2048 * 2048 * 4
+    assert lib.cw_gemm_workspace_bytes(NN, 8192, 2048, 2048, 2, BF16) == 0
+    assert lib.cw_gemm_workspace_bytes(TN, 2048, 2048, 8192, 2, F32) == 0
+    # reduction length that is not a multiple of 32 with B stored [K, N]: 32 rows of B
+    assert lib.cw_gemm_workspace_bytes(NN, 8192, 2048, 12568, 1, BF16) == 32 * 2048 * 2
+    assert lib.cw_gemm_workspace_bytes(TN, 8192, 2048, 12568, 1, BF16) == 32 * 2048 * 2
+    assert lib.cw_gemm_workspace_bytes(NT, 8192, 2048, 12568, 1, BF16) == 0   # B is [N, K]: not provided
+    assert lib.cw_gemm_workspace_bytes(NN, 8192, 2048, 12568, 2, BF16) == 0   # one step only
+    assert lib.cw_gemm_workspace_bytes(NN, 512, 512, 12568, 1, BF16) == 0     # small outputs keep the guarded kernel
+    # token order: direct ranks need no scratch, the sorting network one 64-bit key per padded token
+    assert lib.cw_embed_sort_workspace_bytes(16384) == 0
+    assert lib.cw_embed_sort_workspace_bytes(16385) == 32768 * 8
+    assert lib.cw_embed_sort_ids(-1, None, 0, 8, None, None, None, 0, None) == -1
+    assert lib.cw_embed_sort_ids(4, None, 0, 0, None, None, None, 0, None) == -1
+    assert b"V_loc" in lib.cw_last_error()
+    assert lib.cw_embed_sort_ids(0, None, 0, 8, None, None, None, 0, None) == 0
+    assert lib.cw_embed_sort_ids(20000, None, 0, 8, None, None, None, 0, None) == -1  # null pointers
+    # gradient-norm clipping
+    numels = (C.c_int64 * 3)(65536, 1, 65537)
+    assert lib.cw_multi_norm_workspace_bytes(3, C.cast(numels, C.c_void_p)) == (1 + 1 + 2) * 2 * 4
+    assert lib.cw_clip_coef(0, None, 1.0, 2.0, 1.0, None, None) == -1
+    assert lib.cw_clip_coef(1, None, 1.0, 2.0, 1.0, None, None) == -1
+    # attention: head sizes other than 64 / 128 and dtypes other than bf16 are refused before any launch
+    assert lib.cw_attn_bwd_workspace_bytes(4, 32, 2048) == 4 * 32 * 2048 * 4
+    args = [1, 1, 8, 80, None, None, None, 240, 240, 240, 0.1, 1, None, 80, 80, 80, None, BF16, None]
+    assert lib.cw_attn_fwd(*args) == -3
+    assert b"head size" in lib.cw_last_error()
+    args[3], args[17] = 64, F32
+    assert lib.cw_attn_fwd(*args) == -3
+    # fused LayerNorm backward: the two column outputs come together
+    assert lib.cw_ln_backward_fused(4, 8, None, 8, None, 8, None, None, None, None, 8, None, C.c_void_p(16), None, 0, BF16, None) == -1
+    assert b"both" in lib.cw_last_error()
