@@ -35,6 +35,25 @@ __device__ __forceinline__ int find_tensor(const TensorBatch& b, int block) {
     return t;
 }
 
+// Maximum of absolute values through their bit patterns: for non-negative floats the unsigned order is the
+// float order, +inf sorts above every number and every NaN above +inf, so a NaN gradient makes the maximum
+// NaN, as torch's abs().max() does (fmaxf would drop it).
+__device__ __forceinline__ float abs_max(float a, float b) {
+    const uint32_t ua = __float_as_uint(a) & 0x7fffffffu, ub = __float_as_uint(b) & 0x7fffffffu;
+    return __uint_as_float(ua > ub ? ua : ub);
+}
+__device__ __forceinline__ float wave_abs_max(float v) {
+    v = abs_max(v, dpp_move<kDppXor1>(v));
+    v = abs_max(v, dpp_move<kDppXor2>(v));
+    v = abs_max(v, dpp_move<kDppHalfMirror>(v));
+    v = abs_max(v, dpp_move<kDppMirror>(v));
+    const int iv = __float_as_int(v);
+    float r = __int_as_float(__builtin_amdgcn_readlane(iv, 0));
+    r = abs_max(r, __int_as_float(__builtin_amdgcn_readlane(iv, 16)));
+    r = abs_max(r, __int_as_float(__builtin_amdgcn_readlane(iv, 32)));
+    return abs_max(r, __int_as_float(__builtin_amdgcn_readlane(iv, 48)));
+}
+
 // KIND 0: max |g|;  KIND 2: sum g^2;  KIND 1: sum |g|^p (general p)
 template <typename T, int KIND>
 __global__ __launch_bounds__(kClipThreads) void multi_norm_kernel(const TensorBatch b, float p, float* __restrict__ ws,
@@ -49,7 +68,7 @@ __global__ __launch_bounds__(kClipThreads) void multi_norm_kernel(const TensorBa
     float acc = 0.0f;
     auto add = [&](float x) {
         const float a = fabsf(x);
-        if (KIND == 0) acc = fmaxf(acc, a);
+        if (KIND == 0) acc = abs_max(acc, x);
         else if (KIND == 2) acc = __builtin_fmaf(x, x, acc);
         else acc += __powf(a, p);
     };
@@ -66,13 +85,13 @@ __global__ __launch_bounds__(kClipThreads) void multi_norm_kernel(const TensorBa
     } else {
         for (int64_t i = threadIdx.x; i < len; i += kClipThreads) add(load_elem(g + i));
     }
-    acc = (KIND == 0) ? wave_max(acc) : wave_sum(acc);
+    acc = (KIND == 0) ? wave_abs_max(acc) : wave_sum(acc);
     if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = acc;
     __syncthreads();
     if (threadIdx.x == 0) {
         float r = red[0];
 #pragma unroll
-        for (int w = 1; w < kClipThreads / 64; ++w) r = (KIND == 0) ? fmaxf(r, red[w]) : r + red[w];
+        for (int w = 1; w < kClipThreads / 64; ++w) r = (KIND == 0) ? abs_max(r, red[w]) : r + red[w];
         // the partial and, beside it, the group it belongs to
         ws[2 * (ws_offset + blockIdx.x)] = (KIND == 0) ? r : r * b.factor[t];
         ws[2 * (ws_offset + blockIdx.x) + 1] = (float)b.group[t];
@@ -89,8 +108,8 @@ __global__ __launch_bounds__(256) void norm_finalize_kernel(const float* __restr
         const float v = ws[2 * i];
         const bool tp = ws[2 * i + 1] != 0.0f;
         if (KIND == 0) {
-            a0 = tp ? a0 : fmaxf(a0, v);
-            a1 = tp ? fmaxf(a1, v) : a1;
+            a0 = tp ? a0 : abs_max(a0, v);
+            a1 = tp ? abs_max(a1, v) : a1;
         } else {
             a0 += tp ? 0.0f : v;
             a1 += tp ? v : 0.0f;
@@ -101,7 +120,7 @@ __global__ __launch_bounds__(256) void norm_finalize_kernel(const float* __restr
     __syncthreads();
     if (threadIdx.x < 2) {
         float r = red[threadIdx.x][0];
-        for (int i = 1; i < 256; ++i) r = (KIND == 0) ? fmaxf(r, red[threadIdx.x][i]) : r + red[threadIdx.x][i];
+        for (int i = 1; i < 256; ++i) r = (KIND == 0) ? abs_max(r, red[threadIdx.x][i]) : r + red[threadIdx.x][i];
         out[threadIdx.x] = r;
     }
 }
@@ -139,10 +158,7 @@ __global__ void clip_coef_kernel(const float* __restrict__ sets, int n_sets, flo
     float norm;
     if (__builtin_isinf(norm_type)) {
         norm = 0.0f;
-        for (int i = 0; i < 2 * n_sets; ++i) {
-            const float v = sets[i];
-            norm = (v != v) ? v : fmaxf(norm, v);  // a NaN gradient makes the norm NaN, as torch.max does
-        }
+        for (int i = 0; i < 2 * n_sets; ++i) norm = abs_max(norm, sets[i]);  // NaN-propagating, as torch.max is
     } else {
         float std_sum = 0.0f, tp_sum = 0.0f;
         for (int i = 0; i < n_sets; ++i) {

@@ -109,3 +109,34 @@ def test_clip_grad_norm_with_peer_sums(norm_type):
     assert_parity(a.grad, (ga * coef).float(), torch.float32, "gradient a", scale=10)
     assert_parity(b.grad, (gb * coef).float(), torch.float32, "gradient b", scale=10)
     initialize(None, 1)
+
+
+@pytest.mark.parametrize("norm_type", [2.0, float("inf")])
+@pytest.mark.parametrize("bad", [float("nan"), float("inf")])
+def test_clip_grad_norm_nonfinite_gradients(norm_type, bad):
+    """A NaN or infinite gradient element gives the non-finite total norm torch gives (the maximum norm
+    included: torch's abs().max() propagates NaN), the same scaled gradients, and error_if_nonfinite
+    raises (clip_grad.py:51-57)."""
+    from cubework_amd.clip_grad import clip_grad_norm
+    from cubework_amd.distributed import initialize
+
+    initialize(None, 1)
+    ours = _params([(300, 7), (65,), (70000,)], torch.float32, 3)
+    with torch.no_grad():
+        ours[2].grad[12345] = bad
+    ref = [torch.nn.Parameter(torch.zeros_like(p, device="cpu")) for p in ours]
+    for r, p in zip(ref, ours):
+        r.grad = p.grad.detach().cpu().clone()
+    keep = [p.grad.clone() for p in ours]
+    want = torch.nn.utils.clip_grad_norm_(ref, 1.0, norm_type)
+    got = clip_grad_norm(ours, 1.0, norm_type)
+    torch.cuda.synchronize()
+    assert torch.isnan(got).item() == torch.isnan(want).item() and torch.isinf(got).item() == torch.isinf(want).item()
+    for r, p in zip(ref, ours):
+        assert torch.equal(torch.isnan(p.grad.cpu()), torch.isnan(r.grad))
+        finite = torch.isfinite(r.grad)
+        assert torch.allclose(p.grad.cpu()[finite], r.grad[finite], rtol=1e-5, atol=0)
+    for p, k in zip(ours, keep):
+        p.grad = k
+    with pytest.raises(RuntimeError):
+        clip_grad_norm(ours, 1.0, norm_type, error_if_nonfinite=True)
