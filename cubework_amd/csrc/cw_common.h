@@ -209,7 +209,7 @@ template <int ACT>
 __device__ __forceinline__ float apply_act(float x) {
     if constexpr (ACT == CW_ACT_GELU_TANH) return gelu_tanh(x);
     if constexpr (ACT == CW_ACT_GELU_ERF) return gelu_erf(x);
-    if constexpr (ACT == CW_ACT_RELU) return x > 0.0f ? x : 0.0f;
+    if constexpr (ACT == CW_ACT_RELU) return x < 0.0f ? 0.0f : x;  // NaN stays NaN, as torch.relu leaves it
     return x;
 }
 template <int ACT>

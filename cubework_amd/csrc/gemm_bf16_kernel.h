@@ -184,7 +184,7 @@ template <int EPI>
 __device__ __forceinline__ float epi_act(float x) {
     if constexpr (EPI == CW_EPI_BIAS_GELU_TANH) return gelu_tanh(x);
     if constexpr (EPI == CW_EPI_BIAS_GELU_ERF) return gelu_erf(x);
-    if constexpr (EPI == CW_EPI_BIAS_RELU) return x > 0.0f ? x : 0.0f;
+    if constexpr (EPI == CW_EPI_BIAS_RELU) return x < 0.0f ? 0.0f : x;  // NaN stays NaN, as torch.relu leaves it
     return x;
 }
 

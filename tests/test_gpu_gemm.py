@@ -226,3 +226,23 @@ def test_rejects_bad_arguments():
     lib = _lib.load()
     rc = lib.cw_gemm_ksteps(7, 8, 8, 8, 1, None, 8, None, 8, None, 0, None, 8, None, 0, None, 0, 0, 0, None)
     assert rc < 0 and b"layout" in lib.cw_last_error()
+
+
+@pytest.mark.parametrize("shape", [(64, 128, 64), (4096, 2048, 64)])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+def test_relu_epilogue_keeps_nan(shape, dtype):
+    """torch.relu(NaN) is NaN: a NaN in one row of A reaches exactly that row of the output (register-staged
+    and LDS-DMA kernels, fp32 kernel)."""
+    import oracle
+    from cubework_amd import ops
+
+    M, N, K = shape
+    A = randn((M, K), dtype, 1)
+    B = randn((K, N), dtype, 2, std=0.1)
+    bias = randn((N,), dtype, 3)
+    A[5, 7] = float("nan")
+    want = oracle.gemm_ksteps("NN", [A], [B], bias, "relu")
+    got = ops.gemm_ksteps("NN", [A.cuda()], [B.cuda()], bias.cuda(), "relu").cpu()
+    assert torch.isnan(want[5]).all() and torch.equal(torch.isnan(got), torch.isnan(want))
+    ok = ~torch.isnan(want)
+    assert_parity(got[ok], want[ok], dtype, "relu epilogue beside a NaN row")
