@@ -62,65 +62,145 @@ __global__ __launch_bounds__(256) void zero_rows_kernel(int64_t R, int64_t E, T*
     }
 }
 
-// One block per position i of the sorted order; only the first position of a run of equal ids works.
-// Wavefront w sums tokens i + w, i + w + 4, ... of the run for a slab of 64 x V x NCH columns at a time.
-template <typename T, int NCH>
-__global__ __launch_bounds__(kEmbWaves * 64) void embed_bwd_kernel(int64_t T_rows, int64_t E,
+// One block per position i of the sorted order. A run of fewer than kRunBlocks equal ids is summed by
+// its first block, a column slice per wavefront. The first kRunBlocks positions of a longer run share its
+// work by column slices of 64 vectors (block k takes slices k, k + kRunBlocks, ...); the other positions
+// exit after a few index loads. Inside such a block, wavefront w sums tokens w, w + 8, ... of the run,
+// eight row loads in flight, and finds the run's end as it goes (no scan for the length ahead of the
+// work); the eight sums are added in wavefront order. Everything is a fixed order: bit-reproducible, no atomics. A run of
+// L tokens costs L / 8 row slices per wavefront: token frequencies of real text (one id hundreds of times
+// in a batch) stay in the microseconds.
+constexpr int kRunBlocks = 4;
+constexpr int kRunWaves = 8;
+
+template <typename T>
+__global__ __launch_bounds__(kRunWaves * 64) void embed_bwd_kernel(int64_t T_rows, int64_t E,
                                                                    const int64_t* __restrict__ sorted_ids,
                                                                    const int64_t* __restrict__ order, int64_t vocab_start,
                                                                    int64_t V_loc, int64_t skip_row,
                                                                    const T* __restrict__ d_out, int64_t ldo,
                                                                    T* __restrict__ d_weight, int64_t ldw) {
     constexpr int V = elem<T>::kVec;
-    __shared__ float red[kEmbWaves - 1][NCH * V][64];
+    constexpr int kSlices = 16 / V;      // column slices held in registers at a time: 1024 columns
+    constexpr int kTokens = 8 / kSlices;  // tokens of the run a wavefront loads together
+    __shared__ float red[kRunWaves - 1][kSlices * V][64];
     const int64_t i = blockIdx.x;
     const int64_t id = sorted_ids[i];
-    if (i > 0 && sorted_ids[i - 1] == id) return;
+    // equal predecessors (k) and successors, as far as kRunBlocks - 1 each way: all loads are independent
+    int k = 0, after = 0;
+    bool open = true, open_after = true;
+#pragma unroll
+    for (int j = 1; j < kRunBlocks; ++j) {
+        const bool same = i - j >= 0 && sorted_ids[i - j >= 0 ? i - j : 0] == id;
+        open = open && same;
+        k += open ? 1 : 0;
+        const bool same_after = i + j < T_rows && sorted_ids[i + j < T_rows ? i + j : T_rows - 1] == id;
+        open_after = open_after && same_after;
+        after += open_after ? 1 : 0;
+    }
+    if (k == kRunBlocks - 1 && i - kRunBlocks >= 0 && sorted_ids[i - kRunBlocks] == id) return;  // not among the first
     const int64_t local = id - vocab_start;
     if (local < 0 || local >= V_loc || local == skip_row) return;
-    int64_t run = 1;
-    while (i + run < T_rows && sorted_ids[i + run] == id) ++run;
+    const int sharers = (k + 1 + after) < kRunBlocks ? (k + 1 + after) : kRunBlocks;  // min(run length, kRunBlocks)
+    const int64_t first = i - k;  // first position of the run
 
     const int lane = threadIdx.x & 63;
-    const int wave = threadIdx.x >> 6;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     T* dst = d_weight + local * ldw;
-    for (int64_t col0 = 0; col0 < E; col0 += (int64_t)64 * V * NCH) {
-        float acc[NCH][V];
+    const int64_t slice_cols = (int64_t)64 * V;
+    if (sharers < kRunBlocks) {
+        // A run of one to three tokens (its length is known exactly: sharers), the common case: its first
+        // block does it alone, the wavefronts take a column slice each, no exchange between them.
+        if (k != 0) return;
+        int64_t tok[kRunBlocks - 1];
 #pragma unroll
-        for (int j = 0; j < NCH; ++j)
+        for (int u = 0; u < kRunBlocks - 1; ++u) tok[u] = order[first + u < T_rows ? first + u : T_rows - 1];
+        for (int64_t c = wave * slice_cols + (int64_t)lane * V; c < E; c += kRunWaves * slice_cols) {
+            raw16_t raw[kRunBlocks - 1];
 #pragma unroll
-            for (int e = 0; e < V; ++e) acc[j][e] = 0.0f;
-        for (int64_t r = wave; r < run; r += kEmbWaves) {
-            const T* src = d_out + order[i + r] * ldo + col0;
+            for (int u = 0; u < kRunBlocks - 1; ++u) {
+                raw[u] = raw16_t{0u, 0u, 0u, 0u};
+                if (u < sharers) raw[u] = load_raw_stream(d_out + tok[u] * ldo + c);
+            }
+            float acc[V];
 #pragma unroll
-            for (int j = 0; j < NCH; ++j) {
-                const int64_t c = ((int64_t)j * 64 + lane) * V;
-                if (col0 + c < E) {
-                    float v[V];
-                    unpack_raw(load_raw_stream(src + c), v, (const T*)nullptr);
+            for (int e = 0; e < V; ++e) acc[e] = 0.0f;
 #pragma unroll
-                    for (int e = 0; e < V; ++e) acc[j][e] += v[e];
+            for (int u = 0; u < kRunBlocks - 1; ++u) {
+                float v[V];
+                unpack_raw(raw[u], v, (const T*)nullptr);
+#pragma unroll
+                for (int e = 0; e < V; ++e) acc[e] += v[e];
+            }
+            store_raw_stream(dst + c, pack_raw(acc, (const T*)nullptr));
+        }
+        return;
+    }
+    // this block's slices k, k + sharers, ...: kSlices of them per pass (a run of one token does the whole
+    // row of 4 slices in one pass, as many loads in flight as a longer run has with its tokens)
+    for (int64_t s0 = k; s0 * slice_cols < E; s0 += (int64_t)kSlices * sharers) {
+        int64_t c[kSlices];
+        bool live[kSlices];
+#pragma unroll
+        for (int n = 0; n < kSlices; ++n) {
+            c[n] = (s0 + (int64_t)n * sharers) * slice_cols + (int64_t)lane * V;
+            live[n] = c[n] < E;  // E is a multiple of V on this path
+        }
+        float acc[kSlices][V];
+#pragma unroll
+        for (int n = 0; n < kSlices; ++n)
+#pragma unroll
+            for (int e = 0; e < V; ++e) acc[n][e] = 0.0f;
+        bool more = true;
+        for (int64_t r = first + wave; more; r += kTokens * kRunWaves) {
+            int64_t tok[kTokens];
+            bool in_run[kTokens];
+#pragma unroll
+            for (int u = 0; u < kTokens; ++u) {
+                const int64_t pos = r + u * kRunWaves;
+                const int64_t pc = pos < T_rows ? pos : T_rows - 1;
+                in_run[u] = pos < T_rows && sorted_ids[pc] == id;
+                tok[u] = order[pc];
+            }
+            // positions are the same in all lanes of a wavefront: the branch is a scalar one, and a
+            // wavefront with no token of the run (all but one when the id occurs once) loads nothing
+            raw16_t raw[kTokens][kSlices];
+#pragma unroll
+            for (int u = 0; u < kTokens; ++u) {
+#pragma unroll
+                for (int n = 0; n < kSlices; ++n) raw[u][n] = raw16_t{0u, 0u, 0u, 0u};
+                if (in_run[u]) {
+#pragma unroll
+                    for (int n = 0; n < kSlices; ++n) raw[u][n] = load_raw_stream(d_out + tok[u] * ldo + (live[n] ? c[n] : 0));
                 }
             }
+#pragma unroll
+            for (int u = 0; u < kTokens; ++u)
+#pragma unroll
+                for (int n = 0; n < kSlices; ++n) {
+                    float v[V];
+                    unpack_raw(raw[u][n], v, (const T*)nullptr);
+#pragma unroll
+                    for (int e = 0; e < V; ++e) acc[n][e] += v[e];
+                }
+            more = in_run[kTokens - 1];  // the run is contiguous: once a position is outside it, all later ones are
         }
         if (wave > 0) {
 #pragma unroll
-            for (int j = 0; j < NCH; ++j)
+            for (int n = 0; n < kSlices; ++n)
 #pragma unroll
-                for (int e = 0; e < V; ++e) red[wave - 1][j * V + e][lane] = acc[j][e];
+                for (int e = 0; e < V; ++e) red[wave - 1][n * V + e][lane] = acc[n][e];
         }
         __syncthreads();
         if (wave == 0) {
 #pragma unroll
-            for (int j = 0; j < NCH; ++j) {
-                const int64_t c = ((int64_t)j * 64 + lane) * V;
-                if (col0 + c < E) {
+            for (int n = 0; n < kSlices; ++n) {
+                if (!live[n]) continue;
 #pragma unroll
-                    for (int w = 0; w < kEmbWaves - 1; ++w)
+                for (int w = 0; w < kRunWaves - 1; ++w)
 #pragma unroll
-                        for (int e = 0; e < V; ++e) acc[j][e] += red[w][j * V + e][lane];
-                    store_raw_stream(dst + col0 + c, pack_raw(acc[j], (const T*)nullptr));
-                }
+                    for (int e = 0; e < V; ++e) acc[n][e] += red[w][n * V + e][lane];
+                store_raw_stream(dst + c[n], pack_raw(acc[n], (const T*)nullptr));
             }
         }
         __syncthreads();
@@ -175,12 +255,8 @@ int bwd_impl(int64_t T_rows, int64_t E, const int64_t* sorted_ids, const int64_t
     if (rc != CW_OK || T_rows == 0) return rc;
     const bool vec = w_vec && aligned16(d_out) && ldo % V == 0 && E % V == 0;
     if (vec) {
-        if (E <= 64 * V)
-            hipLaunchKernelGGL((embed_bwd_kernel<T, 1>), dim3((unsigned)T_rows), dim3(kEmbWaves * 64), 0, s, T_rows, E, sorted_ids,
-                               order, vocab_start, V_loc, skip_row, (const T*)d_out, ldo, (T*)d_weight, ldw);
-        else
-            hipLaunchKernelGGL((embed_bwd_kernel<T, 4>), dim3((unsigned)T_rows), dim3(kEmbWaves * 64), 0, s, T_rows, E, sorted_ids,
-                               order, vocab_start, V_loc, skip_row, (const T*)d_out, ldo, (T*)d_weight, ldw);
+        hipLaunchKernelGGL(embed_bwd_kernel<T>, dim3((unsigned)T_rows), dim3(kRunWaves * 64), 0, s, T_rows, E, sorted_ids, order,
+                           vocab_start, V_loc, skip_row, (const T*)d_out, ldo, (T*)d_weight, ldw);
     } else {
         hipLaunchKernelGGL(embed_bwd_generic_kernel<T>, dim3((unsigned)T_rows), dim3(256), 0, s, T_rows, E, sorted_ids, order,
                            vocab_start, V_loc, skip_row, (const T*)d_out, ldo, (T*)d_weight, ldw);

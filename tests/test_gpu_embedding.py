@@ -51,6 +51,26 @@ def test_embedding_forward_backward_parity(case, dtype):
         assert (got_dw.cpu()[untouched] == 0).all(), "rows without tokens are exactly zero"
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("e", [520, 2048, 4104])
+def test_embedding_backward_every_run_length(e, dtype):
+    """Id j occurs j + 1 times (runs of 1 .. 45 tokens in the sorted order, shuffled over the batch): the
+    short-run path, the shared path with its four column-sharing blocks and ragged last slices, and runs
+    that end inside and at the edge of a wavefront's group of tokens all meet the oracle's sums."""
+    import oracle
+    from cubework_amd import ops
+
+    ids = torch.cat([torch.full((j + 1,), 3 + 2 * j, dtype=torch.int64) for j in range(45)])
+    ids = ids[torch.randperm(ids.numel(), generator=torch.Generator().manual_seed(e))]
+    v_loc, start = 100, 0
+    d_out = randn((ids.numel(), e), dtype, 7)
+    want = oracle.vocab_embedding_bwd(ids, d_out, v_loc, start, None)
+    got = ops.embedding_bwd(ids.to(DEV), d_out.to(DEV), v_loc, start, -1)
+    torch.cuda.synchronize()
+    assert_parity(got, want, dtype, "embedding d_weight, runs of 1..45, E=%d" % e)
+    assert (got.cpu()[0:3] == 0).all() and (got.cpu()[4::2][:44] == 0).all(), "rows without tokens are exactly zero"
+
+
 def test_vocab_slices_sum_to_the_full_lookup():
     """Four vocabulary slices: every token is live in exactly one, so the slices' outputs sum (the
     all-reduce of parallel_1d/module.py:454) to F.embedding on the whole table, bit for bit."""
