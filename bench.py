@@ -200,6 +200,15 @@ def bench_other_configs(device, sets):
     us = event_time_us(tn, 50, 10)
     out["gemm_tn_dW_splitk"] = {"us": round(us, 2), "TFLOPs": round(GEMM_FLOP / us / 1e6, 1),
                                 "frac": round(GEMM_FLOP / us / 1e6 / MFMA_BF16_PEAK_TFLOPS, 4)}
+    # config 2's product with float16 operands (what a plain torch.autocast hands the GEMM-type operators):
+    # the same kernel with the other MFMA opcode and conversion
+    a16 = [t.to(torch.float16) for t in sets[0][0]]
+    b16 = [t.to(torch.float16) for t in sets[0][1]]
+    o16 = torch.empty((M, N), dtype=torch.float16, device=device)
+    us = event_time_us(lambda: ops.gemm_ksteps("NN", a16, b16, out=o16), 50, 10)
+    out["gemm_nn_float16"] = {"us": round(us, 2), "TFLOPs": round(GEMM_FLOP / us / 1e6, 1),
+                              "frac": round(GEMM_FLOP / us / 1e6 / MFMA_BF16_PEAK_TFLOPS, 4)}
+    del a16, b16, o16
     # vocabulary-slice classifier of the OPT-1.3B-shaped model (one rank of four: 12568 of 50272 classes):
     # logits = x W^T, and the two gradients. 12568 is not a tile multiple: it is N, M and K in turn.
     xc = _seeded((8192, 2048), 51, 1.0, torch.bfloat16).to(device)

@@ -12,7 +12,7 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.environ.get("CUBEWORK_HIP_LIB") or os.path.join(_HERE, "libcubework_hip.so")
 
 # enums of include/cubework_hip.h
-CW_BF16, CW_F32 = 0, 1
+CW_BF16, CW_F32, CW_F16 = 0, 1, 2
 CW_NN, CW_NT, CW_TN = 0, 1, 2
 CW_EPI_NONE, CW_EPI_BIAS, CW_EPI_BIAS_GELU_TANH, CW_EPI_BIAS_GELU_ERF, CW_EPI_BIAS_RELU = 0, 1, 2, 3, 4
 CW_ACT_NONE, CW_ACT_GELU_TANH, CW_ACT_GELU_ERF, CW_ACT_RELU = 0, 2, 3, 4

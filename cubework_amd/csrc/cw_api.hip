@@ -55,7 +55,7 @@ extern "C" const char* cw_device_arch(void) {
 
 extern "C" int64_t cw_gemm_workspace_bytes(int layout, int64_t M, int64_t N, int64_t K, int n_steps, int io_dtype) {
     if (layout != CW_NN && layout != CW_NT && layout != CW_TN) return 0;
-    if (io_dtype != CW_BF16) return 0;  // the fp32 GEMM is not split
+    if (io_dtype != CW_BF16 && io_dtype != CW_F16) return 0;  // the fp32 GEMM is not split
     const int slices = gemm_bf16_split_slices(M, N, K, n_steps);
     if (slices > 1) return (int64_t)slices * M * N * (int64_t)sizeof(float);
     return gemm_bf16_ktail_workspace_bytes(layout, M, N, K, n_steps);
@@ -78,7 +78,7 @@ extern "C" int cw_gemm_ksteps_ws(int layout, int64_t M, int64_t N, int64_t K, in
         return fail(CW_ERR_INVALID, "cw_gemm_ksteps: bad layout %d", layout);
     if (epilogue < CW_EPI_NONE || epilogue > CW_EPI_BIAS_RELU)
         return fail(CW_ERR_INVALID, "cw_gemm_ksteps: bad epilogue %d", epilogue);
-    if (io_dtype != CW_BF16 && io_dtype != CW_F32)
+    if (io_dtype != CW_BF16 && io_dtype != CW_F32 && io_dtype != CW_F16)
         return fail(CW_ERR_INVALID, "cw_gemm_ksteps: bad io_dtype %d", io_dtype);
     if (M < 0 || N < 0 || K < 0 || M > INT32_MAX || N > INT32_MAX || K > INT32_MAX)
         return fail(CW_ERR_INVALID, "cw_gemm_ksteps: bad shape M=%lld N=%lld K=%lld", (long long)M, (long long)N,
@@ -105,9 +105,9 @@ extern "C" int cw_gemm_ksteps_ws(int layout, int64_t M, int64_t N, int64_t K, in
 
     GemmArgs args;
     memset(&args, 0, sizeof(args));
-    const int vec = (io_dtype == CW_BF16) ? 8 : 4;       // elements per 16 bytes
+    const int vec = (io_dtype == CW_F32) ? 4 : 8;        // elements per 16 bytes
     const uintptr_t out_mask = 15u;                      // outputs / addends move 16 bytes at a time
-    const int out_vec = (io_dtype == CW_BF16) ? 8 : 4;   // elements per 16 bytes
+    const int out_vec = (io_dtype == CW_F32) ? 4 : 8;    // elements per 16 bytes
     args.vec_a = args.vec_b = 1;
     for (int i = 0; i < n_steps; ++i) {
         if (A_steps[i] == nullptr || B_steps[i] == nullptr)
@@ -145,5 +145,6 @@ extern "C" int cw_gemm_ksteps_ws(int layout, int64_t M, int64_t N, int64_t K, in
     args.workspace = workspace_bytes > 0 ? workspace : nullptr;
     args.workspace_bytes = workspace != nullptr ? workspace_bytes : 0;
     hipStream_t s = (hipStream_t)stream;
-    return io_dtype == CW_BF16 ? gemm_bf16_launch(args, layout, epilogue, s) : gemm_f32_launch(args, layout, epilogue, s);
+    return io_dtype == CW_F32 ? gemm_f32_launch(args, layout, epilogue, s)
+                              : gemm_half_launch(args, layout, epilogue, io_dtype == CW_F16, s);
 }

@@ -19,12 +19,21 @@ struct bf16_t {
     uint16_t bits;
 };
 
+// IEEE half precision: what torch's autocast hands the GEMM-type operators by default.
+struct f16_t {
+    uint16_t bits;
+};
+
 template <typename T>
 struct elem;
 
 template <>
 struct elem<bf16_t> {
     static constexpr int kVec = 8;  // elements per 16-byte vector
+};
+template <>
+struct elem<f16_t> {
+    static constexpr int kVec = 8;
 };
 template <>
 struct elem<float> {
@@ -44,6 +53,40 @@ __device__ __forceinline__ uint32_t pack_bf16x2(float lo, float hi) {
     return f32_to_bf16_bits(lo) | (f32_to_bf16_bits(hi) << 16);
 }
 
+// fp16 <-> fp32: v_cvt_f32_f16 is exact, v_cvt_f16_f32 rounds to nearest even (the mode the kernels run in),
+// overflow goes to infinity as torch's conversion does.
+__device__ __forceinline__ float f16_bits_to_f32(uint32_t h) {
+    return static_cast<float>(__builtin_bit_cast(_Float16, static_cast<uint16_t>(h)));
+}
+__device__ __forceinline__ uint32_t f32_to_f16_bits(float f) {
+    return static_cast<uint32_t>(__builtin_bit_cast(uint16_t, static_cast<_Float16>(f)));
+}
+__device__ __forceinline__ uint32_t pack_f16x2(float lo, float hi) {
+    typedef _Float16 half2_t __attribute__((ext_vector_type(2)));
+    const half2_t h = {static_cast<_Float16>(lo), static_cast<_Float16>(hi)};
+    return __builtin_bit_cast(uint32_t, h);
+}
+
+// The two 16-bit element types share every kernel; what differs is the conversion.
+template <typename T>
+struct half_conv;
+template <>
+struct half_conv<bf16_t> {
+    static __device__ __forceinline__ float lo(uint32_t w) { return __uint_as_float(w << 16); }
+    static __device__ __forceinline__ float hi(uint32_t w) { return __uint_as_float(w & 0xffff0000u); }
+    static __device__ __forceinline__ float one(uint32_t bits) { return bf16_bits_to_f32(bits); }
+    static __device__ __forceinline__ uint32_t pack2(float a, float b) { return pack_bf16x2(a, b); }
+};
+template <>
+struct half_conv<f16_t> {
+    static __device__ __forceinline__ float lo(uint32_t w) { return f16_bits_to_f32(w & 0xffffu); }
+    static __device__ __forceinline__ float hi(uint32_t w) { return f16_bits_to_f32(w >> 16); }
+    static __device__ __forceinline__ float one(uint32_t bits) { return f16_bits_to_f32(bits); }
+    static __device__ __forceinline__ uint32_t pack2(float a, float b) { return pack_f16x2(a, b); }
+};
+
+__device__ __forceinline__ float load_elem(const f16_t* p) { return f16_bits_to_f32(p->bits); }
+__device__ __forceinline__ void store_elem(f16_t* p, float v) { p->bits = static_cast<uint16_t>(f32_to_f16_bits(v)); }
 __device__ __forceinline__ float load_elem(const bf16_t* p) { return bf16_bits_to_f32(p->bits); }
 __device__ __forceinline__ float load_elem(const float* p) { return *p; }
 __device__ __forceinline__ void store_elem(bf16_t* p, float v) { p->bits = static_cast<uint16_t>(f32_to_bf16_bits(v)); }
@@ -61,6 +104,23 @@ __device__ __forceinline__ void load_vec(const bf16_t* p, float (&v)[8]) {
     v[5] = __uint_as_float(u.z & 0xffff0000u);
     v[6] = __uint_as_float(u.w << 16);
     v[7] = __uint_as_float(u.w & 0xffff0000u);
+}
+__device__ __forceinline__ void load_vec(const f16_t* p, float (&v)[8]) {
+    const uint4 u = *reinterpret_cast<const uint4*>(p);
+    const uint32_t w[4] = {u.x, u.y, u.z, u.w};
+#pragma unroll
+    for (int d = 0; d < 4; ++d) {
+        v[2 * d] = half_conv<f16_t>::lo(w[d]);
+        v[2 * d + 1] = half_conv<f16_t>::hi(w[d]);
+    }
+}
+__device__ __forceinline__ void store_vec(f16_t* p, const float (&v)[8]) {
+    uint4 u;
+    u.x = pack_f16x2(v[0], v[1]);
+    u.y = pack_f16x2(v[2], v[3]);
+    u.z = pack_f16x2(v[4], v[5]);
+    u.w = pack_f16x2(v[6], v[7]);
+    *reinterpret_cast<uint4*>(p) = u;
 }
 __device__ __forceinline__ void load_vec(const float* p, float (&v)[4]) {
     const float4 u = *reinterpret_cast<const float4*>(p);
@@ -102,6 +162,21 @@ __device__ __forceinline__ void unpack_raw(raw16_t u, float (&v)[8], const bf16_
     v[5] = __uint_as_float(u.z & 0xffff0000u);
     v[6] = __uint_as_float(u.w << 16);
     v[7] = __uint_as_float(u.w & 0xffff0000u);
+}
+__device__ __forceinline__ void unpack_raw(raw16_t u, float (&v)[8], const f16_t*) {
+#pragma unroll
+    for (int d = 0; d < 4; ++d) {
+        v[2 * d] = half_conv<f16_t>::lo(u[d]);
+        v[2 * d + 1] = half_conv<f16_t>::hi(u[d]);
+    }
+}
+__device__ __forceinline__ raw16_t pack_raw(const float (&v)[8], const f16_t*) {
+    raw16_t u;
+    u.x = pack_f16x2(v[0], v[1]);
+    u.y = pack_f16x2(v[2], v[3]);
+    u.z = pack_f16x2(v[4], v[5]);
+    u.w = pack_f16x2(v[6], v[7]);
+    return u;
 }
 __device__ __forceinline__ void unpack_raw(raw16_t u, float (&v)[4], const float*) {
     v[0] = __uint_as_float(u.x);

@@ -208,12 +208,15 @@ extern "C" int64_t cw_colsum_workspace_bytes(int64_t M, int64_t N) {
 extern "C" int cw_colsum(int64_t M, int64_t N, const void* dY, int64_t ld, float* out, void* workspace,
                          int64_t workspace_bytes, int io_dtype, void* stream) {
     if (M < 0 || N <= 0) return fail(CW_ERR_INVALID, "cw_colsum: bad shape M=%lld N=%lld", (long long)M, (long long)N);
-    if (io_dtype != CW_BF16 && io_dtype != CW_F32) return fail(CW_ERR_INVALID, "cw_colsum: bad io_dtype %d", io_dtype);
+    if (io_dtype != CW_BF16 && io_dtype != CW_F32 && io_dtype != CW_F16)
+        return fail(CW_ERR_INVALID, "cw_colsum: bad io_dtype %d", io_dtype);
     if (out == nullptr) return fail(CW_ERR_INVALID, "cw_colsum: out is NULL");
     hipStream_t s = (hipStream_t)stream;
     if (M == 0) return finalize_col_partials(nullptr, 0, N, 1, N, out, nullptr, s);  // zero fill
     if (dY == nullptr || workspace == nullptr || ld < N)
         return fail(CW_ERR_INVALID, "cw_colsum: null pointer or ld < N");
+    if (io_dtype == CW_F16)
+        return colsum_impl<f16_t, 0>(M, N, dY, ld, nullptr, 0, nullptr, 0, 0, out, workspace, workspace_bytes, s);
     return io_dtype == CW_BF16
                ? colsum_impl<bf16_t, 0>(M, N, dY, ld, nullptr, 0, nullptr, 0, 0, out, workspace, workspace_bytes, s)
                : colsum_impl<float, 0>(M, N, dY, ld, nullptr, 0, nullptr, 0, 0, out, workspace, workspace_bytes, s);
@@ -224,7 +227,7 @@ extern "C" int cw_act_bwd_colsum(int activation, int64_t M, int64_t N, const voi
                                  void* workspace, int64_t workspace_bytes, int io_dtype, void* stream) {
     if (M < 0 || N <= 0)
         return fail(CW_ERR_INVALID, "cw_act_bwd_colsum: bad shape M=%lld N=%lld", (long long)M, (long long)N);
-    if (io_dtype != CW_BF16 && io_dtype != CW_F32)
+    if (io_dtype != CW_BF16 && io_dtype != CW_F32 && io_dtype != CW_F16)
         return fail(CW_ERR_INVALID, "cw_act_bwd_colsum: bad io_dtype %d", io_dtype);
     if (activation != CW_ACT_NONE && activation != CW_ACT_GELU_TANH && activation != CW_ACT_GELU_ERF &&
         activation != CW_ACT_RELU)
@@ -238,6 +241,9 @@ extern "C" int cw_act_bwd_colsum(int activation, int64_t M, int64_t N, const voi
         return fail(CW_ERR_INVALID, "cw_act_bwd_colsum: null pointer or leading dimension < N");
     if (dbias != nullptr && workspace == nullptr)
         return fail(CW_ERR_INVALID, "cw_act_bwd_colsum: workspace is NULL");
+    if (io_dtype == CW_F16)
+        return colsum_impl<f16_t, 1>(M, N, dY, ld_dy, preact, ld_pre, dPre, ld_dpre, activation, dbias, workspace,
+                                     workspace_bytes, s);
     return io_dtype == CW_BF16 ? colsum_impl<bf16_t, 1>(M, N, dY, ld_dy, preact, ld_pre, dPre, ld_dpre, activation, dbias,
                                                         workspace, workspace_bytes, s)
                                : colsum_impl<float, 1>(M, N, dY, ld_dy, preact, ld_pre, dPre, ld_dpre, activation, dbias,

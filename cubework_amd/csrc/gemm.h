@@ -1,4 +1,4 @@
-// Kernel argument block shared by the bf16 and fp32 block-GEMM kernels.
+// Kernel argument block shared by the bf16 / fp16 and fp32 block-GEMM kernels.
 #pragma once
 
 #include "cw_common.h"
@@ -50,7 +50,8 @@ int gemm_bf16_split_slices(int64_t M, int64_t N, int64_t K, int n_steps);
 // Scratch for finishing a reduction length that is not a multiple of 32 on the LDS-DMA kernel (0: not used).
 int64_t gemm_bf16_ktail_workspace_bytes(int layout, int64_t M, int64_t N, int64_t K, int n_steps);
 
-int gemm_bf16_launch(const GemmArgs& args, int layout, int epilogue, hipStream_t s);
+// bf16 (f16 = false) or fp16 (f16 = true) operands and outputs
+int gemm_half_launch(const GemmArgs& args, int layout, int epilogue, bool f16, hipStream_t s);
 int gemm_f32_launch(const GemmArgs& args, int layout, int epilogue, hipStream_t s);
 
 }  // namespace cw

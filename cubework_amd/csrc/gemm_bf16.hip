@@ -1,4 +1,4 @@
-// bf16 block GEMM: choice of kernel and tile configuration.
+// bf16 / fp16 block GEMM: choice of kernel and tile configuration (the same for both element types).
 //   - large tile-aligned problems (>= 128 tiles of 256x256, K a multiple of 64,
 //     16-byte aligned rows, at most 4 k-steps and 2 addends): the LDS-DMA
 //     kernel (gemm_bf16_dma.h);
@@ -25,6 +25,14 @@ int gemm_bf16_dma_split_launch_nn(const GemmArgs& args, int slices, hipStream_t 
 int gemm_bf16_dma_split_launch_nt(const GemmArgs& args, int slices, hipStream_t s);
 int gemm_bf16_dma_split_launch_tn(const GemmArgs& args, int slices, hipStream_t s);
 
+int gemm_f16_dma_launch_nn(const GemmArgs& args, int epilogue, hipStream_t s, const void* tail_a, const void* tail_b);
+int gemm_f16_dma_launch_nt(const GemmArgs& args, int epilogue, hipStream_t s, const void* tail_a, const void* tail_b);
+int gemm_f16_dma_launch_tn(const GemmArgs& args, int epilogue, hipStream_t s, const void* tail_a, const void* tail_b);
+
+int gemm_f16_dma_split_launch_nn(const GemmArgs& args, int slices, hipStream_t s);
+int gemm_f16_dma_split_launch_nt(const GemmArgs& args, int slices, hipStream_t s);
+int gemm_f16_dma_split_launch_tn(const GemmArgs& args, int slices, hipStream_t s);
+
 int gemm_bf16_split_slices(int64_t M, int64_t N, int64_t K, int n_steps) {
     if (M <= 0 || N <= 0 || K <= 0 || n_steps <= 0 || n_steps > kRingMaxSteps) return 1;
     if ((M % 256) != 0 || (N % 256) != 0 || (K % 64) != 0) return 1;
@@ -39,13 +47,12 @@ namespace {
 
 // C = epilogue(sum over slices of partial + addends + bias). One thread per 8
 // consecutive columns of a row; slices are added in index order.
-template <int EPI>
+template <int EPI, typename E>
 __global__ __launch_bounds__(256) void splitk_reduce_kernel(const float* __restrict__ partial, int slices, int64_t M,
-                                                            int64_t N, const bf16_t* __restrict__ bias,
-                                                            const bf16_t* __restrict__ add0,
-                                                            const bf16_t* __restrict__ add1, int64_t ldadd,
-                                                            bf16_t* __restrict__ C, int64_t ldc,
-                                                            bf16_t* __restrict__ preact, int64_t ldp) {
+                                                            int64_t N, const E* __restrict__ bias,
+                                                            const E* __restrict__ add0, const E* __restrict__ add1,
+                                                            int64_t ldadd, E* __restrict__ C, int64_t ldc,
+                                                            E* __restrict__ preact, int64_t ldp) {
     const int64_t vec_per_row = N / 8;
     const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
     if (idx >= M * vec_per_row) return;
@@ -66,44 +73,44 @@ __global__ __launch_bounds__(256) void splitk_reduce_kernel(const float* __restr
     }
     float t[8];
     if (EPI != CW_EPI_NONE && bias != nullptr) {
-        unpack_raw(load_raw(bias + col), t, (const bf16_t*)nullptr);
+        unpack_raw(load_raw(bias + col), t, (const E*)nullptr);
 #pragma unroll
         for (int e = 0; e < 8; ++e) v[e] += t[e];
     }
     if (add0 != nullptr) {
-        unpack_raw(load_raw_stream(add0 + row * ldadd + col), t, (const bf16_t*)nullptr);
+        unpack_raw(load_raw_stream(add0 + row * ldadd + col), t, (const E*)nullptr);
 #pragma unroll
         for (int e = 0; e < 8; ++e) v[e] += t[e];
     }
     if (add1 != nullptr) {
-        unpack_raw(load_raw_stream(add1 + row * ldadd + col), t, (const bf16_t*)nullptr);
+        unpack_raw(load_raw_stream(add1 + row * ldadd + col), t, (const E*)nullptr);
 #pragma unroll
         for (int e = 0; e < 8; ++e) v[e] += t[e];
     }
-    if (preact != nullptr) store_raw_stream(preact + row * ldp + col, pack_raw(v, (const bf16_t*)nullptr));
+    if (preact != nullptr) store_raw_stream(preact + row * ldp + col, pack_raw(v, (const E*)nullptr));
 #pragma unroll
     for (int e = 0; e < 8; ++e) v[e] = gemm_bf16::epi_act<EPI>(v[e]);
-    store_raw_stream(C + row * ldc + col, pack_raw(v, (const bf16_t*)nullptr));
+    store_raw_stream(C + row * ldc + col, pack_raw(v, (const E*)nullptr));
 }
 
-template <int EPI>
+template <int EPI, typename E>
 int launch_splitk_reduce(const GemmArgs& a, int slices, hipStream_t s) {
     const int64_t threads = (int64_t)a.M * (a.N / 8);
-    hipLaunchKernelGGL(splitk_reduce_kernel<EPI>, dim3((unsigned)((threads + 255) / 256)), dim3(256), 0, s,
-                       (const float*)a.workspace, slices, (int64_t)a.M, (int64_t)a.N, (const bf16_t*)a.bias,
-                       (const bf16_t*)(a.n_addends > 0 ? a.addend[0] : nullptr),
-                       (const bf16_t*)(a.n_addends > 1 ? a.addend[1] : nullptr), a.ldadd, (bf16_t*)a.C, a.ldc,
-                       (bf16_t*)a.preact, a.ldp);
+    hipLaunchKernelGGL((splitk_reduce_kernel<EPI, E>), dim3((unsigned)((threads + 255) / 256)), dim3(256), 0, s,
+                       (const float*)a.workspace, slices, (int64_t)a.M, (int64_t)a.N, (const E*)a.bias,
+                       (const E*)(a.n_addends > 0 ? a.addend[0] : nullptr),
+                       (const E*)(a.n_addends > 1 ? a.addend[1] : nullptr), a.ldadd, (E*)a.C, a.ldc, (E*)a.preact, a.ldp);
     return check_launch("splitk_reduce_kernel");
 }
 
+template <typename E>
 int splitk_reduce(const GemmArgs& a, int slices, int epilogue, hipStream_t s) {
     switch (epilogue) {
-        case CW_EPI_NONE: return launch_splitk_reduce<CW_EPI_NONE>(a, slices, s);
-        case CW_EPI_BIAS: return launch_splitk_reduce<CW_EPI_BIAS>(a, slices, s);
-        case CW_EPI_BIAS_GELU_TANH: return launch_splitk_reduce<CW_EPI_BIAS_GELU_TANH>(a, slices, s);
-        case CW_EPI_BIAS_GELU_ERF: return launch_splitk_reduce<CW_EPI_BIAS_GELU_ERF>(a, slices, s);
-        case CW_EPI_BIAS_RELU: return launch_splitk_reduce<CW_EPI_BIAS_RELU>(a, slices, s);
+        case CW_EPI_NONE: return launch_splitk_reduce<CW_EPI_NONE, E>(a, slices, s);
+        case CW_EPI_BIAS: return launch_splitk_reduce<CW_EPI_BIAS, E>(a, slices, s);
+        case CW_EPI_BIAS_GELU_TANH: return launch_splitk_reduce<CW_EPI_BIAS_GELU_TANH, E>(a, slices, s);
+        case CW_EPI_BIAS_GELU_ERF: return launch_splitk_reduce<CW_EPI_BIAS_GELU_ERF, E>(a, slices, s);
+        case CW_EPI_BIAS_RELU: return launch_splitk_reduce<CW_EPI_BIAS_RELU, E>(a, slices, s);
         default: return fail(CW_ERR_INVALID, "cw_gemm_ksteps: bad epilogue %d", epilogue);
     }
 }
@@ -140,26 +147,30 @@ static bool dma_kernel_enabled() {
     return enabled;
 }
 
-static int staged_launch(const GemmArgs& a, int layout, int epilogue, bool big, bool exact, hipStream_t s) {
+static int staged_launch(const GemmArgs& a, int layout, int epilogue, bool big, bool exact, bool f16, hipStream_t s) {
     switch (layout) {
-        case CW_NN: return gemm_bf16_launch_nn(a, epilogue, big, exact, s);
-        case CW_NT: return gemm_bf16_launch_nt(a, epilogue, big, exact, s);
-        case CW_TN: return gemm_bf16_launch_tn(a, epilogue, big, exact, s);
+        case CW_NN: return f16 ? gemm_f16_launch_nn(a, epilogue, big, exact, s) : gemm_bf16_launch_nn(a, epilogue, big, exact, s);
+        case CW_NT: return f16 ? gemm_f16_launch_nt(a, epilogue, big, exact, s) : gemm_bf16_launch_nt(a, epilogue, big, exact, s);
+        case CW_TN: return f16 ? gemm_f16_launch_tn(a, epilogue, big, exact, s) : gemm_bf16_launch_tn(a, epilogue, big, exact, s);
         default: return fail(CW_ERR_INVALID, "cw_gemm_ksteps: bad layout %d", layout);
     }
 }
 
-static int dma_launch(const GemmArgs& a, int layout, int epilogue, hipStream_t s, const void* tail_a = nullptr,
+static int dma_launch(const GemmArgs& a, int layout, int epilogue, bool f16, hipStream_t s, const void* tail_a = nullptr,
                       const void* tail_b = nullptr) {
     switch (layout) {
-        case CW_NN: return gemm_bf16_dma_launch_nn(a, epilogue, s, tail_a, tail_b);
-        case CW_NT: return gemm_bf16_dma_launch_nt(a, epilogue, s, tail_a, tail_b);
-        case CW_TN: return gemm_bf16_dma_launch_tn(a, epilogue, s, tail_a, tail_b);
+        case CW_NN:
+            return f16 ? gemm_f16_dma_launch_nn(a, epilogue, s, tail_a, tail_b) : gemm_bf16_dma_launch_nn(a, epilogue, s, tail_a, tail_b);
+        case CW_NT:
+            return f16 ? gemm_f16_dma_launch_nt(a, epilogue, s, tail_a, tail_b) : gemm_bf16_dma_launch_nt(a, epilogue, s, tail_a, tail_b);
+        case CW_TN:
+            return f16 ? gemm_f16_dma_launch_tn(a, epilogue, s, tail_a, tail_b) : gemm_bf16_dma_launch_tn(a, epilogue, s, tail_a, tail_b);
         default: return fail(CW_ERR_INVALID, "cw_gemm_ksteps: bad layout %d", layout);
     }
 }
 
-int gemm_bf16_launch(const GemmArgs& args, int layout, int epilogue, hipStream_t s) {
+// f16: the operands, bias, addends and outputs are IEEE half instead of bfloat16; everything else is shared.
+int gemm_half_launch(const GemmArgs& args, int layout, int epilogue, bool f16, hipStream_t s) {
     // the unguarded kernels address operands with 32-bit byte offsets
     const int64_t max_dim = args.M > args.N ? (args.M > args.K ? args.M : args.K) : (args.N > args.K ? args.N : args.K);
     const bool fits32 = (max_dim + 64) * (args.lda > args.ldb ? args.lda : args.ldb) * 2 < ((int64_t)1 << 32);
@@ -176,7 +187,7 @@ int gemm_bf16_launch(const GemmArgs& args, int layout, int epilogue, hipStream_t
     // full tile in each direction and 16-byte steps wherever a tile origin moves along a contiguous
     // dimension (N always: the output and a [K, N] operand; M for a [K, M] operand).
     const bool edges_ok = args.M >= 256 && args.N >= 256 && (args.N % 8) == 0 && (layout != CW_TN || (args.M % 8) == 0);
-    if (big && all_vec && ring_ok && edges_ok && (args.K % gemm_bf16::kBK) == 0) return dma_launch(args, layout, epilogue, s);
+    if (big && all_vec && ring_ok && edges_ok && (args.K % gemm_bf16::kBK) == 0) return dma_launch(args, layout, epilogue, f16, s);
     // A reduction length that is not a multiple of the k tile (a vocabulary slice as K: 12568 = 392 x 32 +
     // 24), with B stored [K, N]: the regular step covers the first K - K % 32 columns, one more step of 32
     // covers [K-32, K) with a copy of B's last 32 rows whose overlapping rows are zero. The copy (64 bytes
@@ -196,7 +207,7 @@ int gemm_bf16_launch(const GemmArgs& args, int layout, int epilogue, hipStream_t
         const void* tail_a = layout == CW_TN ? a0 + (int64_t)(args.K - 32) * args.lda : a0 + (args.K - 32);
         GemmArgs main_part = args;
         main_part.K = args.K - kr;
-        return dma_launch(main_part, layout, epilogue, s, tail_a, tail_b);
+        return dma_launch(main_part, layout, epilogue, f16, s, tail_a, tail_b);
     }
     const int slices = gemm_bf16_split_slices(args.M, args.N, args.K, args.n_steps);
     if (slices > 1 && all_vec && args.n_addends <= kRingMaxAddends && dma_kernel_enabled() &&
@@ -204,15 +215,15 @@ int gemm_bf16_launch(const GemmArgs& args, int layout, int epilogue, hipStream_t
         args.workspace_bytes >= (int64_t)slices * args.M * args.N * (int64_t)sizeof(float)) {
         int rc;
         switch (layout) {
-            case CW_NN: rc = gemm_bf16_dma_split_launch_nn(args, slices, s); break;
-            case CW_NT: rc = gemm_bf16_dma_split_launch_nt(args, slices, s); break;
-            case CW_TN: rc = gemm_bf16_dma_split_launch_tn(args, slices, s); break;
+            case CW_NN: rc = f16 ? gemm_f16_dma_split_launch_nn(args, slices, s) : gemm_bf16_dma_split_launch_nn(args, slices, s); break;
+            case CW_NT: rc = f16 ? gemm_f16_dma_split_launch_nt(args, slices, s) : gemm_bf16_dma_split_launch_nt(args, slices, s); break;
+            case CW_TN: rc = f16 ? gemm_f16_dma_split_launch_tn(args, slices, s) : gemm_bf16_dma_split_launch_tn(args, slices, s); break;
             default: return fail(CW_ERR_INVALID, "cw_gemm_ksteps: bad layout %d", layout);
         }
         if (rc != CW_OK) return rc;
-        return splitk_reduce(args, slices, epilogue, s);
+        return f16 ? splitk_reduce<f16_t>(args, slices, epilogue, s) : splitk_reduce<bf16_t>(args, slices, epilogue, s);
     }
-    return staged_launch(args, layout, epilogue, big, exact, s);
+    return staged_launch(args, layout, epilogue, big, exact, f16, s);
 }
 
 }  // namespace cw

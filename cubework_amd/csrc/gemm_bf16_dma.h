@@ -1,7 +1,7 @@
 // SUMMA block GEMM for gfx950, large tile-aligned problems.
 //
 //   - 256x256 tile of C per 256-thread block (4 wavefronts, 2x2, 128x128 each =
-//     4x4 v_mfma_f32_32x32x16_bf16 tiles = 256 fp32 accumulators per lane);
+//     4x4 v_mfma_f32_32x32x16_bf16 (E = f16_t: _f16) tiles = 256 fp32 accumulators per lane);
 //   - operands stream global -> LDS through the load unit itself
 //     (global_load_lds_dwordx4): no staging registers, no LDS write
 //     instructions, no transposition ALU work;
@@ -123,7 +123,7 @@ struct FragReader {
 // SPLIT: blockIdx.y selects one of gridDim.y equal slices of every step's k
 // range; the block writes its fp32 partial tile to args.partial and
 // splitk_reduce_kernel finishes the sum and the epilogue.
-template <bool TRANS_A, bool TRANS_B, int EPI, int NS, bool SPLIT>
+template <bool TRANS_A, bool TRANS_B, int EPI, int NS, bool SPLIT, typename E>
 __global__ __launch_bounds__(kThreads) void gemm_bf16_dma_kernel(const RingArgs args) {
     extern __shared__ __attribute__((aligned(16))) uint16_t lds[];
     lds_char* lds_base = (lds_char*)lds;
@@ -261,7 +261,7 @@ __global__ __launch_bounds__(kThreads) void gemm_bf16_dma_kernel(const RingArgs 
             gemm_bf16::static_for<4>([&](auto i) {
                 gemm_bf16::static_for<4>([&](auto j) {
                     constexpr int I = i.value, J = j.value, Q = I * 4 + J;
-                    acc[I][J] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(bfr[0][J], af[0][I], acc[I][J], 0, 0, 0);
+                    acc[I][J] = gemm_bf16::mfma_32x32x16<E>(bfr[0][J], af[0][I], acc[I][J]);
                     if constexpr (Q < 4) af[1][Q] = fa.template read<Q, 1>(sa);
                     else if constexpr (Q < 8) bfr[1][Q - 4] = fb.template read<Q - 4, 1>(sb);
                     else if constexpr ((Q & 1) == 0) dma_one<TRANS_B, (Q - 8) / 2>(is_b, ldb_bytes, is_k0, b_even, b_odd, st + kOperBytes, wave);
@@ -282,7 +282,7 @@ __global__ __launch_bounds__(kThreads) void gemm_bf16_dma_kernel(const RingArgs 
             gemm_bf16::static_for<4>([&](auto i) {
                 gemm_bf16::static_for<4>([&](auto j) {
                     constexpr int I = i.value, J = j.value, Q = I * 4 + J;
-                    acc[I][J] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(bfr[1][J], af[1][I], acc[I][J], 0, 0, 0);
+                    acc[I][J] = gemm_bf16::mfma_32x32x16<E>(bfr[1][J], af[1][I], acc[I][J]);
                     if constexpr (Q < 8 && (Q & 1) == 0) dma_one<TRANS_A, Q / 2>(is_a, lda_bytes, is_k0, a_even, a_odd, st, wave);
                     else if constexpr (Q >= 8 && Q < 12) af[0][Q - 8] = fa.template read<Q - 8, 0>(na);
                     else if constexpr (Q >= 12) bfr[0][Q - 12] = fb.template read<Q - 12, 0>(nb);
@@ -312,7 +312,7 @@ __global__ __launch_bounds__(kThreads) void gemm_bf16_dma_kernel(const RingArgs 
                     *reinterpret_cast<raw16_t*>(part + (int64_t)i * 32 * N + j * 32 + 8 * g) = u;
                 }
     } else {
-        gemm_bf16::gemm_epilogue_slabs<EPI>(acc, args, bias_raw, lds, m0, n0, wm, wn, lane, tid);
+        gemm_bf16::gemm_epilogue_slabs<EPI, E>(acc, args, bias_raw, lds, m0, n0, wm, wn, lane, tid);
     }
 }
 
@@ -338,7 +338,7 @@ inline RingArgs to_ring_args(const GemmArgs& g) {
 
 // tail_a / tail_b != nullptr: the extra short step (k extent kBK) that finishes a reduction length which is
 // not a multiple of the k tile; gargs.K is then the part covered by the regular steps.
-template <bool TA, bool TB, int EPI, int NS>
+template <bool TA, bool TB, int EPI, int NS, typename E>
 int launch_dma_cfg(const GemmArgs& gargs, hipStream_t s, const void* tail_a = nullptr, const void* tail_b = nullptr) {
     RingArgs args = to_ring_args(gargs);
     if (tail_a != nullptr && tail_b != nullptr && gargs.n_steps < kRingMaxSteps) {
@@ -346,7 +346,7 @@ int launch_dma_cfg(const GemmArgs& gargs, hipStream_t s, const void* tail_a = nu
         args.B[gargs.n_steps] = tail_b;
         args.k_tail = kBK;
     }
-    auto kern = gemm_bf16_dma_kernel<TA, TB, EPI, NS, false>;
+    auto kern = gemm_bf16_dma_kernel<TA, TB, EPI, NS, false, E>;
     constexpr size_t lds = lds_bytes_dma<NS>();
     static_assert(lds <= 160 * 1024, "LDS image does not fit the CU");
     hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
@@ -361,11 +361,11 @@ constexpr int kStages = 4;
 
 // Split-k launch: `slices` blocks per output tile, partial sums to the
 // caller's scratch. The epilogue is left to splitk_reduce.
-template <bool TA, bool TB>
+template <bool TA, bool TB, typename E>
 int launch_dma_split(const GemmArgs& gargs, int slices, hipStream_t s) {
     RingArgs args = to_ring_args(gargs);
     args.partial = reinterpret_cast<float*>(gargs.workspace);
-    auto kern = gemm_bf16_dma_kernel<TA, TB, CW_EPI_NONE, kStages, true>;
+    auto kern = gemm_bf16_dma_kernel<TA, TB, CW_EPI_NONE, kStages, true, E>;
     constexpr size_t lds = lds_bytes_dma<kStages>();
     hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
     if (e != hipSuccess) return fail(CW_ERR_LAUNCH, "hipFuncSetAttribute(gemm_bf16_ring, split): %s", hipGetErrorString(e));
@@ -375,14 +375,14 @@ int launch_dma_split(const GemmArgs& gargs, int slices, hipStream_t s) {
     return check_launch("gemm_bf16_dma_kernel (split k)");
 }
 
-template <bool TA, bool TB>
+template <bool TA, bool TB, typename E>
 int launch_dma(const GemmArgs& args, int epilogue, hipStream_t s, const void* tail_a = nullptr, const void* tail_b = nullptr) {
     switch (epilogue) {
-        case CW_EPI_NONE: return launch_dma_cfg<TA, TB, CW_EPI_NONE, kStages>(args, s, tail_a, tail_b);
-        case CW_EPI_BIAS: return launch_dma_cfg<TA, TB, CW_EPI_BIAS, kStages>(args, s, tail_a, tail_b);
-        case CW_EPI_BIAS_GELU_TANH: return launch_dma_cfg<TA, TB, CW_EPI_BIAS_GELU_TANH, kStages>(args, s, tail_a, tail_b);
-        case CW_EPI_BIAS_GELU_ERF: return launch_dma_cfg<TA, TB, CW_EPI_BIAS_GELU_ERF, kStages>(args, s, tail_a, tail_b);
-        case CW_EPI_BIAS_RELU: return launch_dma_cfg<TA, TB, CW_EPI_BIAS_RELU, kStages>(args, s, tail_a, tail_b);
+        case CW_EPI_NONE: return launch_dma_cfg<TA, TB, CW_EPI_NONE, kStages, E>(args, s, tail_a, tail_b);
+        case CW_EPI_BIAS: return launch_dma_cfg<TA, TB, CW_EPI_BIAS, kStages, E>(args, s, tail_a, tail_b);
+        case CW_EPI_BIAS_GELU_TANH: return launch_dma_cfg<TA, TB, CW_EPI_BIAS_GELU_TANH, kStages, E>(args, s, tail_a, tail_b);
+        case CW_EPI_BIAS_GELU_ERF: return launch_dma_cfg<TA, TB, CW_EPI_BIAS_GELU_ERF, kStages, E>(args, s, tail_a, tail_b);
+        case CW_EPI_BIAS_RELU: return launch_dma_cfg<TA, TB, CW_EPI_BIAS_RELU, kStages, E>(args, s, tail_a, tail_b);
         default: return fail(CW_ERR_INVALID, "cw_gemm_ksteps: bad epilogue %d", epilogue);
     }
 }

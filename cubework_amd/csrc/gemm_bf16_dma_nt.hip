@@ -4,11 +4,11 @@
 namespace cw {
 
 int gemm_bf16_dma_launch_nt(const GemmArgs& args, int epilogue, hipStream_t s, const void* tail_a, const void* tail_b) {
-    return gemm_dma::launch_dma<false, false>(args, epilogue, s, tail_a, tail_b);
+    return gemm_dma::launch_dma<false, false, bf16_t>(args, epilogue, s, tail_a, tail_b);
 }
 
 int gemm_bf16_dma_split_launch_nt(const GemmArgs& args, int slices, hipStream_t s) {
-    return gemm_dma::launch_dma_split<false, false>(args, slices, s);
+    return gemm_dma::launch_dma_split<false, false, bf16_t>(args, slices, s);
 }
 
 }  // namespace cw

@@ -4,11 +4,11 @@
 namespace cw {
 
 int gemm_bf16_dma_launch_tn(const GemmArgs& args, int epilogue, hipStream_t s, const void* tail_a, const void* tail_b) {
-    return gemm_dma::launch_dma<true, true>(args, epilogue, s, tail_a, tail_b);
+    return gemm_dma::launch_dma<true, true, bf16_t>(args, epilogue, s, tail_a, tail_b);
 }
 
 int gemm_bf16_dma_split_launch_tn(const GemmArgs& args, int slices, hipStream_t s) {
-    return gemm_dma::launch_dma_split<true, true>(args, slices, s);
+    return gemm_dma::launch_dma_split<true, true, bf16_t>(args, slices, s);
 }
 
 }  // namespace cw

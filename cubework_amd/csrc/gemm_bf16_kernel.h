@@ -1,5 +1,6 @@
 // SUMMA block GEMM for gfx950: C = act(sum_i op(A_i) op(B_i) + addends + bias),
-// bf16 operands, fp32 accumulation in v_mfma_f32_32x32x16_bf16.
+// 16-bit operands (bf16, or fp16 with E = f16_t: the same kernels, another MFMA opcode and conversion),
+// fp32 accumulation in v_mfma_f32_32x32x16_bf16 / _f16.
 //
 // Shape of the kernel
 //   - one 256-thread block (4 wavefronts, 2x2) per BM x BN tile of C; a
@@ -40,6 +41,16 @@ typedef float f32x16_t __attribute__((ext_vector_type(16)));
 // address spaces become memcpy calls that keep the array in scratch memory.
 typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
 typedef uint32_t u32x2_t __attribute__((ext_vector_type(2)));
+typedef _Float16 f16x8_t __attribute__((ext_vector_type(8)));
+
+// acc += a b for the element type E; fragments travel as 8 x 16 bits whatever the type.
+template <typename E>
+__device__ __forceinline__ f32x16_t mfma_32x32x16(bf16x8_t a, bf16x8_t b, f32x16_t acc) {
+    if constexpr (std::is_same<E, f16_t>::value)
+        return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8_t, a), __builtin_bit_cast(f16x8_t, b), acc, 0, 0, 0);
+    else
+        return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, acc, 0, 0, 0);
+}
 
 // Compile-time loop: f(std::integral_constant<int, I>) for I in [0, N).
 template <int... Is, typename F>
@@ -188,16 +199,17 @@ __device__ __forceinline__ float epi_act(float x) {
     return x;
 }
 
-__device__ __forceinline__ void load4_bf16(const uint16_t* __restrict__ p, int n_valid, bool vec_ok, float (&v)[4]) {
+template <typename E>
+__device__ __forceinline__ void load4_half(const uint16_t* __restrict__ p, int n_valid, bool vec_ok, float (&v)[4]) {
     if (vec_ok && n_valid >= 4) {
         const u32x2_t u = *reinterpret_cast<const u32x2_t*>(p);
-        v[0] = __uint_as_float(u.x << 16);
-        v[1] = __uint_as_float(u.x & 0xffff0000u);
-        v[2] = __uint_as_float(u.y << 16);
-        v[3] = __uint_as_float(u.y & 0xffff0000u);
+        v[0] = half_conv<E>::lo(u.x);
+        v[1] = half_conv<E>::hi(u.x);
+        v[2] = half_conv<E>::lo(u.y);
+        v[3] = half_conv<E>::hi(u.y);
     } else {
 #pragma unroll
-        for (int e = 0; e < 4; ++e) v[e] = e < n_valid ? bf16_bits_to_f32(p[e]) : 0.0f;
+        for (int e = 0; e < 4; ++e) v[e] = e < n_valid ? half_conv<E>::one(p[e]) : 0.0f;
     }
 }
 
@@ -257,7 +269,7 @@ __device__ __forceinline__ void tile_store(const uint16_t* __restrict__ lds_c, u
 //               col  n = n0 + wn*(BN/2) + j*32 + 8*(v/4) + 4*(lane>>5) + (v%4)
 // FAST: the tile is entirely in bounds and every pointer / leading dimension
 // allows the vector accesses (checked on the host): no per-element guards.
-template <int BM, int BN, int TM, int TN, int EPI, bool FAST, typename Args>
+template <int BM, int BN, int TM, int TN, int EPI, bool FAST, typename E, typename Args>
 __device__ __forceinline__ void gemm_epilogue(f32x16_t (&acc)[TM][TN], const Args& args, uint16_t* lds, int m0,
                                               int n0, int wm, int wn, int lane, int tid) {
     constexpr int WTM = BM / 2, WTN = BN / 2;
@@ -278,7 +290,7 @@ __device__ __forceinline__ void gemm_epilogue(f32x16_t (&acc)[TM][TN], const Arg
             for (int g = 0; g < 4; ++g) {
                 const int ncol = n0 + col_l + j * 32 + 8 * g;
                 if (use_bias && (FAST || ncol < N)) {
-                    load4_bf16(bias + ncol, FAST ? 4 : N - ncol, FAST || args.vec_bias != 0, bv[g]);
+                    load4_half<E>(bias + ncol, FAST ? 4 : N - ncol, FAST || args.vec_bias != 0, bv[g]);
                 } else {
 #pragma unroll
                     for (int e = 0; e < 4; ++e) bv[g][e] = 0.0f;
@@ -297,8 +309,8 @@ __device__ __forceinline__ void gemm_epilogue(f32x16_t (&acc)[TM][TN], const Arg
 #pragma unroll 1
                         for (int a = 0; a < args.n_addends; ++a) {
                             float t[4];
-                            load4_bf16(reinterpret_cast<const uint16_t*>(pick_ptr(args.addend, a)) + (int64_t)mrow * args.ldadd + ncol,
-                                       FAST ? 4 : N - ncol, FAST || args.vec_add != 0, t);
+                            load4_half<E>(reinterpret_cast<const uint16_t*>(pick_ptr(args.addend, a)) + (int64_t)mrow * args.ldadd + ncol,
+                                          FAST ? 4 : N - ncol, FAST || args.vec_add != 0, t);
 #pragma unroll
                             for (int e = 0; e < 4; ++e) v[e] += t[e];
                         }
@@ -308,8 +320,8 @@ __device__ __forceinline__ void gemm_epilogue(f32x16_t (&acc)[TM][TN], const Arg
                         for (int e = 0; e < 4; ++e) v[e] = epi_act<EPI>(v[e]);
                     }
                     u32x2_t p;
-                    p.x = pack_bf16x2(v[0], v[1]);
-                    p.y = pack_bf16x2(v[2], v[3]);
+                    p.x = half_conv<E>::pack2(v[0], v[1]);
+                    p.y = half_conv<E>::pack2(v[2], v[3]);
                     *reinterpret_cast<u32x2_t*>(lds_c + (row_l + i * 32) * CP + col_l + j * 32 + 8 * g) = p;
                 }
             }
@@ -334,7 +346,7 @@ __device__ __forceinline__ void gemm_epilogue(f32x16_t (&acc)[TM][TN], const Arg
 // is enough: a buffer is rewritten two slabs after it was read.
 // bias_raw[j][g]: the lane's 4 bias values (bf16 pairs) for accumulator
 // columns j*32 + 8g .. +3, loaded by the caller ahead of the k loop.
-template <int EPI, typename Args>
+template <int EPI, typename E, typename Args>
 __device__ __forceinline__ void gemm_epilogue_slabs(f32x16_t (&acc)[4][4], const Args& args,
                                                     const u32x2_t (&bias_raw)[4][4], uint16_t* lds, int m0, int n0,
                                                     int wm, int wn, int lane, int tid) {
@@ -355,17 +367,17 @@ __device__ __forceinline__ void gemm_epilogue_slabs(f32x16_t (&acc)[4][4], const
             for (int g = 0; g < 4; ++g) {
                 const u32x2_t b = bias_raw[j][g];
                 float v[4];
-                v[0] = acc[I][j][4 * g] + __uint_as_float(b.x << 16);
-                v[1] = acc[I][j][4 * g + 1] + __uint_as_float(b.x & 0xffff0000u);
-                v[2] = acc[I][j][4 * g + 2] + __uint_as_float(b.y << 16);
-                v[3] = acc[I][j][4 * g + 3] + __uint_as_float(b.y & 0xffff0000u);
+                v[0] = acc[I][j][4 * g] + half_conv<E>::lo(b.x);
+                v[1] = acc[I][j][4 * g + 1] + half_conv<E>::hi(b.x);
+                v[2] = acc[I][j][4 * g + 2] + half_conv<E>::lo(b.y);
+                v[3] = acc[I][j][4 * g + 3] + half_conv<E>::hi(b.y);
                 if (args.n_addends > 0) {
                     const int ncol = n0 + col_l + j * 32 + 8 * g;
 #pragma unroll 1
                     for (int a = 0; a < args.n_addends; ++a) {
                         float t[4];
-                        load4_bf16(reinterpret_cast<const uint16_t*>(pick_ptr(args.addend, a)) + (int64_t)mrow * args.ldadd + ncol,
-                                   4, true, t);
+                        load4_half<E>(reinterpret_cast<const uint16_t*>(pick_ptr(args.addend, a)) + (int64_t)mrow * args.ldadd + ncol,
+                                      4, true, t);
 #pragma unroll
                         for (int e = 0; e < 4; ++e) v[e] += t[e];
                     }
@@ -375,8 +387,8 @@ __device__ __forceinline__ void gemm_epilogue_slabs(f32x16_t (&acc)[4][4], const
                     for (int e = 0; e < 4; ++e) v[e] = epi_act<EPI>(v[e]);
                 }
                 u32x2_t p;
-                p.x = pack_bf16x2(v[0], v[1]);
-                p.y = pack_bf16x2(v[2], v[3]);
+                p.x = half_conv<E>::pack2(v[0], v[1]);
+                p.y = half_conv<E>::pack2(v[2], v[3]);
                 *reinterpret_cast<u32x2_t*>(dst + j * 32 + 8 * g) = p;
             }
         }
@@ -407,7 +419,7 @@ __device__ __forceinline__ void gemm_epilogue_slabs(f32x16_t (&acc)[4][4], const
     });
 }
 
-template <int BM, int BN, bool TRANS_A, bool TRANS_B, bool GUARD, int EPI>
+template <int BM, int BN, bool TRANS_A, bool TRANS_B, bool GUARD, int EPI, typename E>
 __global__ __launch_bounds__(kThreads) void gemm_bf16_kernel(const GemmArgs args) {
     constexpr int WTM = BM / 2, WTN = BN / 2;  // wavefront sub-tile
     constexpr int TM = WTM / 32, TN = WTN / 32;
@@ -514,13 +526,13 @@ __global__ __launch_bounds__(kThreads) void gemm_bf16_kernel(const GemmArgs args
             for (int i = 0; i < TM; ++i)
 #pragma unroll
                 for (int j = 0; j < TN; ++j)
-                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(bfr[ks & 1][j], af[ks & 1][i], acc[i][j], 0, 0, 0);
+                    acc[i][j] = mfma_32x32x16<E>(bfr[ks & 1][j], af[ks & 1][i], acc[i][j]);
         }
         if (kt + 1 < KT) commit_loads(cur ^ 1);
         __syncthreads();
     }
 
-    gemm_epilogue<BM, BN, TM, TN, EPI, !GUARD>(acc, args, lds, m0, n0, wm, wn, lane, tid);
+    gemm_epilogue<BM, BN, TM, TN, EPI, !GUARD, E>(acc, args, lds, m0, n0, wm, wn, lane, tid);
 }
 
 template <int BM, int BN>
@@ -530,9 +542,9 @@ constexpr size_t lds_bytes() {
     return stages > ctile ? stages : ctile;
 }
 
-template <int BM, int BN, bool TA, bool TB, bool GUARD, int EPI>
+template <int BM, int BN, bool TA, bool TB, bool GUARD, int EPI, typename E>
 int launch_cfg(const GemmArgs& args, hipStream_t s) {
-    auto kern = gemm_bf16_kernel<BM, BN, TA, TB, GUARD, EPI>;
+    auto kern = gemm_bf16_kernel<BM, BN, TA, TB, GUARD, EPI, E>;
     constexpr size_t lds = lds_bytes<BM, BN>();
     static_assert(lds <= 160 * 1024, "LDS tile does not fit the CU");
     if (lds > 48 * 1024) {
@@ -545,34 +557,37 @@ int launch_cfg(const GemmArgs& args, hipStream_t s) {
     return check_launch("gemm_bf16_kernel");
 }
 
-template <int BM, int BN, bool TA, bool TB, bool GUARD>
+template <int BM, int BN, bool TA, bool TB, bool GUARD, typename E>
 int launch_epi(const GemmArgs& args, int epilogue, hipStream_t s) {
     switch (epilogue) {
-        case CW_EPI_NONE: return launch_cfg<BM, BN, TA, TB, GUARD, CW_EPI_NONE>(args, s);
-        case CW_EPI_BIAS: return launch_cfg<BM, BN, TA, TB, GUARD, CW_EPI_BIAS>(args, s);
-        case CW_EPI_BIAS_GELU_TANH: return launch_cfg<BM, BN, TA, TB, GUARD, CW_EPI_BIAS_GELU_TANH>(args, s);
-        case CW_EPI_BIAS_GELU_ERF: return launch_cfg<BM, BN, TA, TB, GUARD, CW_EPI_BIAS_GELU_ERF>(args, s);
-        case CW_EPI_BIAS_RELU: return launch_cfg<BM, BN, TA, TB, GUARD, CW_EPI_BIAS_RELU>(args, s);
+        case CW_EPI_NONE: return launch_cfg<BM, BN, TA, TB, GUARD, CW_EPI_NONE, E>(args, s);
+        case CW_EPI_BIAS: return launch_cfg<BM, BN, TA, TB, GUARD, CW_EPI_BIAS, E>(args, s);
+        case CW_EPI_BIAS_GELU_TANH: return launch_cfg<BM, BN, TA, TB, GUARD, CW_EPI_BIAS_GELU_TANH, E>(args, s);
+        case CW_EPI_BIAS_GELU_ERF: return launch_cfg<BM, BN, TA, TB, GUARD, CW_EPI_BIAS_GELU_ERF, E>(args, s);
+        case CW_EPI_BIAS_RELU: return launch_cfg<BM, BN, TA, TB, GUARD, CW_EPI_BIAS_RELU, E>(args, s);
         default: return fail(CW_ERR_INVALID, "cw_gemm_ksteps: bad epilogue %d", epilogue);
     }
 }
 
 // All tile configurations of one operand orientation. `big` selects 256x256
 // tiles, `exact` the unguarded kernels (tile-multiple, 16-byte aligned shapes).
-template <bool TA, bool TB>
+template <bool TA, bool TB, typename E>
 int launch_orientation(const GemmArgs& args, int epilogue, bool big, bool exact, hipStream_t s) {
     if (big)
-        return exact ? launch_epi<256, 256, TA, TB, false>(args, epilogue, s)
-                     : launch_epi<256, 256, TA, TB, true>(args, epilogue, s);
-    return exact ? launch_epi<128, 128, TA, TB, false>(args, epilogue, s)
-                 : launch_epi<128, 128, TA, TB, true>(args, epilogue, s);
+        return exact ? launch_epi<256, 256, TA, TB, false, E>(args, epilogue, s)
+                     : launch_epi<256, 256, TA, TB, true, E>(args, epilogue, s);
+    return exact ? launch_epi<128, 128, TA, TB, false, E>(args, epilogue, s)
+                 : launch_epi<128, 128, TA, TB, true, E>(args, epilogue, s);
 }
 
 }  // namespace gemm_bf16
 
-// One translation unit per orientation (gemm_bf16_nn/nt/tn.hip).
+// One translation unit per orientation and element type (gemm_bf16_nn/nt/tn.hip, gemm_f16_nn/nt/tn.hip).
 int gemm_bf16_launch_nn(const GemmArgs& args, int epilogue, bool big, bool exact, hipStream_t s);
 int gemm_bf16_launch_nt(const GemmArgs& args, int epilogue, bool big, bool exact, hipStream_t s);
 int gemm_bf16_launch_tn(const GemmArgs& args, int epilogue, bool big, bool exact, hipStream_t s);
+int gemm_f16_launch_nn(const GemmArgs& args, int epilogue, bool big, bool exact, hipStream_t s);
+int gemm_f16_launch_nt(const GemmArgs& args, int epilogue, bool big, bool exact, hipStream_t s);
+int gemm_f16_launch_tn(const GemmArgs& args, int epilogue, bool big, bool exact, hipStream_t s);
 
 }  // namespace cw

@@ -4,7 +4,7 @@
 namespace cw {
 
 int gemm_bf16_launch_nn(const GemmArgs& args, int epilogue, bool big, bool exact, hipStream_t s) {
-    return gemm_bf16::launch_orientation<false, true>(args, epilogue, big, exact, s);
+    return gemm_bf16::launch_orientation<false, true, bf16_t>(args, epilogue, big, exact, s);
 }
 
 }  // namespace cw

@@ -4,7 +4,7 @@
 namespace cw {
 
 int gemm_bf16_launch_nt(const GemmArgs& args, int epilogue, bool big, bool exact, hipStream_t s) {
-    return gemm_bf16::launch_orientation<false, false>(args, epilogue, big, exact, s);
+    return gemm_bf16::launch_orientation<false, false, bf16_t>(args, epilogue, big, exact, s);
 }
 
 }  // namespace cw

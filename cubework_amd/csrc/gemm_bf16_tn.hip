@@ -4,7 +4,7 @@
 namespace cw {
 
 int gemm_bf16_launch_tn(const GemmArgs& args, int epilogue, bool big, bool exact, hipStream_t s) {
-    return gemm_bf16::launch_orientation<true, true>(args, epilogue, big, exact, s);
+    return gemm_bf16::launch_orientation<true, true, bf16_t>(args, epilogue, big, exact, s);
 }
 
 }  // namespace cw

@@ -3,14 +3,35 @@
 The reference wraps its GEMM-type Functions in custom_fwd(cast_inputs=float16)
 and its LayerNorm / loss Functions in custom_fwd(cast_inputs=float32)
 (cubework/module/parallel_2d/_operation.py:17,96,176,255,309,363;
-cubework/module/loss/loss_1d.py:13). The MI355X kernels take bf16 and fp32,
-so inside an autocast region GEMM-type operators cast to bfloat16; outside
-autocast nothing is cast, as in the reference.
+cubework/module/loss/loss_1d.py:13). Here the GEMM-type operators cast to the
+dtype the autocast region was opened with: float16 under a plain
+torch.autocast("cuda") / torch.cuda.amp.autocast(), which is what the
+reference's training scripts use (benchmark/opt/train.py:85-86) and so gives
+the reference's dtype, and bfloat16 under torch.autocast("cuda",
+dtype=torch.bfloat16), where the reference would still cast to float16.
+Outside autocast nothing is cast, as in the reference.
 """
 import functools
 
 import torch
 
-gemm_fwd = functools.partial(torch.amp.custom_fwd, device_type="cuda", cast_inputs=torch.bfloat16)
+_GEMM_CAST_DTYPES = (torch.float16, torch.bfloat16)
+
+
+def gemm_fwd():
+    """custom_fwd whose cast_inputs follows the autocast dtype (float16 unless the region asks for bfloat16)."""
+    def decorate(fwd):
+        variants = {dt: torch.amp.custom_fwd(fwd, device_type="cuda", cast_inputs=dt) for dt in _GEMM_CAST_DTYPES}
+
+        @functools.wraps(fwd)
+        def wrapper(*args, **kwargs):
+            dt = torch.float16
+            if torch.is_autocast_enabled("cuda") and torch.get_autocast_dtype("cuda") in variants:
+                dt = torch.get_autocast_dtype("cuda")
+            return variants[dt](*args, **kwargs)
+        return wrapper
+    return decorate
+
+
 fp32_fwd = functools.partial(torch.amp.custom_fwd, device_type="cuda", cast_inputs=torch.float32)
 bwd = functools.partial(torch.amp.custom_bwd, device_type="cuda")

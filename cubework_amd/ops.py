@@ -2,8 +2,10 @@
 (device memory and streams are torch's; the arithmetic is the HIP library's),
 pass raw pointers and the current stream.
 
-Every function requires CUDA (ROCm) tensors of dtype bfloat16 or float32 and
-raises instead of falling back to torch arithmetic.
+Every function requires CUDA (ROCm) tensors of dtype bfloat16 or float32 (the
+GEMM and column-sum wrappers also take float16, the type autocast hands the
+GEMM-type operators by default) and raises instead of falling back to torch
+arithmetic.
 """
 import ctypes
 from typing import Optional, Sequence, Tuple
@@ -11,7 +13,7 @@ from typing import Optional, Sequence, Tuple
 import torch
 
 from . import _lib
-from ._lib import (CW_ACT_GELU_ERF, CW_ACT_GELU_TANH, CW_ACT_NONE, CW_ACT_RELU, CW_BF16, CW_EPI_BIAS,
+from ._lib import (CW_ACT_GELU_ERF, CW_ACT_GELU_TANH, CW_ACT_NONE, CW_ACT_RELU, CW_BF16, CW_F16, CW_EPI_BIAS,
                    CW_EPI_BIAS_GELU_ERF, CW_EPI_BIAS_GELU_TANH, CW_EPI_BIAS_RELU, CW_EPI_NONE, CW_F32, CW_LN_ONE_PASS,
                    CW_LN_TWO_PASS, CW_NN, CW_NT, CW_TN)
 
@@ -28,12 +30,15 @@ def epilogue_code(has_bias: bool, activation: Optional[str]) -> int:
             CW_ACT_RELU: CW_EPI_BIAS_RELU}[act]
 
 
-def _dtype_code(t: torch.Tensor) -> int:
+def _dtype_code(t: torch.Tensor, half_ok: bool = False) -> int:
     if t.dtype == torch.bfloat16:
         return CW_BF16
     if t.dtype == torch.float32:
         return CW_F32
-    raise TypeError("cubework_amd kernels take bfloat16 or float32 tensors, got %s" % t.dtype)
+    if t.dtype == torch.float16 and half_ok:
+        return CW_F16
+    raise TypeError("this cubework_amd kernel takes %s tensors, got %s"
+                    % ("bfloat16, float16 or float32" if half_ok else "bfloat16 or float32", t.dtype))
 
 
 def _require_device(*tensors):
@@ -90,7 +95,7 @@ def gemm_ksteps(layout: str, A_steps: Sequence[torch.Tensor], B_steps: Sequence[
     B_steps = [_rows(b) for b in B_steps]
     _require_device(*A_steps, *B_steps, bias, *addends)
     a0, b0 = A_steps[0], B_steps[0]
-    dt = _dtype_code(a0)
+    dt = _dtype_code(a0, half_ok=True)
     if layout == "NN":
         M, K, N, Kb = a0.shape[0], a0.shape[1], b0.shape[1], b0.shape[0]
     elif layout == "NT":
@@ -152,7 +157,7 @@ def bias_act(x: torch.Tensor, bias: Optional[torch.Tensor], activation: Optional
     out = torch.empty((M, N), dtype=x2.dtype, device=x2.device)
     tadd = _ptr_table([x2])
     rc = lib.cw_gemm_ksteps(CW_NN, M, N, 0, 0, None, 0, None, 0, _p(bias), epilogue_code(bias is not None, activation),
-                            _p(out), _ld(out), None, 0, tadd, 1, _ld(x2), _dtype_code(x2), _stream())
+                            _p(out), _ld(out), None, 0, tadd, 1, _ld(x2), _dtype_code(x2, half_ok=True), _stream())
     _lib.check(rc, "cw_gemm_ksteps (bias/activation only)")
     return out.reshape(shape)
 
@@ -170,7 +175,7 @@ def colsum(dy: torch.Tensor) -> torch.Tensor:
     M, N = dy.shape
     out = torch.empty(N, dtype=torch.float32, device=dy.device)
     ws = _workspace(M, N, dy.device)
-    rc = lib.cw_colsum(M, N, _p(dy), _ld(dy), _p(out), _p(ws), ws.numel(), _dtype_code(dy), _stream())
+    rc = lib.cw_colsum(M, N, _p(dy), _ld(dy), _p(out), _p(ws), ws.numel(), _dtype_code(dy, half_ok=True), _stream())
     _lib.check(rc, "cw_colsum")
     return out
 
@@ -188,8 +193,8 @@ def act_bwd_colsum(activation: Optional[str], dy: torch.Tensor, preact: torch.Te
     dbias = torch.empty(N, dtype=torch.float32, device=dy.device) if want_dbias else None
     ws = _workspace(M, N, dy.device) if want_dbias else None
     rc = lib.cw_act_bwd_colsum(ACTIVATIONS[activation], M, N, _p(dy), _ld(dy), _p(preact), _ld(preact), _p(dpre),
-                               _ld(dpre), _p(dbias), _p(ws), ws.numel() if ws is not None else 0, _dtype_code(dy),
-                               _stream())
+                               _ld(dpre), _p(dbias), _p(ws), ws.numel() if ws is not None else 0,
+                               _dtype_code(dy, half_ok=True), _stream())
     _lib.check(rc, "cw_act_bwd_colsum")
     return dpre, dbias
 

@@ -17,7 +17,8 @@
  *   - re-entrant and callable from any thread (the autograd engine calls the
  *     backward entry points from its own device thread);
  *   - io_dtype selects the storage type of activations/weights (CW_BF16 or
- *     CW_F32); statistics, losses and all accumulation are fp32.
+ *     CW_F32; CW_F16 where an entry point says so); statistics, losses and all
+ *     accumulation are fp32.
  *
  * Citations name the reference code (kurisusnowdeng/Cubework) each entry
  * point stands in for; paths are relative to the reference tree.
@@ -40,7 +41,12 @@ typedef enum {
     CW_ERR_DEVICE = -5       /* current device is not gfx950             */
 } cw_status;
 
-typedef enum { CW_BF16 = 0, CW_F32 = 1 } cw_dtype;
+/* CW_F16 (IEEE half, the type the reference's GEMM-type Functions cast to under autocast:
+ * custom_fwd(cast_inputs=torch.float16), cubework/module/parallel_2d/_operation.py:17,96,176,255,363) is
+ * taken by the GEMM and column-sum entry points only (cw_gemm_ksteps, cw_gemm_ksteps_ws, cw_colsum,
+ * cw_act_bwd_colsum): the reference runs LayerNorm and the loss in fp32 under autocast, and so do their
+ * entry points here. */
+typedef enum { CW_BF16 = 0, CW_F32 = 1, CW_F16 = 2 } cw_dtype;
 
 /* Operand orientation of the block GEMM, per k-step i:
  *   CW_NN: C[M,N] += A_i[M,K] * B_i[K,N]      (summa_AB,  Linear2D/3D forward)

@@ -222,7 +222,9 @@ def test_rejects_bad_arguments():
     with pytest.raises(RuntimeError):
         ops.gemm_ksteps("NN", [a.cpu()], [a.cpu()])
     with pytest.raises(TypeError):
-        ops.gemm_ksteps("NN", [a.half()], [a.half()])
+        ops.gemm_ksteps("NN", [a.double()], [a.double()])
+    with pytest.raises(TypeError):
+        ops.gemm_ksteps("NN", [a.half()], [a])  # operands of two dtypes
     lib = _lib.load()
     rc = lib.cw_gemm_ksteps(7, 8, 8, 8, 1, None, 8, None, 8, None, 0, None, 8, None, 0, None, 0, 0, 0, None)
     assert rc < 0 and b"layout" in lib.cw_last_error()
