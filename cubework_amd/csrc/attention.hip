@@ -1,4 +1,4 @@
-// Fused causal attention core for gfx950, head sizes 64 and 128, bf16:
+// Fused causal attention core for gfx950, head sizes 64 and 128, bf16 (or fp16: E = f16_t):
 //   O = softmax(scale * Q K^T + causal mask) V        per (batch, head)
 // (benchmark/opt/opt.py:81-117 of the reference: scaled bmm, additive mask,
 // softmax, bmm). One pass over K/V per block of queries with a running
@@ -51,7 +51,7 @@ struct AttnArgs {
 // NP: head size / 64. A tile of NP x 64 columns is NP images side by side ("panels"); everything that
 // runs over the head dimension runs over NP times as many 16-wide k blocks (scores) or 32-wide output
 // blocks (O^T). Head size 64 keeps two blocks per compute unit, 128 has the registers and LDS of one.
-template <int NP>
+template <int NP, typename E>
 __global__ __launch_bounds__(kThreads, NP == 1 ? 2 : 1) void attn_fwd_kernel(const AttnArgs a) {
     constexpr int kStage = 2 * NP * kImage;  // K panels (row images), then V panels (transpose images)
     __shared__ __attribute__((aligned(16))) char lds_raw[2 * kStage];
@@ -157,7 +157,7 @@ __global__ __launch_bounds__(kThreads, NP == 1 ? 2 : 1) void attn_fwd_kernel(con
                     const bf16x8_t kf = read_rows<32 * kt>(ks + (kb >> 2) * kImage, ro, kb & 3);
 #pragma unroll
                     for (int qt = 0; qt < kQT; ++qt)
-                        st[qt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf, qf[qt][kb], st[qt], 0, 0, 0);
+                        st[qt] = mfma16<E>(kf, qf[qt][kb], st[qt]);
                 }
                 bf16x8_t pb[kQT][2];
 #pragma unroll
@@ -194,9 +194,9 @@ __global__ __launch_bounds__(kThreads, NP == 1 ? 2 : 1) void attn_fwd_kernel(con
                         p[e] = __builtin_amdgcn_exp2f(__builtin_fmaf(st[qt][e], a.scale_log2e, -m_use));
                     // k slot j of 16-block kvb <-> e = 8 kvb + j. The row sum is taken over the rounded
                     // probabilities, the values the second product uses.
-                    pb[qt][0] = pack_slots(p, 0);
-                    pb[qt][1] = pack_slots(p, 1);
-                    l_run[qt] += sum_slots(pb[qt][1], sum_slots(pb[qt][0], 0.0f));
+                    pb[qt][0] = pack_slots<E>(p, 0);
+                    pb[qt][1] = pack_slots<E>(p, 1);
+                    l_run[qt] += sum_slots<E>(pb[qt][1], sum_slots<E>(pb[qt][0], 0.0f));
                 }
                 // O^T += V^T P^T over the 32 kv rows of this half tile
 #pragma unroll
@@ -205,8 +205,8 @@ __global__ __launch_bounds__(kThreads, NP == 1 ? 2 : 1) void attn_fwd_kernel(con
                     const bf16x8_t vf1 = read_transposed<32 * kt + 16>(vs + (dt >> 1) * kImage, ro, dt & 1);
 #pragma unroll
                     for (int qt = 0; qt < kQT; ++qt) {
-                        oacc[qt][dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf0, pb[qt][0], oacc[qt][dt], 0, 0, 0);
-                        oacc[qt][dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf1, pb[qt][1], oacc[qt][dt], 0, 0, 0);
+                        oacc[qt][dt] = mfma16<E>(vf0, pb[qt][0], oacc[qt][dt]);
+                        oacc[qt][dt] = mfma16<E>(vf1, pb[qt][1], oacc[qt][dt]);
                     }
                 }
             };
@@ -226,7 +226,7 @@ __global__ __launch_bounds__(kThreads, NP == 1 ? 2 : 1) void attn_fwd_kernel(con
         if (qi < S) {
             uint16_t* orow = a.o + b * a.ob + (int64_t)qi * a.os + h * a.oh;
 #pragma unroll
-            for (int p = 0; p < NP; ++p) store_row_pieces(orow + 64 * p, oacc[qt] + 2 * p, inv, half);
+            for (int p = 0; p < NP; ++p) store_row_pieces<E>(orow + 64 * p, oacc[qt] + 2 * p, inv, half);
             if (half == 0 && a.lse != nullptr)
                 a.lse[(int64_t)bh * S + qi] = (m_run[qt] + __builtin_amdgcn_logf(l_tot)) * kLn2;  // natural-log LSE of scale*s
         }
@@ -243,7 +243,7 @@ extern "C" int cw_attn_fwd(int64_t B, int64_t H, int64_t S, int64_t D, const voi
                            int64_t out_stride_b, int64_t out_stride_s, int64_t out_stride_h, float* lse,
                            int io_dtype, void* stream) {
     if (B < 0 || H < 0 || S < 0 || D <= 0) return fail(CW_ERR_INVALID, "cw_attn_fwd: bad shape B=%lld H=%lld S=%lld D=%lld", (long long)B, (long long)H, (long long)S, (long long)D);
-    if (io_dtype != CW_BF16) return fail(CW_ERR_UNSUPPORTED, "cw_attn_fwd: only bf16 is provided");
+    if (io_dtype != CW_BF16 && io_dtype != CW_F16) return fail(CW_ERR_UNSUPPORTED, "cw_attn_fwd: only bf16 and fp16 are provided");
     if (D != 64 && D != 128) return fail(CW_ERR_UNSUPPORTED, "cw_attn_fwd: head size %lld is not provided (64 and 128)", (long long)D);
     if (B == 0 || H == 0 || S == 0) return CW_OK;
     if (q == nullptr || k == nullptr || v == nullptr || out == nullptr) return fail(CW_ERR_INVALID, "cw_attn_fwd: null pointer");
@@ -268,7 +268,13 @@ extern "C" int cw_attn_fwd(int64_t B, int64_t H, int64_t S, int64_t D, const voi
     a.causal = causal ? 1 : 0;
     a.n_qblocks = (int)((S + kQPerBlock - 1) / kQPerBlock);
     const dim3 grid((unsigned)(a.n_qblocks * B * H));
-    if (D == 64) hipLaunchKernelGGL(attn_fwd_kernel<1>, grid, dim3(kThreads), 0, (hipStream_t)stream, a);
-    else hipLaunchKernelGGL(attn_fwd_kernel<2>, grid, dim3(kThreads), 0, (hipStream_t)stream, a);
+    hipStream_t s = (hipStream_t)stream;
+    if (io_dtype == CW_F16) {
+        if (D == 64) hipLaunchKernelGGL((attn_fwd_kernel<1, f16_t>), grid, dim3(kThreads), 0, s, a);
+        else hipLaunchKernelGGL((attn_fwd_kernel<2, f16_t>), grid, dim3(kThreads), 0, s, a);
+    } else {
+        if (D == 64) hipLaunchKernelGGL((attn_fwd_kernel<1, bf16_t>), grid, dim3(kThreads), 0, s, a);
+        else hipLaunchKernelGGL((attn_fwd_kernel<2, bf16_t>), grid, dim3(kThreads), 0, s, a);
+    }
     return check_launch("attn_fwd_kernel");
 }

@@ -1,4 +1,4 @@
-// Backward of the fused attention core for gfx950 (head sizes 64 and 128, bf16):
+// Backward of the fused attention core for gfx950 (head sizes 64 and 128; bf16, or fp16 with E = f16_t):
 // given Q, K, V, O, dO and the forward's log-sum-exp L (natural log),
 //   P_ij  = exp(scale q_i.k_j - L_i)              (recomputed, never stored)
 //   D_i   = sum_d dO_id O_id
@@ -61,7 +61,7 @@ struct BwdArgs {
 };
 
 // ---- D_i = sum_d dO_id O_id : one group of LPR = head size / 8 lanes per (b, h, i) row -------------
-template <int LPR>
+template <int LPR, typename E>
 __global__ __launch_bounds__(256) void attn_delta_kernel(const BwdArgs a) {
     constexpr int kRows = 256 / LPR;
     const int64_t row = (int64_t)blockIdx.x * kRows + (threadIdx.x / LPR);  // (bh, i) flattened
@@ -73,8 +73,8 @@ __global__ __launch_bounds__(256) void attn_delta_kernel(const BwdArgs a) {
     const int b = bh / a.H, h = bh - b * a.H;
     const int64_t off = b * a.ob + (int64_t)i * a.os + h * a.oh + sub * 8;
     float x[8], y[8];
-    unpack_raw(load_raw(a.o + off), x, (const bf16_t*)nullptr);
-    unpack_raw(load_raw(a.d_o + off), y, (const bf16_t*)nullptr);
+    unpack_raw(load_raw(a.o + off), x, (const E*)nullptr);
+    unpack_raw(load_raw(a.d_o + off), y, (const E*)nullptr);
     float s = 0.0f;
 #pragma unroll
     for (int e = 0; e < 8; ++e) s += x[e] * y[e];
@@ -87,7 +87,7 @@ __global__ __launch_bounds__(256) void attn_delta_kernel(const BwdArgs a) {
 
 // ---- dQ ---------------------------------------------------------------------
 // LDS per stage: K row images, K transpose images, V row images (NP = head size / 64 panels of each).
-template <int NP>
+template <int NP, typename E>
 __global__ __launch_bounds__(kThreads, 1) void attn_dq_kernel(const BwdArgs a) {
     constexpr int kStage = 3 * NP * kImage;
     __shared__ __attribute__((aligned(16))) char lds_raw[2 * kStage];
@@ -177,8 +177,8 @@ __global__ __launch_bounds__(kThreads, 1) void attn_dq_kernel(const BwdArgs a) {
                 }
 #pragma unroll
                 for (int kb = 0; kb < 4 * NP; ++kb) {
-                    st = __builtin_amdgcn_mfma_f32_32x32x16_bf16(read_rows<32 * kt>(k_rows + (kb >> 2) * kImage, ro, kb & 3), qf[kb], st, 0, 0, 0);
-                    dpt = __builtin_amdgcn_mfma_f32_32x32x16_bf16(read_rows<32 * kt>(v_rows + (kb >> 2) * kImage, ro, kb & 3), dof[kb], dpt, 0, 0, 0);
+                    st = mfma16<E>(read_rows<32 * kt>(k_rows + (kb >> 2) * kImage, ro, kb & 3), qf[kb], st);
+                    dpt = mfma16<E>(read_rows<32 * kt>(v_rows + (kb >> 2) * kImage, ro, kb & 3), dof[kb], dpt);
                 }
                 // element e: key kv0 + 32 kt + 8 (e / 4) + 4 half + e % 4, query qi
                 float ds[16];
@@ -191,12 +191,12 @@ __global__ __launch_bounds__(kThreads, 1) void attn_dq_kernel(const BwdArgs a) {
 #pragma unroll
                     for (int e = 0; e < 16; ++e) ds[e] = (32 * kt + 8 * (e >> 2) + (e & 3) > lim) ? 0.0f : ds[e];
                 }
-                const bf16x8_t dsb0 = pack_slots(ds, 0), dsb1 = pack_slots(ds, 1);
+                const bf16x8_t dsb0 = pack_slots<E>(ds, 0), dsb1 = pack_slots<E>(ds, 1);
 #pragma unroll
                 for (int dt = 0; dt < 2 * NP; ++dt) {
                     lds_char* kt_img = k_tr + (dt >> 1) * kImage;
-                    dq[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(read_transposed<32 * kt>(kt_img, ro, dt & 1), dsb0, dq[dt], 0, 0, 0);
-                    dq[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(read_transposed<32 * kt + 16>(kt_img, ro, dt & 1), dsb1, dq[dt], 0, 0, 0);
+                    dq[dt] = mfma16<E>(read_transposed<32 * kt>(kt_img, ro, dt & 1), dsb0, dq[dt]);
+                    dq[dt] = mfma16<E>(read_transposed<32 * kt + 16>(kt_img, ro, dt & 1), dsb1, dq[dt]);
                 }
             };
             half_tile(std::integral_constant<int, 0>{});
@@ -208,7 +208,7 @@ __global__ __launch_bounds__(kThreads, 1) void attn_dq_kernel(const BwdArgs a) {
     if (qi < S) {
         uint16_t* grow = a.dq + b * a.gb + (int64_t)qi * a.gs + h * a.gh;
 #pragma unroll
-        for (int p = 0; p < NP; ++p) store_row_pieces(grow + 64 * p, dq + 2 * p, a.scale, half);
+        for (int p = 0; p < NP; ++p) store_row_pieces<E>(grow + 64 * p, dq + 2 * p, a.scale, half);
     }
 }
 
@@ -221,7 +221,7 @@ constexpr int dkdv_stage_bytes() { return 4 * NP * kImage + 2 * kTile * 4; }
 
 // KG: groups of 32 key rows per wavefront. With two, every A operand read from LDS (Q, dO, their
 // transposes) feeds two MFMAs instead of one.
-template <int NP, int NW, int KG>
+template <int NP, int NW, int KG, typename E>
 __global__ __launch_bounds__(NW * 64, 1) void attn_dkdv_kernel(const BwdArgs a) {
     constexpr int kKeysPerWave = KG * kRowsPerWave;
     constexpr int kDkdvStage = dkdv_stage_bytes<NP>();
@@ -345,8 +345,8 @@ __global__ __launch_bounds__(NW * 64, 1) void attn_dkdv_kernel(const BwdArgs a) 
                     const bf16x8_t ga = read_rows<32 * qt>(g_rows + (kb >> 2) * kImage, ro, kb & 3);
 #pragma unroll
                     for (int kg = 0; kg < KG; ++kg) {
-                        s_acc[kg] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(qa, kf[kg][kb], s_acc[kg], 0, 0, 0);
-                        dp_acc[kg] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ga, vf[kg][kb], dp_acc[kg], 0, 0, 0);
+                        s_acc[kg] = mfma16<E>(qa, kf[kg][kb], s_acc[kg]);
+                        dp_acc[kg] = mfma16<E>(ga, vf[kg][kb], dp_acc[kg]);
                     }
                 }
                 bf16x8_t pb[KG][2], dsb[KG][2];
@@ -376,8 +376,8 @@ __global__ __launch_bounds__(NW * 64, 1) void attn_dkdv_kernel(const BwdArgs a) 
                     }
 #pragma unroll
                     for (int sl = 0; sl < 2; ++sl) {
-                        pb[kg][sl] = pack_slots(p, sl);
-                        dsb[kg][sl] = pack_slots(ds, sl);
+                        pb[kg][sl] = pack_slots<E>(p, sl);
+                        dsb[kg][sl] = pack_slots<E>(ds, sl);
                     }
                 }
 #pragma unroll
@@ -390,8 +390,8 @@ __global__ __launch_bounds__(NW * 64, 1) void attn_dkdv_kernel(const BwdArgs a) 
                         const bf16x8_t qtr = sl == 0 ? read_transposed<32 * qt>(qi_img, ro, dt & 1) : read_transposed<32 * qt + 16>(qi_img, ro, dt & 1);
 #pragma unroll
                         for (int kg = 0; kg < KG; ++kg) {
-                            dv[kg][dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(gt, pb[kg][sl], dv[kg][dt], 0, 0, 0);
-                            dk[kg][dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(qtr, dsb[kg][sl], dk[kg][dt], 0, 0, 0);
+                            dv[kg][dt] = mfma16<E>(gt, pb[kg][sl], dv[kg][dt]);
+                            dk[kg][dt] = mfma16<E>(qtr, dsb[kg][sl], dk[kg][dt]);
                         }
                     }
                 }
@@ -411,11 +411,41 @@ __global__ __launch_bounds__(NW * 64, 1) void attn_dkdv_kernel(const BwdArgs a) 
             uint16_t* dvrow = a.dv + b * a.gb + (int64_t)kvi * a.gs + h * a.gh;
 #pragma unroll
             for (int p = 0; p < NP; ++p) {
-                store_row_pieces(dkrow + 64 * p, dk[kg] + 2 * p, a.scale, half);
-                store_row_pieces(dvrow + 64 * p, dv[kg] + 2 * p, 1.0f, half);
+                store_row_pieces<E>(dkrow + 64 * p, dk[kg] + 2 * p, a.scale, half);
+                store_row_pieces<E>(dvrow + 64 * p, dv[kg] + 2 * p, 1.0f, half);
             }
         }
     }
+}
+
+// The three launches of the backward for element type E.
+template <typename E>
+int launch_bwd(const BwdArgs& a, int64_t B, int64_t H, int64_t S, int64_t D, int64_t nblk, hipStream_t s) {
+    const int64_t rows = B * H * S;
+    if (D == 64) hipLaunchKernelGGL((attn_delta_kernel<8, E>), dim3((unsigned)((rows + 31) / 32)), dim3(256), 0, s, a);
+    else hipLaunchKernelGGL((attn_delta_kernel<16, E>), dim3((unsigned)((rows + 15) / 16)), dim3(256), 0, s, a);
+    int rc = check_launch("attn_delta_kernel");
+    if (rc != CW_OK) return rc;
+    if (D == 64) hipLaunchKernelGGL((attn_dq_kernel<1, E>), dim3((unsigned)(nblk * B * H)), dim3(kThreads), 0, s, a);
+    else hipLaunchKernelGGL((attn_dq_kernel<2, E>), dim3((unsigned)(nblk * B * H)), dim3(kThreads), 0, s, a);
+    rc = check_launch("attn_dq_kernel");
+    if (rc != CW_OK) return rc;
+    if (D == 64) {
+        constexpr int lds_bytes = 2 * dkdv_stage_bytes<1>();
+        auto kern = attn_dkdv_kernel<1, kDkdvWaves, kDkdvGroups, E>;
+        hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes);
+        if (e != hipSuccess) return fail(CW_ERR_LAUNCH, "hipFuncSetAttribute(attn_dkdv_kernel): %s", hipGetErrorString(e));
+        hipLaunchKernelGGL(kern, dim3((unsigned)(nblk * B * H)), dim3(kDkdvWaves * 64), lds_bytes, s, a);
+    } else {
+        constexpr int lds_bytes = 2 * dkdv_stage_bytes<2>();
+        auto kern = attn_dkdv_kernel<2, 4, 1, E>;
+        const int64_t nkv = (S + 4 * kRowsPerWave - 1) / (4 * kRowsPerWave);
+        if (nkv * B * H > INT32_MAX) return fail(CW_ERR_INVALID, "cw_attn_bwd: S or B*H too large");
+        hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes);
+        if (e != hipSuccess) return fail(CW_ERR_LAUNCH, "hipFuncSetAttribute(attn_dkdv_kernel): %s", hipGetErrorString(e));
+        hipLaunchKernelGGL(kern, dim3((unsigned)(nkv * B * H)), dim3(4 * 64), lds_bytes, s, a);
+    }
+    return check_launch("attn_dkdv_kernel");
 }
 
 }  // namespace
@@ -436,7 +466,7 @@ extern "C" int cw_attn_bwd(int64_t B, int64_t H, int64_t S, int64_t D, const voi
                            int io_dtype, void* stream) {
     if (B < 0 || H < 0 || S < 0 || D <= 0)
         return fail(CW_ERR_INVALID, "cw_attn_bwd: bad shape B=%lld H=%lld S=%lld D=%lld", (long long)B, (long long)H, (long long)S, (long long)D);
-    if (io_dtype != CW_BF16) return fail(CW_ERR_UNSUPPORTED, "cw_attn_bwd: only bf16 is provided");
+    if (io_dtype != CW_BF16 && io_dtype != CW_F16) return fail(CW_ERR_UNSUPPORTED, "cw_attn_bwd: only bf16 and fp16 are provided");
     if (D != 64 && D != 128) return fail(CW_ERR_UNSUPPORTED, "cw_attn_bwd: head size %lld is not provided (64 and 128)", (long long)D);
     if (B == 0 || H == 0 || S == 0) return CW_OK;
     if (q == nullptr || k == nullptr || v == nullptr || out == nullptr || d_out == nullptr || lse == nullptr ||
@@ -470,29 +500,5 @@ extern "C" int cw_attn_bwd(int64_t B, int64_t H, int64_t S, int64_t D, const voi
     a.causal = causal ? 1 : 0;
     a.D = (int)D;
     hipStream_t s = (hipStream_t)stream;
-    const int64_t rows = B * H * S;
-    if (D == 64) hipLaunchKernelGGL(attn_delta_kernel<8>, dim3((unsigned)((rows + 31) / 32)), dim3(256), 0, s, a);
-    else hipLaunchKernelGGL(attn_delta_kernel<16>, dim3((unsigned)((rows + 15) / 16)), dim3(256), 0, s, a);
-    int rc = check_launch("attn_delta_kernel");
-    if (rc != CW_OK) return rc;
-    if (D == 64) hipLaunchKernelGGL(attn_dq_kernel<1>, dim3((unsigned)(nblk * B * H)), dim3(kThreads), 0, s, a);
-    else hipLaunchKernelGGL(attn_dq_kernel<2>, dim3((unsigned)(nblk * B * H)), dim3(kThreads), 0, s, a);
-    rc = check_launch("attn_dq_kernel");
-    if (rc != CW_OK) return rc;
-    if (D == 64) {
-        constexpr int lds_bytes = 2 * dkdv_stage_bytes<1>();
-        auto kern = attn_dkdv_kernel<1, kDkdvWaves, kDkdvGroups>;
-        hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes);
-        if (e != hipSuccess) return fail(CW_ERR_LAUNCH, "hipFuncSetAttribute(attn_dkdv_kernel): %s", hipGetErrorString(e));
-        hipLaunchKernelGGL(kern, dim3((unsigned)(nblk * B * H)), dim3(kDkdvWaves * 64), lds_bytes, s, a);
-    } else {
-        constexpr int lds_bytes = 2 * dkdv_stage_bytes<2>();
-        auto kern = attn_dkdv_kernel<2, 4, 1>;
-        const int64_t nkv = (S + 4 * kRowsPerWave - 1) / (4 * kRowsPerWave);
-        if (nkv * B * H > INT32_MAX) return fail(CW_ERR_INVALID, "cw_attn_bwd: S or B*H too large");
-        hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes);
-        if (e != hipSuccess) return fail(CW_ERR_LAUNCH, "hipFuncSetAttribute(attn_dkdv_kernel): %s", hipGetErrorString(e));
-        hipLaunchKernelGGL(kern, dim3((unsigned)(nkv * B * H)), dim3(4 * 64), lds_bytes, s, a);
-    }
-    return check_launch("attn_dkdv_kernel");
+    return io_dtype == CW_F16 ? launch_bwd<f16_t>(a, B, H, S, D, nblk, s) : launch_bwd<bf16_t>(a, B, H, S, D, nblk, s);
 }

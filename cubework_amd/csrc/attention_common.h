@@ -1,4 +1,4 @@
-// Pieces shared by the attention forward and backward kernels (gfx950, bf16):
+// Pieces shared by the attention forward and backward kernels (gfx950; bf16, or fp16 with E = f16_t):
 // LDS tile images of 64 columns (a head of 128 is two of them side by side),
 // MFMA operand reads, tile loader.
 #pragma once
@@ -12,6 +12,8 @@ namespace attn {
 
 typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
 typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+typedef _Float16 f16x8_t __attribute__((ext_vector_type(8)));
+typedef _Float16 f16x2_t __attribute__((ext_vector_type(2)));
 typedef float f32x16_t __attribute__((ext_vector_type(16)));
 typedef float f32x4_t __attribute__((ext_vector_type(4)));
 typedef short s16x4_t __attribute__((ext_vector_type(4)));
@@ -64,32 +66,60 @@ __device__ __forceinline__ bf16x8_t read_transposed(lds_char* img, const ReadOff
     return __builtin_bit_cast(bf16x8_t, (s16x8_t)__builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
 }
 
-// bf16 B operand from 8 consecutive accumulator elements (k slot j <-> element 8 blk + j).
-__device__ __forceinline__ bf16x8_t pack_slots(const float (&x)[16], int blk) {
-    bf16x8_t r;
-#pragma unroll
-    for (int j = 0; j < 8; ++j) r[j] = (__bf16)x[8 * blk + j];
-    return r;
+// Operands travel as 8 x 16 bits (bf16x8_t) whatever the element type E (bf16_t or f16_t); these are
+// the places where the type matters.
+template <typename E>
+__device__ __forceinline__ f32x16_t mfma16(bf16x8_t a, bf16x8_t b, f32x16_t acc) {
+    if constexpr (std::is_same<E, f16_t>::value)
+        return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8_t, a), __builtin_bit_cast(f16x8_t, b), acc, 0, 0, 0);
+    else
+        return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, acc, 0, 0, 0);
 }
-// Sum of the 8 bf16 values of an operand, in fp32 (v_dot2 with ones).
+// B operand from 8 consecutive accumulator elements (k slot j <-> element 8 blk + j), rounded to E.
+template <typename E>
+__device__ __forceinline__ bf16x8_t pack_slots(const float (&x)[16], int blk) {
+    if constexpr (std::is_same<E, f16_t>::value) {
+        f16x8_t r;
+#pragma unroll
+        for (int j = 0; j < 8; ++j) r[j] = (_Float16)x[8 * blk + j];
+        return __builtin_bit_cast(bf16x8_t, r);
+    } else {
+        bf16x8_t r;
+#pragma unroll
+        for (int j = 0; j < 8; ++j) r[j] = (__bf16)x[8 * blk + j];
+        return r;
+    }
+}
+// Sum of the 8 values of an operand, in fp32 (v_dot2 with ones).
+template <typename E>
 __device__ __forceinline__ float sum_slots(bf16x8_t v, float acc) {
-    const bf16x2_t ones = {(__bf16)1.0f, (__bf16)1.0f};
-    acc = __builtin_amdgcn_fdot2_f32_bf16(__builtin_shufflevector(v, v, 0, 1), ones, acc, false);
-    acc = __builtin_amdgcn_fdot2_f32_bf16(__builtin_shufflevector(v, v, 2, 3), ones, acc, false);
-    acc = __builtin_amdgcn_fdot2_f32_bf16(__builtin_shufflevector(v, v, 4, 5), ones, acc, false);
-    acc = __builtin_amdgcn_fdot2_f32_bf16(__builtin_shufflevector(v, v, 6, 7), ones, acc, false);
+    if constexpr (std::is_same<E, f16_t>::value) {
+        const f16x8_t h = __builtin_bit_cast(f16x8_t, v);
+        const f16x2_t ones = {(_Float16)1.0f, (_Float16)1.0f};
+        acc = __builtin_amdgcn_fdot2(__builtin_shufflevector(h, h, 0, 1), ones, acc, false);
+        acc = __builtin_amdgcn_fdot2(__builtin_shufflevector(h, h, 2, 3), ones, acc, false);
+        acc = __builtin_amdgcn_fdot2(__builtin_shufflevector(h, h, 4, 5), ones, acc, false);
+        acc = __builtin_amdgcn_fdot2(__builtin_shufflevector(h, h, 6, 7), ones, acc, false);
+    } else {
+        const bf16x2_t ones = {(__bf16)1.0f, (__bf16)1.0f};
+        acc = __builtin_amdgcn_fdot2_f32_bf16(__builtin_shufflevector(v, v, 0, 1), ones, acc, false);
+        acc = __builtin_amdgcn_fdot2_f32_bf16(__builtin_shufflevector(v, v, 2, 3), ones, acc, false);
+        acc = __builtin_amdgcn_fdot2_f32_bf16(__builtin_shufflevector(v, v, 4, 5), ones, acc, false);
+        acc = __builtin_amdgcn_fdot2_f32_bf16(__builtin_shufflevector(v, v, 6, 7), ones, acc, false);
+    }
     return acc;
 }
 
 // Lane (row = lane % 32, half = lane / 32) holds, of a transposed 64 x 32 result, the values
-// d = 32 dt + 8 (e / 4) + 4 half + e % 4 of its row: write them, times `mul`, as bf16.
+// d = 32 dt + 8 (e / 4) + 4 half + e % 4 of its row: write them, times `mul`, as E.
+template <typename E>
 __device__ __forceinline__ void store_row_pieces(uint16_t* rowp, const f32x16_t* acc, float mul, int half) {
 #pragma unroll
     for (int dt = 0; dt < 2; ++dt)
 #pragma unroll
         for (int g = 0; g < 4; ++g) {
-            const uint2 w = make_uint2(pack_bf16x2(acc[dt][4 * g] * mul, acc[dt][4 * g + 1] * mul),
-                                       pack_bf16x2(acc[dt][4 * g + 2] * mul, acc[dt][4 * g + 3] * mul));
+            const uint2 w = make_uint2(half_conv<E>::pack2(acc[dt][4 * g] * mul, acc[dt][4 * g + 1] * mul),
+                                       half_conv<E>::pack2(acc[dt][4 * g + 2] * mul, acc[dt][4 * g + 3] * mul));
             *reinterpret_cast<uint2*>(rowp + 32 * dt + 8 * g + 4 * half) = w;
         }
 }

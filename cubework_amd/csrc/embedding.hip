@@ -5,8 +5,9 @@
 //           row is never read, only written as zeros.
 // backward: d_weight[r, :] = sum over tokens with id - start == r of d_out[t, :]
 //           (autograd of F.embedding), deterministic: the caller supplies the token order sorted
-//           by id, one block owns one run of equal ids, its wavefronts split the run and are
-//           combined in a fixed order. No atomics.
+//           by id; a run of equal ids is summed by the blocks at its first positions (column
+//           slices), whose wavefronts stride the run's tokens and are combined in a fixed order.
+//           No atomics.
 // Both are HBM-streaming kernels: 16-byte accesses, one wavefront per row.
 #include "cw_common.h"
 

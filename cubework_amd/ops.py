@@ -409,7 +409,7 @@ def attn_fwd(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, scale: Optional[
     out = torch.empty((B, S, H, D), dtype=q.dtype, device=q.device)
     lse = torch.empty((B, H, S), dtype=torch.float32, device=q.device) if want_lse else None
     rc = lib.cw_attn_fwd(B, H, S, D, _p(q), _p(k), _p(v), strides[0], strides[1], strides[2], scale, 1 if causal else 0,
-                         _p(out), out.stride(0), out.stride(1), out.stride(2), _p(lse), _dtype_code(q), _stream())
+                         _p(out), out.stride(0), out.stride(1), out.stride(2), _p(lse), _dtype_code(q, half_ok=True), _stream())
     _lib.check(rc, "cw_attn_fwd")
     out = out.view(B, S, H * D)
     return (out, lse) if want_lse else out
@@ -439,7 +439,7 @@ def attn_bwd(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, out: torch.Tenso
     ws = torch.empty(max(ws_bytes, 16), dtype=torch.uint8, device=q.device)
     rc = lib.cw_attn_bwd(B, H, S, D, _p(q), _p(k), _p(v), strides[0], strides[1], strides[2], _p(out4), _p(dout4),
                          ostr[0], ostr[1], ostr[2], _p(lse), scale, 1 if causal else 0, _p(dq), _p(dk), _p(dv),
-                         gstrides[0], gstrides[1], gstrides[2], _p(ws), ws.numel(), _dtype_code(q), _stream())
+                         gstrides[0], gstrides[1], gstrides[2], _p(ws), ws.numel(), _dtype_code(q, half_ok=True), _stream())
     _lib.check(rc, "cw_attn_bwd")
 
 

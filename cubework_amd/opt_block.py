@@ -39,7 +39,7 @@ class OPTBlock(nn.Module):
         self.fc2 = cube_nn.Linear(ffn, hidden, dtype=dtype)
 
     def _attention_core(self, qkv: torch.Tensor) -> torch.Tensor:
-        if self.head_dim in (64, 128) and qkv.dtype == torch.bfloat16 and qkv.is_cuda:
+        if self.head_dim in (64, 128) and qkv.dtype in (torch.bfloat16, torch.float16) and qkv.is_cuda:
             return ops.attention_core(qkv, self.heads)
         b, s, _ = qkv.shape
         qkv = qkv.view(b, s, self.heads, 3 * self.head_dim).permute(0, 2, 1, 3)

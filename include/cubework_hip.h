@@ -43,9 +43,9 @@ typedef enum {
 
 /* CW_F16 (IEEE half, the type the reference's GEMM-type Functions cast to under autocast:
  * custom_fwd(cast_inputs=torch.float16), cubework/module/parallel_2d/_operation.py:17,96,176,255,363) is
- * taken by the GEMM and column-sum entry points only (cw_gemm_ksteps, cw_gemm_ksteps_ws, cw_colsum,
- * cw_act_bwd_colsum): the reference runs LayerNorm and the loss in fp32 under autocast, and so do their
- * entry points here. */
+ * taken by the GEMM, column-sum and attention entry points only (cw_gemm_ksteps, cw_gemm_ksteps_ws,
+ * cw_colsum, cw_act_bwd_colsum, cw_attn_fwd, cw_attn_bwd): the reference runs LayerNorm and the loss in
+ * fp32 under autocast, and so do their entry points here. */
 typedef enum { CW_BF16 = 0, CW_F32 = 1, CW_F16 = 2 } cw_dtype;
 
 /* Operand orientation of the block GEMM, per k-step i:
@@ -368,7 +368,7 @@ int cw_multi_scale(int n_tensors, void* const* grads, const int64_t* numels, con
  * stride in c; opt.py:72-76 makes them [b, s, heads, 3*d] slices), out
  * likewise with its own strides ([b, s, heads*d] as opt.py:123-128 leaves it).
  * lse (optional, [B,H,S] fp32) receives log sum_j exp(scale * q.k_j) for the
- * backward. D = 64 or 128 and CW_BF16 only in this build (CW_ERR_UNSUPPORTED
+ * backward. D = 64 or 128, CW_BF16 or CW_F16 in this build (CW_ERR_UNSUPPORTED
  * else); token strides below 2^23 elements.
  */
 int cw_attn_fwd(int64_t B, int64_t H, int64_t S, int64_t D,

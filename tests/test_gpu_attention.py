@@ -185,3 +185,37 @@ def test_attention_head_size_128_autograd():
     dq, dk, dv = oracle.attention_core_backward(qc, kc, vc, d_out)
     want = torch.cat([dq, dk, dv], dim=-1).permute(0, 2, 1, 3).reshape(b, s, h * 3 * d)
     assert_parity(g1, want, torch.bfloat16, "d qkv, head size 128", scale=2)
+
+
+@pytest.mark.parametrize("d", [64, 128])
+@pytest.mark.parametrize("shape", [(2, 256, 2), (1, 100, 2), (1, 257, 1), (1, 1, 1), (1, 700, 2)])
+@pytest.mark.parametrize("causal", [True, False])
+def test_attention_float16(shape, causal, d):
+    """float16 q/k/v (what the projections return under a plain autocast): forward, log-sum-exp and the three
+    gradients against the oracle at the float16 bar (probabilities and dS are rounded to 11 significand bits
+    instead of bfloat16's 8 on their way into the second MFMA)."""
+    import oracle
+    from cubework_amd import ops
+
+    b, s, h = shape
+    f16 = torch.float16
+    qkv = _qkv(b, s, h, d, seed=5 * s + h, std=1.2).to(f16)
+    d_out = randn((b, s, h * d), f16, seed=s + 19)
+    qc, kc, vc = oracle.split_qkv(qkv, h)
+    want, want_lse = oracle.attention_core(qc, kc, vc, causal=causal, return_lse=True)
+    want_g = oracle.attention_core_backward(qc, kc, vc, d_out, causal=causal)
+    dev = qkv.to(DEV)
+    q, k, v = _views(dev, h, d)
+    out, lse = ops.attn_fwd(q, k, v, causal=causal, want_lse=True)
+    g = torch.full((b, s, h, 3 * d), float("nan"), dtype=f16, device=DEV)
+    ops.attn_bwd(q, k, v, out, d_out.to(DEV), lse, g[..., :d], g[..., d:2 * d], g[..., 2 * d:], causal=causal)
+    torch.cuda.synchronize()
+    assert out.dtype == f16
+    assert_parity(out, want, f16, "float16 attention out d=%d %s" % (d, shape))
+    assert_parity(lse, want_lse, torch.float32, "float16 attention lse d=%d %s" % (d, shape), scale=100)
+    if s == 1:  # dq and dk are exactly zero: judged against the size of the whole gradient
+        assert_parity(g.permute(0, 2, 1, 3), torch.cat(want_g, dim=-1), f16, "float16 attention grads d=%d %s" % (d, shape))
+        return
+    for name, got, ref in (("dq", g[..., :d], want_g[0]), ("dk", g[..., d:2 * d], want_g[1]), ("dv", g[..., 2 * d:], want_g[2])):
+        assert_parity(got.permute(0, 2, 1, 3), ref, f16, "float16 attention %s d=%d %s causal=%s" % (name, d, shape, causal),
+                      scale=2)

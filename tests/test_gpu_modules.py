@@ -297,6 +297,33 @@ def test_vocab_parallel_loss_one_rank_of_four(dtype):
     assert torch.equal(x.detach(), before), "the caller's logits must stay intact"
 
 
+@pytest.mark.parametrize("amp_dtype", [torch.float16, torch.bfloat16])
+def test_opt_block_under_autocast(amp_dtype):
+    """fp32 parameters and input inside torch.autocast, as the reference's training scripts run
+    (benchmark/opt/train.py:85-86): the four Linear2D cast to the autocast dtype (float16 by default, the
+    reference's custom_fwd dtype), LayerNorm2D runs in fp32, the fused attention core takes the projections'
+    dtype; output and every gradient against the same block in fp32 torch."""
+    from cubework_amd.distributed import initialize
+    from cubework_amd.opt_block import OPTBlock, opt_block_reference
+
+    initialize("2d", 1)
+    torch.manual_seed(0)
+    blk = OPTBlock(hidden=256, heads=4, ffn=1024, dtype=torch.float32, activation="gelu_tanh").to(DEV)
+    x = _leaf(randn((2, 64, 256), torch.float32, 1).to(DEV))
+    dy = randn((2, 64, 256), torch.float32, 2).to(DEV)
+    with torch.autocast("cuda", dtype=amp_dtype):
+        y = blk(x)
+    y.backward(dy)
+    xr = _leaf(x.detach().cpu())
+    ref, params = opt_block_reference(blk, xr)
+    ref.backward(dy.cpu())
+    assert_parity(y, ref.detach(), amp_dtype, "block forward under autocast", scale=5)
+    assert_parity(x.grad, xr.grad, amp_dtype, "block dX under autocast", scale=8)
+    for name, prm in blk.named_parameters():
+        assert prm.grad is not None and prm.grad.dtype == torch.float32, name
+        assert_parity(prm.grad, params[name].grad, amp_dtype, name + ".grad under autocast", scale=8)
+
+
 @pytest.mark.parametrize("activation", ["gelu_tanh", "relu"])
 def test_opt_block_shapes_small(activation):
     """A reduced OPT decoder layer (benchmark/opt/opt.py:135-211 shapes: pre-LN,
