@@ -32,4 +32,5 @@ from .vpce import vpce_fwd_local, vpce_finalize, vpce_bwd, vpce_reference_full  
 from .attention import split_qkv, attention_core, attention_core_backward, attention_brute_force  # noqa: F401
 from .embedding import vocab_embedding_fwd, vocab_embedding_bwd  # noqa: F401
 from .clip_grad import clip_grad_norm  # noqa: F401
+from .opt_block import opt_block_reference  # noqa: F401
 from . import grid  # noqa: F401

@@ -304,7 +304,8 @@ def test_opt_block_under_autocast(amp_dtype):
     reference's custom_fwd dtype), LayerNorm2D runs in fp32, the fused attention core takes the projections'
     dtype; output and every gradient against the same block in fp32 torch."""
     from cubework_amd.distributed import initialize
-    from cubework_amd.opt_block import OPTBlock, opt_block_reference
+    from cubework_amd.opt_block import OPTBlock
+    from oracle import opt_block_reference
 
     initialize("2d", 1)
     torch.manual_seed(0)
@@ -334,7 +335,8 @@ def test_opt_block_shapes_small(activation):
     moves a whole term of fc1's weight gradient, which is not a rounding-sized
     difference; the smooth GeLU variant is compared in full."""
     from cubework_amd.distributed import initialize
-    from cubework_amd.opt_block import OPTBlock, opt_block_reference
+    from cubework_amd.opt_block import OPTBlock
+    from oracle import opt_block_reference
 
     initialize("2d", 1)
     torch.manual_seed(0)

@@ -27,22 +27,23 @@ def _gemm_cases():
     return cases
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
 @pytest.mark.parametrize("case", _gemm_cases())
-def test_random_gemm(case):
+def test_random_gemm(case, dtype):
     import oracle
     from cubework_amd import ops
 
     layout, M, N, K, steps = case
     a_shape = (K, M) if layout == "TN" else (M, K)
     b_shape = (N, K) if layout == "NT" else (K, N)
-    A = [randn(a_shape, torch.bfloat16, 7 * s + M) for s in range(steps)]
-    B = [randn(b_shape, torch.bfloat16, 7 * s + N + 1, std=0.05) for s in range(steps)]
-    bias = randn((N,), torch.bfloat16, K, std=0.3)
+    A = [randn(a_shape, dtype, 7 * s + M) for s in range(steps)]
+    B = [randn(b_shape, dtype, 7 * s + N + 1, std=0.05) for s in range(steps)]
+    bias = randn((N,), dtype, K, std=0.3)
     act = ["relu", "gelu_tanh", None][(M + N + K) % 3]
     want = oracle.gemm_ksteps(layout, A, B, bias, act)
     got = ops.gemm_ksteps(layout, [a.to(DEV) for a in A], [b.to(DEV) for b in B], bias.to(DEV), act)
     torch.cuda.synchronize()
-    assert_parity(got, want, torch.bfloat16, "gemm %s" % (case,))
+    assert_parity(got, want, dtype, "gemm %s %s" % (case, dtype))
 
 
 def _attn_cases():
