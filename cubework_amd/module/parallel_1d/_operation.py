@@ -30,9 +30,12 @@ class _LinearNT(torch.autograd.Function):
     @gemm_fwd()
     def forward(ctx, input_, weight, bias, activation):
         x2 = input_.reshape(-1, input_.shape[-1])
-        need_pre = activation is not None
+        # ReLU needs no separate pre-activation: its derivative [pre > 0] is [out > 0], so the output serves
+        need_pre = activation is not None and activation != "relu"
         res = ops.gemm_ksteps("NT", [x2], [weight], bias, activation, want_preact=need_pre)
         out, pre = res if need_pre else (res, None)
+        if activation == "relu":
+            pre = out
         ctx.save_for_backward(x2, weight, pre)
         ctx.meta = (input_.shape, activation, bias is not None, None if bias is None else bias.dtype)
         return out.reshape(input_.shape[:-1] + (weight.shape[0],))

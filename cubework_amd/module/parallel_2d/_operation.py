@@ -39,9 +39,12 @@ class _SUMMA_AB(torch.autograd.Function):
         A_steps = [broadcast(A2, row_parallel_mode.rank_by_idx(i), row_parallel_mode) for i in range(summa_dim)]
         B_steps = [broadcast(B2, col_parallel_mode.rank_by_idx(i), col_parallel_mode) for i in range(summa_dim)]
         bias_full = None if bias is None else all_gather(bias, -1, col_parallel_mode)
-        need_pre = activation is not None
+        # ReLU needs no separate pre-activation: its derivative [pre > 0] is [out > 0], so the output serves
+        need_pre = activation is not None and activation != "relu"
         res = ops.gemm_ksteps("NN", A_steps, B_steps, bias_full, activation, want_preact=need_pre)
         out, pre = res if need_pre else (res, None)
+        if activation == "relu":
+            pre = out
         ctx.save_for_backward(A, B, pre)
         ctx.meta = (summa_dim, row_parallel_mode, col_parallel_mode, activation, bias is not None,
                     None if bias is None else bias.dtype, A.shape, B.shape)

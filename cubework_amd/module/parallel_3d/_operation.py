@@ -33,9 +33,12 @@ class _Linear3D(torch.autograd.Function):
         x2 = _flat(x)
         pre = None
         if output_parallel_mode.world_size == 1:
-            need_pre = activation is not None
+            # ReLU needs no separate pre-activation: its derivative [pre > 0] is [out > 0], so the output serves
+            need_pre = activation is not None and activation != "relu"
             res = ops.gemm_ksteps("NN", [x2], [w], bias, activation, want_preact=need_pre)
             out, pre = res if need_pre else (res, None)
+            if activation == "relu":
+                pre = out
             out = out.reshape(x.shape[:-1] + (w.shape[-1],))
         else:
             assert activation is None, "a fused activation needs the whole reduction on this rank"
