@@ -2,8 +2,8 @@
 backward of each layer against the reference tests' own oracles — plain torch
 on the master tensors (tests/test_2d/check_2d_modules.py:77, tests/test_1d/
 check_1d_modules.py:74,144, tests/test_3d/check_3d_modules.py:132) — at
-tensor-parallel size 1, and as one rank of a 2 x 2 grid / of 4 vocabulary
-slices with the peers' data pre-staged.
+tensor-parallel size 1, and as one rank of a 2 x 2 grid / of a 1D pair / of a
+2 x 2 x 2 cube / of 4 vocabulary slices with the peers' data pre-staged.
 """
 import pytest
 import torch
@@ -207,6 +207,169 @@ def test_linear2d_one_rank_of_2x2_grid():
     sent_row = dict(row.outbox["reduce"])
     assert_parity(sent_row[0], gemm("NT", [dC], [shard(W_master, q, 0, j)]), dt, "product sent to column 0", scale=10)
     assert not any(row.inbox.values()) and not any(col.inbox.values())
+
+
+@pytest.mark.parametrize("rank", [0, 1])
+def test_linear1d_col_row_one_rank_of_two(rank):
+    """Column-parallel then row-parallel Linear1D (the Megatron MLP the reference's 1D mode builds from two
+    `Linear`s, parallel_1d/module.py:38-58) as one rank of two, the peer's partial product and input gradient
+    pre-staged; checked against the master computation as tests/test_1d/check_1d_modules.py:38-150 does."""
+    from cubework_amd.distributed import initialize, pm
+    from cubework_amd.module.parallel_1d import Linear1D_Col, Linear1D_Row
+
+    p, other = 2, 1 - rank
+    T_, IN, HID, OUT = 48, 128, 256, 192
+    dt = torch.float32
+    X = randn((T_, IN), dt, 0)
+    W1, b1 = randn((HID, IN), dt, 1, std=0.05), randn((HID,), dt, 2)
+    W2, b2 = randn((OUT, HID), dt, 3, std=0.05), randn((OUT,), dt, 4)
+    dY = randn((T_, OUT), dt, 5)
+    Xr, W1r, b1r, W2r, b2r = (_leaf(t) for t in (X, W1, b1, W2, b2))
+    ref = F.linear(F.gelu(F.linear(Xr, W1r, b1r), approximate="tanh"), W2r, b2r)
+    ref.backward(dY)
+    rows = lambda t, r: torch.chunk(t, p, dim=0)[r]   # noqa: E731  column-parallel: output features
+    cols = lambda t, r: torch.chunk(t, p, dim=-1)[r]  # noqa: E731  row-parallel: input features
+
+    initialize("1d", p, rank=rank)
+    col = Linear1D_Col(IN, HID, activation="gelu_tanh").to(DEV)
+    row = Linear1D_Row(HID, OUT).to(DEV)
+    assert col.weight.shape == (HID // p, IN) and col.bias.shape == (HID // p,)
+    assert row.weight.shape == (OUT, HID // p) and row.bias.shape == (OUT,)
+    with torch.no_grad():
+        col.weight.copy_(rows(W1, rank)); col.bias.copy_(rows(b1, rank))
+        row.weight.copy_(cols(W2, rank)); row.bias.copy_(b2)
+    d = lambda t: t.to(DEV)  # noqa: E731
+    mode = pm.PARALLEL_1D
+    h_other = F.gelu(F.linear(X, rows(W1, other), rows(b1, other)), approximate="tanh")
+    mode.stage("all_reduce", [d(h_other @ cols(W2, other).t())])          # the peer's partial product
+    x = _leaf(d(X))
+    y = row(col(x))
+    assert_parity(y, ref.detach(), dt, "Linear1D col->row forward", scale=10)
+    # backward: the peer's share of the input gradient arrives through the all-reduce of reduce_grad
+    pre_other = F.linear(X, rows(W1, other), rows(b1, other))
+    _g = _leaf(pre_other)
+    F.gelu(_g, approximate="tanh").backward(dY @ cols(W2, other))
+    mode.stage("all_reduce", [d(_g.grad @ rows(W1, other))])
+    y.backward(d(dY))
+    assert_parity(x.grad, Xr.grad, dt, "dX", scale=10)
+    assert_parity(col.weight.grad, rows(W1r.grad, rank), dt, "column-parallel dW shard", scale=10)
+    assert_parity(col.bias.grad, rows(b1r.grad, rank), dt, "column-parallel dbias shard", scale=30)
+    assert_parity(row.weight.grad, cols(W2r.grad, rank), dt, "row-parallel dW shard", scale=10)
+    assert_parity(row.bias.grad, b2r.grad, dt, "row-parallel dbias", scale=30)
+    assert not any(mode.inbox.values())
+
+
+def test_linear3d_one_rank_of_2x2x2_cube():
+    """Linear3D as rank (input 1, weight 0, output 1) of a depth-2 cube with the reference test's shard layout
+    (tests/test_3d/check_3d_modules.py:40-110: j = input rank, i = weight rank, k = output rank), every
+    gather / reduce-scatter the operator performs pre-staged from the master tensors."""
+    from cubework_amd.distributed import initialize
+    from cubework_amd.module.parallel_3d import Linear3D
+
+    dep, j, i, k = 2, 1, 0, 1
+    B_, S_, IN, OUT = 8, 4, 128, 256
+    dt = torch.float32
+    A_m = randn((B_, S_, IN), dt, 0)
+    W_m = randn((IN, OUT), dt, 1, std=0.05)
+    b_m = randn((OUT,), dt, 2)
+    G_m = randn((B_, S_, OUT), dt, 3)
+    ch = lambda t, dim, r: torch.chunk(t, dep, dim=dim)[r]  # noqa: E731
+    a_shard = lambda jj, ii, kk: ch(ch(ch(A_m, 0, ii), -1, kk), 0, jj)    # noqa: E731  [B/d^2, S, IN/d]
+    w_shard = lambda jj, ii, kk: ch(ch(ch(W_m, 0, kk), -1, jj), -1, ii)   # noqa: E731  [IN/d, OUT/d^2]
+    c_shard = lambda t, jj, ii, kk: ch(ch(ch(t, 0, ii), -1, jj), 0, kk)   # noqa: E731  [B/d^2, S, OUT/d]
+    a_rows = lambda ii, kk: ch(ch(A_m, 0, ii), -1, kk)                    # noqa: E731  gathered over the input group
+    w_blk = lambda jj, kk: ch(ch(W_m, 0, kk), -1, jj)                     # noqa: E731  gathered over the weight group
+    g_rows = lambda ii, jj: ch(ch(G_m, 0, ii), -1, jj)                    # noqa: E731  gathered over the output group
+
+    initialize("3d", dep ** 3, coords=(j, i, k))
+    layer = Linear3D(IN, OUT).to(DEV)
+    in_mode, w_mode, out_mode = layer.input_parallel_mode, layer.weight_parallel_mode, layer.output_parallel_mode
+    assert (in_mode.local_rank, w_mode.local_rank, out_mode.local_rank) == (j, i, k)
+    assert layer.weight.shape == (IN // dep, OUT // dep ** 2) and layer.bias.shape == (OUT // dep,)
+    with torch.no_grad():
+        layer.weight.copy_(w_shard(j, i, k))
+        layer.bias.copy_(ch(b_m, 0, j))
+    d = lambda t: t.to(DEV)  # noqa: E731
+    in_mode.stage("all_gather", [d(a_shard(jj, i, k)) for jj in range(dep)])
+    w_mode.stage("all_gather", [d(w_shard(j, ii, k)) for ii in range(dep)])
+    out_mode.stage("reduce_scatter", [d(a_rows(i, kk) @ w_blk(j, kk)) for kk in range(dep) if kk != k])
+    x = _leaf(d(a_shard(j, i, k)))
+    out = layer(x)
+    A_r, W_r, b_r = _leaf(A_m), _leaf(W_m), _leaf(b_m)
+    C_m = A_r @ W_r + b_r
+    C_m.backward(G_m)
+    assert_parity(out, c_shard(C_m.detach(), j, i, k), dt, "Linear3D forward shard", scale=10)
+
+    flat = lambda t: t.reshape(-1, t.shape[-1])  # noqa: E731
+    out_mode.stage("all_gather", [d(c_shard(G_m, j, i, kk)) for kk in range(dep)])
+    w_mode.stage("all_reduce", [d(flat(g_rows(ii, j)).sum(0)) for ii in range(dep) if ii != i])
+    w_mode.stage("reduce_scatter", [d(flat(a_rows(ii, k)).t() @ flat(g_rows(ii, j))) for ii in range(dep) if ii != i])
+    in_mode.stage("reduce_scatter", [d(g_rows(i, jj) @ w_blk(jj, k).t()) for jj in range(dep) if jj != j])
+    out.backward(d(c_shard(G_m, j, i, k)))
+    assert_parity(x.grad, a_shard_of(A_r.grad, dep, j, i, k), dt, "dA shard", scale=10)
+    assert_parity(layer.weight.grad, ch(ch(ch(W_r.grad, 0, k), -1, j), -1, i), dt, "dW shard", scale=10)
+    assert_parity(layer.bias.grad, ch(b_r.grad, 0, j), dt, "dbias shard", scale=30)
+    assert not any(in_mode.inbox.values()) and not any(w_mode.inbox.values()) and not any(out_mode.inbox.values())
+
+
+def test_layernorm3d_one_rank_of_2x2x2_cube():
+    """LayerNorm3D (two-pass statistics, parallel_3d/_operation.py:256-313) as rank (input 0, weight 1,
+    output 1) of a depth-2 cube with the shard layout of tests/test_3d/check_3d_modules.py:137-173: the
+    output-group peer holds the other half of every row, the other row shards contribute to dgamma / dbeta."""
+    import oracle
+    from cubework_amd.distributed import initialize
+    from cubework_amd.module.parallel_3d import LayerNorm3D
+
+    dep, j, i, k = 2, 0, 1, 1
+    R, H, eps = 16, 512, 1e-6
+    dt = torch.float32
+    A = randn((R, H), dt, 0)
+    dY = randn((R, H), dt, 1)
+    gamma = torch.rand(H, generator=torch.Generator().manual_seed(2)) * 0.2 + 0.9
+    beta = randn((H,), dt, 3, std=0.02)
+    ch = lambda t, dim, r: torch.chunk(t, dep, dim=dim)[r]  # noqa: E731
+    rows_of = lambda t, jj, ii: ch(ch(t, 0, ii), 0, jj)     # noqa: E731
+
+    initialize("3d", dep ** 3, coords=(j, i, k))
+    norm = LayerNorm3D(H, eps).to(DEV)
+    assert norm.weight.shape == (H // dep,)
+    with torch.no_grad():
+        norm.weight.copy_(ch(gamma, 0, k))
+        norm.bias.copy_(ch(beta, 0, k))
+    out_mode, ixw_mode = norm.output_parallel_mode, norm.input_x_weight_parallel_mode
+    d = lambda t: t.to(DEV)  # noqa: E731
+    my_rows, peer_k = rows_of(A, j, i), 1 - k
+    mean = my_rows.mean(-1)
+    out_mode.stage("all_reduce", [d(ch(my_rows, -1, peer_k).sum(-1))])                           # sum x
+    out_mode.stage("all_reduce", [d(((ch(my_rows, -1, peer_k) - mean[:, None]) ** 2).sum(-1))])  # sum (x - mean)^2
+    x = _leaf(d(ch(my_rows, -1, k)))
+    y = norm(x)
+    Ar, gr, br = _leaf(A), _leaf(gamma), _leaf(beta)
+    ref = F.layer_norm(Ar, (H,), gr, br, eps)
+    ref.backward(dY)
+    assert_parity(y, ch(rows_of(ref.detach(), j, i), -1, k), dt, "LayerNorm3D forward shard", scale=20)
+
+    var = A.var(-1, unbiased=False)
+    mr = torch.stack([A.mean(-1), 1.0 / torch.sqrt(var + eps)], dim=-1)
+    rs_peer, _, _ = oracle.ln2d_backward_partials(ch(rows_of(dY, j, i), -1, peer_k), ch(my_rows, -1, peer_k),
+                                                  rows_of(mr, j, i), ch(gamma, 0, peer_k))
+    out_mode.stage("all_reduce", [d(rs_peer)])
+    others = [(jj, ii) for jj in range(dep) for ii in range(dep) if (jj, ii) != (j, i)]
+    parts = [oracle.ln2d_backward_partials(ch(rows_of(dY, jj, ii), -1, k), ch(rows_of(A, jj, ii), -1, k),
+                                           rows_of(mr, jj, ii), ch(gamma, 0, k)) for jj, ii in others]
+    ixw_mode.stage("all_reduce", [d(p_[1]) for p_ in parts])
+    ixw_mode.stage("all_reduce", [d(p_[2]) for p_ in parts])
+    y.backward(d(ch(rows_of(dY, j, i), -1, k)))
+    assert_parity(x.grad, ch(rows_of(Ar.grad, j, i), -1, k), dt, "dX shard", scale=20)
+    assert_parity(norm.weight.grad, ch(gr.grad, 0, k), dt, "dgamma shard", scale=100)
+    assert_parity(norm.bias.grad, ch(br.grad, 0, k), dt, "dbeta shard", scale=100)
+    assert not any(out_mode.inbox.values()) and not any(ixw_mode.inbox.values())
+
+
+def a_shard_of(t, dep, j, i, k):
+    """The activation shard of rank (input j, weight i, output k): rows chunk i then j, columns chunk k."""
+    ch = lambda x, dim, r: torch.chunk(x, dep, dim=dim)[r]  # noqa: E731
+    return ch(ch(ch(t, 0, i), -1, k), 0, j)
 
 
 def test_linear2d_missing_peer_data_is_an_error():
