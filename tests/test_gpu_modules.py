@@ -372,6 +372,105 @@ def a_shard_of(t, dep, j, i, k):
     return ch(ch(ch(t, 0, i), -1, k), 0, j)
 
 
+def test_classifier2d_one_rank_of_2x2_grid():
+    """Classifier2D (parallel_2d/_operation.py:364-419) as rank (row 1, col 0) of a 2 x 2 grid with the shard
+    layout of tests/test_2d/check_2d_modules.py:345-403: the column peers' weight slices, the row peer's
+    partial product and the column peers' gradient contributions pre-staged."""
+    from oracle.grid import shard
+    from cubework_amd.distributed import initialize, pm
+    from cubework_amd.module.parallel_2d import Classifier2D
+
+    q, i, j = 2, 1, 0
+    B_, S_, IN, NC = 8, 4, 256, 40
+    dt = torch.float32
+    A_m = randn((B_ * S_, IN), dt, 0)
+    W_m = randn((NC, IN), dt, 1, std=0.05)
+    b_m = randn((NC,), dt, 2)
+    G_m = randn((B_ * S_, NC), dt, 3)
+    ch = lambda t, dim, r: torch.chunk(t, q, dim=dim)[r]  # noqa: E731
+    w_shard = lambda ii, jj: ch(ch(W_m, -1, jj), -1, ii)   # noqa: E731  [NC, IN/q^2]
+
+    initialize("2d", q * q, row=i, col=j)
+    head = Classifier2D(IN, NC).to(DEV)
+    assert head.weight.shape == (NC, IN // q ** 2) and head.bias.shape == (NC,)
+    with torch.no_grad():
+        head.weight.copy_(w_shard(i, j))
+        head.bias.copy_(b_m)
+    row, col = pm.PARALLEL_2D_ROW, pm.PARALLEL_2D_COL
+    d = lambda t: t.to(DEV)  # noqa: E731
+    col.stage("all_gather", [d(w_shard(ii, j)) for ii in range(q)])
+    row.stage("all_reduce", [d(shard(A_m, q, i, jj) @ ch(W_m, -1, jj).t()) for jj in range(q) if jj != j])
+    x = _leaf(d(shard(A_m, q, i, j)))
+    out = head(x)
+    Ar, Wr, br = _leaf(A_m), _leaf(W_m), _leaf(b_m)
+    C_m = F.linear(Ar, Wr, br)
+    C_m.backward(G_m)
+    assert_parity(out, ch(C_m.detach(), 0, i), dt, "Classifier2D forward rows", scale=10)
+    col.stage("reduce_scatter", [d(ch(G_m, 0, ii).t() @ shard(A_m, q, ii, j)) for ii in range(q) if ii != i])
+    col.stage("all_reduce", [d(ch(G_m, 0, ii).sum(0)) for ii in range(q) if ii != i])
+    out.backward(d(ch(G_m, 0, i)))
+    assert_parity(x.grad, shard(Ar.grad, q, i, j), dt, "dA shard", scale=10)
+    assert_parity(head.weight.grad, ch(ch(Wr.grad, -1, j), -1, i), dt, "dW shard", scale=10)
+    assert_parity(head.bias.grad, br.grad, dt, "dbias", scale=30)
+    assert not any(row.inbox.values()) and not any(col.inbox.values())
+
+
+@pytest.mark.parametrize("pos", [(0, 1), (1, 0)])
+def test_vocab_parallel_classifier2d_one_rank_of_2x2_grid(pos):
+    """VocabParallelClassifier2D (summa_ABT forward, summa_AB / summa_ATB backward: the lm head of the 2D
+    models) as one rank of a 2 x 2 grid with the shard layout of tests/test_2d/check_2d_modules.py:422-478."""
+    import oracle
+    from oracle.grid import bias_shard, shard
+    from cubework_amd.distributed import initialize, pm
+    from cubework_amd.module.parallel_2d import VocabParallelClassifier2D
+
+    q = 2
+    i, j = pos
+    oi, oj = 1 - i, 1 - j
+    T_, IN, V = 32, 256, 512
+    dt = torch.float32
+    A_m = randn((T_, IN), dt, 0)
+    W_m = randn((V, IN), dt, 1, std=0.05)
+    b_m = randn((V,), dt, 2)
+    G_m = randn((T_, V), dt, 3)
+    a, w, g_ = (lambda r, c: shard(A_m, q, r, c)), (lambda r, c: shard(W_m, q, r, c)), (lambda r, c: shard(G_m, q, r, c))  # noqa: E731
+
+    initialize("2d", q * q, row=i, col=j)
+    head = VocabParallelClassifier2D(IN, V).to(DEV)
+    assert head.weight.shape == (V // q, IN // q) and head.bias.shape == (V // q ** 2,)
+    with torch.no_grad():
+        head.weight.copy_(w(i, j))
+        head.bias.copy_(bias_shard(b_m, q, i, j))
+    row, col = pm.PARALLEL_2D_ROW, pm.PARALLEL_2D_COL
+    d = lambda t: t.to(DEV)  # noqa: E731
+    gemm = oracle.gemm_ksteps
+    # forward, summa_ABT: the weight block of the other grid row arrives by broadcast; my output block
+    # C[i, j] = sum_k A[i, k] W[j, k]^T collects the row peer's product
+    col.stage("broadcast", d(w(oi, j)))
+    row.stage("reduce", [d(gemm("NT", [a(i, oj)], [w(j, oj)]))])
+    gathered = [None, None]
+    gathered[oi] = d(bias_shard(b_m, q, oi, j))
+    col.stage("all_gather", gathered)
+    x = _leaf(d(a(i, j)))
+    out = head(x)
+    Ar, Wr, br = _leaf(A_m), _leaf(W_m), _leaf(b_m)
+    C_m = F.linear(Ar, Wr, br)
+    C_m.backward(G_m)
+    assert_parity(out, shard(C_m.detach(), q, i, j), dt, "logits shard", scale=10)
+    # backward: bias column sums of the column peer; summa_AB (dA[i, j] = sum_t G[i, t] W[t, j]) and
+    # summa_ATB (dW[i, j] = sum_t G[t, i]^T A[t, j]) with their broadcasts and the column peer's product
+    col.stage("reduce_scatter", [d(oracle.colsum(g_(oi, j)))])
+    row.stage("broadcast", d(g_(i, oj)))
+    col.stage("broadcast", d(w(oi, j)))
+    row.stage("broadcast", d(g_(i, oj)))
+    col.stage("reduce", [d(gemm("TN", [g_(oi, i)], [a(oi, j)]))])
+    out.backward(d(g_(i, j)))
+    assert_parity(x.grad, shard(Ar.grad, q, i, j), dt, "dA shard", scale=10)
+    assert_parity(head.weight.grad, shard(Wr.grad, q, i, j), dt, "dW shard", scale=10)
+    assert_parity(head.bias.grad, bias_shard(br.grad, q, i, j), dt, "dbias shard", scale=30)
+    assert not any(row.inbox.values()) and not any(col.inbox.values())
+
+
 def test_linear2d_missing_peer_data_is_an_error():
     from cubework_amd.distributed import MissingPeerData, initialize
     from cubework_amd.module.parallel_2d import Linear2D
