@@ -559,6 +559,38 @@ def test_vocab_parallel_loss_one_rank_of_four(dtype):
     assert torch.equal(x.detach(), before), "the caller's logits must stay intact"
 
 
+def test_vocab_parallel_loss2d_one_rank_of_2x2_grid():
+    """VocabParallelCrossEntropyLoss2D as rank (row 1, col 0) of a 2 x 2 grid
+    (tests/test_2d/check_2d_modules.py:635-661): the classes are split over the grid columns, the tokens over
+    the grid rows; the row peer's per-token statistics and the column peer's mean loss are pre-staged."""
+    import oracle
+    from oracle.grid import shard
+    from cubework_amd.distributed import initialize, pm
+    from cubework_amd.module.loss import VocabParallelCrossEntropyLoss2D
+
+    q, i, j = 2, 1, 0
+    oi, oj = 1 - i, 1 - j
+    T, V = 64, 600
+    dt = torch.float32
+    full = randn((T, V), dt, 0, std=2.0)
+    t = torch.randint(0, V, (T,), generator=torch.Generator().manual_seed(1))
+    t_rows = torch.chunk(t, q)[i]
+    initialize("2d", q * q, row=i, col=j)
+    peer = oracle.vpce_fwd_local(shard(full, q, i, oj), t_rows, oj * (V // q))
+    pm.PARALLEL_2D_ROW.stage("vpce_stats", [pk.unsqueeze(0).to(DEV) for pk in peer])
+    pm.PARALLEL_2D_COL.stage("all_reduce", [F.cross_entropy(torch.chunk(full, q)[oi], torch.chunk(t, q)[oi]).to(DEV)])
+    crit = VocabParallelCrossEntropyLoss2D()
+    x = _leaf(shard(full, q, i, j).contiguous().to(DEV))
+    loss = crit(x, t.to(DEV))
+    loss.backward()
+    fr = _leaf(full)
+    ref = F.cross_entropy(fr, t)
+    ref.backward()
+    assert_parity(loss, ref.detach(), dt, "mean loss", scale=10)
+    assert_parity(x.grad, shard(fr.grad, q, i, j), dt, "logits grad shard", scale=10)
+    assert not any(pm.PARALLEL_2D_ROW.inbox.values()) and not any(pm.PARALLEL_2D_COL.inbox.values())
+
+
 @pytest.mark.parametrize("amp_dtype", [torch.float16, torch.bfloat16])
 def test_opt_block_under_autocast(amp_dtype):
     """fp32 parameters and input inside torch.autocast, as the reference's training scripts run
