@@ -8,8 +8,18 @@
 // two tiles per compute unit: both are then resident at once and no partial
 // last round of tiles remains (config-1 forward: 1024 tiles of 128x128 are
 // 1 1/3 rounds of the 768 that fit).
+//
+// Large aligned problems (at least 128 tiles of 256x256) take gemm_f32_ring_kernel instead: the ring of LDS
+// stages filled by the load unit that the 16-bit kernel uses (gemm_bf16_dma.h), with a k extent of 16 per
+// stage. There is no register staging, no LDS write instruction and no fragment read right behind the
+// barrier, so a wavefront arrives at the one barrier per stage with the next products' operands already
+// in registers.
+#include <cstdlib>
+#include <cstring>
+
 #include "cw_common.h"
 #include "gemm.h"
+#include "gemm_bf16_kernel.h"
 
 namespace cw {
 
@@ -266,6 +276,303 @@ __global__ __launch_bounds__(kFThreads, BM == 256 ? 2 : 3) void gemm_f32_kernel(
     }
 }
 
+// ---------------------------------------------------------------------------------------------------
+// Ring kernel: 256x256 tile per 256-thread block (2x2 wavefronts of 128x128 = 4x4 MFMA blocks, 256
+// accumulators per lane), NS stages of k = 16 in LDS (16 KB per operand and stage), filled by
+// global_load_lds_dwordx4 (lane l writes LDS bytes [16 l, 16 l + 16) of the instruction's 1 KB, so an
+// image's swizzle is applied on the global side).
+//   k-contiguous operand ([rows][k] in memory): image [256 rows][16 k], 64 B per row, 16-byte chunk c of
+//     row r at position c ^ ((r >> 2) & 3); a lane reads its row's k = 4h .. 4h+3 and 8+4h .. 8+4h+3
+//     (h = lane / 32) with two ds_read_b128;
+//   k-slow operand ([k][rows] in memory): image [16 k][256 rows], 1 KB per k row, the 128-byte group g of
+//     k row k at position g ^ ((k >> 2) & 1), which puts the two half-wavefronts of a read (k rows 4 apart)
+//     on different banks; one ds_read_b32 per product.
+// Both kinds consume k in the order k(s, h) = 4h + s (s < 4), 8 + 4h + (s - 4): steps 0..3 ("lo") and 4..7
+// ("hi") of a stage. Per stage: products of lo, barrier, products of hi; the hi operands are read during
+// the lo products and the next stage's lo operands during the hi products, the eight load instructions of
+// the tile NS-1 ahead are spread over both. The loads are inline asm and counted by hand (dma_wait), as in
+// the 16-bit kernel.
+namespace ring {
+
+typedef __attribute__((address_space(3))) char lds_char;
+typedef float f32x4_t __attribute__((ext_vector_type(4)));
+constexpr int kTile = 256, kBK = 16, kThreads = 256, kStages = 4;
+constexpr int kOperBytes = kTile * kBK * 4;  // 16384
+constexpr int kStageBytes = 2 * kOperBytes;
+constexpr int kDmaPerTile = 8;
+
+__device__ __forceinline__ void dma16(const char* gbase, uint32_t voff, uint32_t lds_addr) {
+    asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, %2" : : "s"(lds_addr), "v"(voff), "s"(gbase) : "memory", "m0");
+}
+template <int N>
+__device__ __forceinline__ void dma_wait() {
+    asm volatile("s_waitcnt vmcnt(%0)" : : "n"(N) : "memory");
+}
+
+// Byte offset, inside the span of one load instruction, of the 16 bytes this lane fetches.
+template <bool KSLOW>
+__device__ __forceinline__ uint32_t lane_voff(int lane, int wave, int64_t ld, int row0) {
+    if constexpr (!KSLOW) {
+        const int r = lane >> 2, c = (lane & 3) ^ (lane >> 4);  // 16 rows x 64 B; swizzle (row >> 2) & 3 = lane >> 4
+        return (uint32_t)((((int64_t)(row0 + r)) * ld + c * 4) * 4);
+    } else {
+        const int c = lane ^ ((wave & 1) << 3);  // k row = 4 wave + I: (k >> 2) & 1 = wave & 1
+        return (uint32_t)((row0 + 4 * c) * 4);
+    }
+}
+// Load instruction I (of 4) of this wavefront for one operand of the tile at k0.
+template <bool KSLOW, int I>
+__device__ __forceinline__ void dma_one(const char* gbase, int64_t ld_bytes, int k0, uint32_t voff, uint32_t lds_oper, int wave) {
+    if constexpr (!KSLOW) {
+        const int row = wave * 64 + I * 16;
+        dma16(gbase + ((int64_t)row * ld_bytes + (int64_t)k0 * 4), voff, lds_oper + row * 64);
+    } else {
+        const int k = wave * 4 + I;
+        dma16(gbase + (int64_t)(k0 + k) * ld_bytes, voff, lds_oper + k * 1024);
+    }
+}
+
+// Operand values of one half stage: v[block of 32 rows][step].
+struct Frag {
+    float v[4][4];
+};
+
+template <bool KSLOW>
+struct Reader {
+    uint32_t off[4];  // k-contiguous: [0] lo, [1] hi; k-slow: [block]
+    __device__ __forceinline__ void init(int lane, int wrow) {
+        const int r = lane & 31, h = lane >> 5;
+        if constexpr (!KSLOW) {
+            const int swz = (r >> 2) & 3;
+            off[0] = (uint32_t)((wrow + r) * 64 + ((h ^ swz) << 4));
+            off[1] = (uint32_t)((wrow + r) * 64 + (((2 + h) ^ swz) << 4));
+            off[2] = off[3] = 0;
+        } else {
+#pragma unroll
+            for (int t = 0; t < 4; ++t) off[t] = (uint32_t)(4 * h * 1024 + (((wrow >> 5) + (t ^ h)) << 7) + r * 4);
+        }
+    }
+    // Read number Q of a half stage (HI: steps 4..7) into f: 4 reads (one per block) for a k-contiguous
+    // operand, 16 (block Q / 4, step Q % 4) for a k-slow one.
+    template <int Q, bool HI>
+    __device__ __forceinline__ void read(lds_char* oper, Frag& f) const {
+        if constexpr (!KSLOW) {
+            const f32x4_t x = *(__attribute__((address_space(3))) const f32x4_t*)(oper + off[HI ? 1 : 0] + Q * 2048);
+            f.v[Q][0] = x[0]; f.v[Q][1] = x[1]; f.v[Q][2] = x[2]; f.v[Q][3] = x[3];
+        } else {
+            constexpr int T = Q >> 2, S = Q & 3;
+            f.v[T][S] = *(__attribute__((address_space(3))) const float*)(oper + off[T] + ((HI ? 8 : 0) + S) * 1024);
+        }
+    }
+    static constexpr int kReads = KSLOW ? 16 : 4;
+};
+
+#define CW_F32_PIN() __builtin_amdgcn_sched_barrier(0)
+
+// One 32 x 32 block of the result through a wavefront-private LDS patch (as f32_store_block), activation
+// chosen at run time; whole tile in bounds, 16-byte aligned rows.
+__device__ __forceinline__ void store_block(const f32x16_t& blk, float* patch, const RingArgs& args, int epilogue, int row0,
+                                            int col0, int lane) {
+#pragma unroll
+    for (int v = 0; v < 16; ++v) patch[(8 * (v >> 2) + 4 * (lane >> 5) + (v & 3)) * kPatchPitch + (lane & 31)] = blk[v];
+    const int c4 = 4 * (lane & 7);
+    const int col = col0 + c4;
+    float4 bv = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+    if (epilogue != CW_EPI_NONE && args.bias != nullptr) bv = *reinterpret_cast<const float4*>(reinterpret_cast<const float*>(args.bias) + col);
+    float* C = reinterpret_cast<float*>(args.C);
+    float* P = reinterpret_cast<float*>(args.preact);
+#pragma unroll
+    for (int pass = 0; pass < 4; ++pass) {
+        const int r = (lane >> 3) + 8 * pass;
+        const int64_t row = row0 + r;
+        const float4 t = *reinterpret_cast<const float4*>(patch + r * kPatchPitch + c4);
+        float x[4] = {t.x + bv.x, t.y + bv.y, t.z + bv.z, t.w + bv.w};
+#pragma unroll 1
+        for (int a = 0; a < args.n_addends; ++a) {
+            const float4 ad = *reinterpret_cast<const float4*>(reinterpret_cast<const float*>(gemm_bf16::pick_ptr(args.addend, a)) + row * args.ldadd + col);
+            x[0] += ad.x; x[1] += ad.y; x[2] += ad.z; x[3] += ad.w;
+        }
+        if (P != nullptr) *reinterpret_cast<float4*>(P + row * args.ldp + col) = make_float4(x[0], x[1], x[2], x[3]);
+        if (epilogue == CW_EPI_BIAS_GELU_TANH) {
+#pragma unroll
+            for (int e = 0; e < 4; ++e) x[e] = gelu_tanh(x[e]);
+        } else if (epilogue == CW_EPI_BIAS_GELU_ERF) {
+#pragma unroll
+            for (int e = 0; e < 4; ++e) x[e] = gelu_erf(x[e]);
+        } else if (epilogue == CW_EPI_BIAS_RELU) {
+#pragma unroll
+            for (int e = 0; e < 4; ++e) x[e] = x[e] < 0.0f ? 0.0f : x[e];  // NaN stays NaN, as torch.relu leaves it
+        }
+        *reinterpret_cast<float4*>(C + row * args.ldc + col) = make_float4(x[0], x[1], x[2], x[3]);
+    }
+}
+
+template <bool A_KSLOW, bool B_KSLOW>
+__global__ __launch_bounds__(kThreads) void gemm_f32_ring_kernel(const RingArgs args, int epilogue) {
+    constexpr int NS = kStages;
+    extern __shared__ __attribute__((aligned(16))) float lds_f[];
+    lds_char* lds_base = (lds_char*)lds_f;
+    const uint32_t lds_addr0 = (uint32_t)(uintptr_t)lds_base;
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int wm = wave >> 1, wn = wave & 1;
+    const int M = args.M, N = args.N, K = args.K;
+    // the last tile of a row or column of tiles is moved back to end at the edge (it overlaps its neighbour;
+    // both compute the shared elements from the same operands in the same order)
+    const int tiles_m = (M + kTile - 1) / kTile, tiles_n = (N + kTile - 1) / kTile;
+    const int total = tiles_m * tiles_n;
+    int tile;
+    {
+        const int pid = blockIdx.x;
+        const int per_xcd = (total + 7) / 8;
+        tile = (pid & 7) * per_xcd + (pid >> 3);
+        if (tile >= total) return;
+    }
+    constexpr int GROUP_M = 8;
+    const int group = tile / (GROUP_M * tiles_n);
+    const int first_m = group * GROUP_M;
+    const int gsz = (tiles_m - first_m) < GROUP_M ? (tiles_m - first_m) : GROUP_M;
+    const int in_group = tile - group * GROUP_M * tiles_n;
+    int m0 = (first_m + in_group % gsz) * kTile;
+    int n0 = (in_group / gsz) * kTile;
+    m0 = m0 + kTile > M ? M - kTile : m0;
+    n0 = n0 + kTile > N ? N - kTile : n0;
+
+    const int kt_per_step = K / kBK;
+    const int KT = kt_per_step * args.n_steps;
+    const uint32_t a_voff = lane_voff<A_KSLOW>(lane, wave, args.lda, m0);
+    const uint32_t b_voff = lane_voff<B_KSLOW>(lane, wave, args.ldb, n0);
+    const int64_t lda_bytes = args.lda * 4, ldb_bytes = args.ldb * 4;
+
+    Reader<A_KSLOW> ra;
+    Reader<B_KSLOW> rb;
+    ra.init(lane, wm * 128);
+    rb.init(lane, wn * 128);
+
+    f32x16_t acc[4][4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+#pragma unroll
+            for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.0f;
+
+    // the tile whose loads are issued next; past the last tile the position stays on it (harmless duplicate
+    // loads into a free stage keep the load counting the same in every iteration)
+    int is_kt = 0, is_step = 0, is_k0 = 0, is_stage = 0;
+    const char* is_a = reinterpret_cast<const char*>(args.A[0]);
+    const char* is_b = reinterpret_cast<const char*>(args.B[0]);
+    auto issue_advance = [&]() {
+        if (is_kt + 1 < KT) {
+            ++is_kt;
+            is_k0 += kBK;
+            if (is_k0 >= K) {
+                is_k0 = 0;
+                ++is_step;
+                is_a = reinterpret_cast<const char*>(gemm_bf16::pick_ptr(args.A, is_step));
+                is_b = reinterpret_cast<const char*>(gemm_bf16::pick_ptr(args.B, is_step));
+            }
+        }
+        is_stage = (is_stage + 1 == NS) ? 0 : is_stage + 1;
+    };
+
+    // prologue: tiles 0 .. NS-3 in flight, plus the A part of tile NS-2
+    for (int p = 0; p < NS - 2; ++p) {
+        const uint32_t st = lds_addr0 + is_stage * kStageBytes;
+        gemm_bf16::static_for<4>([&](auto I) {
+            dma_one<A_KSLOW, I.value>(is_a, lda_bytes, is_k0, a_voff, st, wave);
+            dma_one<B_KSLOW, I.value>(is_b, ldb_bytes, is_k0, b_voff, st + kOperBytes, wave);
+        });
+        issue_advance();
+    }
+    {
+        const uint32_t st = lds_addr0 + is_stage * kStageBytes;
+        gemm_bf16::static_for<4>([&](auto I) { dma_one<A_KSLOW, I.value>(is_a, lda_bytes, is_k0, a_voff, st, wave); });
+    }
+    dma_wait<kDmaPerTile*(NS - 3) + 4>();
+    __builtin_amdgcn_s_barrier();
+    asm volatile("" ::: "memory");
+
+    Frag a_lo, a_hi, b_lo, b_hi;
+    gemm_bf16::static_for<Reader<A_KSLOW>::kReads>([&](auto q) { ra.template read<q.value, false>(lds_base, a_lo); });
+    gemm_bf16::static_for<Reader<B_KSLOW>::kReads>([&](auto q) { rb.template read<q.value, false>(lds_base + kOperBytes, b_lo); });
+
+    constexpr int NRA = Reader<A_KSLOW>::kReads, NRB = Reader<B_KSLOW>::kReads;
+    int cur = 0;
+    for (int kt = 0; kt < KT; ++kt) {
+        lds_char* sa = lds_base + cur * kStageBytes;
+        lds_char* sb = sa + kOperBytes;
+        const int nxt = (cur + 1 == NS) ? 0 : cur + 1;
+        lds_char* na = lds_base + nxt * kStageBytes;
+        lds_char* nb = na + kOperBytes;
+
+        // ---- products of steps 0..3; behind them the reads of steps 4..7 and the B part of the tile whose
+        //      A part went out in the previous iteration
+        CW_F32_PIN();
+        {
+            const uint32_t st = lds_addr0 + is_stage * kStageBytes;
+            gemm_bf16::static_for<64>([&](auto qq) {
+                constexpr int Q = qq.value, S = Q >> 4, I = (Q >> 2) & 3, J = Q & 3;
+                acc[I][J] = __builtin_amdgcn_mfma_f32_32x32x2f32(a_lo.v[I][S], b_lo.v[J][S], acc[I][J], 0, 0, 0);
+                if constexpr (Q < NRA) ra.template read<Q, true>(sa, a_hi);
+                else if constexpr (Q < NRA + NRB) rb.template read<Q - NRA, true>(sb, b_hi);
+                else if constexpr (Q < NRA + NRB + 4) dma_one<B_KSLOW, Q - NRA - NRB>(is_b, ldb_bytes, is_k0, b_voff, st + kOperBytes, wave);
+                CW_F32_PIN();
+            });
+            issue_advance();
+        }
+        // ---- tile kt+1 complete for everybody, stage of tile kt-1 free
+        dma_wait<kDmaPerTile*(NS - 3)>();
+        __builtin_amdgcn_s_barrier();
+        asm volatile("" ::: "memory");
+        CW_F32_PIN();
+        // ---- products of steps 4..7; behind them the A part of tile kt+NS-1 and the reads of (kt+1, steps 0..3)
+        {
+            const uint32_t st = lds_addr0 + is_stage * kStageBytes;
+            gemm_bf16::static_for<64>([&](auto qq) {
+                constexpr int Q = qq.value, S = Q >> 4, I = (Q >> 2) & 3, J = Q & 3;
+                acc[I][J] = __builtin_amdgcn_mfma_f32_32x32x2f32(a_hi.v[I][S], b_hi.v[J][S], acc[I][J], 0, 0, 0);
+                if constexpr (Q < 4) dma_one<A_KSLOW, Q>(is_a, lda_bytes, is_k0, a_voff, st, wave);
+                else if constexpr (Q < 4 + NRA) ra.template read<Q - 4, false>(na, a_lo);
+                else if constexpr (Q < 4 + NRA + NRB) rb.template read<Q - 4 - NRA, false>(nb, b_lo);
+                CW_F32_PIN();
+            });
+        }
+        cur = nxt;
+    }
+    dma_wait<0>();
+    __syncthreads();
+    // acc[i][j][v]: row m0 + wm*128 + i*32 + 8 (v/4) + 4 (lane/32) + v%4, column n0 + wn*128 + j*32 + lane%32
+    float* patch = lds_f + wave * 32 * kPatchPitch;
+    gemm_bf16::static_for<16>([&](auto b) {
+        constexpr int I = b.value >> 2, J = b.value & 3;
+        store_block(acc[I][J], patch, args, epilogue, m0 + wm * 128 + I * 32, n0 + wn * 128 + J * 32, lane);
+    });
+}
+
+template <bool AS, bool BS>
+int launch(const GemmArgs& g, int epilogue, hipStream_t s) {
+    RingArgs r = {};
+    for (int i = 0; i < g.n_steps && i < kRingMaxSteps; ++i) { r.A[i] = g.A[i]; r.B[i] = g.B[i]; }
+    for (int i = 0; i < g.n_addends && i < kRingMaxAddends; ++i) r.addend[i] = g.addend[i];
+    r.bias = g.bias; r.C = g.C; r.preact = g.preact;
+    r.lda = g.lda; r.ldb = g.ldb; r.ldc = g.ldc; r.ldp = g.ldp; r.ldadd = g.ldadd;
+    r.M = g.M; r.N = g.N; r.K = g.K; r.n_steps = g.n_steps; r.n_addends = g.n_addends;
+    r.vec_bias = 1; r.vec_add = 1; r.k_tail = 0; r.partial = nullptr;
+    auto kern = gemm_f32_ring_kernel<AS, BS>;
+    constexpr int lds = kStages * kStageBytes;
+    static_assert(lds <= 160 * 1024, "LDS image does not fit the CU");
+    hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, lds);
+    if (e != hipSuccess) return fail(CW_ERR_LAUNCH, "hipFuncSetAttribute(gemm_f32_ring): %s", hipGetErrorString(e));
+    const int tiles = ((g.M + kTile - 1) / kTile) * ((g.N + kTile - 1) / kTile);
+    hipLaunchKernelGGL(kern, dim3(((tiles + 7) / 8) * 8), dim3(kThreads), lds, s, r, epilogue);
+    return check_launch("gemm_f32_ring_kernel");
+}
+
+}  // namespace ring
+
 template <int BM, bool AK, bool BK_, bool GUARD>
 int launch_f32(const GemmArgs& args, int epilogue, hipStream_t s) {
     const int tiles = ((args.M + BM - 1) / BM) * ((args.N + kFBN - 1) / kFBN);
@@ -289,6 +596,30 @@ int launch_f32_layout(const GemmArgs& args, int layout, int epilogue, hipStream_
 int gemm_f32_launch(const GemmArgs& args, int layout, int epilogue, hipStream_t s) {
     if (epilogue < CW_EPI_NONE || epilogue > CW_EPI_BIAS_RELU)
         return fail(CW_ERR_INVALID, "cw_gemm_ksteps: bad epilogue %d", epilogue);
+    // ring kernel: many 256x256 tiles, every pointer and leading dimension good for 16-byte accesses, the
+    // reduction a multiple of the stage's k extent, byte offsets within 32 bits
+    {
+        const int64_t tiles256 = ((int64_t)(args.M + 255) / 256) * ((args.N + 255) / 256);
+        const int64_t max_dim = args.M > args.N ? (args.M > args.K ? args.M : args.K) : (args.N > args.K ? args.N : args.K);
+        const bool fits32 = (max_dim + 64) * (args.lda > args.ldb ? args.lda : args.ldb) * 4 < ((int64_t)1 << 32);
+        const bool all_vec = args.vec_a && args.vec_b && args.vec_c && (args.preact == nullptr || args.vec_p) &&
+                             (args.n_addends == 0 || args.vec_add) &&
+                             (args.bias == nullptr || (reinterpret_cast<uintptr_t>(args.bias) & 15u) == 0);
+        static const bool ring_enabled = [] {
+            const char* v = std::getenv("CW_GEMM_IMPL");
+            return !(v != nullptr && std::strcmp(v, "staged") == 0);
+        }();
+        if (ring_enabled && tiles256 >= 128 && all_vec && fits32 && args.M >= 256 && args.N >= 256 && (args.N % 4) == 0 &&
+            (layout != CW_TN || (args.M % 4) == 0) && args.K >= ring::kBK && (args.K % ring::kBK) == 0 && args.n_steps >= 1 &&
+            args.n_steps <= kRingMaxSteps && args.n_addends <= kRingMaxAddends) {
+            switch (layout) {
+                case CW_NN: return ring::launch<false, true>(args, epilogue, s);
+                case CW_NT: return ring::launch<false, false>(args, epilogue, s);
+                case CW_TN: return ring::launch<true, true>(args, epilogue, s);
+                default: return fail(CW_ERR_INVALID, "cw_gemm_ksteps: bad layout %d", layout);
+            }
+        }
+    }
     const bool vec = args.vec_a && args.vec_b && (args.N % kFBN) == 0 && (args.K % kFBK) == 0;
     // 256-row tiles when they still give every compute unit two tiles
     const int64_t tall_tiles = ((int64_t)(args.M + 255) / 256) * ((args.N + kFBN - 1) / kFBN);

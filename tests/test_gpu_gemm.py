@@ -143,6 +143,18 @@ def test_fp32_tall_tiles(layout):
     _run(layout, 4100, 4104, 40, 1, torch.float32, act="relu", n_add=1, preact=True, seed=17)
 
 
+@pytest.mark.parametrize("layout", LAYOUTS)
+def test_fp32_ring_kernel(layout):
+    """fp32 outputs of at least 128 tiles of 256 x 256 with aligned operands: the LDS-ring kernel. Several
+    k-steps (the ring runs across the seam between two steps' allocations), addend, pre-activation copy and
+    activation; the shortest reduction the ring takes (one stage); M and N that are not tile multiples
+    (last tiles moved back to the edge); padded leading dimensions."""
+    _run(layout, 4096, 2048, 64, 3, torch.float32, act="gelu_tanh", n_add=1, preact=True, seed=21)
+    _run(layout, 2048, 4096, 16, 1, torch.float32, act=None, bias=False, seed=22)
+    _run(layout, 4104, 2060, 48, 2, torch.float32, act="relu", n_add=2, preact=True, seed=23)
+    _run(layout, 4096, 2048, 32, 1, torch.float32, act="gelu_erf", pad_a=4, pad_b=8, seed=24)
+
+
 def test_fp32_linear1d_col_shape():
     # BASELINE config 1: x [8,512,1024] fp32, W [4096,1024], b zeros -> F.linear
     import oracle
