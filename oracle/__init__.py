@@ -15,6 +15,8 @@ line by line in torch, and is pinned by
   * torch library routines the reference's tests use as their own oracle
     (A @ W + b, nn.LayerNorm, F.cross_entropy),
   * for the attention core: pure-Python float64 loops, F.scaled_dot_product_attention and its autograd,
+  * for the OPT decoder layer: the composition of the functions above, its residual paths (identity with
+    zeroed branch outputs), causality, and the agreement of both weight orientations,
   * invariants (split-invariance of statistics, sum of softmax gradient = 0,
     k-step sum == concatenated GEMM, grid composition == master result).
 Parity status: every function below is pinned by at least one such check in
