@@ -278,7 +278,8 @@ __global__ __launch_bounds__(kFThreads, BM == 256 ? 2 : 3) void gemm_f32_kernel(
 
 // ---------------------------------------------------------------------------------------------------
 // Ring kernel: 256x256 tile per 256-thread block (2x2 wavefronts of 128x128 = 4x4 MFMA blocks, 256
-// accumulators per lane), NS stages of k = 16 in LDS (16 KB per operand and stage), filled by
+// accumulators per lane; 128x128 and 128x64 tiles, two workgroups per compute unit, for outputs with fewer
+// tiles), NS stages of k = 16 in LDS (64 bytes per row, operand and stage), filled by
 // global_load_lds_dwordx4 (lane l writes LDS bytes [16 l, 16 l + 16) of the instruction's 1 KB, so an
 // image's swizzle is applied on the global side).
 //   k-contiguous operand ([rows][k] in memory): image [256 rows][16 k], 64 B per row, 16-byte chunk c of
@@ -296,10 +297,10 @@ namespace ring {
 
 typedef __attribute__((address_space(3))) char lds_char;
 typedef float f32x4_t __attribute__((ext_vector_type(4)));
-constexpr int kTile = 256, kBK = 16, kThreads = 256, kStages = 4;
-constexpr int kOperBytes = kTile * kBK * 4;  // 16384
-constexpr int kStageBytes = 2 * kOperBytes;
-constexpr int kDmaPerTile = 8;
+constexpr int kBK = 16, kThreads = 256, kStages = 4;
+// A tile is 64 TI x 64 TJ (TI, TJ in {1, 2, 4}): 2x2 wavefronts of TI x TJ blocks of 32 x 32. An operand of
+// ROWS = 64 T rows takes ROWS * 64 bytes per stage and T load instructions per wavefront.
+constexpr int oper_bytes(int t) { return 64 * t * kBK * 4; }
 
 __device__ __forceinline__ void dma16(const char* gbase, uint32_t voff, uint32_t lds_addr) {
     asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, %2" : : "s"(lds_addr), "v"(voff), "s"(gbase) : "memory", "m0");
@@ -310,25 +311,28 @@ __device__ __forceinline__ void dma_wait() {
 }
 
 // Byte offset, inside the span of one load instruction, of the 16 bytes this lane fetches.
-template <bool KSLOW>
+template <bool KSLOW, int T>
 __device__ __forceinline__ uint32_t lane_voff(int lane, int wave, int64_t ld, int row0) {
     if constexpr (!KSLOW) {
         const int r = lane >> 2, c = (lane & 3) ^ (lane >> 4);  // 16 rows x 64 B; swizzle (row >> 2) & 3 = lane >> 4
         return (uint32_t)((((int64_t)(row0 + r)) * ld + c * 4) * 4);
     } else {
-        const int c = lane ^ ((wave & 1) << 3);  // k row = 4 wave + I: (k >> 2) & 1 = wave & 1
-        return (uint32_t)((row0 + 4 * c) * 4);
+        // an instruction's 1 KB holds 4 / T k rows of 16 T chunks; the wavefront's T instructions cover
+        // k rows 4 wave .. 4 wave + 3, so (k >> 2) & 1 = wave & 1
+        constexpr int kChunks = 16 * T;
+        const int kr = lane / kChunks, c = (lane % kChunks) ^ ((wave & 1) << 3);
+        return (uint32_t)((((int64_t)kr) * ld + row0 + 4 * c) * 4);
     }
 }
-// Load instruction I (of 4) of this wavefront for one operand of the tile at k0.
-template <bool KSLOW, int I>
+// Load instruction I (of T) of this wavefront for one operand (64 T rows) of the tile at k0.
+template <bool KSLOW, int T, int I>
 __device__ __forceinline__ void dma_one(const char* gbase, int64_t ld_bytes, int k0, uint32_t voff, uint32_t lds_oper, int wave) {
     if constexpr (!KSLOW) {
-        const int row = wave * 64 + I * 16;
+        const int row = (wave * T + I) * 16;
         dma16(gbase + ((int64_t)row * ld_bytes + (int64_t)k0 * 4), voff, lds_oper + row * 64);
     } else {
-        const int k = wave * 4 + I;
-        dma16(gbase + (int64_t)(k0 + k) * ld_bytes, voff, lds_oper + k * 1024);
+        const int k = wave * 4 + I * (4 / T);
+        dma16(gbase + (int64_t)(k0 + k) * ld_bytes, voff, lds_oper + k * (256 * T));
     }
 }
 
@@ -337,7 +341,7 @@ struct Frag {
     float v[4][4];
 };
 
-template <bool KSLOW>
+template <bool KSLOW, int T>
 struct Reader {
     uint32_t off[4];  // k-contiguous: [0] lo, [1] hi; k-slow: [block]
     __device__ __forceinline__ void init(int lane, int wrow) {
@@ -349,22 +353,22 @@ struct Reader {
             off[2] = off[3] = 0;
         } else {
 #pragma unroll
-            for (int t = 0; t < 4; ++t) off[t] = (uint32_t)(4 * h * 1024 + (((wrow >> 5) + (t ^ h)) << 7) + r * 4);
+            for (int t = 0; t < 4; ++t) off[t] = (uint32_t)(4 * h * (256 * T) + ((((wrow >> 5) + t) ^ h) << 7) + r * 4);
         }
     }
-    // Read number Q of a half stage (HI: steps 4..7) into f: 4 reads (one per block) for a k-contiguous
-    // operand, 16 (block Q / 4, step Q % 4) for a k-slow one.
+    // Read number Q of a half stage (HI: steps 4..7) into f: T reads (one per block) for a k-contiguous
+    // operand, 4 T (block Q / 4, step Q % 4) for a k-slow one.
     template <int Q, bool HI>
     __device__ __forceinline__ void read(lds_char* oper, Frag& f) const {
         if constexpr (!KSLOW) {
             const f32x4_t x = *(__attribute__((address_space(3))) const f32x4_t*)(oper + off[HI ? 1 : 0] + Q * 2048);
             f.v[Q][0] = x[0]; f.v[Q][1] = x[1]; f.v[Q][2] = x[2]; f.v[Q][3] = x[3];
         } else {
-            constexpr int T = Q >> 2, S = Q & 3;
-            f.v[T][S] = *(__attribute__((address_space(3))) const float*)(oper + off[T] + ((HI ? 8 : 0) + S) * 1024);
+            constexpr int B = Q >> 2, S = Q & 3;
+            f.v[B][S] = *(__attribute__((address_space(3))) const float*)(oper + off[B] + ((HI ? 8 : 0) + S) * (256 * T));
         }
     }
-    static constexpr int kReads = KSLOW ? 16 : 4;
+    static constexpr int kReads = KSLOW ? 4 * T : T;
 };
 
 #define CW_F32_PIN() __builtin_amdgcn_sched_barrier(0)
@@ -407,9 +411,12 @@ __device__ __forceinline__ void store_block(const f32x16_t& blk, float* patch, c
     }
 }
 
-template <bool A_KSLOW, bool B_KSLOW>
-__global__ __launch_bounds__(kThreads) void gemm_f32_ring_kernel(const RingArgs args, int epilogue) {
+template <int TI, int TJ, bool A_KSLOW, bool B_KSLOW>
+__global__ __launch_bounds__(kThreads, (TI * TJ <= 4) ? 2 : 1) void gemm_f32_ring_kernel(const RingArgs args, int epilogue) {
     constexpr int NS = kStages;
+    constexpr int BM = 64 * TI, BN = 64 * TJ;
+    constexpr int kOperA = oper_bytes(TI), kStageBytes = oper_bytes(TI) + oper_bytes(TJ);
+    constexpr int kDmaPerTile = TI + TJ;  // load instructions per wavefront and tile
     extern __shared__ __attribute__((aligned(16))) float lds_f[];
     lds_char* lds_base = (lds_char*)lds_f;
     const uint32_t lds_addr0 = (uint32_t)(uintptr_t)lds_base;
@@ -421,7 +428,7 @@ __global__ __launch_bounds__(kThreads) void gemm_f32_ring_kernel(const RingArgs 
     const int M = args.M, N = args.N, K = args.K;
     // the last tile of a row or column of tiles is moved back to end at the edge (it overlaps its neighbour;
     // both compute the shared elements from the same operands in the same order)
-    const int tiles_m = (M + kTile - 1) / kTile, tiles_n = (N + kTile - 1) / kTile;
+    const int tiles_m = (M + BM - 1) / BM, tiles_n = (N + BN - 1) / BN;
     const int total = tiles_m * tiles_n;
     int tile;
     {
@@ -435,27 +442,27 @@ __global__ __launch_bounds__(kThreads) void gemm_f32_ring_kernel(const RingArgs 
     const int first_m = group * GROUP_M;
     const int gsz = (tiles_m - first_m) < GROUP_M ? (tiles_m - first_m) : GROUP_M;
     const int in_group = tile - group * GROUP_M * tiles_n;
-    int m0 = (first_m + in_group % gsz) * kTile;
-    int n0 = (in_group / gsz) * kTile;
-    m0 = m0 + kTile > M ? M - kTile : m0;
-    n0 = n0 + kTile > N ? N - kTile : n0;
+    int m0 = (first_m + in_group % gsz) * BM;
+    int n0 = (in_group / gsz) * BN;
+    m0 = m0 + BM > M ? M - BM : m0;
+    n0 = n0 + BN > N ? N - BN : n0;
 
     const int kt_per_step = K / kBK;
     const int KT = kt_per_step * args.n_steps;
-    const uint32_t a_voff = lane_voff<A_KSLOW>(lane, wave, args.lda, m0);
-    const uint32_t b_voff = lane_voff<B_KSLOW>(lane, wave, args.ldb, n0);
+    const uint32_t a_voff = lane_voff<A_KSLOW, TI>(lane, wave, args.lda, m0);
+    const uint32_t b_voff = lane_voff<B_KSLOW, TJ>(lane, wave, args.ldb, n0);
     const int64_t lda_bytes = args.lda * 4, ldb_bytes = args.ldb * 4;
 
-    Reader<A_KSLOW> ra;
-    Reader<B_KSLOW> rb;
-    ra.init(lane, wm * 128);
-    rb.init(lane, wn * 128);
+    Reader<A_KSLOW, TI> ra;
+    Reader<B_KSLOW, TJ> rb;
+    ra.init(lane, wm * (BM / 2));
+    rb.init(lane, wn * (BN / 2));
 
-    f32x16_t acc[4][4];
+    f32x16_t acc[TI][TJ];
 #pragma unroll
-    for (int i = 0; i < 4; ++i)
+    for (int i = 0; i < TI; ++i)
 #pragma unroll
-        for (int j = 0; j < 4; ++j)
+        for (int j = 0; j < TJ; ++j)
 #pragma unroll
             for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.0f;
 
@@ -481,44 +488,50 @@ __global__ __launch_bounds__(kThreads) void gemm_f32_ring_kernel(const RingArgs 
     // prologue: tiles 0 .. NS-3 in flight, plus the A part of tile NS-2
     for (int p = 0; p < NS - 2; ++p) {
         const uint32_t st = lds_addr0 + is_stage * kStageBytes;
-        gemm_bf16::static_for<4>([&](auto I) {
-            dma_one<A_KSLOW, I.value>(is_a, lda_bytes, is_k0, a_voff, st, wave);
-            dma_one<B_KSLOW, I.value>(is_b, ldb_bytes, is_k0, b_voff, st + kOperBytes, wave);
-        });
+        gemm_bf16::static_for<TI>([&](auto I) { dma_one<A_KSLOW, TI, I.value>(is_a, lda_bytes, is_k0, a_voff, st, wave); });
+        gemm_bf16::static_for<TJ>([&](auto I) { dma_one<B_KSLOW, TJ, I.value>(is_b, ldb_bytes, is_k0, b_voff, st + kOperA, wave); });
         issue_advance();
     }
     {
         const uint32_t st = lds_addr0 + is_stage * kStageBytes;
-        gemm_bf16::static_for<4>([&](auto I) { dma_one<A_KSLOW, I.value>(is_a, lda_bytes, is_k0, a_voff, st, wave); });
+        gemm_bf16::static_for<TI>([&](auto I) { dma_one<A_KSLOW, TI, I.value>(is_a, lda_bytes, is_k0, a_voff, st, wave); });
     }
-    dma_wait<kDmaPerTile*(NS - 3) + 4>();
+    dma_wait<kDmaPerTile*(NS - 3) + TI>();
     __builtin_amdgcn_s_barrier();
     asm volatile("" ::: "memory");
 
+    constexpr int NRA = Reader<A_KSLOW, TI>::kReads, NRB = Reader<B_KSLOW, TJ>::kReads;
     Frag a_lo, a_hi, b_lo, b_hi;
-    gemm_bf16::static_for<Reader<A_KSLOW>::kReads>([&](auto q) { ra.template read<q.value, false>(lds_base, a_lo); });
-    gemm_bf16::static_for<Reader<B_KSLOW>::kReads>([&](auto q) { rb.template read<q.value, false>(lds_base + kOperBytes, b_lo); });
+    gemm_bf16::static_for<NRA>([&](auto q) { ra.template read<q.value, false>(lds_base, a_lo); });
+    gemm_bf16::static_for<NRB>([&](auto q) { rb.template read<q.value, false>(lds_base + kOperA, b_lo); });
 
-    constexpr int NRA = Reader<A_KSLOW>::kReads, NRB = Reader<B_KSLOW>::kReads;
+    constexpr int NM = 4 * TI * TJ;            // products of a half stage
+    constexpr int NOPS = NRA + NRB + TI + TJ;  // memory instructions of a stage, spread evenly behind them
+    constexpr int NOP1 = NRA + NRB + TJ, NOP2 = TI + NRA + NRB;
+    static_assert(NOP1 + NOP2 == 2 * NOPS - TI - TJ, "operation count");
     int cur = 0;
     for (int kt = 0; kt < KT; ++kt) {
         lds_char* sa = lds_base + cur * kStageBytes;
-        lds_char* sb = sa + kOperBytes;
+        lds_char* sb = sa + kOperA;
         const int nxt = (cur + 1 == NS) ? 0 : cur + 1;
         lds_char* na = lds_base + nxt * kStageBytes;
-        lds_char* nb = na + kOperBytes;
+        lds_char* nb = na + kOperA;
 
         // ---- products of steps 0..3; behind them the reads of steps 4..7 and the B part of the tile whose
         //      A part went out in the previous iteration
         CW_F32_PIN();
         {
             const uint32_t st = lds_addr0 + is_stage * kStageBytes;
-            gemm_bf16::static_for<64>([&](auto qq) {
-                constexpr int Q = qq.value, S = Q >> 4, I = (Q >> 2) & 3, J = Q & 3;
+            gemm_bf16::static_for<NM>([&](auto qq) {
+                constexpr int Q = qq.value, S = Q / (TI * TJ), I = (Q / TJ) % TI, J = Q % TJ;
                 acc[I][J] = __builtin_amdgcn_mfma_f32_32x32x2f32(a_lo.v[I][S], b_lo.v[J][S], acc[I][J], 0, 0, 0);
-                if constexpr (Q < NRA) ra.template read<Q, true>(sa, a_hi);
-                else if constexpr (Q < NRA + NRB) rb.template read<Q - NRA, true>(sb, b_hi);
-                else if constexpr (Q < NRA + NRB + 4) dma_one<B_KSLOW, Q - NRA - NRB>(is_b, ldb_bytes, is_k0, b_voff, st + kOperBytes, wave);
+                constexpr int first = Q * NOP1 / NM, last = (Q + 1) * NOP1 / NM;
+                gemm_bf16::static_for<last - first>([&](auto oo) {
+                    constexpr int O = first + oo.value;
+                    if constexpr (O < NRA) ra.template read<O, true>(sa, a_hi);
+                    else if constexpr (O < NRA + NRB) rb.template read<O - NRA, true>(sb, b_hi);
+                    else dma_one<B_KSLOW, TJ, O - NRA - NRB>(is_b, ldb_bytes, is_k0, b_voff, st + kOperA, wave);
+                });
                 CW_F32_PIN();
             });
             issue_advance();
@@ -531,12 +544,16 @@ __global__ __launch_bounds__(kThreads) void gemm_f32_ring_kernel(const RingArgs 
         // ---- products of steps 4..7; behind them the A part of tile kt+NS-1 and the reads of (kt+1, steps 0..3)
         {
             const uint32_t st = lds_addr0 + is_stage * kStageBytes;
-            gemm_bf16::static_for<64>([&](auto qq) {
-                constexpr int Q = qq.value, S = Q >> 4, I = (Q >> 2) & 3, J = Q & 3;
+            gemm_bf16::static_for<NM>([&](auto qq) {
+                constexpr int Q = qq.value, S = Q / (TI * TJ), I = (Q / TJ) % TI, J = Q % TJ;
                 acc[I][J] = __builtin_amdgcn_mfma_f32_32x32x2f32(a_hi.v[I][S], b_hi.v[J][S], acc[I][J], 0, 0, 0);
-                if constexpr (Q < 4) dma_one<A_KSLOW, Q>(is_a, lda_bytes, is_k0, a_voff, st, wave);
-                else if constexpr (Q < 4 + NRA) ra.template read<Q - 4, false>(na, a_lo);
-                else if constexpr (Q < 4 + NRA + NRB) rb.template read<Q - 4 - NRA, false>(nb, b_lo);
+                constexpr int first = Q * NOP2 / NM, last = (Q + 1) * NOP2 / NM;
+                gemm_bf16::static_for<last - first>([&](auto oo) {
+                    constexpr int O = first + oo.value;
+                    if constexpr (O < TI) dma_one<A_KSLOW, TI, O>(is_a, lda_bytes, is_k0, a_voff, st, wave);
+                    else if constexpr (O < TI + NRA) ra.template read<O - TI, false>(na, a_lo);
+                    else rb.template read<O - TI - NRA, false>(nb, b_lo);
+                });
                 CW_F32_PIN();
             });
         }
@@ -544,15 +561,15 @@ __global__ __launch_bounds__(kThreads) void gemm_f32_ring_kernel(const RingArgs 
     }
     dma_wait<0>();
     __syncthreads();
-    // acc[i][j][v]: row m0 + wm*128 + i*32 + 8 (v/4) + 4 (lane/32) + v%4, column n0 + wn*128 + j*32 + lane%32
+    // acc[i][j][v]: row m0 + wm*(BM/2) + i*32 + 8 (v/4) + 4 (lane/32) + v%4, column n0 + wn*(BN/2) + j*32 + lane%32
     float* patch = lds_f + wave * 32 * kPatchPitch;
-    gemm_bf16::static_for<16>([&](auto b) {
-        constexpr int I = b.value >> 2, J = b.value & 3;
-        store_block(acc[I][J], patch, args, epilogue, m0 + wm * 128 + I * 32, n0 + wn * 128 + J * 32, lane);
+    gemm_bf16::static_for<TI * TJ>([&](auto b) {
+        constexpr int I = b.value / TJ, J = b.value % TJ;
+        store_block(acc[I][J], patch, args, epilogue, m0 + wm * (BM / 2) + I * 32, n0 + wn * (BN / 2) + J * 32, lane);
     });
 }
 
-template <bool AS, bool BS>
+template <int TI, int TJ, bool AS, bool BS>
 int launch(const GemmArgs& g, int epilogue, hipStream_t s) {
     RingArgs r = {};
     for (int i = 0; i < g.n_steps && i < kRingMaxSteps; ++i) { r.A[i] = g.A[i]; r.B[i] = g.B[i]; }
@@ -561,14 +578,26 @@ int launch(const GemmArgs& g, int epilogue, hipStream_t s) {
     r.lda = g.lda; r.ldb = g.ldb; r.ldc = g.ldc; r.ldp = g.ldp; r.ldadd = g.ldadd;
     r.M = g.M; r.N = g.N; r.K = g.K; r.n_steps = g.n_steps; r.n_addends = g.n_addends;
     r.vec_bias = 1; r.vec_add = 1; r.k_tail = 0; r.partial = nullptr;
-    auto kern = gemm_f32_ring_kernel<AS, BS>;
-    constexpr int lds = kStages * kStageBytes;
+    auto kern = gemm_f32_ring_kernel<TI, TJ, AS, BS>;
+    constexpr int stages = kStages * (oper_bytes(TI) + oper_bytes(TJ));
+    constexpr int patches = 4 * 32 * kPatchPitch * 4;
+    constexpr int lds = stages > patches ? stages : patches;
     static_assert(lds <= 160 * 1024, "LDS image does not fit the CU");
     hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, lds);
     if (e != hipSuccess) return fail(CW_ERR_LAUNCH, "hipFuncSetAttribute(gemm_f32_ring): %s", hipGetErrorString(e));
-    const int tiles = ((g.M + kTile - 1) / kTile) * ((g.N + kTile - 1) / kTile);
+    const int tiles = ((g.M + 64 * TI - 1) / (64 * TI)) * ((g.N + 64 * TJ - 1) / (64 * TJ));
     hipLaunchKernelGGL(kern, dim3(((tiles + 7) / 8) * 8), dim3(kThreads), lds, s, r, epilogue);
     return check_launch("gemm_f32_ring_kernel");
+}
+
+template <int TI, int TJ>
+int launch_layout(const GemmArgs& g, int layout, int epilogue, hipStream_t s) {
+    switch (layout) {
+        case CW_NN: return launch<TI, TJ, false, true>(g, epilogue, s);
+        case CW_NT: return launch<TI, TJ, false, false>(g, epilogue, s);
+        case CW_TN: return launch<TI, TJ, true, true>(g, epilogue, s);
+        default: return fail(CW_ERR_INVALID, "cw_gemm_ksteps: bad layout %d", layout);
+    }
 }
 
 }  // namespace ring
@@ -609,16 +638,16 @@ int gemm_f32_launch(const GemmArgs& args, int layout, int epilogue, hipStream_t 
             const char* v = std::getenv("CW_GEMM_IMPL");
             return !(v != nullptr && std::strcmp(v, "staged") == 0);
         }();
-        if (ring_enabled && tiles256 >= 128 && all_vec && fits32 && args.M >= 256 && args.N >= 256 && (args.N % 4) == 0 &&
-            (layout != CW_TN || (args.M % 4) == 0) && args.K >= ring::kBK && (args.K % ring::kBK) == 0 && args.n_steps >= 1 &&
-            args.n_steps <= kRingMaxSteps && args.n_addends <= kRingMaxAddends) {
-            switch (layout) {
-                case CW_NN: return ring::launch<false, true>(args, epilogue, s);
-                case CW_NT: return ring::launch<false, false>(args, epilogue, s);
-                case CW_TN: return ring::launch<true, true>(args, epilogue, s);
-                default: return fail(CW_ERR_INVALID, "cw_gemm_ksteps: bad layout %d", layout);
-            }
-        }
+        const bool ring_ok = ring_enabled && all_vec && fits32 && (args.N % 4) == 0 && (layout != CW_TN || (args.M % 4) == 0) &&
+                             args.K >= ring::kBK && (args.K % ring::kBK) == 0 && args.n_steps >= 1 &&
+                             args.n_steps <= kRingMaxSteps && args.n_addends <= kRingMaxAddends;
+        // the largest tile that still gives every compute unit work: 256 x 256 (one workgroup per unit), else
+        // 128 x 128 or 128 x 64 (two per unit)
+        const int64_t tiles128 = ((int64_t)(args.M + 127) / 128) * ((args.N + 127) / 128);
+        const int64_t tiles128x64 = ((int64_t)(args.M + 127) / 128) * ((args.N + 63) / 64);
+        if (ring_ok && tiles256 >= 128 && args.M >= 256 && args.N >= 256) return ring::launch_layout<4, 4>(args, layout, epilogue, s);
+        if (ring_ok && tiles128 >= 384 && args.M >= 128 && args.N >= 128) return ring::launch_layout<2, 2>(args, layout, epilogue, s);
+        if (ring_ok && tiles128x64 >= 256 && args.M >= 128 && args.N >= 64) return ring::launch_layout<2, 1>(args, layout, epilogue, s);
     }
     const bool vec = args.vec_a && args.vec_b && (args.N % kFBN) == 0 && (args.K % kFBK) == 0;
     // 256-row tiles when they still give every compute unit two tiles

@@ -155,6 +155,18 @@ def test_fp32_ring_kernel(layout):
     _run(layout, 4096, 2048, 32, 1, torch.float32, act="gelu_erf", pad_a=4, pad_b=8, seed=24)
 
 
+@pytest.mark.parametrize("layout", LAYOUTS)
+def test_fp32_ring_kernel_smaller_tiles(layout):
+    """Outputs with too few 256 x 256 tiles for the chip: the ring kernel with 128 x 128 tiles (3072 x 2048:
+    384 of them) and with 128 x 64 tiles (config 1's gradient shapes, 4096 x 1024), exact and with ragged
+    edges, several k-steps, addends and the pre-activation copy."""
+    _run(layout, 3072, 2048, 48, 2, torch.float32, act="gelu_tanh", n_add=1, preact=True, seed=31)
+    _run(layout, 3080, 2052, 32, 1, torch.float32, act="relu", n_add=2, preact=True, seed=32)
+    _run(layout, 4096, 1024, 64, 3, torch.float32, act=None, n_add=1, preact=True, seed=33)
+    _run(layout, 4100, 1028, 16, 1, torch.float32, act="gelu_erf", seed=34)
+    _run(layout, 4096, 1024, 32, 1, torch.float32, act=None, bias=False, pad_a=4, pad_b=12, seed=35)
+
+
 def test_fp32_linear1d_col_shape():
     # BASELINE config 1: x [8,512,1024] fp32, W [4096,1024], b zeros -> F.linear
     import oracle
