@@ -231,6 +231,14 @@ def bench_other_configs(device, sets):
     flop1 = 2.0 * 4096 * 1024 * 4096
     out["linear1d_fp32_fwd"] = {"us": round(us, 2), "TFLOPs": round(flop1 / us / 1e6, 1),
                                 "frac_fp32_mfma": round(flop1 / us / 1e6 / 157.3, 4)}
+    # config 1 backward: dX = dY W (NN, [4096,4096] x [4096,1024]) and dW = dY^T X (TN), the same FLOP each
+    dy1 = _seeded((4096, 4096), 3, 1.0, torch.float32).to(device)
+    for name, fn in (("linear1d_fp32_dX", lambda: ops.gemm_ksteps("NN", [dy1], [w1])),
+                     ("linear1d_fp32_dW", lambda: ops.gemm_ksteps("TN", [dy1], [x1]))):
+        us = event_time_us(fn, 30, 5)
+        out[name] = {"us": round(us, 2), "TFLOPs": round(flop1 / us / 1e6, 1),
+                     "frac_fp32_mfma": round(flop1 / us / 1e6 / 157.3, 4)}
+    del dy1
     # vocab-parallel embedding (rank 1 of 4 of OPT's 50272 x 2048 table, 8192 tokens): bytes = ids + the rows
     # actually read (about a quarter of the tokens are live) + the output written
     e_tok, e_dim, e_vloc = 8192, 2048, 12568

@@ -1,0 +1,63 @@
+"""The entry points enqueue work on the caller's stream and neither allocate nor synchronise, so a sequence
+of them can be recorded into a HIP graph (torch.cuda.graph) and replayed: every replay must reproduce the
+eager results bit for bit, also with other work and synchronisations between the replays."""
+import pytest
+import torch
+
+from tests.util import randn
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+
+
+def _pipeline(x, w1, b1, w2, gamma, beta, targets, ids, table_rows):
+    from cubework_amd import ops
+
+    h = ops.gemm_ksteps("NN", [x], [w1], b1, "gelu_tanh")                      # LDS-ring kernel
+    y, _ = ops.ln_forward_fused(h, 1e-5, gamma, beta)
+    small = ops.gemm_ksteps("TN", [y], [x])                                    # few tiles, long k: split k with scratch
+    logits = ops.gemm_ksteps("NT", [y], [w2])
+    mx, se, pr, mask = ops.vpce_fwd_local(logits, targets, 0)
+    loss, gmax, gsum = ops.vpce_finalize(mx[None], se[None], pr[None], mask[None])
+    grad = ops.vpce_bwd(logits, targets, 0, gmax, gsum, None, 1.0 / targets.numel())
+    dw = ops.embedding_bwd(ids, y, table_rows, 0)
+    qkv = ops.gemm_ksteps("NN", [y], [w1[:, :768].contiguous()])               # 4 heads of 64: q, k, v side by side
+    att = ops.attention_core(qkv.view(4, -1, 768), 4)
+    return h, y, small, loss, grad, dw, att
+
+
+def test_entry_points_replay_from_a_graph():
+    T, H, V = 4096, 2048, 1024
+    x = randn((T, H), torch.bfloat16, 0).to(DEV)
+    w1 = randn((H, H), torch.bfloat16, 1, std=0.03).to(DEV)
+    b1 = randn((H,), torch.bfloat16, 2, std=0.1).to(DEV)
+    w2 = randn((V, H), torch.bfloat16, 3, std=0.03).to(DEV)
+    gamma = (1.0 + 0.1 * randn((H,), torch.float32, 4)).to(torch.bfloat16).to(DEV)
+    beta = randn((H,), torch.bfloat16, 5, std=0.1).to(DEV)
+    targets = torch.randint(0, V, (T,), generator=torch.Generator().manual_seed(6)).to(DEV)
+    ids = torch.randint(0, 300, (T,), generator=torch.Generator().manual_seed(7)).to(DEV)
+    args = (x, w1, b1, w2, gamma, beta, targets, ids, 300)
+
+    eager = [t.clone() for t in _pipeline(*args)]
+    torch.cuda.synchronize()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        _pipeline(*args)
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        outs = _pipeline(*args)
+    for replay in range(3):
+        for t in outs:
+            t.fill_(float("nan")) if t.is_floating_point() else t.zero_()
+        graph.replay()
+        torch.cuda.synchronize()
+        for name, got, want in zip(("gemm", "layernorm", "split-k gemm", "loss", "logits grad", "embedding grad", "attention"),
+                                   outs, eager):
+            assert torch.equal(got, want), "%s differs on replay %d" % (name, replay)
+        # the program's own eager work between replays
+        again = _pipeline(*args)
+        torch.cuda.synchronize()
+        assert torch.equal(again[0], eager[0])
