@@ -71,6 +71,25 @@ def test_embedding_backward_every_run_length(e, dtype):
     assert (got.cpu()[0:3] == 0).all() and (got.cpu()[4::2][:44] == 0).all(), "rows without tokens are exactly zero"
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+def test_embedding_backward_one_id_thousands_of_times(dtype):
+    """Token frequencies of text: one id 3000 times among 5000 tokens (a run that every wavefront of the
+    sharing blocks walks for many rounds), the rest spread over the table; compared in float64."""
+    from cubework_amd import ops
+
+    g = torch.Generator().manual_seed(3)
+    ids = torch.randint(0, 400, (5000,), generator=g)
+    ids[torch.randperm(5000, generator=g)[:3000]] = 17
+    e, v_loc = 1032, 400
+    d_out = randn((5000, e), dtype, 8)
+    want = torch.zeros((v_loc, e), dtype=torch.float64).index_add_(0, ids, d_out.double())
+    got = ops.embedding_bwd(ids.to(DEV), d_out.to(DEV), v_loc, 0, -1)
+    again = ops.embedding_bwd(ids.to(DEV), d_out.to(DEV), v_loc, 0, -1)
+    torch.cuda.synchronize()
+    assert torch.equal(got, again)
+    assert_parity(got, want, dtype, "embedding d_weight with a run of 3000", scale=20 if dtype == torch.float32 else 1)
+
+
 def test_vocab_slices_sum_to_the_full_lookup():
     """Four vocabulary slices: every token is live in exactly one, so the slices' outputs sum (the
     all-reduce of parallel_1d/module.py:454) to F.embedding on the whole table, bit for bit."""
