@@ -33,6 +33,8 @@ int gemm_f16_dma_split_launch_nn(const GemmArgs& args, int slices, hipStream_t s
 int gemm_f16_dma_split_launch_nt(const GemmArgs& args, int slices, hipStream_t s);
 int gemm_f16_dma_split_launch_tn(const GemmArgs& args, int slices, hipStream_t s);
 
+int gemm_half_small_launch(const GemmArgs& args, int layout, int epilogue, bool f16, hipStream_t s);
+
 int gemm_bf16_split_slices(int64_t M, int64_t N, int64_t K, int n_steps) {
     if (M <= 0 || N <= 0 || K <= 0 || n_steps <= 0 || n_steps > kRingMaxSteps) return 1;
     if ((M % 256) != 0 || (N % 256) != 0 || (K % 64) != 0) return 1;
@@ -187,6 +189,20 @@ int gemm_half_launch(const GemmArgs& args, int layout, int epilogue, bool f16, h
     // full tile in each direction and 16-byte steps wherever a tile origin moves along a contiguous
     // dimension (N always: the output and a [K, N] operand; M for a [K, M] operand).
     const bool edges_ok = args.M >= 256 && args.N >= 256 && (args.N % 8) == 0 && (layout != CW_TN || (args.M % 8) == 0);
+    // Fewer than 160 tiles of 256 x 256 (at 128 .. 159 of them the large tiles leave 40 % of the compute units
+    // idle, and four times as many small tiles fill them): the ring kernel with 128 x 128 tiles, unless a long
+    // reduction over few tiles is better served by splitting k (below; measured on 2048 x 2048 outputs: the
+    // small tiles win up to a reduction length of 8192, the split from 16384).
+    const int slices = gemm_bf16_split_slices(args.M, args.N, args.K, args.n_steps);
+    {
+        const int64_t tiles128 = (int64_t)((args.M + 127) / 128) * ((args.N + 127) / 128);
+        const bool splits = slices > 1 && args.workspace != nullptr && aligned16(args.workspace) &&
+                            args.workspace_bytes >= (int64_t)slices * args.M * args.N * (int64_t)sizeof(float);
+        if (tiles256 < 160 && all_vec && ring_ok && args.M >= 128 && args.N >= 128 && (args.N % 8) == 0 &&
+            (layout != CW_TN || (args.M % 8) == 0) && args.K >= 64 && (args.K % 64) == 0 &&
+            args.lda < ((int64_t)1 << 23) && args.ldb < ((int64_t)1 << 23) && ((tiles128 >= 192 && (int64_t)args.K * args.n_steps < 12288) || !splits))
+            return gemm_half_small_launch(args, layout, epilogue, f16, s);
+    }
     if (big && all_vec && ring_ok && edges_ok && (args.K % gemm_bf16::kBK) == 0) return dma_launch(args, layout, epilogue, f16, s);
     // A reduction length that is not a multiple of the k tile (a vocabulary slice as K: 12568 = 392 x 32 +
     // 24), with B stored [K, N]: the regular step covers the first K - K % 32 columns, one more step of 32
@@ -209,7 +225,6 @@ int gemm_half_launch(const GemmArgs& args, int layout, int epilogue, bool f16, h
         main_part.K = args.K - kr;
         return dma_launch(main_part, layout, epilogue, f16, s, tail_a, tail_b);
     }
-    const int slices = gemm_bf16_split_slices(args.M, args.N, args.K, args.n_steps);
     if (slices > 1 && all_vec && args.n_addends <= kRingMaxAddends && dma_kernel_enabled() &&
         args.workspace != nullptr && aligned16(args.workspace) &&
         args.workspace_bytes >= (int64_t)slices * args.M * args.N * (int64_t)sizeof(float)) {

@@ -113,6 +113,19 @@ def test_bf16_ragged_big_config(layout):
     _run(layout, 4100, 2056, 136, 2, torch.bfloat16, act="gelu_erf", seed=5)
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("layout", LAYOUTS)
+def test_half_small_tile_ring(layout, dtype):
+    """Outputs with fewer than 128 tiles of 256 x 256, aligned operands and a reduction that is a multiple of
+    64: the ring kernel with 128 x 128 tiles. One and several k-steps, a single k tile, M and N that are not
+    tile multiples (last tiles moved back), every epilogue piece, padded leading dimensions."""
+    _run(layout, 2048, 2048, 512, 1, dtype, act="gelu_tanh", seed=41)
+    _run(layout, 256, 384, 192, 3, dtype, act=None, n_add=2, preact=True, seed=42)
+    _run(layout, 128, 128, 64, 1, dtype, act="relu", seed=43)
+    _run(layout, 392, 264, 128, 2, dtype, act="gelu_erf", n_add=1, preact=True, seed=44)
+    _run(layout, 1024, 136, 320, 1, dtype, act=None, bias=False, pad_a=8, pad_b=24, seed=45)
+
+
 @pytest.mark.parametrize("act", [None, "gelu_tanh", "gelu_erf", "relu"])
 def test_bf16_epilogues_with_preact_and_addends(act):
     _run("NN", 384, 256, 128, 2, torch.bfloat16, act=act, n_add=2, preact=True, seed=7)
