@@ -57,7 +57,12 @@ extern "C" int64_t cw_gemm_workspace_bytes(int layout, int64_t M, int64_t N, int
     if (layout != CW_NN && layout != CW_NT && layout != CW_TN) return 0;
     if (io_dtype != CW_BF16 && io_dtype != CW_F16) return 0;  // the fp32 GEMM is not split
     const int slices = gemm_bf16_split_slices(M, N, K, n_steps);
-    if (slices > 1) return (int64_t)slices * M * N * (int64_t)sizeof(float);
+    if (slices > 1) {
+        // shapes the 128 x 128 ring kernel takes in preference to the split (gemm_half_launch) need none
+        const int64_t tiles128 = ((M + 127) / 128) * ((N + 127) / 128);
+        if (tiles128 >= 192 && K * n_steps < 12288) return 0;
+        return (int64_t)slices * M * N * (int64_t)sizeof(float);
+    }
     return gemm_bf16_ktail_workspace_bytes(layout, M, N, K, n_steps);
 }
 

@@ -65,6 +65,8 @@ def test_scratch_sizes_and_refusals_of_the_later_entry_points():
     # split-k: few tiles, long reduction (config-2 weight gradient: 64 tiles x 4 slices of fp32 partials)
     assert lib.cw_gemm_workspace_bytes(TN, 2048, 2048, 8192, 2, BF16) == 4 * 2048 * 2048 * 4
     assert lib.cw_gemm_workspace_bytes(NN, 8192, 2048, 2048, 2, BF16) == 0
+    assert lib.cw_gemm_workspace_bytes(TN, 2048, 2048, 2048, 1, BF16) == 0    # 256 tiles of 128 x 128: the small-tile ring kernel
+    assert lib.cw_gemm_workspace_bytes(TN, 1024, 1024, 2048, 1, BF16) > 0     # 64 small tiles: split k
     assert lib.cw_gemm_workspace_bytes(TN, 2048, 2048, 8192, 2, F32) == 0
     # reduction length that is not a multiple of 32 with B stored [K, N]: 32 rows of B
     assert lib.cw_gemm_workspace_bytes(NN, 8192, 2048, 12568, 1, BF16) == 32 * 2048 * 2
