@@ -142,14 +142,6 @@ __device__ __forceinline__ float sum_halves(float v) {
 // is applied on the global side: the lane fetches the chunk that belongs at its position. No staging
 // registers, no LDS write instructions. The compiler does not see these loads (inline asm); the kernel
 // waits for them itself (dma_wait) before the barrier that publishes the tile.
-__device__ __forceinline__ void dma16(const char* gbase, uint32_t voff, uint32_t lds_addr) {
-    asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, %2" : : "s"(lds_addr), "v"(voff), "s"(gbase) : "memory", "m0");
-}
-// Waits until at most N of this thread's loads are in flight (loads complete in issue order).
-template <int N>
-__device__ __forceinline__ void dma_wait() {
-    asm volatile("s_waitcnt vmcnt(%0)" : : "n"(N) : "memory");
-}
 
 // Which chunk (row, 16-byte column) of a 64-row tile lives at chunk position p of an image.
 __device__ __forceinline__ void row_image_source(int p, int& r, int& c) {

@@ -201,6 +201,20 @@ __device__ __forceinline__ raw16_t pack_raw(const float (&v)[4], const float*) {
     return u;
 }
 
+// ---- loads straight into LDS ----------------------------------------------
+// global_load_lds_dwordx4: lane l of the issuing wavefront fetches 16 bytes at gbase + voff and the load
+// unit writes them at LDS address lds_addr + 16 l (M0 holds lds_addr): no staging registers, no LDS write
+// instructions. The compiler does not see these loads (inline asm); a kernel that uses them counts them and
+// waits with dma_wait<N> (at most N of this thread's loads still in flight; loads complete in issue order)
+// before the barrier that publishes the data.
+__device__ __forceinline__ void dma16(const char* gbase, uint32_t voff, uint32_t lds_addr) {
+    asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, %2" : : "s"(lds_addr), "v"(voff), "s"(gbase) : "memory", "m0");
+}
+template <int N>
+__device__ __forceinline__ void dma_wait() {
+    asm volatile("s_waitcnt vmcnt(%0)" : : "n"(N) : "memory");
+}
+
 // ---- wavefront (64 lanes) reductions ------------------------------------
 // Within a row of 16 lanes the partner values come through DPP operand
 // modifiers of the adds themselves (no LDS traffic); the four row results are

@@ -53,13 +53,6 @@ constexpr int kOperBytes = kTile * kBK * 2;  // 16384
 constexpr int kStageBytes = 2 * kOperBytes;  // 32768
 constexpr int kDmaPerTile = 8;               // load instructions per wavefront per tile
 
-__device__ __forceinline__ void dma16(const char* gbase, uint32_t voff, uint32_t lds_addr) {
-    asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, %2" : : "s"(lds_addr), "v"(voff), "s"(gbase) : "memory", "m0");
-}
-template <int N>
-__device__ __forceinline__ void dma_wait() {
-    asm volatile("s_waitcnt vmcnt(%0)" : : "n"(N) : "memory");
-}
 
 template <bool TRANS>
 __device__ __forceinline__ void dma_lane_offsets(int lane, int64_t ld, int row0, uint32_t& even, uint32_t& odd) {

@@ -302,13 +302,6 @@ constexpr int kBK = 16, kThreads = 256, kStages = 4;
 // ROWS = 64 T rows takes ROWS * 64 bytes per stage and T load instructions per wavefront.
 constexpr int oper_bytes(int t) { return 64 * t * kBK * 4; }
 
-__device__ __forceinline__ void dma16(const char* gbase, uint32_t voff, uint32_t lds_addr) {
-    asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, %2" : : "s"(lds_addr), "v"(voff), "s"(gbase) : "memory", "m0");
-}
-template <int N>
-__device__ __forceinline__ void dma_wait() {
-    asm volatile("s_waitcnt vmcnt(%0)" : : "n"(N) : "memory");
-}
 
 // Byte offset, inside the span of one load instruction, of the 16 bytes this lane fetches.
 template <bool KSLOW, int T>
