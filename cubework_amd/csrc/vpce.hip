@@ -181,6 +181,11 @@ __device__ __forceinline__ void store_grad(bf16_t* p, const float (&v)[V]) {
     store_raw_stream(p, pack_raw(v, (const bf16_t*)nullptr));
 }
 template <int V>
+__device__ __forceinline__ void store_grad(f16_t* p, const float (&v)[V]) {
+    static_assert(V == 8, "fp16 gradients are written 8 at a time");
+    store_raw_stream(p, pack_raw(v, (const f16_t*)nullptr));
+}
+template <int V>
 __device__ __forceinline__ void store_grad(float* p, const float (&v)[V]) {
 #pragma unroll
     for (int e = 0; e < V; e += 4) {
@@ -206,14 +211,14 @@ __device__ __forceinline__ void grad_vector(raw16_t raw, int64_t i, int64_t tcol
     store_grad<V>(gr + i * V, v);
 }
 
-// fp32 gradient of bf16 logits: four logits (8 bytes) in, four floats (16 bytes) out per lane, so that the
+// fp32 gradient of 16-bit logits: four logits (8 bytes) in, four floats (16 bytes) out per lane, so that the
 // stores of one instruction cover one contiguous 1 KB span. With 16-byte loads a lane would write 32
 // bytes in two stores that each leave every other 16 bytes to the next instruction.
 typedef uint32_t raw8_t __attribute__((ext_vector_type(2)));
+template <typename T>
 __device__ __forceinline__ void grad_quad(raw8_t raw, int64_t i, int64_t tcol, float m2, float scale, float dl,
                                           float* __restrict__ gr) {
-    float v[4] = {__uint_as_float(raw.x << 16), __uint_as_float(raw.x & 0xffff0000u), __uint_as_float(raw.y << 16),
-                  __uint_as_float(raw.y & 0xffff0000u)};
+    float v[4] = {half_conv<T>::lo(raw.x), half_conv<T>::hi(raw.x), half_conv<T>::lo(raw.y), half_conv<T>::hi(raw.y)};
 #pragma unroll
     for (int e = 0; e < 4; ++e) v[e] = __builtin_amdgcn_exp2f(__builtin_fmaf(v[e], kLog2e, -m2)) * scale;
     const int64_t rel = tcol - i * 4;
@@ -244,10 +249,13 @@ __global__ __launch_bounds__(kCeBlock) void vpce_bwd_kernel(int64_t T_rows, int6
         const int64_t t = targets[row];
         const bool masked = (t < vocab_start) || (t >= vocab_start + V_cols);
         const int64_t tcol = masked ? -1 : (t - vocab_start);
-        if (vec_ok && std::is_same<T, bf16_t>::value && std::is_same<G, float>::value) {
+        bool done = false;
+        if constexpr (sizeof(T) == 2 && std::is_same<G, float>::value) {
+          if (vec_ok) {
+            done = true;
             constexpr int U = 2 * kCeBwdUnroll;
             const int64_t nq = V_cols / 4;
-            const bf16_t* xb = reinterpret_cast<const bf16_t*>(xr);
+            const uint16_t* xb = reinterpret_cast<const uint16_t*>(xr);
             float* gf = reinterpret_cast<float*>(gr);
             int64_t i = tid;
             for (; i + (U - 1) * kCeBlock < nq; i += U * kCeBlock) {
@@ -256,16 +264,19 @@ __global__ __launch_bounds__(kCeBlock) void vpce_bwd_kernel(int64_t T_rows, int6
                 for (int u = 0; u < U; ++u)
                     raw[u] = __builtin_nontemporal_load(reinterpret_cast<const raw8_t*>(xb + (i + u * kCeBlock) * 4));
 #pragma unroll
-                for (int u = 0; u < U; ++u) grad_quad(raw[u], i + u * kCeBlock, tcol, m2, scale, dl, gf);
+                for (int u = 0; u < U; ++u) grad_quad<T>(raw[u], i + u * kCeBlock, tcol, m2, scale, dl, gf);
             }
             for (; i < nq; i += kCeBlock)
-                grad_quad(__builtin_nontemporal_load(reinterpret_cast<const raw8_t*>(xb + i * 4)), i, tcol, m2, scale, dl, gf);
+                grad_quad<T>(__builtin_nontemporal_load(reinterpret_cast<const raw8_t*>(xb + i * 4)), i, tcol, m2, scale, dl, gf);
             for (int64_t c = nq * 4 + tid; c < V_cols; c += kCeBlock) {
                 float y = __builtin_amdgcn_exp2f(__builtin_fmaf(load_elem(xr + c), kLog2e, -m2)) * scale;
                 if (c == tcol) y -= dl;
                 store_elem(gr + c, y);
             }
-        } else if (vec_ok) {
+          }
+        }
+        if (done) continue;
+        if (vec_ok) {
             const int64_t nvec = V_cols / V;
             int64_t i = tid;
             for (; i + (kCeBwdUnroll - 1) * kCeBlock < nvec; i += kCeBwdUnroll * kCeBlock) {
@@ -319,7 +330,8 @@ extern "C" int cw_vpce_fwd_local(int64_t T, int64_t V, const void* logits, int64
                                  int64_t vocab_start, float* out_max, float* out_sumexp, float* out_pred,
                                  uint8_t* out_mask, int io_dtype, void* stream) {
     if (T < 0 || V <= 0) return fail(CW_ERR_INVALID, "cw_vpce_fwd_local: bad shape T=%lld V=%lld", (long long)T, (long long)V);
-    if (io_dtype != CW_BF16 && io_dtype != CW_F32) return fail(CW_ERR_INVALID, "cw_vpce_fwd_local: bad io_dtype %d", io_dtype);
+    if (io_dtype != CW_BF16 && io_dtype != CW_F32 && io_dtype != CW_F16)
+        return fail(CW_ERR_INVALID, "cw_vpce_fwd_local: bad io_dtype %d", io_dtype);
     if (vocab_start < 0) return fail(CW_ERR_INVALID, "cw_vpce_fwd_local: negative vocab_start");
     if (T == 0) return CW_OK;
     if (logits == nullptr || targets == nullptr || out_max == nullptr || out_sumexp == nullptr ||
@@ -330,6 +342,11 @@ extern "C" int cw_vpce_fwd_local(int64_t T, int64_t V, const void* logits, int64
         const int vec_ok = aligned16(logits) && (ld % 8) == 0;
         hipLaunchKernelGGL(vpce_fwd_kernel<bf16_t>, dim3(ce_grid(T)), dim3(kCeBlock), 0, s, T, V,
                            (const bf16_t*)logits, ld, targets, vocab_start, out_max, out_sumexp, out_pred, out_mask,
+                           vec_ok);
+    } else if (io_dtype == CW_F16) {
+        const int vec_ok = aligned16(logits) && (ld % 8) == 0;
+        hipLaunchKernelGGL(vpce_fwd_kernel<f16_t>, dim3(ce_grid(T)), dim3(kCeBlock), 0, s, T, V,
+                           (const f16_t*)logits, ld, targets, vocab_start, out_max, out_sumexp, out_pred, out_mask,
                            vec_ok);
     } else {
         const int vec_ok = aligned16(logits) && (ld % 4) == 0;
@@ -357,15 +374,21 @@ extern "C" int cw_vpce_bwd(int64_t T, int64_t V, const void* logits, int64_t ld,
                            float dloss_scale, void* grad, int64_t ld_grad, int io_dtype, int grad_dtype,
                            void* stream) {
     if (T < 0 || V <= 0) return fail(CW_ERR_INVALID, "cw_vpce_bwd: bad shape T=%lld V=%lld", (long long)T, (long long)V);
-    if (io_dtype != CW_BF16 && io_dtype != CW_F32) return fail(CW_ERR_INVALID, "cw_vpce_bwd: bad io_dtype %d", io_dtype);
-    if (grad_dtype != CW_BF16 && grad_dtype != CW_F32) return fail(CW_ERR_INVALID, "cw_vpce_bwd: bad grad_dtype %d", grad_dtype);
-    if (io_dtype == CW_F32 && grad_dtype == CW_BF16)
-        return fail(CW_ERR_UNSUPPORTED, "cw_vpce_bwd: bf16 gradient of fp32 logits is not provided");
+    if (io_dtype != CW_BF16 && io_dtype != CW_F32 && io_dtype != CW_F16)
+        return fail(CW_ERR_INVALID, "cw_vpce_bwd: bad io_dtype %d", io_dtype);
+    if (grad_dtype != CW_BF16 && grad_dtype != CW_F32 && grad_dtype != CW_F16)
+        return fail(CW_ERR_INVALID, "cw_vpce_bwd: bad grad_dtype %d", grad_dtype);
+    if (grad_dtype != CW_F32 && grad_dtype != io_dtype)
+        return fail(CW_ERR_UNSUPPORTED, "cw_vpce_bwd: the gradient is fp32 or of the logits' type");
     if (T == 0) return CW_OK;
     if (logits == nullptr || targets == nullptr || gmax == nullptr || gsum == nullptr || grad == nullptr || ld < V ||
         ld_grad < V)
         return fail(CW_ERR_INVALID, "cw_vpce_bwd: null pointer or leading dimension < V");
     hipStream_t s = (hipStream_t)stream;
+    if (io_dtype == CW_F16 && grad_dtype == CW_F16)
+        return bwd_impl<f16_t, f16_t>(T, V, logits, ld, targets, vocab_start, gmax, gsum, dloss_rows, dloss_scale, grad, ld_grad, s);
+    if (io_dtype == CW_F16)
+        return bwd_impl<f16_t, float>(T, V, logits, ld, targets, vocab_start, gmax, gsum, dloss_rows, dloss_scale, grad, ld_grad, s);
     if (io_dtype == CW_BF16 && grad_dtype == CW_BF16)
         return bwd_impl<bf16_t, bf16_t>(T, V, logits, ld, targets, vocab_start, gmax, gsum, dloss_rows, dloss_scale, grad, ld_grad, s);
     if (io_dtype == CW_BF16)

@@ -13,13 +13,13 @@ loss_1d.py:20,47-48).
 import torch
 
 from ... import ops
-from .._amp import bwd, fp32_fwd
+from .._amp import bwd, loss_fwd
 
 
 class _VocabParallelCrossEntropy(torch.autograd.Function):
 
     @staticmethod
-    @fp32_fwd()
+    @loss_fwd()
     def forward(ctx, logits, targets, parallel_mode):
         vocab = logits.size(-1)
         vocab_start = parallel_mode.local_rank * vocab

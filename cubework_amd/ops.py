@@ -3,8 +3,8 @@
 pass raw pointers and the current stream.
 
 Every function requires CUDA (ROCm) tensors of dtype bfloat16 or float32 (the
-GEMM and column-sum wrappers also take float16, the type autocast hands the
-GEMM-type operators by default) and raises instead of falling back to torch
+GEMM, column-sum, attention and cross-entropy wrappers also take float16, the
+type autocast hands the GEMM-type operators by default) and raises instead of falling back to torch
 arithmetic.
 """
 import ctypes
@@ -342,7 +342,7 @@ def vpce_fwd_local(logits: torch.Tensor, targets: torch.Tensor, vocab_start: int
     pr = torch.empty(T, dtype=torch.float32, device=dev)
     mk = torch.empty(T, dtype=torch.uint8, device=dev)
     rc = lib.cw_vpce_fwd_local(T, V, _p(logits), _ld(logits), _p(targets), vocab_start, _p(mx), _p(se), _p(pr), _p(mk),
-                               _dtype_code(logits), _stream())
+                               _dtype_code(logits, half_ok=True), _stream())
     _lib.check(rc, "cw_vpce_fwd_local")
     return mx, se, pr, mk
 
@@ -378,7 +378,7 @@ def vpce_bwd(logits: torch.Tensor, targets: torch.Tensor, vocab_start: int, gmax
     if dloss_rows is not None:
         dloss_rows = dloss_rows.reshape(-1).to(torch.float32).contiguous()
     rc = lib.cw_vpce_bwd(T, V, _p(logits), _ld(logits), _p(targets), vocab_start, _p(gmax), _p(gsum), _p(dloss_rows),
-                         dloss_scale, _p(grad), _ld(grad), _dtype_code(logits), _dtype_code(grad), _stream())
+                         dloss_scale, _p(grad), _ld(grad), _dtype_code(logits, half_ok=True), _dtype_code(grad, half_ok=True), _stream())
     _lib.check(rc, "cw_vpce_bwd")
     return grad.reshape(shape)
 

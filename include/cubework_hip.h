@@ -43,9 +43,11 @@ typedef enum {
 
 /* CW_F16 (IEEE half, the type the reference's GEMM-type Functions cast to under autocast:
  * custom_fwd(cast_inputs=torch.float16), cubework/module/parallel_2d/_operation.py:17,96,176,255,363) is
- * taken by the GEMM, column-sum and attention entry points only (cw_gemm_ksteps, cw_gemm_ksteps_ws,
- * cw_colsum, cw_act_bwd_colsum, cw_attn_fwd, cw_attn_bwd): the reference runs LayerNorm and the loss in
- * fp32 under autocast, and so do their entry points here. */
+ * taken by the GEMM, column-sum, attention and cross-entropy entry points (cw_gemm_ksteps,
+ * cw_gemm_ksteps_ws, cw_colsum, cw_act_bwd_colsum, cw_attn_fwd, cw_attn_bwd, cw_vpce_fwd_local,
+ * cw_vpce_bwd): the reference runs LayerNorm in fp32 under autocast, on the fp32 residual stream, and so
+ * does its entry point here; its loss casts the logits to fp32 first, which reading them as 16-bit values
+ * and computing in fp32 reproduces without the copy. */
 typedef enum { CW_BF16 = 0, CW_F32 = 1, CW_F16 = 2 } cw_dtype;
 
 /* Operand orientation of the block GEMM, per k-step i:
@@ -275,7 +277,7 @@ int cw_vpce_finalize(int64_t T, int n_ranks, const float* max_all, const float* 
  * grad[t,c] = (exp(logits[t,c]-gmax[t]) / gsum[t] - [c == target column, in slice]) * dloss
  * with dloss = dloss_rows[t] * dloss_scale (dloss_rows may be NULL = all ones).
  * Recomputes the softmax instead of keeping it (loss_1d.py:55-56,61-79).
- * grad_dtype selects the storage type of grad (CW_BF16 or CW_F32).
+ * grad_dtype selects the storage type of grad: CW_F32 or the logits' type.
  */
 int cw_vpce_bwd(int64_t T, int64_t V, const void* logits, int64_t ld,
                 const int64_t* targets, int64_t vocab_start,

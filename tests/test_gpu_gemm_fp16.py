@@ -100,15 +100,16 @@ def test_f16_colsum_and_act_bwd(shape):
 
 
 def test_f16_refused_where_the_reference_runs_fp32():
-    """LayerNorm and the loss run in fp32 under autocast in the reference (cast_inputs=torch.float32); their
-    wrappers take bfloat16 and float32 only and say so instead of computing something else."""
+    """LayerNorm runs in fp32 under autocast in the reference (cast_inputs=torch.float32) and receives the
+    fp32 residual stream; its wrappers and the embedding's take bfloat16 and float32 only and say so instead
+    of computing something else."""
     from cubework_amd import ops
 
     x = randn((64, 256), F16, 1).to(DEV)
     with pytest.raises(TypeError):
         ops.ln_partial_stats(x)
     with pytest.raises(TypeError):
-        ops.vpce_fwd_local(x, torch.zeros(64, dtype=torch.int64, device=DEV), 0)
+        ops.embedding_fwd(torch.zeros(4, dtype=torch.int64, device=DEV), x, 0)
 
 
 @pytest.mark.parametrize("amp_dtype", [torch.float16, torch.bfloat16])

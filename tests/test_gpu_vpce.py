@@ -61,15 +61,47 @@ def _run_all_ranks(T, V, p, dtype, seed, grad_dtype=None, targets=None):
         assert_parity(grad, ref, gd, "grad rank %d vs autograd" % r, scale=10 if gd == torch.float32 else 1)
 
 
-@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32, torch.float16])
 @pytest.mark.parametrize("shape", [(64, 1024, 4), (37, 1571 * 8, 2), (16, 100, 4), (5, 7, 3), (130, 4104, 1)])
 def test_vpce_all_ranks(shape, dtype):
     T, V, p = shape
     _run_all_ranks(T, V, p, dtype, seed=T + V)
 
 
-def test_vpce_bf16_logits_fp32_grad():
-    _run_all_ranks(32, 2048, 2, torch.bfloat16, seed=3, grad_dtype=torch.float32)
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_vpce_16bit_logits_fp32_grad(dtype):
+    _run_all_ranks(32, 2048, 2, dtype, seed=3, grad_dtype=torch.float32)
+    _run_all_ranks(9, 12568, 1, dtype, seed=4, grad_dtype=torch.float32)
+
+
+@pytest.mark.parametrize("amp_dtype", [torch.float16, torch.bfloat16])
+def test_loss_under_autocast_keeps_16bit_logits(amp_dtype):
+    """Classifier + loss inside torch.autocast: the logits reach the loss in the autocast dtype and are not
+    copied to float32 (the reference's custom_fwd(cast_inputs=torch.float32) does; the cast is exact, so the
+    loss and the gradient are those of F.cross_entropy on the float32 copy)."""
+    from cubework_amd.distributed import initialize
+    from cubework_amd.module.loss import VocabParallelCrossEntropyLoss1D
+
+    initialize("1d", 1)
+    T, V = 96, 2000
+    logits = randn((T, V), amp_dtype, 0, std=2.0).to(DEV).requires_grad_(True)
+    t = _targets(T, V, 1).to(DEV)
+    crit = VocabParallelCrossEntropyLoss1D()
+    torch.cuda.synchronize()
+    torch.cuda.reset_peak_memory_stats()
+    before = torch.cuda.memory_allocated()
+    with torch.autocast("cuda", dtype=amp_dtype):
+        loss = crit(logits, t)
+    loss.backward()
+    torch.cuda.synchronize()
+    assert loss.dtype == torch.float32 and logits.grad.dtype == amp_dtype
+    # one gradient of the logits' size and per-row statistics: no float32 copy (T * V * 4 bytes) was made
+    assert torch.cuda.max_memory_allocated() - before < T * V * 2 + T * V * 4
+    ref_in = logits.detach().float().cpu().requires_grad_(True)
+    ref = torch.nn.functional.cross_entropy(ref_in, t.cpu())
+    ref.backward()
+    assert_parity(loss, ref.detach(), torch.float32, "loss", scale=10)
+    assert_parity(logits.grad, ref_in.grad, amp_dtype, "logits grad")
 
 
 def test_vpce_edge_targets():
