@@ -382,6 +382,10 @@ def main():
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run a plain 256 MiB device copy three times (the known-size kernel that hardware "
                          "counter runs of this script are scaled by)")
+    ap.add_argument("--gemm-counter-run", action="store_true",
+                    help="instead of the benchmark: launch the fp32 ring kernels (config 1 forward and input "
+                         "gradient) and the small-tile 16-bit ring kernel (2048^3) six times each, interleaved with "
+                         "torch.matmul on the same operands - the program of the hardware-counter comparison")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         sys.stderr.write("bench.py measures one rank's share on ONE GPU; --gpus N with N > 1 is not part of this "
@@ -398,6 +402,22 @@ def main():
     torch.cuda.set_device(device)
     lib = _lib.load()
     arch = lib.cw_device_arch().decode()
+    if args.gemm_counter_run:
+        x1 = _seeded((4096, 1024), 1, 1.0, torch.float32).to(device)
+        w1 = _seeded((4096, 1024), 2, 0.03, torch.float32).to(device)
+        dy1 = _seeded((4096, 4096), 3, 1.0, torch.float32).to(device)
+        o1 = torch.empty((4096, 4096), dtype=torch.float32, device=device)
+        a2 = _seeded((2048, 2048), 4, 1.0, torch.bfloat16).to(device)
+        b2 = _seeded((2048, 2048), 5, 0.03, torch.bfloat16).to(device)
+        o2 = torch.empty((2048, 2048), dtype=torch.bfloat16, device=device)
+        for _ in range(6):
+            ops.gemm_ksteps("NT", [x1], [w1], out=o1)
+            torch.matmul(x1, w1.t(), out=o1)
+            ops.gemm_ksteps("NN", [dy1], [w1])
+            ops.gemm_ksteps("NN", [a2], [b2], out=o2)
+            torch.matmul(a2, b2, out=o2)
+        torch.cuda.synchronize()
+        return
 
     n_sets = 3  # 3 x 80 MiB of operands rotate so that no step finds its inputs in the Infinity Cache
     sets, bias = make_gemm_inputs(n_sets, device)
