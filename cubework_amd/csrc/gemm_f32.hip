@@ -634,11 +634,13 @@ int gemm_f32_launch(const GemmArgs& args, int layout, int epilogue, hipStream_t 
         const bool ring_ok = ring_enabled && all_vec && fits32 && (args.N % 4) == 0 && (layout != CW_TN || (args.M % 4) == 0) &&
                              args.K >= ring::kBK && (args.K % ring::kBK) == 0 && args.n_steps >= 1 &&
                              args.n_steps <= kRingMaxSteps && args.n_addends <= kRingMaxAddends;
-        // the largest tile that still gives every compute unit work: 256 x 256 (one workgroup per unit), else
-        // 128 x 128 or 128 x 64 (two per unit)
+        // 256 x 256 tiles (one workgroup per compute unit) for long reductions over many tiles; 128 x 128 or
+        // 128 x 64 (two per unit, one's prologue and epilogue under the other's products) for fewer tiles and for
+        // short reductions (config-1 forward, K = 1024: 241 us against 256 us with the large tiles)
         const int64_t tiles128 = ((int64_t)(args.M + 127) / 128) * ((args.N + 127) / 128);
         const int64_t tiles128x64 = ((int64_t)(args.M + 127) / 128) * ((args.N + 63) / 64);
-        if (ring_ok && tiles256 >= 128 && args.M >= 256 && args.N >= 256) return ring::launch_layout<4, 4>(args, layout, epilogue, s);
+        if (ring_ok && tiles256 >= 128 && args.M >= 256 && args.N >= 256 && (int64_t)args.K * args.n_steps > 2048)
+            return ring::launch_layout<4, 4>(args, layout, epilogue, s);
         if (ring_ok && tiles128 >= 384 && args.M >= 128 && args.N >= 128) return ring::launch_layout<2, 2>(args, layout, epilogue, s);
         if (ring_ok && tiles128x64 >= 256 && args.M >= 128 && args.N >= 64) return ring::launch_layout<2, 1>(args, layout, epilogue, s);
     }

@@ -162,10 +162,14 @@ def test_fp32_ring_kernel(layout):
     k-steps (the ring runs across the seam between two steps' allocations), addend, pre-activation copy and
     activation; the shortest reduction the ring takes (one stage); M and N that are not tile multiples
     (last tiles moved back to the edge); padded leading dimensions."""
-    _run(layout, 4096, 2048, 64, 3, torch.float32, act="gelu_tanh", n_add=1, preact=True, seed=21)
-    _run(layout, 2048, 4096, 16, 1, torch.float32, act=None, bias=False, seed=22)
-    _run(layout, 4104, 2060, 48, 2, torch.float32, act="relu", n_add=2, preact=True, seed=23)
-    _run(layout, 4096, 2048, 32, 1, torch.float32, act="gelu_erf", pad_a=4, pad_b=8, seed=24)
+    # 256 x 256 tiles need a total reduction above 2048 (shorter ones take the 128 x 128 tiles)
+    _run(layout, 4096, 2048, 704, 3, torch.float32, act="gelu_tanh", n_add=1, preact=True, seed=21)
+    _run(layout, 2048, 4096, 2064, 1, torch.float32, act=None, bias=False, seed=22)
+    _run(layout, 4104, 2060, 1040, 2, torch.float32, act="relu", n_add=2, preact=True, seed=23)
+    _run(layout, 4096, 2048, 2080, 1, torch.float32, act="gelu_erf", pad_a=4, pad_b=8, seed=24)
+    # the same outputs with short reductions: 128 x 128 tiles, several rounds of two workgroups per unit
+    _run(layout, 4096, 2048, 64, 3, torch.float32, act="gelu_tanh", n_add=1, preact=True, seed=25)
+    _run(layout, 2048, 4096, 16, 1, torch.float32, act=None, bias=False, seed=26)
 
 
 @pytest.mark.parametrize("layout", LAYOUTS)
