@@ -7,14 +7,14 @@ A "step" is one pass of the hot path over one batch of synthetic input: rank
 (0, 1) of a q = 2 SUMMA grid computing
     out[8192, 2048] = GeLU_tanh(A_0 B_0 + A_1 B_1 + bias)        (bf16, fp32 accumulation)
 with the operands a row/column broadcast would deliver already resident in HBM
-(BASELINE.json configs[1]; 137,438,953,472 FLOP per step). One step is one call
+(the benchmark definition's second configuration; 137,438,953,472 FLOP per step). One step is one call
 of cw_gemm_ksteps through the C ABI = one kernel launch.
 
 Prints ONE JSON line. `value` is TFLOP/s over the timed region (wall clock
 around K steps, synchronised on both sides). `roofline` prices the GEMM kernel
 against the MI355X dense bf16 MFMA peak with the average launch duration from
 HIP events on the launch stream. `aux` reports the bandwidth-bound kernels of
-the same path (LayerNorm2D, vocab-parallel CE; BASELINE.json configs[2], [3])
+the same path (LayerNorm2D, vocab-parallel CE: the third and fourth configurations)
 against the 8 TB/s HBM peak, on buffers rotated through > 512 MiB so that the
 256 MiB Infinity Cache cannot serve them. `cpu_baseline` times the reference's
 CPU path (torch, gloo, world size 1) restated by oracle/ on the host cores, on

@@ -185,7 +185,7 @@ def test_fp32_ring_kernel_smaller_tiles(layout):
 
 
 def test_fp32_linear1d_col_shape():
-    # BASELINE config 1: x [8,512,1024] fp32, W [4096,1024], b zeros -> F.linear
+    # the fp32 Linear1D workload: x [8,512,1024] fp32, W [4096,1024], b zeros -> F.linear
     import oracle
     from cubework_amd import ops
 
@@ -201,7 +201,7 @@ def test_fp32_linear1d_col_shape():
 
 
 def test_kstep_sum_equals_concatenated_gemm():
-    # size-independent property at the BASELINE config-2 shape: two k-steps ==
+    # size-independent property at the benchmark's Linear2D shape: two k-steps ==
     # one GEMM over the concatenated operands (both through the HIP path)
     from cubework_amd import ops
 

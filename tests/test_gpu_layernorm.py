@@ -162,7 +162,7 @@ def test_ln3d_backward_formula_matches():
 
 
 def test_ln_baseline_shape_properties():
-    """BASELINE config 3 at full size, through size-independent properties:
+    """The benchmark's LayerNorm2D workload (16384 x 1024 bf16, H = 2048) at full size, through size-independent properties:
     per-row mean(x_hat) = 0, mean(x_hat^2) = var/(var+eps) over the whole H,
     sum_c dx = 0 and sum_c dx*x_hat = 0 over the whole H, split invariance."""
     from cubework_amd import ops

@@ -136,7 +136,7 @@ def test_vpce_does_not_modify_logits_and_handles_padding():
 
 
 def test_vpce_baseline_shape_properties():
-    """BASELINE config 4 at full size (rank 1 of 4, V_loc = 12568): rows of the
+    """The benchmark's cross-entropy workload at full size (rank 1 of 4, V_loc = 12568): rows of the
     softmax gradient sum to zero across the 4 slices; loss equals logsumexp
     minus the target logit on sampled rows; grad = -dloss*(1-softmax) at the
     target column."""
