@@ -286,9 +286,15 @@ __global__ __launch_bounds__(kTileWaves * 64) void ln_normalize_tile_kernel(
     const int lane = threadIdx.x & 63;
     const int64_t wave = (int64_t)blockIdx.x * kTileWaves + (threadIdx.x >> 6);
     const int64_t step = (int64_t)gridDim.x * kTileWaves * NR;
-    raw16_t g_raw[NCH], b_raw[NCH];
-    load_param_chunks<T, NCH>(gamma, C, lane, g_raw);
-    load_param_chunks<T, NCH>(beta, C, lane, b_raw);
+    // gamma and beta stay in registers across rows while they fit beside the tile; the widest fp32 tile
+    // would pass 256 registers with them (one wavefront per SIMD), so it reads them per chunk from cache
+    constexpr bool kHoldParams = !(sizeof(T) == 4 && NCH * NR >= 8);
+    constexpr int NP = kHoldParams ? NCH : 1;
+    raw16_t g_raw[NP], b_raw[NP];
+    if constexpr (kHoldParams) {
+        load_param_chunks<T, NCH>(gamma, C, lane, g_raw);
+        load_param_chunks<T, NCH>(beta, C, lane, b_raw);
+    }
     for (int64_t row0 = wave * NR; row0 < R; row0 += step) {
         RowTile<T, NCH, NR> t;
         t.load(x, ld, row0, R, C, lane);
@@ -319,8 +325,16 @@ __global__ __launch_bounds__(kTileWaves * 64) void ln_normalize_tile_kernel(
             for (int j = 0; j < NCH; ++j) {
                 float v[V], g[V], b[V];
                 unpack_raw(t.raw[r][j], v, (const T*)nullptr);
-                unpack_raw(g_raw[j], g, (const T*)nullptr);
-                unpack_raw(b_raw[j], b, (const T*)nullptr);
+                if constexpr (kHoldParams) {
+                    unpack_raw(g_raw[j], g, (const T*)nullptr);
+                    unpack_raw(b_raw[j], b, (const T*)nullptr);
+                } else {
+                    const bool ok = chunk_valid<T>(j, lane, C);
+                    const int64_t c0 = ok ? ((int64_t)j * 64 + lane) * V : 0;
+                    const raw16_t zero = {0u, 0u, 0u, 0u};
+                    unpack_raw(gamma != nullptr ? load_raw(gamma + c0) : zero, g, (const T*)nullptr);
+                    unpack_raw(beta != nullptr ? load_raw(beta + c0) : zero, b, (const T*)nullptr);
+                }
 #pragma unroll
                 for (int e = 0; e < V; ++e) {
                     float xh = (v[e] - mean) * rstd;
@@ -484,6 +498,151 @@ __global__ __launch_bounds__(NWAVES * 64) void ln_bwd_partials_kernel(
         const int64_t c = ((int64_t)(rem / V) * 64 + l) * V + (rem % V);
         if (c < C) out[(int64_t)set * C + c] = total;
     });
+}
+
+// Backward partials for rows too wide for one wavefront's registers: `wpr` wavefronts share a row, each
+// owning a segment of NCH chunks (kSeg columns), and a block works on blockDim/64/wpr rows at a time. The
+// segments' row sums meet in LDS (one barrier per trip, slots alternating between trips so that no second
+// barrier is needed), after which every wavefront has the row's totals and, with FUSE_DX, writes its
+// segment of dx from the registers that hold the row. The next trip's rows are loaded before the barrier.
+// The dgamma/dbeta accumulators of the row groups are added through LDS at the end, in a fixed order.
+// The launcher chooses wpr so that every segment starts inside the row.
+template <typename T, int NCH, int MAXW, bool FUSE_DX>
+__global__ __launch_bounds__(MAXW * 64, 4) void ln_bwd_split_kernel(
+    int64_t R, int64_t C, const T* __restrict__ dY, int64_t ld_dy, const T* __restrict__ x, int64_t ld_x,
+    const float* __restrict__ mean_rstd, const T* __restrict__ gamma, float* __restrict__ row_sums,
+    float* __restrict__ col_ws, int want_cols, T* __restrict__ dx, int64_t ld_dx, float inv_h, int wpr) {
+    constexpr int V = elem<T>::kVec;
+    constexpr int kSeg = NCH * 64 * V;
+    constexpr int NA = NCH * V;  // accumulators of one set (dgamma or dbeta) in a lane
+    constexpr bool kPrefetch = sizeof(T) == 4;  // 16-bit rows leave no registers for a second pair of tiles
+    extern __shared__ float lds_red[];
+    __shared__ float lds_sums[2][MAXW][2];
+    const int lane = threadIdx.x & 63;
+    const int wave = threadIdx.x >> 6;
+    const int nrg = (int)(blockDim.x >> 6) / wpr;
+    const int rg = wave / wpr, seg = wave - rg * wpr;
+    const int64_t col0 = (int64_t)seg * kSeg;
+    const int64_t Cs = C - col0;  // columns from the segment's start to the end of the row
+    dY += col0;
+    x += col0;
+    if (gamma != nullptr) gamma += col0;
+    if (FUSE_DX) dx += col0;
+
+    raw16_t g_raw[NCH];
+    load_param_chunks<T, NCH>(gamma, Cs, lane, g_raw);
+    float acc[2 * NA];  // [0, NA): dgamma, [NA, 2*NA): dbeta
+#pragma unroll
+    for (int i = 0; i < 2 * NA; ++i) acc[i] = 0.0f;
+
+    const int64_t step = (int64_t)gridDim.x * nrg;
+    int64_t base = (int64_t)blockIdx.x * nrg;  // the same for every wavefront of the block: uniform trip count
+    RowTile<T, NCH, 1> tdy, tx;
+    if (base < R) {
+        tdy.load(dY, ld_dy, base + rg, R, Cs, lane);
+        tx.load(x, ld_x, base + rg, R, Cs, lane);
+    }
+    for (int trip = 0; base < R; base += step, ++trip) {
+        RowTile<T, NCH, 1> ndy, nx;
+        const bool more = kPrefetch && base + step < R;
+        if (more) {
+            ndy.load(dY, ld_dy, base + step + rg, R, Cs, lane);
+            nx.load(x, ld_x, base + step + rg, R, Cs, lane);
+        }
+        const int64_t row = base + rg;
+        const bool live = row < R;
+        const int64_t row_c = live ? row : R - 1;
+        const float mean = mean_rstd[2 * row_c];
+        const float rstd = mean_rstd[2 * row_c + 1];
+        float s1 = 0.0f, s2 = 0.0f;
+#pragma unroll
+        for (int j = 0; j < NCH; ++j) {
+            float dy[V], xv[V], g[V];
+            unpack_raw(tdy.raw[0][j], dy, (const T*)nullptr);
+            unpack_raw(tx.raw[0][j], xv, (const T*)nullptr);
+            unpack_raw(g_raw[j], g, (const T*)nullptr);
+#pragma unroll
+            for (int e = 0; e < V; ++e) {
+                const float d = live ? dy[e] : 0.0f;  // a row past the end adds nothing to the column sums
+                const float xh = (xv[e] - mean) * rstd;
+                const float gd = gamma != nullptr ? d * g[e] : d;
+                s1 += gd;
+                s2 += gd * xh;
+                acc[j * V + e] += d * xh;
+                acc[NA + j * V + e] += d;
+            }
+        }
+        s1 = wave_sum(s1);
+        s2 = wave_sum(s2);
+        if (lane == 0) {
+            lds_sums[trip & 1][wave][0] = s1;
+            lds_sums[trip & 1][wave][1] = s2;
+        }
+        __syncthreads();
+        s1 = 0.0f;
+        s2 = 0.0f;
+        for (int w = 0; w < wpr; ++w) {
+            s1 += lds_sums[trip & 1][rg * wpr + w][0];
+            s2 += lds_sums[trip & 1][rg * wpr + w][1];
+        }
+        if (seg == 0 && lane == 0 && live) {
+            row_sums[2 * row] = s1;
+            row_sums[2 * row + 1] = s2;
+        }
+        if (FUSE_DX) {
+            const float c1 = s1 * inv_h, c2 = s2 * inv_h;
+#pragma unroll
+            for (int j = 0; j < NCH; ++j) {
+                float dy[V], xv[V], g[V];
+                unpack_raw(tdy.raw[0][j], dy, (const T*)nullptr);
+                unpack_raw(tx.raw[0][j], xv, (const T*)nullptr);
+                unpack_raw(g_raw[j], g, (const T*)nullptr);
+#pragma unroll
+                for (int e = 0; e < V; ++e) {
+                    const float xh = (xv[e] - mean) * rstd;
+                    const float gg = gamma != nullptr ? dy[e] * g[e] : dy[e];
+                    dy[e] = (gg - xh * c2 - c1) * rstd;
+                }
+                if (live && chunk_valid<T>(j, lane, Cs))
+                    store_raw_stream(dx + row * ld_dx + ((int64_t)j * 64 + lane) * V, pack_raw(dy, (const T*)nullptr));
+            }
+        }
+        if (more) {
+            tdy = ndy;
+            tx = nx;
+        } else if (!kPrefetch && base + step < R) {
+            tdy.load(dY, ld_dy, base + step + rg, R, Cs, lane);
+            tx.load(x, ld_x, base + step + rg, R, Cs, lane);
+        }
+    }
+    if (!want_cols) return;
+
+    // row groups 1.. hand their accumulators to group 0, one set and one group at a time
+    float* red = lds_red + ((int64_t)seg * NA) * 64 + lane;
+    for (int set = 0; set < 2; ++set) {
+        for (int g = 1; g < nrg; ++g) {
+            __syncthreads();
+            if (rg == g) {
+#pragma unroll
+                for (int i = 0; i < NA; ++i) red[i * 64] = acc[set * NA + i];
+            }
+            __syncthreads();
+            if (rg == 0) {
+#pragma unroll
+                for (int i = 0; i < NA; ++i) acc[set * NA + i] += red[i * 64];
+            }
+        }
+    }
+    if (rg != 0) return;
+    float* out = col_ws + (int64_t)blockIdx.x * 2 * C + col0;
+#pragma unroll
+    for (int set = 0; set < 2; ++set)
+#pragma unroll
+        for (int j = 0; j < NCH; ++j)
+            if (chunk_valid<T>(j, lane, Cs)) {
+#pragma unroll
+                for (int e = 0; e < V; ++e) out[(int64_t)set * C + ((int64_t)j * 64 + lane) * V + e] = acc[set * NA + j * V + e];
+            }
 }
 
 // Backward partials for shapes the vector kernel does not take (ragged C,
@@ -673,6 +832,56 @@ int bwd_partials_launch(int64_t R, int64_t C, const void* dY, int64_t ld_dy, con
                                                              want_cols, nullptr, 0, s);
 }
 
+// Rows of more than kSplitMinChunks chunks go to the split kernel: kSplitChunks chunks per wavefront, blocks
+// of kSplitBlockWaves wavefronts (of as many as a row needs, up to 16, for the widest rows).
+constexpr int kSplitChunks = 2;
+constexpr int kSplitBlockWaves = 8;
+constexpr int64_t kSplitMaxBlocks = 512;
+
+constexpr int kSplitMinChunks = 4;
+
+bool split_takes(int64_t nch) { return nch > kSplitMinChunks && (nch + kSplitChunks - 1) / kSplitChunks <= 16; }
+
+struct SplitShape {
+    int wpr, nrg;
+    int64_t blocks;
+};
+
+SplitShape split_shape(int64_t R, int64_t nch) {
+    SplitShape sh;
+    sh.wpr = (int)((nch + kSplitChunks - 1) / kSplitChunks);
+    sh.nrg = sh.wpr >= kSplitBlockWaves ? 1 : kSplitBlockWaves / sh.wpr;
+    sh.blocks = (R + sh.nrg - 1) / sh.nrg;
+    if (sh.blocks > kSplitMaxBlocks) sh.blocks = kSplitMaxBlocks;
+    if (sh.blocks < 1) sh.blocks = 1;
+    return sh;
+}
+
+template <typename T, int MAXW, bool FUSE_DX>
+int bwd_split_launch_as(const SplitShape& sh, int64_t R, int64_t C, const void* dY, int64_t ld_dy, const void* x,
+                        int64_t ld_x, const float* mean_rstd, const void* gamma, float* row_sums, float* ws,
+                        int want_cols, void* dx, int64_t ld_dx, hipStream_t s) {
+    constexpr int V = elem<T>::kVec;
+    const size_t lds = sh.nrg > 1 ? (size_t)sh.wpr * kSplitChunks * V * 64 * sizeof(float) : 0;
+    hipLaunchKernelGGL((ln_bwd_split_kernel<T, kSplitChunks, MAXW, FUSE_DX>), dim3((unsigned)sh.blocks),
+                       dim3(sh.wpr * sh.nrg * 64), lds, s, R, C, (const T*)dY, ld_dy, (const T*)x, ld_x, mean_rstd,
+                       (const T*)gamma, row_sums, ws, want_cols, (T*)dx, ld_dx, 1.0f / (float)C, sh.wpr);
+    return check_launch("ln_bwd_split_kernel");
+}
+
+template <typename T>
+int bwd_split_launch(const SplitShape& sh, int64_t R, int64_t C, const void* dY, int64_t ld_dy, const void* x,
+                     int64_t ld_x, const float* mean_rstd, const void* gamma, float* row_sums, float* ws,
+                     int want_cols, void* dx, int64_t ld_dx, hipStream_t s) {
+    const bool wide = sh.wpr * sh.nrg > kSplitBlockWaves;
+#define CW_SPLIT(MAXW, FUSE)                                                                                         \
+    bwd_split_launch_as<T, MAXW, FUSE>(sh, R, C, dY, ld_dy, x, ld_x, mean_rstd, gamma, row_sums, ws, want_cols, dx, \
+                                       ld_dx, s)
+    if (dx != nullptr) return wide ? CW_SPLIT(16, true) : CW_SPLIT(kSplitBlockWaves, true);
+    return wide ? CW_SPLIT(16, false) : CW_SPLIT(kSplitBlockWaves, false);
+#undef CW_SPLIT
+}
+
 constexpr int64_t kGenericSlabRows = 64;
 
 // dx != nullptr asks for the fused backward (C is the whole hidden size); *dx_done tells whether the
@@ -690,7 +899,17 @@ int bwd_partials_impl(int64_t R, int64_t C, const void* dY, int64_t ld_dy, const
     const int64_t nch = (C + 64 * V - 1) / (64 * V);
     int64_t nparts = 0;
     int rc;
-    if (vec && nch <= 8) {
+    if (vec && split_takes(nch)) {
+        const SplitShape sh = split_shape(R, nch);
+        nparts = sh.blocks;
+        if (want_cols && workspace_bytes < nparts * 2 * C * (int64_t)sizeof(float))
+            return fail(CW_ERR_INVALID, "cw_ln_bwd_partials: workspace too small (%lld bytes)", (long long)workspace_bytes);
+        void* fdx = (dx != nullptr && rows_vec_ok<T>(dx, ld_dx)) ? dx : nullptr;
+        rc = bwd_split_launch<T>(sh, R, C, dY, ld_dy, x, ld_x, mean_rstd, gamma, row_sums, (float*)workspace, want_cols,
+                                 fdx, ld_dx, s);
+        if (rc != CW_OK) return rc;
+        if (dx_done != nullptr) *dx_done = fdx != nullptr;
+    } else if (vec && nch <= 8) {
         const int rows_per_trip = nch <= 1 ? 16 * 2 : (nch <= 2 ? 16 : (nch <= 4 ? 8 : 4));
         nparts = bwd_blocks(R, rows_per_trip);
         if (want_cols && workspace_bytes < nparts * 2 * C * (int64_t)sizeof(float))
@@ -763,7 +982,7 @@ int check_rc(const char* fn, int64_t R, int64_t C, int io_dtype) {
 // Upper bound of the column-partial scratch cw_ln_bwd_partials can need.
 int64_t ln_bwd_workspace_bytes(int64_t R, int64_t C) {
     int64_t parts = (R + kGenericSlabRows - 1) / kGenericSlabRows;
-    if (parts < 256) parts = 256;
+    if (parts < kSplitMaxBlocks) parts = kSplitMaxBlocks;
     return parts * 2 * C * (int64_t)sizeof(float);
 }
 

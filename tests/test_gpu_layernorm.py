@@ -10,7 +10,8 @@ from tests.util import assert_parity, rand_uniform, randn
 pytestmark = pytest.mark.gpu
 
 DEV = "cuda:0"
-SHAPES = [(64, 1024), (33, 520), (16, 100), (5, 7), (300, 2048), (9, 4096), (3, 8200), (7, 512), (1, 256), (2050, 264)]
+SHAPES = [(64, 1024), (33, 520), (16, 100), (5, 7), (300, 2048), (9, 4096), (3, 8200), (7, 512), (1, 256), (2050, 264),
+          (1500, 3072), (5, 16384), (2, 16392)]
 
 
 def _inputs(R, C, dtype, seed):
@@ -87,11 +88,13 @@ def test_ln_fused_matches_nn_layernorm(shape, mode, dtype):
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
 @pytest.mark.parametrize("affine", [True, False])
-@pytest.mark.parametrize("shape", [(64, 1024), (17, 200), (4, 2048), (1000, 512), (33, 4096), (5, 1001), (3, 5000), (300, 64)])
+@pytest.mark.parametrize("shape", [(64, 1024), (17, 200), (4, 2048), (1000, 512), (33, 4096), (5, 1001), (3, 5000), (300, 64),
+                                   (70, 8192), (9, 12288), (600, 3072), (2100, 2560), (3, 16384), (2, 20480)])
 def test_ln_backward_fused_matches_autograd(shape, affine, dtype):
     """Rows complete on this rank: one pass gives dx, dgamma, dbeta. Against F.layer_norm's autograd, and
     bit-identical to the two-kernel path (partials, then dx with H = C) that it replaces. Shapes cover
-    every chunk count of the one-pass kernel, ragged widths and the generic fallback."""
+    every chunk count of the one-pass kernel, the kernel that splits wide rows over wavefronts (blocks of one
+    to four row groups, several trips, rows past the end), ragged widths and the generic fallback."""
     from cubework_amd import ops
 
     R, C = shape
