@@ -349,6 +349,93 @@ __global__ __launch_bounds__(kTileWaves * 64) void ln_normalize_tile_kernel(
     }
 }
 
+// Fused forward for rows wider than a wavefront's registers: `wpr` wavefronts share a row, NCH chunks each
+// (the launcher chooses wpr so that every segment starts inside the row), and a block works on
+// blockDim/64/wpr rows at a time. The segments' moments meet in LDS, one barrier per exchange: one exchange
+// per row for one-pass statistics, two for two-pass; the slots alternate between trips so that a wavefront
+// a trip ahead never overwrites sums that another still reads. The row is read from memory once; gamma and
+// beta come from cache per chunk; the next trip's rows are loaded before the barrier.
+template <typename T, int NCH, int MAXW>
+__global__ __launch_bounds__(MAXW * 64) void ln_forward_split_kernel(
+    int64_t R, int64_t C, const T* __restrict__ x, int64_t ld, int mode, float inv_h, float eps,
+    const T* __restrict__ gamma, const T* __restrict__ beta, T* __restrict__ y, int64_t ldy,
+    float* __restrict__ mean_rstd, int wpr) {
+    constexpr int V = elem<T>::kVec;
+    __shared__ float lds_sums[2][2][MAXW][2];  // [trip parity][exchange][wavefront][moment]
+    const int lane = threadIdx.x & 63;
+    const int wave = threadIdx.x >> 6;
+    const int nrg = (int)(blockDim.x >> 6) / wpr;
+    const int rg = wave / wpr, seg = wave - rg * wpr;
+    const int64_t col0 = (int64_t)seg * (NCH * 64 * V);
+    const int64_t Cs = C - col0;  // columns from the segment's start to the end of the row
+    x += col0;
+    y += col0;
+    if (gamma != nullptr) gamma += col0;
+    if (beta != nullptr) beta += col0;
+
+    // totals of (a, b) over the wavefronts of this row group, the same in every lane of the group
+    auto exchange = [&](int parity, int which, float& a, float& b) {
+        if (lane == 0) {
+            lds_sums[parity][which][wave][0] = a;
+            lds_sums[parity][which][wave][1] = b;
+        }
+        __syncthreads();
+        a = 0.0f;
+        b = 0.0f;
+        for (int w = 0; w < wpr; ++w) {
+            a += lds_sums[parity][which][rg * wpr + w][0];
+            b += lds_sums[parity][which][rg * wpr + w][1];
+        }
+    };
+
+    const int64_t step = (int64_t)gridDim.x * nrg;
+    int64_t base = (int64_t)blockIdx.x * nrg;  // the same for every wavefront of the block: uniform trip count
+    RowTile<T, NCH, 1> t;
+    if (base < R) t.load(x, ld, base + rg, R, Cs, lane);
+    for (int trip = 0; base < R; base += step, ++trip) {
+        RowTile<T, NCH, 1> next;
+        const bool more = base + step < R;
+        if (more) next.load(x, ld, base + step + rg, R, Cs, lane);
+        const int64_t row = base + rg;
+        const bool live = row < R;
+        float s1, s2, mean, rstd;
+        tile_moments(t, 0, Cs, 0.0f, lane, s1, s2);
+        exchange(trip & 1, 0, s1, s2);
+        if (mode == CW_LN_TWO_PASS) {
+            const float mu = s1 * inv_h;
+            float d1, d2;
+            tile_moments(t, 0, Cs, mu, lane, d1, d2);
+            exchange(trip & 1, 1, d1, d2);
+            finish_stats(mode, mu, d2, inv_h, eps, mean, rstd);
+        } else {
+            finish_stats(mode, s1, s2, inv_h, eps, mean, rstd);
+        }
+        if (mean_rstd != nullptr && seg == 0 && lane == 0 && live) {
+            mean_rstd[2 * row] = mean;
+            mean_rstd[2 * row + 1] = rstd;
+        }
+#pragma unroll
+        for (int j = 0; j < NCH; ++j) {
+            const bool ok = chunk_valid<T>(j, lane, Cs);
+            const int64_t c0 = ok ? ((int64_t)j * 64 + lane) * V : 0;
+            const raw16_t zero = {0u, 0u, 0u, 0u};
+            float v[V], g[V], b[V];
+            unpack_raw(t.raw[0][j], v, (const T*)nullptr);
+            unpack_raw(gamma != nullptr ? load_raw(gamma + c0) : zero, g, (const T*)nullptr);
+            unpack_raw(beta != nullptr ? load_raw(beta + c0) : zero, b, (const T*)nullptr);
+#pragma unroll
+            for (int e = 0; e < V; ++e) {
+                float xh = (v[e] - mean) * rstd;
+                if (gamma != nullptr) xh *= g[e];
+                if (beta != nullptr) xh += b[e];
+                v[e] = xh;
+            }
+            if (live && ok) store_raw_stream(y + row * ldy + c0, pack_raw(v, (const T*)nullptr));
+        }
+        if (more) t = next;
+    }
+}
+
 template <typename T, int NCH, int NR>
 __global__ __launch_bounds__(kTileWaves * 64) void ln_bwd_dx_tile_kernel(
     int64_t R, int64_t C, const T* __restrict__ dY, int64_t ld_dy, const T* __restrict__ x, int64_t ld_x,
@@ -515,7 +602,8 @@ __global__ __launch_bounds__(MAXW * 64, 4) void ln_bwd_split_kernel(
     constexpr int V = elem<T>::kVec;
     constexpr int kSeg = NCH * 64 * V;
     constexpr int NA = NCH * V;  // accumulators of one set (dgamma or dbeta) in a lane
-    constexpr bool kPrefetch = sizeof(T) == 4;  // 16-bit rows leave no registers for a second pair of tiles
+    // 16-bit rows and segments of more than two chunks leave no registers for a second pair of tiles
+    constexpr bool kPrefetch = sizeof(T) == 4 && NCH <= 2;
     extern __shared__ float lds_red[];
     __shared__ float lds_sums[2][MAXW][2];
     const int lane = threadIdx.x & 63;
@@ -774,6 +862,11 @@ int stats_impl(int64_t R, int64_t C, const void* x, int64_t ld, int mode, const 
     return check_launch("ln_stats_kernel");
 }
 
+// The fused forward of rows of more than 8 chunks: chunks per wavefront and wavefronts per block of
+// ln_forward_split_kernel (blocks of as many wavefronts as a row needs, up to 16, for the widest rows).
+constexpr int kFwdSplitChunks = 4;
+constexpr int kFwdSplitBlockWaves = 8;
+
 template <typename T, bool FUSED>
 int normalize_impl(int64_t R, int64_t C, const void* x, int64_t ld, const float* stats, int mode, int64_t H,
                    float eps, const void* gamma, const void* beta, void* y, int64_t ldy, float* mean_rstd,
@@ -789,6 +882,24 @@ int normalize_impl(int64_t R, int64_t C, const void* x, int64_t ld, const float*
                                (const T*)gamma, (const T*)beta, (T*)y, ldy, mean_rstd);
             return check_launch("ln_normalize_tile_kernel");
         });
+    }
+    if constexpr (FUSED) {
+        const int wpr = (int)((nch + kFwdSplitChunks - 1) / kFwdSplitChunks);
+        if (vec_ok && (C % elem<T>::kVec) == 0 && nch > 8 && wpr <= 16) {
+            const int nrg = wpr >= kFwdSplitBlockWaves ? 1 : kFwdSplitBlockWaves / wpr;
+            int64_t blocks = (R + nrg - 1) / nrg;
+            const int64_t cap = 256 * (16 / (wpr * nrg));
+            if (blocks > cap) blocks = cap;
+            if (wpr * nrg > kFwdSplitBlockWaves)
+                hipLaunchKernelGGL((ln_forward_split_kernel<T, kFwdSplitChunks, 16>), dim3((unsigned)blocks),
+                                   dim3(wpr * nrg * 64), 0, s, R, C, (const T*)x, ld, mode, 1.0f / (float)H, eps,
+                                   (const T*)gamma, (const T*)beta, (T*)y, ldy, mean_rstd, wpr);
+            else
+                hipLaunchKernelGGL((ln_forward_split_kernel<T, kFwdSplitChunks, kFwdSplitBlockWaves>),
+                                   dim3((unsigned)blocks), dim3(wpr * nrg * 64), 0, s, R, C, (const T*)x, ld, mode,
+                                   1.0f / (float)H, eps, (const T*)gamma, (const T*)beta, (T*)y, ldy, mean_rstd, wpr);
+            return check_launch("ln_forward_split_kernel");
+        }
     }
     hipLaunchKernelGGL((ln_normalize_kernel<T, FUSED>), dim3(ln_grid(R)), dim3(kLnBlock), 0, s, R, C, (const T*)x,
                        ld, stats, mode, 1.0f / (float)H, eps, (const T*)gamma, (const T*)beta, (T*)y, ldy,
@@ -832,24 +943,34 @@ int bwd_partials_launch(int64_t R, int64_t C, const void* dY, int64_t ld_dy, con
                                                              want_cols, nullptr, 0, s);
 }
 
-// Rows of more than kSplitMinChunks chunks go to the split kernel: kSplitChunks chunks per wavefront, blocks
-// of kSplitBlockWaves wavefronts (of as many as a row needs, up to 16, for the widest rows).
+// Rows of more than kSplitMinChunks chunks go to the split kernel: kSplitChunks chunks per wavefront (three
+// or four for fp32 rows too wide for 16 such wavefronts), blocks of kSplitBlockWaves wavefronts (of as many
+// as a row needs, up to 16, for the widest rows).
 constexpr int kSplitChunks = 2;
 constexpr int kSplitBlockWaves = 8;
 constexpr int64_t kSplitMaxBlocks = 512;
 
 constexpr int kSplitMinChunks = 4;
 
-bool split_takes(int64_t nch) { return nch > kSplitMinChunks && (nch + kSplitChunks - 1) / kSplitChunks <= 16; }
+// chunks per wavefront of the split kernel for rows of nch chunks, 0 if it does not take them
+template <typename T>
+int split_chunks(int64_t nch) {
+    if (nch <= kSplitMinChunks) return 0;
+    if ((nch + kSplitChunks - 1) / kSplitChunks <= 16) return kSplitChunks;
+    if (sizeof(T) == 4 && (nch + 2) / 3 <= 16) return 3;
+    if (sizeof(T) == 4 && (nch + 3) / 4 <= 16) return 4;
+    return 0;
+}
 
 struct SplitShape {
-    int wpr, nrg;
+    int chunks, wpr, nrg;
     int64_t blocks;
 };
 
-SplitShape split_shape(int64_t R, int64_t nch) {
+SplitShape split_shape(int64_t R, int64_t nch, int chunks) {
     SplitShape sh;
-    sh.wpr = (int)((nch + kSplitChunks - 1) / kSplitChunks);
+    sh.chunks = chunks;
+    sh.wpr = (int)((nch + chunks - 1) / chunks);
     sh.nrg = sh.wpr >= kSplitBlockWaves ? 1 : kSplitBlockWaves / sh.wpr;
     sh.blocks = (R + sh.nrg - 1) / sh.nrg;
     if (sh.blocks > kSplitMaxBlocks) sh.blocks = kSplitMaxBlocks;
@@ -857,13 +978,13 @@ SplitShape split_shape(int64_t R, int64_t nch) {
     return sh;
 }
 
-template <typename T, int MAXW, bool FUSE_DX>
+template <typename T, int NCH, int MAXW, bool FUSE_DX>
 int bwd_split_launch_as(const SplitShape& sh, int64_t R, int64_t C, const void* dY, int64_t ld_dy, const void* x,
                         int64_t ld_x, const float* mean_rstd, const void* gamma, float* row_sums, float* ws,
                         int want_cols, void* dx, int64_t ld_dx, hipStream_t s) {
     constexpr int V = elem<T>::kVec;
-    const size_t lds = sh.nrg > 1 ? (size_t)sh.wpr * kSplitChunks * V * 64 * sizeof(float) : 0;
-    hipLaunchKernelGGL((ln_bwd_split_kernel<T, kSplitChunks, MAXW, FUSE_DX>), dim3((unsigned)sh.blocks),
+    const size_t lds = sh.nrg > 1 ? (size_t)sh.wpr * NCH * V * 64 * sizeof(float) : 0;
+    hipLaunchKernelGGL((ln_bwd_split_kernel<T, NCH, MAXW, FUSE_DX>), dim3((unsigned)sh.blocks),
                        dim3(sh.wpr * sh.nrg * 64), lds, s, R, C, (const T*)dY, ld_dy, (const T*)x, ld_x, mean_rstd,
                        (const T*)gamma, row_sums, ws, want_cols, (T*)dx, ld_dx, 1.0f / (float)C, sh.wpr);
     return check_launch("ln_bwd_split_kernel");
@@ -874,11 +995,16 @@ int bwd_split_launch(const SplitShape& sh, int64_t R, int64_t C, const void* dY,
                      int64_t ld_x, const float* mean_rstd, const void* gamma, float* row_sums, float* ws,
                      int want_cols, void* dx, int64_t ld_dx, hipStream_t s) {
     const bool wide = sh.wpr * sh.nrg > kSplitBlockWaves;
-#define CW_SPLIT(MAXW, FUSE)                                                                                         \
-    bwd_split_launch_as<T, MAXW, FUSE>(sh, R, C, dY, ld_dy, x, ld_x, mean_rstd, gamma, row_sums, ws, want_cols, dx, \
-                                       ld_dx, s)
-    if (dx != nullptr) return wide ? CW_SPLIT(16, true) : CW_SPLIT(kSplitBlockWaves, true);
-    return wide ? CW_SPLIT(16, false) : CW_SPLIT(kSplitBlockWaves, false);
+#define CW_SPLIT(NCH, MAXW, FUSE)                                                                               \
+    bwd_split_launch_as<T, NCH, MAXW, FUSE>(sh, R, C, dY, ld_dy, x, ld_x, mean_rstd, gamma, row_sums, ws, want_cols, \
+                                            dx, ld_dx, s)
+    if constexpr (sizeof(T) == 4) {
+        // three or four chunks: only rows that need more than eight such wavefronts, in one row group
+        if (sh.chunks == 3) return dx != nullptr ? CW_SPLIT(3, 16, true) : CW_SPLIT(3, 16, false);
+        if (sh.chunks == 4) return dx != nullptr ? CW_SPLIT(4, 16, true) : CW_SPLIT(4, 16, false);
+    }
+    if (dx != nullptr) return wide ? CW_SPLIT(kSplitChunks, 16, true) : CW_SPLIT(kSplitChunks, kSplitBlockWaves, true);
+    return wide ? CW_SPLIT(kSplitChunks, 16, false) : CW_SPLIT(kSplitChunks, kSplitBlockWaves, false);
 #undef CW_SPLIT
 }
 
@@ -899,8 +1025,8 @@ int bwd_partials_impl(int64_t R, int64_t C, const void* dY, int64_t ld_dy, const
     const int64_t nch = (C + 64 * V - 1) / (64 * V);
     int64_t nparts = 0;
     int rc;
-    if (vec && split_takes(nch)) {
-        const SplitShape sh = split_shape(R, nch);
+    if (vec && split_chunks<T>(nch) != 0) {
+        const SplitShape sh = split_shape(R, nch, split_chunks<T>(nch));
         nparts = sh.blocks;
         if (want_cols && workspace_bytes < nparts * 2 * C * (int64_t)sizeof(float))
             return fail(CW_ERR_INVALID, "cw_ln_bwd_partials: workspace too small (%lld bytes)", (long long)workspace_bytes);

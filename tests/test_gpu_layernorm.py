@@ -60,7 +60,8 @@ def test_ln2d_forward_backward_with_peer_partials(shape, dtype):
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
 @pytest.mark.parametrize("mode", ["one_pass", "two_pass"])
-@pytest.mark.parametrize("shape", [(64, 1024), (17, 200), (4, 2048)])
+@pytest.mark.parametrize("shape", [(64, 1024), (17, 200), (4, 2048), (33, 4096), (70, 8192), (9, 12288), (2100, 2560),
+                                   (1100, 5120), (3, 16384), (2, 20480)])
 def test_ln_fused_matches_nn_layernorm(shape, mode, dtype):
     """tensor-parallel size 1: against F.layer_norm and its autograd, the
     oracle the reference's 3D test uses (tests/test_3d/check_3d_modules.py:132)."""
@@ -89,7 +90,8 @@ def test_ln_fused_matches_nn_layernorm(shape, mode, dtype):
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
 @pytest.mark.parametrize("affine", [True, False])
 @pytest.mark.parametrize("shape", [(64, 1024), (17, 200), (4, 2048), (1000, 512), (33, 4096), (5, 1001), (3, 5000), (300, 64),
-                                   (70, 8192), (9, 12288), (600, 3072), (2100, 2560), (3, 16384), (2, 20480)])
+                                   (70, 8192), (9, 12288), (600, 3072), (2100, 2560), (3, 16384), (2, 20480),
+                                   (600, 10240)])
 def test_ln_backward_fused_matches_autograd(shape, affine, dtype):
     """Rows complete on this rank: one pass gives dx, dgamma, dbeta. Against F.layer_norm's autograd, and
     bit-identical to the two-kernel path (partials, then dx with H = C) that it replaces. Shapes cover
