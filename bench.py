@@ -136,6 +136,26 @@ def bench_bandwidth_kernels(device):
         out[name] = {"us": round(us, 2), "GBps": round(nbytes / us / 1e3, 1), "frac": round(nbytes / us / 1e3 / HBM_PEAK_GBPS, 3),
                      "bytes": nbytes}
     del xs, dys
+    # wide rows held whole by the rank: the fp32 residual stream under autocast (hidden 2048 and 4096) and a
+    # 16-bit hidden size of 4096; fused forward (x read, y written) and fused backward (dy, x read, dx written)
+    for tag, Rw, Cw, dt in (("fp32_8192x2048", 8192, 2048, torch.float32), ("fp32_4096x4096", 4096, 4096, torch.float32),
+                            ("bf16_8192x4096", 8192, 4096, torch.bfloat16)):
+        nw = 6
+        es = 4 if dt == torch.float32 else 2
+        xw = [_seeded((Rw, Cw), 400 + k, 1.0, dt).to(device) for k in range(nw)]
+        dw = [_seeded((Rw, Cw), 500 + k, 1.0, dt).to(device) for k in range(nw)]
+        gw = torch.ones(Cw, dtype=dt, device=device)
+        bw = torch.zeros(Cw, dtype=dt, device=device)
+        mrw = ops.ln_forward_fused(xw[0], 1e-5, gw, bw)[1]
+        for name, nbytes, fn in (
+                ("ln_forward_fused_" + tag, 2 * Rw * Cw * es + 2 * Cw * es + 8 * Rw,
+                 lambda: ops.ln_forward_fused(rot(xw), 1e-5, gw, bw)),
+                ("ln_backward_fused_" + tag, 3 * Rw * Cw * es + Cw * es + 8 * Rw + 8 * Cw,
+                 lambda: ops.ln_backward_fused(rot(dw), xw[i[0] % nw], mrw, gw))):
+            us = graph_time_us(fn, 2 * nw)
+            out[name] = {"us": round(us, 2), "GBps": round(nbytes / us / 1e3, 1),
+                         "frac": round(nbytes / us / 1e3 / HBM_PEAK_GBPS, 3), "bytes": nbytes}
+        del xw, dw
     T, V, V0 = 8192, 12568, 12568
     lg = [_seeded((T, V), 300 + k, 2.0, torch.bfloat16).to(device) for k in range(3)]  # 3 x 196 MiB
     tg = torch.randint(0, 50272, (T,), generator=torch.Generator().manual_seed(9)).to(device)
