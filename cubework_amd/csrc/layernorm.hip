@@ -349,6 +349,54 @@ __global__ __launch_bounds__(kTileWaves * 64) void ln_normalize_tile_kernel(
     }
 }
 
+// Partial statistics of rows wider than a wavefront's registers, laid out like ln_forward_split_kernel:
+// `wpr` wavefronts share a row and add their moments through LDS (one barrier per row).
+template <typename T, int NCH, int MAXW>
+__global__ __launch_bounds__(MAXW * 64) void ln_stats_split_kernel(int64_t R, int64_t C, const T* __restrict__ x,
+                                                                   int64_t ld, int mode,
+                                                                   const float* __restrict__ mean,
+                                                                   float* __restrict__ stats, int wpr) {
+    constexpr int V = elem<T>::kVec;
+    __shared__ float lds_sums[2][MAXW][2];  // [trip parity][wavefront][moment]
+    const int lane = threadIdx.x & 63;
+    const int wave = threadIdx.x >> 6;
+    const int nrg = (int)(blockDim.x >> 6) / wpr;
+    const int rg = wave / wpr, seg = wave - rg * wpr;
+    const int64_t col0 = (int64_t)seg * (NCH * 64 * V);
+    const int64_t Cs = C - col0;
+    x += col0;
+    const bool centred = mode == CW_LN_TWO_PASS && mean != nullptr;
+    const int64_t step = (int64_t)gridDim.x * nrg;
+    int64_t base = (int64_t)blockIdx.x * nrg;
+    RowTile<T, NCH, 1> t;
+    if (base < R) t.load(x, ld, base + rg, R, Cs, lane);
+    for (int trip = 0; base < R; base += step, ++trip) {
+        RowTile<T, NCH, 1> next;
+        const bool more = base + step < R;
+        if (more) next.load(x, ld, base + step + rg, R, Cs, lane);
+        const int64_t row = base + rg;
+        const float mu = centred ? mean[row < R ? row : R - 1] : 0.0f;
+        float s1, s2;
+        tile_moments(t, 0, Cs, mu, lane, s1, s2);
+        if (lane == 0) {
+            lds_sums[trip & 1][wave][0] = s1;
+            lds_sums[trip & 1][wave][1] = s2;
+        }
+        __syncthreads();
+        if (seg == 0 && lane == 0 && row < R) {
+            s1 = 0.0f;
+            s2 = 0.0f;
+            for (int w = 0; w < wpr; ++w) {
+                s1 += lds_sums[trip & 1][rg * wpr + w][0];
+                s2 += lds_sums[trip & 1][rg * wpr + w][1];
+            }
+            stats[2 * row] = s1;
+            stats[2 * row + 1] = (mode == CW_LN_TWO_PASS && mean == nullptr) ? 0.0f : s2;
+        }
+        if (more) t = next;
+    }
+}
+
 // Fused forward for rows wider than a wavefront's registers: `wpr` wavefronts share a row, NCH chunks each
 // (the launcher chooses wpr so that every segment starts inside the row), and a block works on
 // blockDim/64/wpr rows at a time. The segments' moments meet in LDS, one barrier per exchange: one exchange
@@ -844,6 +892,31 @@ bool rows_vec_ok(const void* p, int64_t ld) {
     return aligned16(p) && (ld % elem<T>::kVec) == 0;
 }
 
+// Chunks per wavefront and wavefronts per block of the forward-side split kernels (statistics, fused
+// forward) for rows of more than 8 chunks; blocks of as many wavefronts as a row needs, up to 16, for the
+// widest rows.
+constexpr int kFwdSplitChunks = 4;
+constexpr int kFwdSplitBlockWaves = 8;
+
+struct FwdSplitShape {
+    int wpr, nrg;
+    int64_t blocks;
+    bool takes, wide;
+};
+
+FwdSplitShape fwd_split_shape(int64_t R, int64_t nch) {
+    FwdSplitShape sh;
+    sh.wpr = (int)((nch + kFwdSplitChunks - 1) / kFwdSplitChunks);
+    sh.takes = nch > 8 && sh.wpr <= 16;
+    sh.nrg = sh.wpr >= kFwdSplitBlockWaves ? 1 : kFwdSplitBlockWaves / sh.wpr;
+    sh.wide = sh.wpr * sh.nrg > kFwdSplitBlockWaves;
+    sh.blocks = (R + sh.nrg - 1) / sh.nrg;
+    const int64_t cap = sh.takes ? 256 * (16 / (sh.wpr * sh.nrg)) : 1;  // 16 wavefronts per CU
+    if (sh.blocks > cap) sh.blocks = cap;
+    if (sh.blocks < 1) sh.blocks = 1;
+    return sh;
+}
+
 template <typename T>
 int stats_impl(int64_t R, int64_t C, const void* x, int64_t ld, int mode, const float* mean, float* stats,
                hipStream_t s) {
@@ -857,15 +930,21 @@ int stats_impl(int64_t R, int64_t C, const void* x, int64_t ld, int mode, const 
             return check_launch("ln_stats_tile_kernel");
         });
     }
+    const FwdSplitShape sh = fwd_split_shape(R, nch);
+    if (vec_ok && (C % elem<T>::kVec) == 0 && sh.takes) {
+        const dim3 grid((unsigned)sh.blocks), block(sh.wpr * sh.nrg * 64);
+        if (sh.wide)
+            hipLaunchKernelGGL((ln_stats_split_kernel<T, kFwdSplitChunks, 16>), grid, block, 0, s, R, C, (const T*)x,
+                               ld, mode, mean, stats, sh.wpr);
+        else
+            hipLaunchKernelGGL((ln_stats_split_kernel<T, kFwdSplitChunks, kFwdSplitBlockWaves>), grid, block, 0, s,
+                               R, C, (const T*)x, ld, mode, mean, stats, sh.wpr);
+        return check_launch("ln_stats_split_kernel");
+    }
     hipLaunchKernelGGL(ln_stats_kernel<T>, dim3(ln_grid(R)), dim3(kLnBlock), 0, s, R, C, (const T*)x, ld, mode,
                        mean, stats, vec_ok);
     return check_launch("ln_stats_kernel");
 }
-
-// The fused forward of rows of more than 8 chunks: chunks per wavefront and wavefronts per block of
-// ln_forward_split_kernel (blocks of as many wavefronts as a row needs, up to 16, for the widest rows).
-constexpr int kFwdSplitChunks = 4;
-constexpr int kFwdSplitBlockWaves = 8;
 
 template <typename T, bool FUSED>
 int normalize_impl(int64_t R, int64_t C, const void* x, int64_t ld, const float* stats, int mode, int64_t H,
@@ -884,20 +963,17 @@ int normalize_impl(int64_t R, int64_t C, const void* x, int64_t ld, const float*
         });
     }
     if constexpr (FUSED) {
-        const int wpr = (int)((nch + kFwdSplitChunks - 1) / kFwdSplitChunks);
-        if (vec_ok && (C % elem<T>::kVec) == 0 && nch > 8 && wpr <= 16) {
-            const int nrg = wpr >= kFwdSplitBlockWaves ? 1 : kFwdSplitBlockWaves / wpr;
-            int64_t blocks = (R + nrg - 1) / nrg;
-            const int64_t cap = 256 * (16 / (wpr * nrg));
-            if (blocks > cap) blocks = cap;
-            if (wpr * nrg > kFwdSplitBlockWaves)
-                hipLaunchKernelGGL((ln_forward_split_kernel<T, kFwdSplitChunks, 16>), dim3((unsigned)blocks),
-                                   dim3(wpr * nrg * 64), 0, s, R, C, (const T*)x, ld, mode, 1.0f / (float)H, eps,
-                                   (const T*)gamma, (const T*)beta, (T*)y, ldy, mean_rstd, wpr);
+        const FwdSplitShape sh = fwd_split_shape(R, nch);
+        if (vec_ok && (C % elem<T>::kVec) == 0 && sh.takes) {
+            const dim3 grid((unsigned)sh.blocks), block(sh.wpr * sh.nrg * 64);
+            if (sh.wide)
+                hipLaunchKernelGGL((ln_forward_split_kernel<T, kFwdSplitChunks, 16>), grid, block, 0, s, R, C,
+                                   (const T*)x, ld, mode, 1.0f / (float)H, eps, (const T*)gamma, (const T*)beta,
+                                   (T*)y, ldy, mean_rstd, sh.wpr);
             else
-                hipLaunchKernelGGL((ln_forward_split_kernel<T, kFwdSplitChunks, kFwdSplitBlockWaves>),
-                                   dim3((unsigned)blocks), dim3(wpr * nrg * 64), 0, s, R, C, (const T*)x, ld, mode,
-                                   1.0f / (float)H, eps, (const T*)gamma, (const T*)beta, (T*)y, ldy, mean_rstd, wpr);
+                hipLaunchKernelGGL((ln_forward_split_kernel<T, kFwdSplitChunks, kFwdSplitBlockWaves>), grid, block, 0,
+                                   s, R, C, (const T*)x, ld, mode, 1.0f / (float)H, eps, (const T*)gamma,
+                                   (const T*)beta, (T*)y, ldy, mean_rstd, sh.wpr);
             return check_launch("ln_forward_split_kernel");
         }
     }
@@ -973,6 +1049,8 @@ SplitShape split_shape(int64_t R, int64_t nch, int chunks) {
     sh.wpr = (int)((nch + chunks - 1) / chunks);
     sh.nrg = sh.wpr >= kSplitBlockWaves ? 1 : kSplitBlockWaves / sh.wpr;
     sh.blocks = (R + sh.nrg - 1) / sh.nrg;
+    const int64_t cap = 256 * (16 / (sh.wpr * sh.nrg));  // 16 wavefronts per CU; at most kSplitMaxBlocks
+    if (sh.blocks > cap) sh.blocks = cap;
     if (sh.blocks > kSplitMaxBlocks) sh.blocks = kSplitMaxBlocks;
     if (sh.blocks < 1) sh.blocks = 1;
     return sh;
@@ -1082,7 +1160,8 @@ int bwd_dx_impl(int64_t R, int64_t C, const void* dY, int64_t ld_dy, const void*
     const int vec_ok = rows_vec_ok<T>(dY, ld_dy) && rows_vec_ok<T>(x, ld_x) && rows_vec_ok<T>(dx, ld_dx) &&
                        (gamma == nullptr || aligned16(gamma));
     const int64_t nch = row_chunks<T>(C);
-    if (vec_ok && (C % elem<T>::kVec) == 0 && nch <= 8) {
+    // rows of more than 4 chunks are faster on the looping kernel (the 8-chunk tile needs 160-240 registers)
+    if (vec_ok && (C % elem<T>::kVec) == 0 && nch <= 4) {
         return dispatch_tile(nch, [&](auto nch_c, auto nr_c) {
             constexpr int NCH = decltype(nch_c)::value, NR = decltype(nr_c)::value;
             hipLaunchKernelGGL((ln_bwd_dx_tile_kernel<T, NCH, NR>), dim3(tile_grid(R, NR)), dim3(kTileWaves * 64), 0,

@@ -148,7 +148,7 @@ int cw_gemm_ksteps_ws(int layout, int64_t M, int64_t N, int64_t K, int n_steps,
 
 /* ---- bias / activation backward ---------------------------------------- */
 /*
- * Number of bytes of scratch cw_colsum / cw_act_bwd_colsum / cw_ln_bwd_partials
+ * Number of bytes of scratch cw_colsum / cw_act_bwd_colsum / cw_ln_bwd_partials / cw_ln_backward_fused
  * need for an [M,N] operand.
  */
 int64_t cw_colsum_workspace_bytes(int64_t M, int64_t N);

@@ -121,14 +121,17 @@ def test_ln_backward_fused_matches_autograd(shape, affine, dtype):
     assert torch.equal(dg, dg2) and torch.equal(db, db2)
 
 
-def test_ln3d_two_pass_with_peer():
+@pytest.mark.parametrize("shape", [(40, 512), (700, 3072), (3, 9216), (5, 20480)])
+def test_ln3d_two_pass_with_peer(shape):
     """3D flavour on one rank of a depth-2 output group: mean exchange, then
-    the centred second moment (parallel_3d/_operation.py:273-276)."""
+    the centred second moment (parallel_3d/_operation.py:273-276). The wide shapes take the statistics
+    kernel that splits a row over wavefronts (several trips; one 16-wavefront group) and the looping one."""
     import oracle
     from cubework_amd import ops
     from cubework_amd._lib import CW_LN_TWO_PASS
 
-    R, C, H, eps = 40, 512, 1024, 1e-12
+    R, C = shape
+    H, eps = 2 * C, 1e-12
     x, dy, gamma, beta = _inputs(R, C, torch.float32, 21)
     x_peer = randn((R, C), torch.float32, 99)
     s_local = ops.ln_partial_stats(x.to(DEV), CW_LN_TWO_PASS, None)
