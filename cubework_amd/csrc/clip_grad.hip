@@ -212,7 +212,8 @@ extern "C" int cw_multi_norm_partials(int n_tensors, const void* const* grads, c
                                       float* out2, void* workspace, int64_t workspace_bytes, int io_dtype,
                                       void* stream) {
     if (n_tensors < 0) return fail(CW_ERR_INVALID, "cw_multi_norm_partials: negative tensor count");
-    if (io_dtype != CW_BF16 && io_dtype != CW_F32) return fail(CW_ERR_INVALID, "cw_multi_norm_partials: bad io_dtype %d", io_dtype);
+    if (io_dtype != CW_BF16 && io_dtype != CW_F32 && io_dtype != CW_F16)
+        return fail(CW_ERR_INVALID, "cw_multi_norm_partials: bad io_dtype %d", io_dtype);
     if (out2 == nullptr || workspace == nullptr) return fail(CW_ERR_INVALID, "cw_multi_norm_partials: null output or workspace");
     if (!(norm_type > 0.0f)) return fail(CW_ERR_INVALID, "cw_multi_norm_partials: norm_type must be positive (inf for the maximum norm)");
     if (n_tensors > 0 && (grads == nullptr || numels == nullptr)) return fail(CW_ERR_INVALID, "cw_multi_norm_partials: null tables");
@@ -233,6 +234,8 @@ extern "C" int cw_multi_norm_partials(int n_tensors, const void* const* grads, c
 #define CW_LAUNCH_NORM(T, KIND) hipLaunchKernelGGL((multi_norm_kernel<T, KIND>), dim3(blocks), dim3(kClipThreads), 0, s, b, norm_type, ws, offset)
         if (io_dtype == CW_BF16) {
             if (kind == 0) CW_LAUNCH_NORM(bf16_t, 0); else if (kind == 2) CW_LAUNCH_NORM(bf16_t, 2); else CW_LAUNCH_NORM(bf16_t, 1);
+        } else if (io_dtype == CW_F16) {
+            if (kind == 0) CW_LAUNCH_NORM(f16_t, 0); else if (kind == 2) CW_LAUNCH_NORM(f16_t, 2); else CW_LAUNCH_NORM(f16_t, 1);
         } else {
             if (kind == 0) CW_LAUNCH_NORM(float, 0); else if (kind == 2) CW_LAUNCH_NORM(float, 2); else CW_LAUNCH_NORM(float, 1);
         }
@@ -259,7 +262,8 @@ extern "C" int cw_clip_coef(int n_sets, const float* sets, float tp_scale, float
 extern "C" int cw_multi_scale(int n_tensors, void* const* grads, const int64_t* numels, const float* coef,
                               int io_dtype, void* stream) {
     if (n_tensors < 0) return fail(CW_ERR_INVALID, "cw_multi_scale: negative tensor count");
-    if (io_dtype != CW_BF16 && io_dtype != CW_F32) return fail(CW_ERR_INVALID, "cw_multi_scale: bad io_dtype %d", io_dtype);
+    if (io_dtype != CW_BF16 && io_dtype != CW_F32 && io_dtype != CW_F16)
+        return fail(CW_ERR_INVALID, "cw_multi_scale: bad io_dtype %d", io_dtype);
     if (coef == nullptr) return fail(CW_ERR_INVALID, "cw_multi_scale: coef is NULL");
     if (n_tensors > 0 && (grads == nullptr || numels == nullptr)) return fail(CW_ERR_INVALID, "cw_multi_scale: null tables");
     for (int i = 0; i < n_tensors; ++i)
@@ -273,6 +277,7 @@ extern "C" int cw_multi_scale(int n_tensors, void* const* grads, const int64_t* 
         const int blocks = b.first_block[b.n];
         if (blocks == 0) continue;
         if (io_dtype == CW_BF16) hipLaunchKernelGGL(multi_scale_kernel<bf16_t>, dim3(blocks), dim3(kClipThreads), 0, s, b, coef);
+        else if (io_dtype == CW_F16) hipLaunchKernelGGL(multi_scale_kernel<f16_t>, dim3(blocks), dim3(kClipThreads), 0, s, b, coef);
         else hipLaunchKernelGGL(multi_scale_kernel<float>, dim3(blocks), dim3(kClipThreads), 0, s, b, coef);
         const int rc = check_launch("multi_scale_kernel");
         if (rc != CW_OK) return rc;

@@ -317,4 +317,13 @@ __device__ __forceinline__ float act_grad(int act, float x) {
     }
 }
 
+// Calls f with a null pointer to the element type io_dtype names (CW_BF16, CW_F16, otherwise float):
+// `with_elem_type(dt, [&](auto* tag) { using T = std::remove_pointer_t<decltype(tag)>; ... })`.
+template <typename F>
+int with_elem_type(int io_dtype, F&& f) {
+    if (io_dtype == CW_BF16) return f((bf16_t*)nullptr);
+    if (io_dtype == CW_F16) return f((f16_t*)nullptr);
+    return f((float*)nullptr);
+}
+
 }  // namespace cw

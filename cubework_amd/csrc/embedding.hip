@@ -9,6 +9,8 @@
 //           slices), whose wavefronts stride the run's tokens and are combined in a fixed order.
 //           No atomics.
 // Both are HBM-streaming kernels: 16-byte accesses, one wavefront per row.
+#include <type_traits>
+
 #include "cw_common.h"
 
 namespace cw {
@@ -273,26 +275,30 @@ using namespace cw;
 extern "C" int cw_embed_fwd(int64_t T, int64_t E, const int64_t* ids, int64_t vocab_start, int64_t V_loc,
                             const void* weight, int64_t ldw, void* out, int64_t ldo, int io_dtype, void* stream) {
     if (T < 0 || E <= 0 || V_loc <= 0) return fail(CW_ERR_INVALID, "cw_embed_fwd: bad shape T=%lld E=%lld V_loc=%lld", (long long)T, (long long)E, (long long)V_loc);
-    if (io_dtype != CW_BF16 && io_dtype != CW_F32) return fail(CW_ERR_INVALID, "cw_embed_fwd: bad io_dtype %d", io_dtype);
+    if (io_dtype != CW_BF16 && io_dtype != CW_F32 && io_dtype != CW_F16)
+        return fail(CW_ERR_INVALID, "cw_embed_fwd: bad io_dtype %d", io_dtype);
     if (T == 0) return CW_OK;
     if (ids == nullptr || weight == nullptr || out == nullptr || ldw < E || ldo < E)
         return fail(CW_ERR_INVALID, "cw_embed_fwd: null pointer or leading dimension < E");
     hipStream_t s = (hipStream_t)stream;
-    return io_dtype == CW_BF16 ? fwd_impl<bf16_t>(T, E, ids, vocab_start, V_loc, weight, ldw, out, ldo, s)
-                               : fwd_impl<float>(T, E, ids, vocab_start, V_loc, weight, ldw, out, ldo, s);
+    return with_elem_type(io_dtype, [&](auto* tag) {
+        return fwd_impl<std::remove_pointer_t<decltype(tag)>>(T, E, ids, vocab_start, V_loc, weight, ldw, out, ldo, s);
+    });
 }
 
 extern "C" int cw_embed_bwd(int64_t T, int64_t E, const int64_t* sorted_ids, const int64_t* order, int64_t vocab_start,
                             int64_t V_loc, int64_t skip_row, const void* d_out, int64_t ldo, void* d_weight,
                             int64_t ldw, int io_dtype, void* stream) {
     if (T < 0 || E <= 0 || V_loc <= 0) return fail(CW_ERR_INVALID, "cw_embed_bwd: bad shape T=%lld E=%lld V_loc=%lld", (long long)T, (long long)E, (long long)V_loc);
-    if (io_dtype != CW_BF16 && io_dtype != CW_F32) return fail(CW_ERR_INVALID, "cw_embed_bwd: bad io_dtype %d", io_dtype);
+    if (io_dtype != CW_BF16 && io_dtype != CW_F32 && io_dtype != CW_F16)
+        return fail(CW_ERR_INVALID, "cw_embed_bwd: bad io_dtype %d", io_dtype);
     if (T > INT32_MAX) return fail(CW_ERR_INVALID, "cw_embed_bwd: too many tokens");
     if (d_weight == nullptr || ldw < E) return fail(CW_ERR_INVALID, "cw_embed_bwd: d_weight is NULL or ldw < E");
     if (T > 0 && (sorted_ids == nullptr || order == nullptr || d_out == nullptr || ldo < E))
         return fail(CW_ERR_INVALID, "cw_embed_bwd: null pointer or leading dimension < E");
     hipStream_t s = (hipStream_t)stream;
-    return io_dtype == CW_BF16
-               ? bwd_impl<bf16_t>(T, E, sorted_ids, order, vocab_start, V_loc, skip_row, d_out, ldo, d_weight, ldw, s)
-               : bwd_impl<float>(T, E, sorted_ids, order, vocab_start, V_loc, skip_row, d_out, ldo, d_weight, ldw, s);
+    return with_elem_type(io_dtype, [&](auto* tag) {
+        return bwd_impl<std::remove_pointer_t<decltype(tag)>>(T, E, sorted_ids, order, vocab_start, V_loc, skip_row, d_out,
+                                                              ldo, d_weight, ldw, s);
+    });
 }

@@ -1178,7 +1178,8 @@ int bwd_dx_impl(int64_t R, int64_t C, const void* dY, int64_t ld_dy, const void*
 
 int check_rc(const char* fn, int64_t R, int64_t C, int io_dtype) {
     if (R < 0 || C <= 0) return fail(CW_ERR_INVALID, "%s: bad shape R=%lld C=%lld", fn, (long long)R, (long long)C);
-    if (io_dtype != CW_BF16 && io_dtype != CW_F32) return fail(CW_ERR_INVALID, "%s: bad io_dtype %d", fn, io_dtype);
+    if (io_dtype != CW_BF16 && io_dtype != CW_F32 && io_dtype != CW_F16)
+        return fail(CW_ERR_INVALID, "%s: bad io_dtype %d", fn, io_dtype);
     return CW_OK;
 }
 
@@ -1203,8 +1204,9 @@ extern "C" int cw_ln_partial_stats(int64_t R, int64_t C, const void* x, int64_t 
     if (R == 0) return CW_OK;
     if (x == nullptr || stats == nullptr || ld < C) return fail(CW_ERR_INVALID, "cw_ln_partial_stats: null pointer or ld < C");
     hipStream_t s = (hipStream_t)stream;
-    return io_dtype == CW_BF16 ? stats_impl<bf16_t>(R, C, x, ld, mode, mean, stats, s)
-                               : stats_impl<float>(R, C, x, ld, mode, mean, stats, s);
+    return with_elem_type(io_dtype, [&](auto* tag) {
+        return stats_impl<std::remove_pointer_t<decltype(tag)>>(R, C, x, ld, mode, mean, stats, s);
+    });
 }
 
 extern "C" int cw_ln_normalize(int64_t R, int64_t C, const void* x, int64_t ld, const float* stats, int mode,
@@ -1218,9 +1220,10 @@ extern "C" int cw_ln_normalize(int64_t R, int64_t C, const void* x, int64_t ld, 
     if (x == nullptr || y == nullptr || stats == nullptr || ld < C || ldy < C)
         return fail(CW_ERR_INVALID, "cw_ln_normalize: null pointer or leading dimension < C");
     hipStream_t s = (hipStream_t)stream;
-    return io_dtype == CW_BF16
-               ? normalize_impl<bf16_t, false>(R, C, x, ld, stats, mode, H, eps, gamma, beta, y, ldy, mean_rstd, s)
-               : normalize_impl<float, false>(R, C, x, ld, stats, mode, H, eps, gamma, beta, y, ldy, mean_rstd, s);
+    return with_elem_type(io_dtype, [&](auto* tag) {
+        return normalize_impl<std::remove_pointer_t<decltype(tag)>, false>(R, C, x, ld, stats, mode, H, eps, gamma, beta,
+                                                                           y, ldy, mean_rstd, s);
+    });
 }
 
 extern "C" int cw_ln_forward_fused(int64_t R, int64_t C, const void* x, int64_t ld, int mode, float eps,
@@ -1233,9 +1236,10 @@ extern "C" int cw_ln_forward_fused(int64_t R, int64_t C, const void* x, int64_t 
     if (x == nullptr || y == nullptr || ld < C || ldy < C)
         return fail(CW_ERR_INVALID, "cw_ln_forward_fused: null pointer or leading dimension < C");
     hipStream_t s = (hipStream_t)stream;
-    return io_dtype == CW_BF16
-               ? normalize_impl<bf16_t, true>(R, C, x, ld, nullptr, mode, C, eps, gamma, beta, y, ldy, mean_rstd, s)
-               : normalize_impl<float, true>(R, C, x, ld, nullptr, mode, C, eps, gamma, beta, y, ldy, mean_rstd, s);
+    return with_elem_type(io_dtype, [&](auto* tag) {
+        return normalize_impl<std::remove_pointer_t<decltype(tag)>, true>(R, C, x, ld, nullptr, mode, C, eps, gamma, beta,
+                                                                          y, ldy, mean_rstd, s);
+    });
 }
 
 extern "C" int cw_ln_bwd_partials(int64_t R, int64_t C, const void* dY, int64_t ld_dy, const void* x, int64_t ld_x,
@@ -1251,10 +1255,10 @@ extern "C" int cw_ln_bwd_partials(int64_t R, int64_t C, const void* dY, int64_t 
         return fail(CW_ERR_INVALID, "cw_ln_bwd_partials: null pointer or leading dimension < C");
     if (dgamma != nullptr && workspace == nullptr) return fail(CW_ERR_INVALID, "cw_ln_bwd_partials: workspace is NULL");
     hipStream_t s = (hipStream_t)stream;
-    return io_dtype == CW_BF16 ? bwd_partials_impl<bf16_t>(R, C, dY, ld_dy, x, ld_x, mean_rstd, gamma, row_sums, dgamma,
-                                                           dbeta, workspace, workspace_bytes, s)
-                               : bwd_partials_impl<float>(R, C, dY, ld_dy, x, ld_x, mean_rstd, gamma, row_sums, dgamma,
-                                                          dbeta, workspace, workspace_bytes, s);
+    return with_elem_type(io_dtype, [&](auto* tag) {
+        return bwd_partials_impl<std::remove_pointer_t<decltype(tag)>>(R, C, dY, ld_dy, x, ld_x, mean_rstd, gamma, row_sums,
+                                                                       dgamma, dbeta, workspace, workspace_bytes, s);
+    });
 }
 
 namespace cw {
@@ -1286,11 +1290,11 @@ extern "C" int cw_ln_backward_fused(int64_t R, int64_t C, const void* dY, int64_
         return fail(CW_ERR_INVALID, "cw_ln_backward_fused: null pointer or leading dimension < C");
     if (dgamma != nullptr && workspace == nullptr) return fail(CW_ERR_INVALID, "cw_ln_backward_fused: workspace is NULL");
     hipStream_t s = (hipStream_t)stream;
-    return io_dtype == CW_BF16
-               ? backward_fused_impl<bf16_t>(R, C, dY, ld_dy, x, ld_x, mean_rstd, gamma, row_sums, dx, ld_dx, dgamma, dbeta,
-                                             workspace, workspace_bytes, s)
-               : backward_fused_impl<float>(R, C, dY, ld_dy, x, ld_x, mean_rstd, gamma, row_sums, dx, ld_dx, dgamma, dbeta,
-                                            workspace, workspace_bytes, s);
+    return with_elem_type(io_dtype, [&](auto* tag) {
+        return backward_fused_impl<std::remove_pointer_t<decltype(tag)>>(R, C, dY, ld_dy, x, ld_x, mean_rstd, gamma, row_sums,
+                                                                         dx, ld_dx, dgamma, dbeta, workspace,
+                                                                         workspace_bytes, s);
+    });
 }
 
 extern "C" int cw_ln_bwd_dx(int64_t R, int64_t C, const void* dY, int64_t ld_dy, const void* x, int64_t ld_x,
@@ -1304,7 +1308,8 @@ extern "C" int cw_ln_bwd_dx(int64_t R, int64_t C, const void* dY, int64_t ld_dy,
         ld_x < C || ld_dx < C)
         return fail(CW_ERR_INVALID, "cw_ln_bwd_dx: null pointer or leading dimension < C");
     hipStream_t s = (hipStream_t)stream;
-    return io_dtype == CW_BF16
-               ? bwd_dx_impl<bf16_t>(R, C, dY, ld_dy, x, ld_x, mean_rstd, gamma, row_sums, H, dx, ld_dx, s)
-               : bwd_dx_impl<float>(R, C, dY, ld_dy, x, ld_x, mean_rstd, gamma, row_sums, H, dx, ld_dx, s);
+    return with_elem_type(io_dtype, [&](auto* tag) {
+        return bwd_dx_impl<std::remove_pointer_t<decltype(tag)>>(R, C, dY, ld_dy, x, ld_x, mean_rstd, gamma, row_sums, H, dx,
+                                                                 ld_dx, s);
+    });
 }

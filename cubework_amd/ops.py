@@ -30,15 +30,14 @@ def epilogue_code(has_bias: bool, activation: Optional[str]) -> int:
             CW_ACT_RELU: CW_EPI_BIAS_RELU}[act]
 
 
-def _dtype_code(t: torch.Tensor, half_ok: bool = False) -> int:
+def _dtype_code(t: torch.Tensor) -> int:
     if t.dtype == torch.bfloat16:
         return CW_BF16
     if t.dtype == torch.float32:
         return CW_F32
-    if t.dtype == torch.float16 and half_ok:
+    if t.dtype == torch.float16:
         return CW_F16
-    raise TypeError("this cubework_amd kernel takes %s tensors, got %s"
-                    % ("bfloat16, float16 or float32" if half_ok else "bfloat16 or float32", t.dtype))
+    raise TypeError("the cubework_amd kernels take bfloat16, float16 or float32 tensors, got %s" % t.dtype)
 
 
 def _require_device(*tensors):
@@ -97,7 +96,7 @@ def gemm_ksteps(layout: str, A_steps: Sequence[torch.Tensor], B_steps: Sequence[
     B_steps = [_rows(b) for b in B_steps]
     _require_device(*A_steps, *B_steps, bias, *addends)
     a0, b0 = A_steps[0], B_steps[0]
-    dt = _dtype_code(a0, half_ok=True)
+    dt = _dtype_code(a0)
     if layout == "NN":
         M, K, N, Kb = a0.shape[0], a0.shape[1], b0.shape[1], b0.shape[0]
     elif layout == "NT":
@@ -159,7 +158,7 @@ def bias_act(x: torch.Tensor, bias: Optional[torch.Tensor], activation: Optional
     out = torch.empty((M, N), dtype=x2.dtype, device=x2.device)
     tadd = _ptr_table([x2])
     rc = lib.cw_gemm_ksteps(CW_NN, M, N, 0, 0, None, 0, None, 0, _p(bias), epilogue_code(bias is not None, activation),
-                            _p(out), _ld(out), None, 0, tadd, 1, _ld(x2), _dtype_code(x2, half_ok=True), _stream())
+                            _p(out), _ld(out), None, 0, tadd, 1, _ld(x2), _dtype_code(x2), _stream())
     _lib.check(rc, "cw_gemm_ksteps (bias/activation only)")
     return out.reshape(shape)
 
@@ -177,7 +176,7 @@ def colsum(dy: torch.Tensor) -> torch.Tensor:
     M, N = dy.shape
     out = torch.empty(N, dtype=torch.float32, device=dy.device)
     ws = _workspace(M, N, dy.device)
-    rc = lib.cw_colsum(M, N, _p(dy), _ld(dy), _p(out), _p(ws), ws.numel(), _dtype_code(dy, half_ok=True), _stream())
+    rc = lib.cw_colsum(M, N, _p(dy), _ld(dy), _p(out), _p(ws), ws.numel(), _dtype_code(dy), _stream())
     _lib.check(rc, "cw_colsum")
     return out
 
@@ -196,7 +195,7 @@ def act_bwd_colsum(activation: Optional[str], dy: torch.Tensor, preact: torch.Te
     ws = _workspace(M, N, dy.device) if want_dbias else None
     rc = lib.cw_act_bwd_colsum(ACTIVATIONS[activation], M, N, _p(dy), _ld(dy), _p(preact), _ld(preact), _p(dpre),
                                _ld(dpre), _p(dbias), _p(ws), ws.numel() if ws is not None else 0,
-                               _dtype_code(dy, half_ok=True), _stream())
+                               _dtype_code(dy), _stream())
     _lib.check(rc, "cw_act_bwd_colsum")
     return dpre, dbias
 
@@ -344,7 +343,7 @@ def vpce_fwd_local(logits: torch.Tensor, targets: torch.Tensor, vocab_start: int
     pr = torch.empty(T, dtype=torch.float32, device=dev)
     mk = torch.empty(T, dtype=torch.uint8, device=dev)
     rc = lib.cw_vpce_fwd_local(T, V, _p(logits), _ld(logits), _p(targets), vocab_start, _p(mx), _p(se), _p(pr), _p(mk),
-                               _dtype_code(logits, half_ok=True), _stream())
+                               _dtype_code(logits), _stream())
     _lib.check(rc, "cw_vpce_fwd_local")
     return mx, se, pr, mk
 
@@ -380,7 +379,7 @@ def vpce_bwd(logits: torch.Tensor, targets: torch.Tensor, vocab_start: int, gmax
     if dloss_rows is not None:
         dloss_rows = dloss_rows.reshape(-1).to(torch.float32).contiguous()
     rc = lib.cw_vpce_bwd(T, V, _p(logits), _ld(logits), _p(targets), vocab_start, _p(gmax), _p(gsum), _p(dloss_rows),
-                         dloss_scale, _p(grad), _ld(grad), _dtype_code(logits, half_ok=True), _dtype_code(grad, half_ok=True), _stream())
+                         dloss_scale, _p(grad), _ld(grad), _dtype_code(logits), _dtype_code(grad), _stream())
     _lib.check(rc, "cw_vpce_bwd")
     return grad.reshape(shape)
 
@@ -411,7 +410,7 @@ def attn_fwd(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, scale: Optional[
     out = torch.empty((B, S, H, D), dtype=q.dtype, device=q.device)
     lse = torch.empty((B, H, S), dtype=torch.float32, device=q.device) if want_lse else None
     rc = lib.cw_attn_fwd(B, H, S, D, _p(q), _p(k), _p(v), strides[0], strides[1], strides[2], scale, 1 if causal else 0,
-                         _p(out), out.stride(0), out.stride(1), out.stride(2), _p(lse), _dtype_code(q, half_ok=True), _stream())
+                         _p(out), out.stride(0), out.stride(1), out.stride(2), _p(lse), _dtype_code(q), _stream())
     _lib.check(rc, "cw_attn_fwd")
     out = out.view(B, S, H * D)
     return (out, lse) if want_lse else out
@@ -441,7 +440,7 @@ def attn_bwd(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, out: torch.Tenso
     ws = torch.empty(max(ws_bytes, 16), dtype=torch.uint8, device=q.device)
     rc = lib.cw_attn_bwd(B, H, S, D, _p(q), _p(k), _p(v), strides[0], strides[1], strides[2], _p(out4), _p(dout4),
                          ostr[0], ostr[1], ostr[2], _p(lse), scale, 1 if causal else 0, _p(dq), _p(dk), _p(dv),
-                         gstrides[0], gstrides[1], gstrides[2], _p(ws), ws.numel(), _dtype_code(q, half_ok=True), _stream())
+                         gstrides[0], gstrides[1], gstrides[2], _p(ws), ws.numel(), _dtype_code(q), _stream())
     _lib.check(rc, "cw_attn_bwd")
 
 

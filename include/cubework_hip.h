@@ -16,8 +16,8 @@
  *     enqueued on `stream` (a hipStream_t passed as void*) and the call returns;
  *   - re-entrant and callable from any thread (the autograd engine calls the
  *     backward entry points from its own device thread);
- *   - io_dtype selects the storage type of activations/weights (CW_BF16 or
- *     CW_F32; CW_F16 where an entry point says so); statistics, losses and all
+ *   - io_dtype selects the storage type of activations/weights (CW_BF16,
+ *     CW_F32 or CW_F16); statistics, losses and all
  *     accumulation are fp32.
  *
  * Citations name the reference code (kurisusnowdeng/Cubework) each entry
@@ -41,13 +41,12 @@ typedef enum {
     CW_ERR_DEVICE = -5       /* current device is not gfx950             */
 } cw_status;
 
-/* CW_F16 (IEEE half, the type the reference's GEMM-type Functions cast to under autocast:
- * custom_fwd(cast_inputs=torch.float16), cubework/module/parallel_2d/_operation.py:17,96,176,255,363) is
- * taken by the GEMM, column-sum, attention and cross-entropy entry points (cw_gemm_ksteps,
- * cw_gemm_ksteps_ws, cw_colsum, cw_act_bwd_colsum, cw_attn_fwd, cw_attn_bwd, cw_vpce_fwd_local,
- * cw_vpce_bwd): the reference runs LayerNorm in fp32 under autocast, on the fp32 residual stream, and so
- * does its entry point here; its loss casts the logits to fp32 first, which reading them as 16-bit values
- * and computing in fp32 reproduces without the copy. */
+/* CW_F16 (IEEE half) is the type the reference's GEMM-type Functions cast to under autocast
+ * (custom_fwd(cast_inputs=torch.float16), cubework/module/parallel_2d/_operation.py:17,96,176,255,363) and
+ * the type of every tensor of a model converted with .half(), where nothing casts. Every entry point
+ * takes it. Under autocast the reference runs LayerNorm in fp32 on the fp32 residual stream (CW_F32
+ * here) and casts the logits of its loss to fp32 first, which reading them as 16-bit values and computing
+ * in fp32 reproduces without the copy. */
 typedef enum { CW_BF16 = 0, CW_F32 = 1, CW_F16 = 2 } cw_dtype;
 
 /* Operand orientation of the block GEMM, per k-step i:

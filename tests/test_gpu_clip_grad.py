@@ -25,7 +25,7 @@ def _params(shapes, dtype, seed, tp_every=2):
 SHAPES = [(1000, 33), (7,), (70000,), (256, 256), (1,), (65536,), (65537,), (3, 5, 11)] + [(129, 17)] * 60
 
 
-@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32, torch.float16])
 @pytest.mark.parametrize("norm_type", [2.0, float("inf"), 1.0, 3.0])
 @pytest.mark.parametrize("max_norm", [0.5, 1e9])
 def test_clip_grad_norm_matches_torch(dtype, norm_type, max_norm):
@@ -42,7 +42,12 @@ def test_clip_grad_norm_matches_torch(dtype, norm_type, max_norm):
     torch.cuda.synchronize()
     assert abs(got.item() - want.item()) <= 1e-4 * abs(want.item()), (got.item(), want.item())
     for r, p in zip(ref, ours):
-        assert_parity(p.grad, r.grad, dtype, "clipped gradient")
+        if dtype == torch.float16:
+            # a small clip coefficient takes float16 gradients into the subnormal range (steps of 2^-24), where
+            # a relative bound means nothing: one step of slack on top of the relative tolerance
+            torch.testing.assert_close(p.grad.float().cpu(), r.grad.to(dtype).float(), rtol=1e-3, atol=2.0 ** -24)
+        else:
+            assert_parity(p.grad, r.grad, dtype, "clipped gradient")
 
 
 def test_tensor_parallel_weighting_and_mixed_dtypes():

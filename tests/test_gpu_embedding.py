@@ -17,7 +17,7 @@ def _ids(shape, vocab, seed, hot=None):
     return ids
 
 
-@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32, torch.float16])
 @pytest.mark.parametrize("case", [(4, 37, 1000, 256, 250, 64), (2, 128, 50272, 12568, 12568, 2048),
                                   (1, 5, 64, 64, 0, 8), (3, 11, 300, 100, 100, 52), (1, 1, 16, 4, 12, 520)])
 def test_embedding_forward_backward_parity(case, dtype):
@@ -51,7 +51,7 @@ def test_embedding_forward_backward_parity(case, dtype):
         assert (got_dw.cpu()[untouched] == 0).all(), "rows without tokens are exactly zero"
 
 
-@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32, torch.float16])
 @pytest.mark.parametrize("e", [520, 2048, 4104])
 def test_embedding_backward_every_run_length(e, dtype):
     """Id j occurs j + 1 times (runs of 1 .. 45 tokens in the sorted order, shuffled over the batch): the
@@ -71,7 +71,7 @@ def test_embedding_backward_every_run_length(e, dtype):
     assert (got.cpu()[0:3] == 0).all() and (got.cpu()[4::2][:44] == 0).all(), "rows without tokens are exactly zero"
 
 
-@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32, torch.float16])
 def test_embedding_backward_one_id_thousands_of_times(dtype):
     """Token frequencies of text: one id 3000 times among 5000 tokens (a run that every wavefront of the
     sharing blocks walks for many rounds), the rest spread over the table; compared in float64."""

@@ -9,7 +9,7 @@ import pytest
 import torch
 
 from tests.test_gpu_gemm import LAYOUTS, _run
-from tests.util import assert_parity, randn
+from tests.util import assert_parity, rand_uniform, randn
 
 pytestmark = pytest.mark.gpu
 DEV = "cuda:0"
@@ -99,17 +99,32 @@ def test_f16_colsum_and_act_bwd(shape):
         assert_parity(dbias, want_dbias, torch.float32, "dbias %s" % act, scale=200)
 
 
-def test_f16_refused_where_the_reference_runs_fp32():
-    """LayerNorm runs in fp32 under autocast in the reference (cast_inputs=torch.float32) and receives the
-    fp32 residual stream; its wrappers and the embedding's take bfloat16 and float32 only and say so instead
-    of computing something else."""
-    from cubework_amd import ops
+def test_half_model_layernorm():
+    """model.half() without autocast: nothing casts, so the reference's LayerNorm Functions receive float16
+    (custom_fwd casts only inside an autocast region). The kernels read float16, compute in fp32 and write
+    float16; against F.layer_norm in fp32 on the same values."""
+    from cubework_amd import module as cube_nn
+    from cubework_amd.distributed import initialize
 
-    x = randn((64, 256), F16, 1).to(DEV)
-    with pytest.raises(TypeError):
-        ops.ln_partial_stats(x)
-    with pytest.raises(TypeError):
-        ops.embedding_fwd(torch.zeros(4, dtype=torch.int64, device=DEV), x, 0)
+    initialize("2d", 1)
+    torch.manual_seed(0)
+    ln = cube_nn.LayerNorm(768, dtype=F16).to(DEV)
+    with torch.no_grad():
+        ln.weight.copy_(rand_uniform((768,), F16, 2, 0.9, 1.1))
+        ln.bias.copy_(randn((768,), F16, 3, std=0.02))
+    x = randn((4, 33, 768), F16, 4).to(DEV).requires_grad_(True)
+    dy = randn((4, 33, 768), F16, 5).to(DEV)
+    y = ln(x)
+    assert y.dtype == F16
+    y.backward(dy)
+    xr = x.detach().float().requires_grad_(True)
+    wr = ln.weight.detach().float().requires_grad_(True)
+    br = ln.bias.detach().float().requires_grad_(True)
+    torch.nn.functional.layer_norm(xr, (768,), wr, br, 1e-5).backward(dy.float())
+    assert_parity(y, torch.nn.functional.layer_norm(xr, (768,), wr, br, 1e-5).detach().to(F16), F16, "y")
+    assert_parity(x.grad, xr.grad.to(F16), F16, "dx")
+    assert_parity(ln.weight.grad, wr.grad.to(F16), F16, "dgamma", scale=4)
+    assert_parity(ln.bias.grad, br.grad.to(F16), F16, "dbeta", scale=4)
 
 
 @pytest.mark.parametrize("amp_dtype", [torch.float16, torch.bfloat16])

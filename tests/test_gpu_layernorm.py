@@ -58,7 +58,7 @@ def test_ln2d_forward_backward_with_peer_partials(shape, dtype):
     assert_parity(dx_got, dx_want, dtype, "dx", scale=4 if dtype == torch.float32 else 1)
 
 
-@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32, torch.float16])
 @pytest.mark.parametrize("mode", ["one_pass", "two_pass"])
 @pytest.mark.parametrize("shape", [(64, 1024), (17, 200), (4, 2048), (33, 4096), (70, 8192), (9, 12288), (2100, 2560),
                                    (1100, 5120), (3, 16384), (2, 20480)])
@@ -87,7 +87,7 @@ def test_ln_fused_matches_nn_layernorm(shape, mode, dtype):
     assert_parity(db, br.grad, torch.float32, "dbeta vs autograd", scale=50)
 
 
-@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32, torch.float16])
 @pytest.mark.parametrize("affine", [True, False])
 @pytest.mark.parametrize("shape", [(64, 1024), (17, 200), (4, 2048), (1000, 512), (33, 4096), (5, 1001), (3, 5000), (300, 64),
                                    (70, 8192), (9, 12288), (600, 3072), (2100, 2560), (3, 16384), (2, 20480),
@@ -213,7 +213,7 @@ def test_ln_empty_and_errors():
     assert rc < 0 and b"hidden size" in lib.cw_last_error()
 
 
-@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32, torch.float16])
 @pytest.mark.parametrize("case", [(50, 1024, 0, 3072), (600, 2560, 512, 4096), (40, 4096, 4096, 12288),
                                   (9, 9216, 8, 9232), (33, 3072, 3, 3080)])
 def test_ln_strided_rows(case, dtype):
