@@ -648,3 +648,28 @@ def test_opt_block_shapes_small(activation):
         assert prm.grad is not None and torch.isfinite(prm.grad.float()).all(), name
         if activation != "relu":
             assert_parity(prm.grad, params[name].grad, torch.bfloat16, name + ".grad", scale=5)
+
+
+def test_opt_block_half_model():
+    """The same layer as a float16 model (parameters and activations in float16, no autocast: nothing
+    casts, every operator of the layer receives float16), against the block in fp32 torch."""
+    from cubework_amd.distributed import initialize
+    from cubework_amd.opt_block import OPTBlock
+    from oracle import opt_block_reference
+
+    initialize("2d", 1)
+    torch.manual_seed(0)
+    blk = OPTBlock(hidden=256, heads=4, ffn=1024, dtype=torch.float16, activation="gelu_tanh").to(DEV)
+    x = _leaf(randn((2, 64, 256), torch.float16, 1).to(DEV))
+    dy = randn((2, 64, 256), torch.float16, 2).to(DEV)
+    y = blk(x)
+    assert y.dtype == torch.float16
+    y.backward(dy)
+    xr = _leaf(x.detach().float().cpu())
+    ref, params = opt_block_reference(blk, xr)
+    ref.backward(dy.float().cpu())
+    assert_parity(y, ref.detach(), torch.float16, "block forward", scale=4)
+    assert_parity(x.grad, xr.grad, torch.float16, "block dX", scale=8)
+    for name, prm in blk.named_parameters():
+        assert prm.grad is not None and prm.grad.dtype == torch.float16, name
+        assert_parity(prm.grad, params[name].grad, torch.float16, name + ".grad", scale=8)
