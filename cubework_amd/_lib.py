@@ -50,6 +50,8 @@ SIGNATURES = {
                            _f32, _int, _ptr, _ptr, _ptr, _i64, _i64, _i64, _ptr, _i64, _int, _ptr]),
     "cw_colsum_workspace_bytes": (_i64, [_i64, _i64]),
     "cw_colsum": (_int, [_i64, _i64, _ptr, _i64, _ptr, _ptr, _i64, _int, _ptr]),
+    "cw_colsum_static_max_bytes": (_i64, []),
+    "cw_colsum_static": (_int, [_i64, _i64, _ptr, _i64, _ptr, _int, _ptr]),
     "cw_act_bwd_colsum": (_int, [_int, _i64, _i64, _ptr, _i64, _ptr, _i64, _ptr, _i64, _ptr, _ptr, _i64, _int, _ptr]),
     "cw_ln_partial_stats": (_int, [_i64, _i64, _ptr, _i64, _int, _ptr, _ptr, _int, _ptr]),
     "cw_ln_normalize": (_int, [_i64, _i64, _ptr, _i64, _ptr, _int, _i64, _f32, _ptr, _ptr, _ptr, _i64, _ptr, _int,

@@ -3,6 +3,8 @@
 // tile of 64 vectors of columns, lanes keep their columns' sums in registers,
 // wavefronts are combined in a fixed-order LDS tree, slabs by a finalize
 // kernel (no atomics: bit-reproducible).
+#include <atomic>
+#include <mutex>
 #include <type_traits>
 
 #include "cw_common.h"
@@ -135,6 +137,23 @@ __global__ __launch_bounds__(kFinGroups * 64) void finalize_cols_kernel(const fl
     }
 }
 
+// Row slabs of an [M,N] operand with V elements per 16 bytes: one partial row of N sums per slab.
+void colsum_plan(int64_t M, int64_t N, int V, bool vec, int64_t& slabs, int64_t& rows_per_slab) {
+    if (!vec) {
+        rows_per_slab = kGenericSlabRows;
+        slabs = (M + rows_per_slab - 1) / rows_per_slab;
+        return;
+    }
+    const int64_t coltiles = (N + 64 * V - 1) / (64 * V);
+    slabs = kColBlocks / coltiles;
+    const int64_t max_slabs = (M + kColWaves * kColUnroll - 1) / (kColWaves * kColUnroll);
+    if (slabs > max_slabs) slabs = max_slabs;
+    if (slabs > 512) slabs = 512;  // the bound cw_colsum_workspace_bytes promises
+    if (slabs < 1) slabs = 1;
+    rows_per_slab = (M + slabs - 1) / slabs;
+    slabs = (M + rows_per_slab - 1) / rows_per_slab;
+}
+
 template <typename T, int MODE>
 int colsum_impl(int64_t M, int64_t N, const void* dY, int64_t ld_dy, const void* pre, int64_t ld_pre, void* dPre,
                 int64_t ld_dpre, int act, float* out, void* workspace, int64_t workspace_bytes, hipStream_t s) {
@@ -145,13 +164,7 @@ int colsum_impl(int64_t M, int64_t N, const void* dY, int64_t ld_dy, const void*
     int64_t slabs, rows_per_slab;
     if (vec) {
         const int64_t coltiles = (N + 64 * V - 1) / (64 * V);
-        slabs = kColBlocks / coltiles;
-        const int64_t max_slabs = (M + kColWaves * kColUnroll - 1) / (kColWaves * kColUnroll);
-        if (slabs > max_slabs) slabs = max_slabs;
-        if (slabs > 512) slabs = 512;  // the bound cw_colsum_workspace_bytes promises
-        if (slabs < 1) slabs = 1;
-        rows_per_slab = (M + slabs - 1) / slabs;
-        slabs = (M + rows_per_slab - 1) / rows_per_slab;
+        colsum_plan(M, N, V, true, slabs, rows_per_slab);
         if (want_sum && workspace_bytes < slabs * N * (int64_t)sizeof(float))
             return fail(CW_ERR_INVALID, "column sum: workspace too small (%lld bytes)", (long long)workspace_bytes);
         const size_t lds = tree_reduce_lds_bytes(V, kColWaves);
@@ -166,8 +179,7 @@ int colsum_impl(int64_t M, int64_t N, const void* dY, int64_t ld_dy, const void*
         else if (act == CW_ACT_GELU_ERF) launch(std::integral_constant<int, CW_ACT_GELU_ERF>{});
         else launch(std::integral_constant<int, CW_ACT_RELU>{});
     } else {
-        rows_per_slab = kGenericSlabRows;
-        slabs = (M + rows_per_slab - 1) / rows_per_slab;
+        colsum_plan(M, N, V, false, slabs, rows_per_slab);
         if (want_sum && workspace_bytes < slabs * N * (int64_t)sizeof(float))
             return fail(CW_ERR_INVALID, "column sum: workspace too small (%lld bytes)", (long long)workspace_bytes);
         hipLaunchKernelGGL((colsum_generic_kernel<T, MODE>), dim3((unsigned)((N + 255) / 256), (unsigned)slabs),
@@ -186,6 +198,52 @@ int finalize_col_partials(const float* ws, int64_t nparts, int64_t part_stride, 
     hipLaunchKernelGGL(finalize_cols_kernel, dim3((unsigned)((C + 63) / 64), (unsigned)nsets), dim3(kFinGroups * 64), 0, s, ws,
                        nparts, part_stride, C, out0, out1);
     return check_launch("finalize_cols_kernel");
+}
+
+// ---- library-owned scratch for the entry point that allocates nothing ------------------------------
+// One zero-initialised array per GPU, part of the code object: it exists from the moment the library is
+// loaded on a device until the process ends. `scratch` names it in device code only; host code uses the
+// device address hipGetSymbolAddress reports, looked up once per device with that device current.
+constexpr int64_t kStaticScratchBytes = 4ll << 20;
+static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
+
+namespace {
+constexpr int kMaxDevices = 64;
+std::atomic<void*> g_scratch_ptr[kMaxDevices];
+std::mutex g_scratch_mutex;
+}  // namespace
+
+// Device address of this GPU's copy of `scratch` (nullptr + error text on failure).
+static void* static_scratch_ptr() {
+    int dev = -1;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) {
+        (void)hipGetLastError();
+        fail(CW_ERR_DEVICE, "cw_colsum_static: no current HIP device (or device index above %d)", kMaxDevices - 1);
+        return nullptr;
+    }
+    void* p = g_scratch_ptr[dev].load(std::memory_order_acquire);
+    if (p != nullptr) return p;
+    std::lock_guard<std::mutex> lock(g_scratch_mutex);
+    p = g_scratch_ptr[dev].load(std::memory_order_acquire);
+    if (p != nullptr) return p;
+    const hipError_t e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+    if (e != hipSuccess || p == nullptr) {
+        (void)hipGetLastError();
+        fail(CW_ERR_DEVICE, "cw_colsum_static: hipGetSymbolAddress(scratch) failed on device %d: %s", dev,
+             hipGetErrorString(e));
+        return nullptr;
+    }
+    g_scratch_ptr[dev].store(p, std::memory_order_release);
+    return p;
+}
+
+// Bytes of partial sums cw_colsum's kernels write for an [M,N] operand.
+template <typename T>
+static int64_t colsum_partial_bytes(int64_t M, int64_t N, const void* dY, int64_t ld) {
+    constexpr int V = elem<T>::kVec;
+    int64_t slabs, rows_per_slab;
+    colsum_plan(M, N, V, aligned16(dY) && (ld % V) == 0 && (N % V) == 0, slabs, rows_per_slab);
+    return slabs * N * (int64_t)sizeof(float);
 }
 
 int64_t colsum_workspace_bytes(int64_t M, int64_t N) {
@@ -220,6 +278,33 @@ extern "C" int cw_colsum(int64_t M, int64_t N, const void* dY, int64_t ld, float
     return io_dtype == CW_BF16
                ? colsum_impl<bf16_t, 0>(M, N, dY, ld, nullptr, 0, nullptr, 0, 0, out, workspace, workspace_bytes, s)
                : colsum_impl<float, 0>(M, N, dY, ld, nullptr, 0, nullptr, 0, 0, out, workspace, workspace_bytes, s);
+}
+
+extern "C" int64_t cw_colsum_static_max_bytes(void) { return kStaticScratchBytes; }
+
+extern "C" int cw_colsum_static(int64_t M, int64_t N, const void* dY, int64_t ld, float* out, int io_dtype,
+                                void* stream) {
+    if (M < 0 || N <= 0)
+        return fail(CW_ERR_INVALID, "cw_colsum_static: bad shape M=%lld N=%lld", (long long)M, (long long)N);
+    if (io_dtype != CW_BF16 && io_dtype != CW_F32 && io_dtype != CW_F16)
+        return fail(CW_ERR_INVALID, "cw_colsum_static: bad io_dtype %d", io_dtype);
+    if (out == nullptr) return fail(CW_ERR_INVALID, "cw_colsum_static: out is NULL");
+    hipStream_t s = (hipStream_t)stream;
+    if (M == 0) return finalize_col_partials(nullptr, 0, N, 1, N, out, nullptr, s);  // zero fill
+    if (dY == nullptr || ld < N) return fail(CW_ERR_INVALID, "cw_colsum_static: null pointer or ld < N");
+    const int64_t need = with_elem_type(io_dtype, [&](auto* tag) -> int {
+        using T = std::remove_pointer_t<decltype(tag)>;
+        const int64_t b = colsum_partial_bytes<T>(M, N, dY, ld);
+        return b > kStaticScratchBytes ? -1 : 0;
+    });
+    if (need != 0)
+        return fail(CW_ERR_UNSUPPORTED,
+                    "cw_colsum_static: [%lld, %lld] needs more than the %lld bytes of the library's static scratch "
+                    "(16-byte aligned operands: N <= 1048576; others: ceil(M/64) * N <= 1048576); use cw_colsum",
+                    (long long)M, (long long)N, (long long)kStaticScratchBytes);
+    void* ws = static_scratch_ptr();  // the device address, never the array's name
+    if (ws == nullptr) return CW_ERR_DEVICE;
+    return cw_colsum(M, N, dY, ld, out, ws, kStaticScratchBytes, io_dtype, stream);
 }
 
 extern "C" int cw_act_bwd_colsum(int activation, int64_t M, int64_t N, const void* dY, int64_t ld_dy,

@@ -163,6 +163,21 @@ int cw_colsum(int64_t M, int64_t N, const void* dY, int64_t ld, float* out,
               void* workspace, int64_t workspace_bytes, int io_dtype, void* stream);
 
 /*
+ * cw_colsum for callers that cannot allocate device memory or hand over scratch (code under HIP graph
+ * capture, tight serving loops, harnesses that forbid hipMalloc). It has no counterpart in the reference,
+ * whose torch.sum allocates through torch's caching allocator. Same kernels and same bits as cw_colsum;
+ * the partial sums go through a 4 MiB array that is part of the library's code object (one copy per GPU,
+ * held until the process ends; cw_colsum_static_max_bytes returns its size). Shapes whose partial sums do
+ * not fit are refused with CW_ERR_UNSUPPORTED: with 16-byte aligned dY and ld, N % (16 / element size)
+ * == 0 the limit is N <= 1048576, otherwise ceil(M / 64) * N <= 1048576. Calls on one GPU share the array:
+ * calls that may overlap on the device (two streams, two threads) race; calls on one stream do not. The
+ * first call on a device looks the array's address up (hipGetSymbolAddress): make it outside a capture.
+ * No hipMalloc / hipFree / allocating library routine on any call.
+ */
+int64_t cw_colsum_static_max_bytes(void);
+int cw_colsum_static(int64_t M, int64_t N, const void* dY, int64_t ld, float* out, int io_dtype, void* stream);
+
+/*
  * dPre[M,N] = dY * act'(preact); optionally dbias[N] (fp32) = column sums of
  * dPre (dbias may be NULL, then workspace may be NULL). Backward of the fused
  * activation epilogue of cw_gemm_ksteps; the reference runs it as autograd of
