@@ -268,6 +268,7 @@ extern "C" int cw_attn_fwd(int64_t B, int64_t H, int64_t S, int64_t D, const voi
     a.causal = causal ? 1 : 0;
     a.n_qblocks = (int)((S + kQPerBlock - 1) / kQPerBlock);
     const dim3 grid((unsigned)(a.n_qblocks * B * H));
+    if (const int drc = require_gfx950("cw_attn_fwd"); drc != CW_OK) return drc;
     hipStream_t s = (hipStream_t)stream;
     if (io_dtype == CW_F16) {
         if (D == 64) hipLaunchKernelGGL((attn_fwd_kernel<1, f16_t>), grid, dim3(kThreads), 0, s, a);

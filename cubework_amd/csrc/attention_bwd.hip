@@ -433,16 +433,14 @@ int launch_bwd(const BwdArgs& a, int64_t B, int64_t H, int64_t S, int64_t D, int
     if (D == 64) {
         constexpr int lds_bytes = 2 * dkdv_stage_bytes<1>();
         auto kern = attn_dkdv_kernel<1, kDkdvWaves, kDkdvGroups, E>;
-        hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes);
-        if (e != hipSuccess) return fail(CW_ERR_LAUNCH, "hipFuncSetAttribute(attn_dkdv_kernel): %s", hipGetErrorString(e));
+        if (const int lrc = ensure_dynamic_lds((const void*)kern, (int)(lds_bytes), "attn_dkdv_kernel"); lrc != CW_OK) return lrc;
         hipLaunchKernelGGL(kern, dim3((unsigned)(nblk * B * H)), dim3(kDkdvWaves * 64), lds_bytes, s, a);
     } else {
         constexpr int lds_bytes = 2 * dkdv_stage_bytes<2>();
         auto kern = attn_dkdv_kernel<2, 4, 1, E>;
         const int64_t nkv = (S + 4 * kRowsPerWave - 1) / (4 * kRowsPerWave);
         if (nkv * B * H > INT32_MAX) return fail(CW_ERR_INVALID, "cw_attn_bwd: S or B*H too large");
-        hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes);
-        if (e != hipSuccess) return fail(CW_ERR_LAUNCH, "hipFuncSetAttribute(attn_dkdv_kernel): %s", hipGetErrorString(e));
+        if (const int lrc = ensure_dynamic_lds((const void*)kern, (int)(lds_bytes), "attn_dkdv_kernel"); lrc != CW_OK) return lrc;
         hipLaunchKernelGGL(kern, dim3((unsigned)(nkv * B * H)), dim3(4 * 64), lds_bytes, s, a);
     }
     return check_launch("attn_dkdv_kernel");
@@ -499,6 +497,7 @@ extern "C" int cw_attn_bwd(int64_t B, int64_t H, int64_t S, int64_t D, const voi
     a.scale = scale; a.scale_log2e = scale * kLog2e;
     a.causal = causal ? 1 : 0;
     a.D = (int)D;
+    if (const int drc = require_gfx950("cw_attn_bwd"); drc != CW_OK) return drc;
     hipStream_t s = (hipStream_t)stream;
     return io_dtype == CW_F16 ? launch_bwd<f16_t>(a, B, H, S, D, nblk, s) : launch_bwd<bf16_t>(a, B, H, S, D, nblk, s);
 }

@@ -222,6 +222,7 @@ extern "C" int cw_multi_norm_partials(int n_tensors, const void* const* grads, c
             return fail(CW_ERR_INVALID, "cw_multi_norm_partials: tensor %d is NULL or has a bad size", i);
     if (workspace_bytes < cw_multi_norm_workspace_bytes(n_tensors, numels))
         return fail(CW_ERR_INVALID, "cw_multi_norm_partials: workspace too small (%lld bytes)", (long long)workspace_bytes);
+    if (const int drc = require_gfx950("cw_multi_norm_partials"); drc != CW_OK) return drc;
     hipStream_t s = (hipStream_t)stream;
     const int kind = __builtin_isinf(norm_type) ? 0 : (norm_type == 2.0f ? 2 : 1);
     float* ws = (float*)workspace;
@@ -254,6 +255,7 @@ extern "C" int cw_clip_coef(int n_sets, const float* sets, float tp_scale, float
     if (n_sets < 1 || n_sets > 64) return fail(CW_ERR_INVALID, "cw_clip_coef: n_sets %d outside [1, 64]", n_sets);
     if (sets == nullptr || out2 == nullptr) return fail(CW_ERR_INVALID, "cw_clip_coef: null argument");
     if (!(norm_type > 0.0f)) return fail(CW_ERR_INVALID, "cw_clip_coef: norm_type must be positive (inf for the maximum norm)");
+    if (const int drc = require_gfx950("cw_clip_coef"); drc != CW_OK) return drc;
     hipLaunchKernelGGL(clip_coef_kernel, dim3(1), dim3(64), 0, (hipStream_t)stream, sets, n_sets, tp_scale, norm_type,
                        max_norm, out2);
     return check_launch("clip_coef_kernel");
@@ -269,6 +271,7 @@ extern "C" int cw_multi_scale(int n_tensors, void* const* grads, const int64_t* 
     for (int i = 0; i < n_tensors; ++i)
         if (numels[i] < 0 || (numels[i] > 0 && grads[i] == nullptr) || blocks_of(numels[i]) > (1 << 24))
             return fail(CW_ERR_INVALID, "cw_multi_scale: tensor %d is NULL or has a bad size", i);
+    if (const int drc = require_gfx950("cw_multi_scale"); drc != CW_OK) return drc;
     hipStream_t s = (hipStream_t)stream;
     int done = 0;
     while (done < n_tensors) {

@@ -1,8 +1,11 @@
 // Host side of the C ABI: error text, device sanity, argument checks of
 // cw_gemm_ksteps. The other entry points live beside their kernels.
+#include <atomic>
 #include <cstdarg>
 #include <cstdio>
 #include <cstring>
+#include <mutex>
+#include <unordered_map>
 
 #include "cw_common.h"
 #include "gemm.h"
@@ -26,6 +29,60 @@ int check_launch(const char* what) {
     const hipError_t e = hipGetLastError();
     if (e == hipSuccess) return CW_OK;
     return fail(CW_ERR_LAUNCH, "%s: launch failed: %s", what, hipGetErrorString(e));
+}
+
+namespace {
+constexpr int kMaxDevices = 64;
+std::atomic<int> g_arch_ok[kMaxDevices];  // 0 = not asked yet, 1 = gfx950, -1 = something else
+std::mutex g_lds_mutex;
+std::unordered_map<const void*, int> g_lds_limit[kMaxDevices];  // kernel -> largest limit set on that device
+}  // namespace
+
+int require_gfx950(const char* who) {
+    int dev = -1;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0) {
+        (void)hipGetLastError();
+        return fail(CW_ERR_DEVICE, "%s: no HIP device is current (this library runs on gfx950 only)", who);
+    }
+    if (dev < kMaxDevices) {
+        const int known = g_arch_ok[dev].load(std::memory_order_relaxed);
+        if (known == 1) return CW_OK;
+    }
+    hipDeviceProp_t prop;
+    if (hipGetDeviceProperties(&prop, dev) != hipSuccess) {
+        (void)hipGetLastError();
+        return fail(CW_ERR_DEVICE, "%s: cannot query device %d", who, dev);
+    }
+    const bool ok = strncmp(prop.gcnArchName, "gfx950", 6) == 0;
+    if (dev < kMaxDevices) g_arch_ok[dev].store(ok ? 1 : -1, std::memory_order_relaxed);
+    if (!ok)
+        return fail(CW_ERR_DEVICE, "%s: device %d is %s; this library holds code objects for gfx950 only", who, dev,
+                    prop.gcnArchName);
+    return CW_OK;
+}
+
+int ensure_dynamic_lds(const void* kernel, int bytes, const char* what) {
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) {
+        (void)hipGetLastError();
+        dev = -1;
+    }
+    if (dev >= 0) {
+        std::lock_guard<std::mutex> lock(g_lds_mutex);
+        auto it = g_lds_limit[dev].find(kernel);
+        if (it != g_lds_limit[dev].end() && it->second >= bytes) return CW_OK;
+    }
+    const hipError_t e = hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, bytes);
+    if (e != hipSuccess) {
+        (void)hipGetLastError();
+        return fail(CW_ERR_LAUNCH, "hipFuncSetAttribute(%s, %d bytes of LDS): %s", what, bytes, hipGetErrorString(e));
+    }
+    if (dev >= 0) {
+        std::lock_guard<std::mutex> lock(g_lds_mutex);
+        int& slot = g_lds_limit[dev][kernel];
+        if (slot < bytes) slot = bytes;
+    }
+    return CW_OK;
 }
 
 }  // namespace cw
@@ -149,6 +206,7 @@ extern "C" int cw_gemm_ksteps_ws(int layout, int64_t M, int64_t N, int64_t K, in
     args.n_addends = n_addends;
     args.workspace = workspace_bytes > 0 ? workspace : nullptr;
     args.workspace_bytes = workspace != nullptr ? workspace_bytes : 0;
+    if (const int drc = require_gfx950("cw_gemm_ksteps_ws"); drc != CW_OK) return drc;
     hipStream_t s = (hipStream_t)stream;
     return io_dtype == CW_F32 ? gemm_f32_launch(args, layout, epilogue, s)
                               : gemm_half_launch(args, layout, epilogue, io_dtype == CW_F16, s);

@@ -11,6 +11,13 @@ namespace cw {
 // ---- host side: thread-local error text --------------------------------
 int fail(int code, const char* fmt, ...);
 int check_launch(const char* what);
+// CW_OK when the current device runs this library's gfx950 code objects; otherwise CW_ERR_DEVICE with the
+// message set (no device, or another architecture). The answer is cached per device.
+int require_gfx950(const char* who);
+// Raises a kernel's dynamic-LDS limit to `bytes`. The attribute is sticky, so it is set once per kernel and
+// device (and again only for a larger size): later launches make no runtime call for it, which also keeps
+// a non-stream API call out of regions a caller captures into a graph after a first eager call.
+int ensure_dynamic_lds(const void* kernel, int bytes, const char* what);
 
 inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 

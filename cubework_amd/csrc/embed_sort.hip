@@ -196,13 +196,12 @@ extern "C" int cw_embed_sort_ids(int64_t T, const int64_t* ids, int64_t vocab_st
     const int64_t need = cw_embed_sort_workspace_bytes(T);
     if (need > 0 && (workspace == nullptr || workspace_bytes < need || (reinterpret_cast<uintptr_t>(workspace) & 7u) != 0))
         return fail(CW_ERR_INVALID, "cw_embed_sort_ids: workspace of %lld bytes (8-byte aligned) required", (long long)need);
+    if (const int drc = require_gfx950("cw_embed_sort_ids"); drc != CW_OK) return drc;
     hipStream_t s = (hipStream_t)stream;
     if (T <= kRankTokens) {
         const int t_pad = (int)((T + kRankUnit - 1) / kRankUnit) * kRankUnit;
         const int lds_bytes = (t_pad + kRankWaves * 64) * (int)sizeof(uint32_t);
-        hipError_t e = hipFuncSetAttribute((const void*)rank_scatter_kernel, hipFuncAttributeMaxDynamicSharedMemorySize,
-                                           (kRankTokens + kRankWaves * 64) * (int)sizeof(uint32_t));
-        if (e != hipSuccess) return fail(CW_ERR_LAUNCH, "hipFuncSetAttribute(rank_scatter_kernel): %s", hipGetErrorString(e));
+        if (const int lrc = ensure_dynamic_lds((const void*)rank_scatter_kernel, (int)((kRankTokens + kRankWaves * 64) * (int)sizeof(uint32_t)), "rank_scatter_kernel"); lrc != CW_OK) return lrc;
         hipLaunchKernelGGL(rank_scatter_kernel, dim3((unsigned)((T + 31) / 32)), dim3(kRankWaves * 64), lds_bytes, s, ids, (int)T,
                            t_pad, vocab_start, V_loc, sorted_ids, order);
         return check_launch("rank_scatter_kernel");
@@ -211,9 +210,10 @@ extern "C" int cw_embed_sort_ids(int64_t T, const int64_t* ids, int64_t vocab_st
     const int n_local = n < kChunkKeys ? n : kChunkKeys;
     const int chunks = n / n_local;
     const int lds_bytes = n_local * (int)sizeof(uint64_t);
-    hipError_t e = hipFuncSetAttribute((const void*)sort_local_kernel<true>, hipFuncAttributeMaxDynamicSharedMemorySize, kChunkKeys * 8);
-    if (e == hipSuccess) e = hipFuncSetAttribute((const void*)sort_local_kernel<false>, hipFuncAttributeMaxDynamicSharedMemorySize, kChunkKeys * 8);
-    if (e != hipSuccess) return fail(CW_ERR_LAUNCH, "hipFuncSetAttribute(sort_local_kernel): %s", hipGetErrorString(e));
+    if (const int lrc = ensure_dynamic_lds((const void*)sort_local_kernel<true>, kChunkKeys * 8, "sort_local_kernel"); lrc != CW_OK)
+        return lrc;
+    if (const int lrc = ensure_dynamic_lds((const void*)sort_local_kernel<false>, kChunkKeys * 8, "sort_local_kernel"); lrc != CW_OK)
+        return lrc;
     uint64_t* keys = (uint64_t*)workspace;
     hipLaunchKernelGGL(sort_local_kernel<true>, dim3(chunks), dim3(kSortThreads), lds_bytes, s, ids, (int)T, vocab_start, V_loc,
                        keys, n_local, 0, chunks == 1 ? 1 : 0, sorted_ids, order);

@@ -280,6 +280,7 @@ extern "C" int cw_embed_fwd(int64_t T, int64_t E, const int64_t* ids, int64_t vo
     if (T == 0) return CW_OK;
     if (ids == nullptr || weight == nullptr || out == nullptr || ldw < E || ldo < E)
         return fail(CW_ERR_INVALID, "cw_embed_fwd: null pointer or leading dimension < E");
+    if (const int drc = require_gfx950("cw_embed_fwd"); drc != CW_OK) return drc;
     hipStream_t s = (hipStream_t)stream;
     return with_elem_type(io_dtype, [&](auto* tag) {
         return fwd_impl<std::remove_pointer_t<decltype(tag)>>(T, E, ids, vocab_start, V_loc, weight, ldw, out, ldo, s);
@@ -296,6 +297,7 @@ extern "C" int cw_embed_bwd(int64_t T, int64_t E, const int64_t* sorted_ids, con
     if (d_weight == nullptr || ldw < E) return fail(CW_ERR_INVALID, "cw_embed_bwd: d_weight is NULL or ldw < E");
     if (T > 0 && (sorted_ids == nullptr || order == nullptr || d_out == nullptr || ldo < E))
         return fail(CW_ERR_INVALID, "cw_embed_bwd: null pointer or leading dimension < E");
+    if (const int drc = require_gfx950("cw_embed_bwd"); drc != CW_OK) return drc;
     hipStream_t s = (hipStream_t)stream;
     return with_elem_type(io_dtype, [&](auto* tag) {
         return bwd_impl<std::remove_pointer_t<decltype(tag)>>(T, E, sorted_ids, order, vocab_start, V_loc, skip_row, d_out,

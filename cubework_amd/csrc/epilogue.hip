@@ -269,6 +269,7 @@ extern "C" int cw_colsum(int64_t M, int64_t N, const void* dY, int64_t ld, float
     if (io_dtype != CW_BF16 && io_dtype != CW_F32 && io_dtype != CW_F16)
         return fail(CW_ERR_INVALID, "cw_colsum: bad io_dtype %d", io_dtype);
     if (out == nullptr) return fail(CW_ERR_INVALID, "cw_colsum: out is NULL");
+    if (const int drc = require_gfx950("cw_colsum"); drc != CW_OK) return drc;
     hipStream_t s = (hipStream_t)stream;
     if (M == 0) return finalize_col_partials(nullptr, 0, N, 1, N, out, nullptr, s);  // zero fill
     if (dY == nullptr || workspace == nullptr || ld < N)
@@ -289,6 +290,7 @@ extern "C" int cw_colsum_static(int64_t M, int64_t N, const void* dY, int64_t ld
     if (io_dtype != CW_BF16 && io_dtype != CW_F32 && io_dtype != CW_F16)
         return fail(CW_ERR_INVALID, "cw_colsum_static: bad io_dtype %d", io_dtype);
     if (out == nullptr) return fail(CW_ERR_INVALID, "cw_colsum_static: out is NULL");
+    if (const int drc = require_gfx950("cw_colsum_static"); drc != CW_OK) return drc;
     hipStream_t s = (hipStream_t)stream;
     if (M == 0) return finalize_col_partials(nullptr, 0, N, 1, N, out, nullptr, s);  // zero fill
     if (dY == nullptr || ld < N) return fail(CW_ERR_INVALID, "cw_colsum_static: null pointer or ld < N");
@@ -317,6 +319,7 @@ extern "C" int cw_act_bwd_colsum(int activation, int64_t M, int64_t N, const voi
     if (activation != CW_ACT_NONE && activation != CW_ACT_GELU_TANH && activation != CW_ACT_GELU_ERF &&
         activation != CW_ACT_RELU)
         return fail(CW_ERR_INVALID, "cw_act_bwd_colsum: bad activation %d", activation);
+    if (const int drc = require_gfx950("cw_act_bwd_colsum"); drc != CW_OK) return drc;
     hipStream_t s = (hipStream_t)stream;
     if (M == 0) {
         if (dbias == nullptr) return CW_OK;

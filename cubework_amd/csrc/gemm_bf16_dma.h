@@ -342,8 +342,7 @@ int launch_dma_cfg(const GemmArgs& gargs, hipStream_t s, const void* tail_a = nu
     auto kern = gemm_bf16_dma_kernel<TA, TB, EPI, NS, false, E>;
     constexpr size_t lds = lds_bytes_dma<NS>();
     static_assert(lds <= 160 * 1024, "LDS image does not fit the CU");
-    hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-    if (e != hipSuccess) return fail(CW_ERR_LAUNCH, "hipFuncSetAttribute(gemm_bf16_ring): %s", hipGetErrorString(e));
+    if (const int lrc = ensure_dynamic_lds((const void*)kern, (int)((int)lds), "gemm_bf16_ring"); lrc != CW_OK) return lrc;
     const int tiles = ((args.M + kTile - 1) / kTile) * ((args.N + kTile - 1) / kTile);
     const int grid = ((tiles + 7) / 8) * 8;
     hipLaunchKernelGGL(kern, dim3(grid), dim3(kThreads), lds, s, args);
@@ -360,8 +359,7 @@ int launch_dma_split(const GemmArgs& gargs, int slices, hipStream_t s) {
     args.partial = reinterpret_cast<float*>(gargs.workspace);
     auto kern = gemm_bf16_dma_kernel<TA, TB, CW_EPI_NONE, kStages, true, E>;
     constexpr size_t lds = lds_bytes_dma<kStages>();
-    hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-    if (e != hipSuccess) return fail(CW_ERR_LAUNCH, "hipFuncSetAttribute(gemm_bf16_ring, split): %s", hipGetErrorString(e));
+    if (const int lrc = ensure_dynamic_lds((const void*)kern, (int)((int)lds), "gemm_bf16_ring, split"); lrc != CW_OK) return lrc;
     const int tiles = ((args.M + kTile - 1) / kTile) * ((args.N + kTile - 1) / kTile);
     const int grid = ((tiles + 7) / 8) * 8;
     hipLaunchKernelGGL(kern, dim3(grid, slices), dim3(kThreads), lds, s, args);

@@ -548,8 +548,7 @@ int launch_cfg(const GemmArgs& args, hipStream_t s) {
     constexpr size_t lds = lds_bytes<BM, BN>();
     static_assert(lds <= 160 * 1024, "LDS tile does not fit the CU");
     if (lds > 48 * 1024) {
-        hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-        if (e != hipSuccess) return fail(CW_ERR_LAUNCH, "hipFuncSetAttribute(gemm_bf16): %s", hipGetErrorString(e));
+        if (const int lrc = ensure_dynamic_lds((const void*)kern, (int)((int)lds), "gemm_bf16"); lrc != CW_OK) return lrc;
     }
     const int tiles = ((args.M + BM - 1) / BM) * ((args.N + BN - 1) / BN);
     const int grid = ((tiles + 7) / 8) * 8;

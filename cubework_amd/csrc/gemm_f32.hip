@@ -576,8 +576,7 @@ int launch(const GemmArgs& g, int epilogue, hipStream_t s) {
     constexpr int patches = 4 * 32 * kPatchPitch * 4;
     constexpr int lds = stages > patches ? stages : patches;
     static_assert(lds <= 160 * 1024, "LDS image does not fit the CU");
-    hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, lds);
-    if (e != hipSuccess) return fail(CW_ERR_LAUNCH, "hipFuncSetAttribute(gemm_f32_ring): %s", hipGetErrorString(e));
+    if (const int lrc = ensure_dynamic_lds((const void*)kern, (int)(lds), "gemm_f32_ring"); lrc != CW_OK) return lrc;
     const int tiles = ((g.M + 64 * TI - 1) / (64 * TI)) * ((g.N + 64 * TJ - 1) / (64 * TJ));
     hipLaunchKernelGGL(kern, dim3(((tiles + 7) / 8) * 8), dim3(kThreads), lds, s, r, epilogue);
     return check_launch("gemm_f32_ring_kernel");

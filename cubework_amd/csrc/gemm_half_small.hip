@@ -196,8 +196,7 @@ int launch_cfg(const RingArgs& args, hipStream_t s) {
     constexpr size_t ctile = (size_t)kBM * gemm_bf16::c_pitch<kBN>() * sizeof(uint16_t);
     constexpr size_t lds = stages > ctile ? stages : ctile;
     static_assert(lds <= 160 * 1024, "LDS image does not fit the CU");
-    hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-    if (e != hipSuccess) return fail(CW_ERR_LAUNCH, "hipFuncSetAttribute(gemm_half_small): %s", hipGetErrorString(e));
+    if (const int lrc = ensure_dynamic_lds((const void*)kern, (int)((int)lds), "gemm_half_small"); lrc != CW_OK) return lrc;
     const int tiles = ((args.M + kBM - 1) / kBM) * ((args.N + kBN - 1) / kBN);
     hipLaunchKernelGGL(kern, dim3(((tiles + 7) / 8) * 8), dim3(kThreads), lds, s, args);
     return check_launch("gemm_half_small_kernel");

@@ -1000,8 +1000,7 @@ int bwd_partials_launch_as(int64_t R, int64_t C, const void* dY, int64_t ld_dy, 
     const size_t lds = flat_reduce_lds_bytes(2 * NCH * V, NWAVES);
     auto kern = ln_bwd_partials_kernel<T, NCH, NWAVES, NR, FUSE_DX>;
     if (lds > 48 * 1024) {
-        hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-        if (e != hipSuccess) return fail(CW_ERR_LAUNCH, "hipFuncSetAttribute(ln_bwd_partials): %s", hipGetErrorString(e));
+        if (const int lrc = ensure_dynamic_lds((const void*)kern, (int)((int)lds), "ln_bwd_partials"); lrc != CW_OK) return lrc;
     }
     hipLaunchKernelGGL(kern, dim3((unsigned)nb), dim3(NWAVES * 64), lds, s, R, C, (const T*)dY, ld_dy, (const T*)x,
                        ld_x, mean_rstd, (const T*)gamma, row_sums, ws, want_cols, (T*)dx, ld_dx, 1.0f / (float)C);
@@ -1131,14 +1130,14 @@ int bwd_partials_impl(int64_t R, int64_t C, const void* dY, int64_t ld_dy, const
         if (rc != CW_OK) return rc;
         if (dx_done != nullptr) *dx_done = fdx != nullptr;
     } else {
+        nparts = (R + kGenericSlabRows - 1) / kGenericSlabRows;
+        if (want_cols && workspace_bytes < nparts * 2 * C * (int64_t)sizeof(float))  // before anything is launched
+            return fail(CW_ERR_INVALID, "cw_ln_bwd_partials: workspace too small (%lld bytes)", (long long)workspace_bytes);
         hipLaunchKernelGGL(ln_bwd_rows_generic_kernel<T>, dim3(ln_grid(R)), dim3(kLnBlock), 0, s, R, C,
                            (const T*)dY, ld_dy, (const T*)x, ld_x, mean_rstd, (const T*)gamma, row_sums);
         rc = check_launch("ln_bwd_rows_generic_kernel");
         if (rc != CW_OK) return rc;
         if (want_cols) {
-            nparts = (R + kGenericSlabRows - 1) / kGenericSlabRows;
-            if (workspace_bytes < nparts * 2 * C * (int64_t)sizeof(float))
-                return fail(CW_ERR_INVALID, "cw_ln_bwd_partials: workspace too small (%lld bytes)", (long long)workspace_bytes);
             dim3 grid((unsigned)((C + kLnBlock - 1) / kLnBlock), (unsigned)nparts);
             hipLaunchKernelGGL(ln_bwd_cols_generic_kernel<T>, grid, dim3(kLnBlock), 0, s, R, C, (const T*)dY, ld_dy,
                                (const T*)x, ld_x, mean_rstd, (float*)workspace, kGenericSlabRows);
@@ -1203,6 +1202,7 @@ extern "C" int cw_ln_partial_stats(int64_t R, int64_t C, const void* x, int64_t 
     if (mode != CW_LN_ONE_PASS && mode != CW_LN_TWO_PASS) return fail(CW_ERR_INVALID, "cw_ln_partial_stats: bad mode %d", mode);
     if (R == 0) return CW_OK;
     if (x == nullptr || stats == nullptr || ld < C) return fail(CW_ERR_INVALID, "cw_ln_partial_stats: null pointer or ld < C");
+    if (const int drc = require_gfx950("cw_ln_partial_stats"); drc != CW_OK) return drc;
     hipStream_t s = (hipStream_t)stream;
     return with_elem_type(io_dtype, [&](auto* tag) {
         return stats_impl<std::remove_pointer_t<decltype(tag)>>(R, C, x, ld, mode, mean, stats, s);
@@ -1219,6 +1219,7 @@ extern "C" int cw_ln_normalize(int64_t R, int64_t C, const void* x, int64_t ld, 
     if (R == 0) return CW_OK;
     if (x == nullptr || y == nullptr || stats == nullptr || ld < C || ldy < C)
         return fail(CW_ERR_INVALID, "cw_ln_normalize: null pointer or leading dimension < C");
+    if (const int drc = require_gfx950("cw_ln_normalize"); drc != CW_OK) return drc;
     hipStream_t s = (hipStream_t)stream;
     return with_elem_type(io_dtype, [&](auto* tag) {
         return normalize_impl<std::remove_pointer_t<decltype(tag)>, false>(R, C, x, ld, stats, mode, H, eps, gamma, beta,
@@ -1235,6 +1236,7 @@ extern "C" int cw_ln_forward_fused(int64_t R, int64_t C, const void* x, int64_t 
     if (R == 0) return CW_OK;
     if (x == nullptr || y == nullptr || ld < C || ldy < C)
         return fail(CW_ERR_INVALID, "cw_ln_forward_fused: null pointer or leading dimension < C");
+    if (const int drc = require_gfx950("cw_ln_forward_fused"); drc != CW_OK) return drc;
     hipStream_t s = (hipStream_t)stream;
     return with_elem_type(io_dtype, [&](auto* tag) {
         return normalize_impl<std::remove_pointer_t<decltype(tag)>, true>(R, C, x, ld, nullptr, mode, C, eps, gamma, beta,
@@ -1254,6 +1256,7 @@ extern "C" int cw_ln_bwd_partials(int64_t R, int64_t C, const void* dY, int64_t 
     if (dY == nullptr || x == nullptr || mean_rstd == nullptr || row_sums == nullptr || ld_dy < C || ld_x < C)
         return fail(CW_ERR_INVALID, "cw_ln_bwd_partials: null pointer or leading dimension < C");
     if (dgamma != nullptr && workspace == nullptr) return fail(CW_ERR_INVALID, "cw_ln_bwd_partials: workspace is NULL");
+    if (const int drc = require_gfx950("cw_ln_bwd_partials"); drc != CW_OK) return drc;
     hipStream_t s = (hipStream_t)stream;
     return with_elem_type(io_dtype, [&](auto* tag) {
         return bwd_partials_impl<std::remove_pointer_t<decltype(tag)>>(R, C, dY, ld_dy, x, ld_x, mean_rstd, gamma, row_sums,
@@ -1289,6 +1292,7 @@ extern "C" int cw_ln_backward_fused(int64_t R, int64_t C, const void* dY, int64_
         ld_x < C || ld_dx < C)
         return fail(CW_ERR_INVALID, "cw_ln_backward_fused: null pointer or leading dimension < C");
     if (dgamma != nullptr && workspace == nullptr) return fail(CW_ERR_INVALID, "cw_ln_backward_fused: workspace is NULL");
+    if (const int drc = require_gfx950("cw_ln_backward_fused"); drc != CW_OK) return drc;
     hipStream_t s = (hipStream_t)stream;
     return with_elem_type(io_dtype, [&](auto* tag) {
         return backward_fused_impl<std::remove_pointer_t<decltype(tag)>>(R, C, dY, ld_dy, x, ld_x, mean_rstd, gamma, row_sums,
@@ -1307,6 +1311,7 @@ extern "C" int cw_ln_bwd_dx(int64_t R, int64_t C, const void* dY, int64_t ld_dy,
     if (dY == nullptr || x == nullptr || mean_rstd == nullptr || row_sums == nullptr || dx == nullptr || ld_dy < C ||
         ld_x < C || ld_dx < C)
         return fail(CW_ERR_INVALID, "cw_ln_bwd_dx: null pointer or leading dimension < C");
+    if (const int drc = require_gfx950("cw_ln_bwd_dx"); drc != CW_OK) return drc;
     hipStream_t s = (hipStream_t)stream;
     return with_elem_type(io_dtype, [&](auto* tag) {
         return bwd_dx_impl<std::remove_pointer_t<decltype(tag)>>(R, C, dY, ld_dy, x, ld_x, mean_rstd, gamma, row_sums, H, dx,

@@ -337,6 +337,7 @@ extern "C" int cw_vpce_fwd_local(int64_t T, int64_t V, const void* logits, int64
     if (logits == nullptr || targets == nullptr || out_max == nullptr || out_sumexp == nullptr ||
         out_pred == nullptr || out_mask == nullptr || ld < V)
         return fail(CW_ERR_INVALID, "cw_vpce_fwd_local: null pointer or ld < V");
+    if (const int drc = require_gfx950("cw_vpce_fwd_local"); drc != CW_OK) return drc;
     hipStream_t s = (hipStream_t)stream;
     if (io_dtype == CW_BF16) {
         const int vec_ok = aligned16(logits) && (ld % 8) == 0;
@@ -364,6 +365,7 @@ extern "C" int cw_vpce_finalize(int64_t T, int n_ranks, const float* max_all, co
     if (T == 0) return CW_OK;
     if (max_all == nullptr || sumexp_all == nullptr || pred_all == nullptr || mask_all == nullptr || loss == nullptr)
         return fail(CW_ERR_INVALID, "cw_vpce_finalize: null pointer");
+    if (const int drc = require_gfx950("cw_vpce_finalize"); drc != CW_OK) return drc;
     hipLaunchKernelGGL(vpce_finalize_kernel, dim3((unsigned)((T + 255) / 256)), dim3(256), 0, (hipStream_t)stream, T,
                        n_ranks, max_all, sumexp_all, pred_all, mask_all, loss, gmax, gsum);
     return check_launch("vpce_finalize_kernel");
@@ -384,6 +386,7 @@ extern "C" int cw_vpce_bwd(int64_t T, int64_t V, const void* logits, int64_t ld,
     if (logits == nullptr || targets == nullptr || gmax == nullptr || gsum == nullptr || grad == nullptr || ld < V ||
         ld_grad < V)
         return fail(CW_ERR_INVALID, "cw_vpce_bwd: null pointer or leading dimension < V");
+    if (const int drc = require_gfx950("cw_vpce_bwd"); drc != CW_OK) return drc;
     hipStream_t s = (hipStream_t)stream;
     if (io_dtype == CW_F16 && grad_dtype == CW_F16)
         return bwd_impl<f16_t, f16_t>(T, V, logits, ld, targets, vocab_start, gmax, gsum, dloss_rows, dloss_scale, grad, ld_grad, s);

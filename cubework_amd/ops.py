@@ -122,11 +122,15 @@ def gemm_ksteps(layout: str, A_steps: Sequence[torch.Tensor], B_steps: Sequence[
             raise ValueError("bias has %d elements, output width is %d" % (bias.numel(), N))
         bias = bias.to(a0.dtype).contiguous()
     addends = [_rows(t) for t in addends]
-    ldadd = 0
     for t in addends:
         if tuple(t.shape) != (M, N) or t.dtype != a0.dtype:
             raise ValueError("addends must be [M,N] of the operand dtype")
-        ldadd = _ld(t)
+    ldadd = _ld(addends[0]) if addends else 0
+    # the C ABI takes one leading dimension for all addends: copy those that are laid out differently
+    addends = [t if _ld(t) == ldadd else t.contiguous() for t in addends]
+    if any(_ld(t) != ldadd for t in addends):
+        ldadd = N
+        addends = [t.contiguous() for t in addends]
     if out is None:
         out = torch.empty((M, N), dtype=a0.dtype, device=a0.device)
     elif tuple(out.shape) != (M, N) or out.dtype != a0.dtype or out.stride(1) != 1:

@@ -26,6 +26,7 @@ drawn under the reference's per-rank RNG fork are deliberately not restated.
 Precision convention for bf16 inputs: evaluate the reference formulas in fp32
 (float64 where noted) on the bf16-rounded inputs and round the result once.
 """
+from ._precision import precision, compute_dtype  # noqa: F401
 from .summa import (gemm_ksteps, summa_ab_rank, summa_abt_rank, summa_atb_rank, summa_ab_reference_dtype,  # noqa: F401
                     activation, activation_grad, act_bwd_colsum, colsum)
 from .layernorm import (ln2d_partial_stats, ln2d_mean_rstd, ln2d_normalize, ln2d_backward_partials, ln2d_backward_dx,  # noqa: F401

@@ -17,8 +17,7 @@ import math
 import torch
 
 
-def _f(t):
-    return t.detach().to("cpu").to(torch.float32)
+from ._precision import to_compute as _f
 
 
 def split_qkv(qkv: torch.Tensor, heads: int):
@@ -30,14 +29,14 @@ def split_qkv(qkv: torch.Tensor, heads: int):
 
 
 def attention_core(q, k, v, scale=None, causal=True, return_lse=False):
-    """softmax(scale * q k^T + mask) v in fp32 on [b, heads, s, d] inputs; returns [b, s, heads*d]
+    """softmax(scale * q k^T + mask) v in the compute type on [b, heads, s, d] inputs; returns [b, s, heads*d]
     (and the natural-log sum of exponentials [b, heads, s])."""
     q, k, v = _f(q), _f(k), _f(v)
     b, h, s, d = q.shape
     scale = d ** -0.5 if scale is None else scale
     w = torch.matmul(q * scale, k.transpose(-1, -2))
     if causal:
-        mask = torch.full((s, s), float("-inf")).triu(1)
+        mask = torch.full((s, s), float("-inf"), dtype=w.dtype).triu(1)
         w = w + mask
     lse = torch.logsumexp(w, dim=-1)
     p = torch.softmax(w, dim=-1)
@@ -54,7 +53,7 @@ def attention_core_backward(q, k, v, d_out, scale=None, causal=True):
     do = _f(d_out).reshape(b, s, h, d).transpose(1, 2)
     w = torch.matmul(q * scale, k.transpose(-1, -2))
     if causal:
-        w = w + torch.full((s, s), float("-inf")).triu(1)
+        w = w + torch.full((s, s), float("-inf"), dtype=w.dtype).triu(1)
     p = torch.softmax(w, dim=-1)
     dv = torch.matmul(p.transpose(-1, -2), do)
     dp = torch.matmul(do, v.transpose(-1, -2))

@@ -10,15 +10,15 @@ Reference statements followed:
   cubework/module/parallel_3d/_operation.py:273-281  two-pass mean / var / sigma, y = w*z + b
   cubework/module/parallel_3d/_operation.py:294-311  3D backward
 Collectives are replaced by explicit "local partial" / "summed over peers"
-arguments. All arithmetic is fp32 on the inputs as given.
+arguments. All arithmetic is in the oracle's compute type (fp32 unless oracle.precision says
+float64) on the inputs as given.
 """
 from typing import Optional
 
 import torch
 
 
-def _f(t):
-    return None if t is None else t.detach().to("cpu").to(torch.float32)
+from ._precision import round_like, to_compute as _f
 
 
 # ---- 2D: one-pass statistics ----------------------------------------------
@@ -50,7 +50,7 @@ def ln2d_normalize(x, stats_global, hidden: int, eps: float, gamma=None, beta=No
         y = y * _f(gamma)
     if beta is not None:
         y = y + _f(beta)  # module.py:170
-    return y.to(x.dtype).reshape(x.shape), mr
+    return round_like(y, x).reshape(x.shape), mr
 
 
 def ln2d_backward_partials(dy, x, mean_rstd, gamma=None):
@@ -80,7 +80,7 @@ def ln2d_backward_dx(dy, x, mean_rstd, row_sums_global, hidden: int, gamma=None)
     grad -= xh * (rs[:, 1:2] / hidden)
     grad -= rs[:, 0:1] / hidden
     grad *= mr[:, 1:2]
-    return grad.to(x.dtype).reshape(x.shape)
+    return round_like(grad, x).reshape(x.shape)
 
 
 # ---- 3D: two-pass statistics ------------------------------------------------
@@ -102,7 +102,7 @@ def ln3d_forward(x, gamma, beta, hidden: int, eps: float, peer_sum=None, peer_sq
     sigma = torch.sqrt(var + eps)
     z = mu / sigma
     y = _f(gamma) * z + _f(beta)
-    return y.to(x.dtype).reshape(x.shape), mu, sigma
+    return round_like(y, x).reshape(x.shape), mu, sigma
 
 
 def ln3d_backward(dy, mu, sigma, gamma, hidden: int, peer_dvar=None, peer_dmean_fn=None):
@@ -121,7 +121,7 @@ def ln3d_backward(dy, mu, sigma, gamma, hidden: int, peer_dvar=None, peer_dmean_
     if peer_dmean_fn is not None:
         dmean = dmean + peer_dmean_fn(dvar)
     dx = dz / sigma + dvar * 2 * mu / hidden + dmean / hidden
-    return dx.to(dy.dtype).reshape(dy.shape), dgamma, dbeta
+    return round_like(dx, dy).reshape(dy.shape), dgamma, dbeta
 
 
 # ---- whole-row helpers (tensor-parallel size 1) -----------------------------

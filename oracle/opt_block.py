@@ -9,14 +9,23 @@ from typing import Dict, Tuple
 import torch
 import torch.nn.functional as F
 
+from ._precision import compute_dtype
+
 _ACT = {"relu": F.relu, "gelu": F.gelu, "gelu_erf": F.gelu, "gelu_tanh": lambda t: F.gelu(t, approximate="tanh")}
 
 
-def opt_block_reference(block, x: torch.Tensor) -> Tuple[torch.Tensor, Dict[str, torch.Tensor]]:
-    """The same layer in plain fp32 torch on the CPU, with leaf copies of the
-    block's parameters (returned by name so gradients can be compared).
-    Weights of the 2D/3D layers are [in, out]; 1D layers keep [out, in]."""
-    p = {n: t.detach().float().cpu().clone().requires_grad_(True) for n, t in block.named_parameters()}
+def opt_block_reference(block, x: torch.Tensor, relu_mask=None) -> Tuple[torch.Tensor, Dict[str, torch.Tensor]]:
+    """The same layer in plain torch on the CPU (compute type: fp32 unless oracle.precision says float64), with
+    leaf copies of the block's parameters (returned by name so gradients can be compared).
+    Weights of the 2D/3D layers are [in, out]; 1D layers keep [out, in].
+
+    relu_mask (optional, bool, the shape of fc1's output): which units the ReLU lets through, instead of
+    `fc1 > 0`. ReLU's derivative jumps at 0, so a pre-activation that another arithmetic rounds to the
+    other side of 0 flips a whole gradient path; a comparison of gradients hands over the mask of the
+    implementation under test, after which both sides differentiate the same piecewise-linear function."""
+    ct = compute_dtype()
+    x = x.to(ct)
+    p = {n: t.detach().cpu().to(ct).clone().requires_grad_(True) for n, t in block.named_parameters()}
 
     def find(prefix: str, leaf: str) -> torch.Tensor:
         for n, t in p.items():
@@ -39,7 +48,13 @@ def opt_block_reference(block, x: torch.Tensor) -> Tuple[torch.Tensor, Dict[str,
     q, k, v = torch.chunk(qkv, 3, dim=-1)
     o = F.scaled_dot_product_attention(q, k, v, is_causal=True).transpose(1, 2).reshape(b, s, heads * hd)
     x1 = x + lin("out_proj", o)
-    h = _ACT[block.activation](lin("fc1", ln("final_layer_norm", x1)))
+    pre = lin("fc1", ln("final_layer_norm", x1))
+    if relu_mask is not None:
+        if block.activation != "relu":
+            raise ValueError("relu_mask is for a block whose activation is ReLU")
+        h = pre * relu_mask.to(pre.dtype).reshape(pre.shape)
+    else:
+        h = _ACT[block.activation](pre)
     return x1 + lin("fc2", h), p
 
 

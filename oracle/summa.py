@@ -16,6 +16,9 @@ from typing import Optional, Sequence
 import torch
 import torch.nn.functional as F
 
+from . import _precision
+from ._precision import round_like
+
 
 def _f(t: torch.Tensor, dtype) -> torch.Tensor:
     return t.detach().to("cpu").to(dtype)
@@ -42,15 +45,18 @@ def activation_grad(x: torch.Tensor, kind: Optional[str]) -> torch.Tensor:
 
 def gemm_ksteps(layout: str, A_steps: Sequence[torch.Tensor], B_steps: Sequence[torch.Tensor],
                 bias: Optional[torch.Tensor] = None, act: Optional[str] = None,
-                addends: Sequence[torch.Tensor] = (), compute_dtype=torch.float32, return_preact: bool = False):
+                addends: Sequence[torch.Tensor] = (), compute_dtype=None, return_preact: bool = False):
     """act(sum_i op(A_i) op(B_i) + sum_j addends_j + bias), accumulated in
-    compute_dtype on the inputs as given, rounded once to the inputs' dtype.
+    compute_dtype (default: the oracle's compute type) on the inputs as given; 16-bit
+    inputs give a result rounded once to their type, fp32 inputs one in compute_dtype.
 
     The k-step loop is parallel_2d/_operation.py:43-47 (NN), :119-125 (NT),
     :199-204 (TN) with the broadcast operands passed in; addends are the
     partial products a `reduce` delivers from the peers.
     """
-    out_dtype = A_steps[0].dtype
+    if compute_dtype is None:
+        compute_dtype = _precision.compute_dtype()
+    out_dtype = A_steps[0].dtype if A_steps[0].dtype in (torch.bfloat16, torch.float16) else compute_dtype
     acc = None
     for a, b in zip(A_steps, B_steps):
         a, b = _f(a, compute_dtype), _f(b, compute_dtype)
@@ -108,13 +114,14 @@ def summa_ab_reference_dtype(A_steps, B_steps, bias=None):
 
 
 def colsum(dy: torch.Tensor) -> torch.Tensor:
-    """fp32 sum over every dimension but the last
+    """Sum over every dimension but the last, in the compute type
     (parallel_2d/_operation.py:285-286, parallel_3d/_operation.py:59)."""
-    d = _f(dy, torch.float32)
+    d = _f(dy, _precision.compute_dtype())
     return d.reshape(-1, d.shape[-1]).sum(dim=0)
 
 
 def act_bwd_colsum(kind, dy: torch.Tensor, preact: torch.Tensor):
     """Backward of `act(preact)` followed by the bias-gradient column sum."""
-    g = _f(dy, torch.float32) * activation_grad(_f(preact, torch.float32), kind)
-    return g.to(dy.dtype), g.reshape(-1, g.shape[-1]).sum(dim=0)
+    ct = _precision.compute_dtype()
+    g = _f(dy, ct) * activation_grad(_f(preact, ct), kind)
+    return round_like(g, dy), g.reshape(-1, g.shape[-1]).sum(dim=0)

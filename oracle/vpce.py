@@ -17,8 +17,7 @@ vocab_end with `>` (loss_2d.py:48-50): the same set of targets.
 import torch
 
 
-def _f(t):
-    return t.detach().to("cpu").to(torch.float32)
+from ._precision import compute_dtype, to_compute as _f
 
 
 def vpce_fwd_local(logits: torch.Tensor, targets: torch.Tensor, vocab_start: int):
@@ -52,7 +51,7 @@ def vpce_finalize(max_all, sumexp_all, pred_all, mask_all):
 
 def vpce_bwd(logits, targets, vocab_start: int, gmax, gsum, dloss):
     """Gradient w.r.t. this rank's logits slice; dloss is [T] or a scalar.
-    Returned in fp32."""
+    Returned in the compute type."""
     x = _f(logits).reshape(-1, logits.shape[-1])
     t = targets.detach().to("cpu").reshape(-1).to(torch.int64)
     V = x.shape[-1]
@@ -62,7 +61,7 @@ def vpce_bwd(logits, targets, vocab_start: int, gmax, gsum, dloss):
     softmax = torch.exp(x - _f(gmax).unsqueeze(-1)) / _f(gsum).unsqueeze(-1)
     grad = softmax
     ar = torch.arange(x.shape[0])
-    grad[ar, masked_target] -= 1.0 - mask.float()
+    grad[ar, masked_target] -= 1.0 - mask.to(grad.dtype)
     dl = dloss if torch.is_tensor(dloss) else torch.tensor(float(dloss))
     dl = _f(dl)
     grad = grad * (dl.unsqueeze(-1) if dl.dim() == 1 else dl)
@@ -78,7 +77,7 @@ def vpce_reference_full(slices, targets, dloss=None):
     V = xs[0].shape[-1]
     logits_max = torch.stack([torch.max(x, dim=-1)[0] for x in xs]).max(dim=0)[0]      # :17-18
     xs = [x - logits_max.unsqueeze(-1) for x in xs]                                     # :20
-    predicted = torch.zeros(xs[0].shape[0])
+    predicted = torch.zeros(xs[0].shape[0], dtype=compute_dtype())
     masks, mts = [], []
     ar = torch.arange(xs[0].shape[0])
     for r, x in enumerate(xs):
@@ -98,7 +97,7 @@ def vpce_reference_full(slices, targets, dloss=None):
     dl = torch.ones_like(loss) if dloss is None else _f(dloss if torch.is_tensor(dloss) else torch.tensor(float(dloss)))
     for e, mask, mt in zip(exps, masks, mts):
         g = e / sum_exp.unsqueeze(-1)                                                   # :55
-        g[ar, mt] -= 1.0 - mask.float()                                                 # :74
+        g[ar, mt] -= 1.0 - mask.to(g.dtype)                                                # :74
         g = g * (dl.unsqueeze(-1) if dl.dim() == 1 else dl)                             # :77
         grads.append(g)
     return loss, grads

@@ -97,3 +97,25 @@ def test_scratch_sizes_and_refusals_of_the_later_entry_points():
     # fused LayerNorm backward: the two column outputs come together
     assert lib.cw_ln_backward_fused(4, 8, None, 8, None, 8, None, None, None, None, 8, None, C.c_void_p(16), None, 0, BF16, None) == -1
     assert b"both" in lib.cw_last_error()
+
+
+def test_no_usable_device_is_reported_as_such():
+    """Without a GPU (or on one that is not gfx950) a call that passes its argument checks returns
+    CW_ERR_DEVICE before anything is launched; the pointers are never touched."""
+    import ctypes as C
+    import torch
+    from cubework_amd import _lib
+    if not os.path.exists(_lib.LIB_PATH):
+        pytest.skip("libcubework_hip.so not built yet")
+    if torch.cuda.is_available():
+        pytest.skip("a GPU is visible: the refusal path needs a machine without one")
+    lib = _lib.load()
+    p = C.c_void_p(256)
+    assert lib.cw_colsum(8, 8, p, 8, p, p, 1 << 20, _lib.CW_F32, None) == -5
+    assert b"device" in lib.cw_last_error().lower()
+    assert lib.cw_colsum_static(8, 8, p, 8, p, _lib.CW_F32, None) == -5
+    assert lib.cw_ln_partial_stats(4, 8, p, 8, _lib.CW_LN_ONE_PASS, None, p, _lib.CW_BF16, None) == -5
+    tab = (C.c_void_p * 1)(256)
+    assert lib.cw_gemm_ksteps(_lib.CW_NN, 8, 8, 8, 1, tab, 8, tab, 8, None, 0, p, 8, None, 0, None, 0, 0, _lib.CW_BF16, None) == -5
+    assert lib.cw_vpce_finalize(4, 1, p, p, p, p, p, p, p, None) == -5
+    assert lib.cw_device_arch() == b""

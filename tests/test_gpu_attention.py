@@ -6,6 +6,13 @@ import torch
 from tests.util import assert_parity, randn
 
 pytestmark = pytest.mark.gpu
+
+# The log-sum-exp the forward saves for the backward is stored in fp32 but carries 16-bit accuracy by design: the
+# row sum is taken over the probabilities as rounded for the second MFMA product, so that the output's
+# normaliser is the sum of exactly the weights that multiplied V. Each term is off by at most one 16-bit
+# rounding (2^-8 relative for bf16, 2^-11 for float16), the sum by no more, its logarithm by that much in absolute
+# terms; against the largest |lse| of a case (about 3 to 8) that is below the bars here (achieved: 2e-4 / 3e-5).
+LSE_BAR = {torch.bfloat16: 1e-3, torch.float16: 1.2e-4}
 DEV = "cuda:0"
 
 
@@ -30,12 +37,13 @@ def test_attention_forward_parity(shape, causal):
     b, s, h = shape
     d = 64
     qkv = _qkv(b, s, h, d, seed=s + h, std=1.5)
-    want, want_lse = oracle.attention_core(*oracle.split_qkv(qkv, h), causal=causal, return_lse=True)
+    with oracle.precision(torch.float64):
+        want, want_lse = oracle.attention_core(*oracle.split_qkv(qkv, h), causal=causal, return_lse=True)
     q, k, v = _views(qkv.to(DEV), h, d)
     got, lse = ops.attn_fwd(q, k, v, causal=causal, want_lse=True)
     torch.cuda.synchronize()
     assert_parity(got, want, torch.bfloat16, "attention out %s causal=%s" % (shape, causal))
-    assert_parity(lse, want_lse, torch.float32, "attention lse %s" % (shape,), scale=100)
+    assert_parity(lse, want_lse, torch.float32, "attention lse %s" % (shape,), bar=LSE_BAR[torch.bfloat16])
 
 
 def test_attention_rows_are_convex_combinations():
@@ -108,8 +116,7 @@ def test_attention_backward_parity(shape, causal):
         assert_parity(g.permute(0, 2, 1, 3), torch.cat(want, dim=-1), torch.bfloat16, "attention grads %s" % (shape,))
         return
     for name, got, ref in (("dq", g[..., :d], want[0]), ("dk", g[..., d:2 * d], want[1]), ("dv", g[..., 2 * d:], want[2])):
-        assert_parity(got.permute(0, 2, 1, 3), ref, torch.bfloat16, "attention %s %s causal=%s" % (name, shape, causal),
-                      scale=2)
+        assert_parity(got.permute(0, 2, 1, 3), ref, torch.bfloat16, "attention %s %s causal=%s" % (name, shape, causal))
 
 
 def test_attention_core_autograd_and_reproducibility():
@@ -131,7 +138,7 @@ def test_attention_core_autograd_and_reproducibility():
     qc, kc, vc = oracle.split_qkv(qkv, h)
     dq, dk, dv = oracle.attention_core_backward(qc, kc, vc, d_out)
     want = torch.cat([dq, dk, dv], dim=-1).permute(0, 2, 1, 3).reshape(b, s, h * 3 * d)
-    assert_parity(g1, want, torch.bfloat16, "d qkv", scale=2)
+    assert_parity(g1, want, torch.bfloat16, "d qkv")
     assert_parity(y, oracle.attention_core(qc, kc, vc), torch.bfloat16, "attention_core forward")
 
 
@@ -150,7 +157,8 @@ def test_attention_head_size_128(shape, causal):
     qkv = _qkv(b, s, h, d, seed=3 * s + h, std=1.2)
     d_out = randn((b, s, h * d), torch.bfloat16, seed=s + 17)
     qc, kc, vc = oracle.split_qkv(qkv, h)
-    want, want_lse = oracle.attention_core(qc, kc, vc, causal=causal, return_lse=True)
+    with oracle.precision(torch.float64):
+        want, want_lse = oracle.attention_core(qc, kc, vc, causal=causal, return_lse=True)
     want_g = oracle.attention_core_backward(qc, kc, vc, d_out, causal=causal)
     dev = qkv.to(DEV)
     q, k, v = _views(dev, h, d)
@@ -159,13 +167,12 @@ def test_attention_head_size_128(shape, causal):
     ops.attn_bwd(q, k, v, out, d_out.to(DEV), lse, g[..., :d], g[..., d:2 * d], g[..., 2 * d:], causal=causal)
     torch.cuda.synchronize()
     assert_parity(out, want, torch.bfloat16, "attention out d=128 %s" % (shape,))
-    assert_parity(lse, want_lse, torch.float32, "attention lse d=128 %s" % (shape,), scale=100)
+    assert_parity(lse, want_lse, torch.float32, "attention lse d=128 %s" % (shape,), bar=LSE_BAR[torch.bfloat16])
     if s == 1:
         assert_parity(g.permute(0, 2, 1, 3), torch.cat(want_g, dim=-1), torch.bfloat16, "attention grads d=128 %s" % (shape,))
         return
     for name, got, ref in (("dq", g[..., :d], want_g[0]), ("dk", g[..., d:2 * d], want_g[1]), ("dv", g[..., 2 * d:], want_g[2])):
-        assert_parity(got.permute(0, 2, 1, 3), ref, torch.bfloat16, "attention %s d=128 %s causal=%s" % (name, shape, causal),
-                      scale=2)
+        assert_parity(got.permute(0, 2, 1, 3), ref, torch.bfloat16, "attention %s d=128 %s causal=%s" % (name, shape, causal))
 
 
 def test_attention_head_size_128_autograd():
@@ -184,7 +191,7 @@ def test_attention_head_size_128_autograd():
     qc, kc, vc = oracle.split_qkv(qkv, h)
     dq, dk, dv = oracle.attention_core_backward(qc, kc, vc, d_out)
     want = torch.cat([dq, dk, dv], dim=-1).permute(0, 2, 1, 3).reshape(b, s, h * 3 * d)
-    assert_parity(g1, want, torch.bfloat16, "d qkv, head size 128", scale=2)
+    assert_parity(g1, want, torch.bfloat16, "d qkv, head size 128")
 
 
 @pytest.mark.parametrize("d", [64, 128])
@@ -202,7 +209,8 @@ def test_attention_float16(shape, causal, d):
     qkv = _qkv(b, s, h, d, seed=5 * s + h, std=1.2).to(f16)
     d_out = randn((b, s, h * d), f16, seed=s + 19)
     qc, kc, vc = oracle.split_qkv(qkv, h)
-    want, want_lse = oracle.attention_core(qc, kc, vc, causal=causal, return_lse=True)
+    with oracle.precision(torch.float64):
+        want, want_lse = oracle.attention_core(qc, kc, vc, causal=causal, return_lse=True)
     want_g = oracle.attention_core_backward(qc, kc, vc, d_out, causal=causal)
     dev = qkv.to(DEV)
     q, k, v = _views(dev, h, d)
@@ -212,10 +220,9 @@ def test_attention_float16(shape, causal, d):
     torch.cuda.synchronize()
     assert out.dtype == f16
     assert_parity(out, want, f16, "float16 attention out d=%d %s" % (d, shape))
-    assert_parity(lse, want_lse, torch.float32, "float16 attention lse d=%d %s" % (d, shape), scale=100)
+    assert_parity(lse, want_lse, torch.float32, "float16 attention lse d=%d %s" % (d, shape), bar=LSE_BAR[torch.float16])
     if s == 1:  # dq and dk are exactly zero: judged against the size of the whole gradient
         assert_parity(g.permute(0, 2, 1, 3), torch.cat(want_g, dim=-1), f16, "float16 attention grads d=%d %s" % (d, shape))
         return
     for name, got, ref in (("dq", g[..., :d], want_g[0]), ("dk", g[..., d:2 * d], want_g[1]), ("dv", g[..., 2 * d:], want_g[2])):
-        assert_parity(got.permute(0, 2, 1, 3), ref, f16, "float16 attention %s d=%d %s causal=%s" % (name, d, shape, causal),
-                      scale=2)
+        assert_parity(got.permute(0, 2, 1, 3), ref, f16, "float16 attention %s d=%d %s causal=%s" % (name, d, shape, causal))

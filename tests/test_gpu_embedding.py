@@ -87,7 +87,8 @@ def test_embedding_backward_one_id_thousands_of_times(dtype):
     again = ops.embedding_bwd(ids.to(DEV), d_out.to(DEV), v_loc, 0, -1)
     torch.cuda.synchronize()
     assert torch.equal(got, again)
-    assert_parity(got, want, dtype, "embedding d_weight with a run of 3000", scale=20 if dtype == torch.float32 else 1)
+    # the longest run sums 3000 rows in fp32
+    assert_parity(got, want, dtype, "embedding d_weight with a run of 3000")
 
 
 def test_vocab_slices_sum_to_the_full_lookup():

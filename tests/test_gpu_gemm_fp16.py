@@ -90,13 +90,16 @@ def test_f16_colsum_and_act_bwd(shape):
     M, N = shape
     dy = randn((M, N), F16, 1)
     got = ops.colsum(dy.to(DEV))
-    assert_parity(got, oracle.colsum(dy), torch.float32, "colsum", scale=100)
+    with oracle.precision(torch.float64):
+        want = oracle.colsum(dy)
+    assert_parity(got, want, torch.float32, "colsum")
     pre = randn((M, N), F16, 3, std=1.5)
     for act in ("gelu_tanh", "relu"):
         dpre, dbias = ops.act_bwd_colsum(act, dy.to(DEV), pre.to(DEV))
-        want_dpre, want_dbias = oracle.act_bwd_colsum(act, dy, pre)
+        with oracle.precision(torch.float64):
+            want_dpre, want_dbias = oracle.act_bwd_colsum(act, dy, pre)
         assert_parity(dpre, want_dpre, F16, "dPre %s" % act)
-        assert_parity(dbias, want_dbias, torch.float32, "dbias %s" % act, scale=200)
+        assert_parity(dbias, want_dbias, torch.float32, "dbias %s" % act)
 
 
 def test_half_model_layernorm():
@@ -123,8 +126,8 @@ def test_half_model_layernorm():
     torch.nn.functional.layer_norm(xr, (768,), wr, br, 1e-5).backward(dy.float())
     assert_parity(y, torch.nn.functional.layer_norm(xr, (768,), wr, br, 1e-5).detach().to(F16), F16, "y")
     assert_parity(x.grad, xr.grad.to(F16), F16, "dx")
-    assert_parity(ln.weight.grad, wr.grad.to(F16), F16, "dgamma", scale=4)
-    assert_parity(ln.bias.grad, br.grad.to(F16), F16, "dbeta", scale=4)
+    assert_parity(ln.weight.grad, wr.grad.to(F16), F16, "dgamma")
+    assert_parity(ln.bias.grad, br.grad.to(F16), F16, "dbeta")
 
 
 @pytest.mark.parametrize("amp_dtype", [torch.float16, torch.bfloat16])

@@ -74,7 +74,7 @@ def test_random_attention(case):
         assert_parity(g.permute(0, 2, 1, 3), torch.cat([dq, dk, dv], dim=-1), torch.bfloat16, "attention grads %s" % (case,))
         return
     for name, got, ref in (("dq", g[..., :d], dq), ("dk", g[..., d:2 * d], dk), ("dv", g[..., 2 * d:], dv)):
-        assert_parity(got.permute(0, 2, 1, 3), ref, torch.bfloat16, "attention %s %s" % (name, case), scale=2)
+        assert_parity(got.permute(0, 2, 1, 3), ref, torch.bfloat16, "attention %s %s" % (name, case))
 
 
 def _ln_cases():
@@ -92,14 +92,15 @@ def test_random_layernorm(shape):
     dy = randn((R, C), torch.bfloat16, R + C + 1)
     gamma = (1 + 0.1 * randn((C,), torch.float32, 3)).to(torch.bfloat16)
     beta = randn((C,), torch.bfloat16, 4, std=0.05)
-    y_ref, mr_ref = oracle.ln_forward_full(x, gamma, beta, 1e-5)
-    dx_ref, dg_ref, db_ref = oracle.ln_backward_full(dy, x, mr_ref, gamma)
+    with oracle.precision(torch.float64):
+        y_ref, mr_ref = oracle.ln_forward_full(x, gamma, beta, 1e-5)
+        dx_ref, dg_ref, db_ref = oracle.ln_backward_full(dy, x, mr_ref, gamma)
     xd, dyd, gd, bd = (t.to(DEV) for t in (x, dy, gamma, beta))
     y, mr = ops.ln_forward_fused(xd, 1e-5, gd, bd)
     rs, dgam, dbet = ops.ln_bwd_partials(dyd, xd, mr, gd)
     dx = ops.ln_bwd_dx(dyd, xd, mr, rs, C, gd)
     torch.cuda.synchronize()
     assert_parity(y, y_ref, torch.bfloat16, "ln y %s" % (shape,))
-    assert_parity(dx, dx_ref, torch.bfloat16, "ln dx %s" % (shape,), scale=2)
-    assert_parity(dgam, dg_ref, torch.float32, "ln dgamma %s" % (shape,), scale=100)
-    assert_parity(dbet, db_ref, torch.float32, "ln dbeta %s" % (shape,), scale=100)
+    assert_parity(dx, dx_ref, torch.bfloat16, "ln dx %s" % (shape,))
+    assert_parity(dgam, dg_ref, torch.float32, "ln dgamma %s" % (shape,))
+    assert_parity(dbet, db_ref, torch.float32, "ln dbeta %s" % (shape,))

@@ -1,7 +1,9 @@
 """GPU parity of the vocab-parallel cross-entropy entry points (through the C
 ABI) against the CPU oracle and against F.cross_entropy on the concatenated
 slices (the reference tests' own oracle, tests/test_1d/check_1d_modules.py:499-523).
-Mask, shifted index and gathered logit must be bit-exact.
+Mask, shifted index, gathered logit and row maximum must be bit-exact. The floating-point
+expected values are evaluated in float64 (oracle.precision), the fp32 results (sum of
+exponentials, loss, fp32 gradient) are held to 1e-5 of the largest expected magnitude.
 """
 import pytest
 import torch
@@ -28,37 +30,39 @@ def _run_all_ranks(T, V, p, dtype, seed, grad_dtype=None, targets=None):
     t = _targets(T, V * p, seed + 1) if targets is None else targets
     slices = list(torch.chunk(full, p, dim=-1))
     stats_got, stats_want = [], []
-    for r, s in enumerate(slices):
-        s_dev = s.contiguous().to(DEV)
-        got = ops.vpce_fwd_local(s_dev, t.to(DEV), r * V)
-        want = oracle.vpce_fwd_local(s, t, r * V)
-        # integer / gather part: bit exact
-        assert torch.equal(got[3].cpu(), want[3]), "mask"
-        assert torch.equal(got[2].cpu(), want[2]), "gathered logit"
-        assert torch.equal(got[0].cpu(), want[0]), "row max"
-        assert_parity(got[1], want[1], torch.float32, "sum exp rank %d" % r, scale=10)
-        stats_got.append(got)
-        stats_want.append(want)
-    stk = lambda lst, k: torch.stack([x[k] for x in lst])  # noqa: E731
-    loss_g, gmax_g, gsum_g = ops.vpce_finalize(*(stk(stats_got, k) for k in range(4)))
-    loss_w, gmax_w, gsum_w = oracle.vpce_finalize(*(stk(stats_want, k) for k in range(4)))
-    assert torch.equal(gmax_g.cpu(), gmax_w)
-    assert_parity(gsum_g, gsum_w, torch.float32, "global sum", scale=10)
-    assert_parity(loss_g, loss_w, torch.float32, "loss", scale=10)
-    # the reference tests' oracle
-    logits_ref = full.float().requires_grad_(True)
-    loss_ref = torch.nn.functional.cross_entropy(logits_ref, t, reduction="none")
-    assert_parity(loss_g, loss_ref.detach(), torch.float32, "loss vs F.cross_entropy", scale=10)
-    dl = torch.linspace(0.5, 1.5, T)
-    loss_ref.backward(dl)
-    gd = grad_dtype or dtype
-    for r, s in enumerate(slices):
-        grad = ops.vpce_bwd(s.contiguous().to(DEV), t.to(DEV), r * V, gmax_g, gsum_g, dl.to(DEV), 1.0, grad_dtype=gd)
-        want = oracle.vpce_bwd(s, t, r * V, gmax_w, gsum_w, dl)
-        assert grad.dtype == gd
-        assert_parity(grad, want, gd, "grad rank %d vs oracle" % r, scale=10 if gd == torch.float32 else 1)
-        ref = logits_ref.grad[:, r * V:(r + 1) * V]
-        assert_parity(grad, ref, gd, "grad rank %d vs autograd" % r, scale=10 if gd == torch.float32 else 1)
+    with oracle.precision(torch.float64):
+        for r, s in enumerate(slices):
+            s_dev = s.contiguous().to(DEV)
+            got = ops.vpce_fwd_local(s_dev, t.to(DEV), r * V)
+            want = oracle.vpce_fwd_local(s, t, r * V)
+            # integer / gather part: bit exact (the values are inputs, exact in either precision)
+            assert torch.equal(got[3].cpu(), want[3]), "mask"
+            assert torch.equal(got[2].cpu(), want[2].float()), "gathered logit"
+            assert torch.equal(got[0].cpu(), want[0].float()), "row max"
+            assert_parity(got[1], want[1], torch.float32, "sum exp rank %d" % r)
+            stats_got.append(got)
+            stats_want.append(want)
+        stk = lambda lst, k: torch.stack([x[k] for x in lst])  # noqa: E731
+        loss_g, gmax_g, gsum_g = ops.vpce_finalize(*(stk(stats_got, k) for k in range(4)))
+        loss_w, gmax_w, gsum_w = oracle.vpce_finalize(*(stk(stats_want, k) for k in range(4)))
+        assert torch.equal(gmax_g.cpu(), gmax_w.float())
+        assert_parity(gsum_g, gsum_w, torch.float32, "global sum")
+        assert_parity(loss_g, loss_w, torch.float32, "loss")
+        # the reference tests' oracle
+        logits_ref = full.double().requires_grad_(True)
+        loss_ref = torch.nn.functional.cross_entropy(logits_ref, t, reduction="none")
+        assert_parity(loss_g, loss_ref.detach(), torch.float32, "loss vs F.cross_entropy")
+        dl = torch.linspace(0.5, 1.5, T)
+        loss_ref.backward(dl.double())
+        gd = grad_dtype or dtype
+        for r, s in enumerate(slices):
+            grad = ops.vpce_bwd(s.contiguous().to(DEV), t.to(DEV), r * V, gmax_g, gsum_g, dl.to(DEV), 1.0, grad_dtype=gd)
+            # the kernel is handed the fp32 statistics of the forward; so is the oracle
+            want = oracle.vpce_bwd(s, t, r * V, gmax_g.cpu(), gsum_g.cpu(), dl)
+            assert grad.dtype == gd
+            assert_parity(grad, want, gd, "grad rank %d vs oracle" % r)
+            ref = logits_ref.grad[:, r * V:(r + 1) * V]
+            assert_parity(grad, ref, gd, "grad rank %d vs autograd" % r)
 
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32, torch.float16])
@@ -97,10 +101,10 @@ def test_loss_under_autocast_keeps_16bit_logits(amp_dtype):
     assert loss.dtype == torch.float32 and logits.grad.dtype == amp_dtype
     # one gradient of the logits' size and per-row statistics: no float32 copy (T * V * 4 bytes) was made
     assert torch.cuda.max_memory_allocated() - before < T * V * 2 + T * V * 4
-    ref_in = logits.detach().float().cpu().requires_grad_(True)
+    ref_in = logits.detach().double().cpu().requires_grad_(True)
     ref = torch.nn.functional.cross_entropy(ref_in, t.cpu())
     ref.backward()
-    assert_parity(loss, ref.detach(), torch.float32, "loss", scale=10)
+    assert_parity(loss, ref.detach(), torch.float32, "loss")
     assert_parity(logits.grad, ref_in.grad, amp_dtype, "logits grad")
 
 
@@ -126,9 +130,10 @@ def test_vpce_does_not_modify_logits_and_handles_padding():
     before = parent.clone()
     t = _targets(T, 2 * V, 6).to(DEV)
     got = ops.vpce_fwd_local(view, t, V)
-    want = oracle.vpce_fwd_local(view.cpu(), t.cpu(), V)
-    assert torch.equal(got[2].cpu(), want[2]) and torch.equal(got[3].cpu(), want[3])
-    assert_parity(got[1], want[1], torch.float32, "sumexp", scale=10)
+    with oracle.precision(torch.float64):
+        want = oracle.vpce_fwd_local(view.cpu(), t.cpu(), V)
+    assert torch.equal(got[2].cpu(), want[2].float()) and torch.equal(got[3].cpu(), want[3])
+    assert_parity(got[1], want[1], torch.float32, "sumexp")
     loss, gmax, gsum = ops.vpce_finalize(*(g.unsqueeze(0) for g in got))
     ops.vpce_bwd(view, t, V, gmax, gsum, None, 0.25)
     torch.cuda.synchronize()
@@ -153,7 +158,7 @@ def test_vpce_baseline_shape_properties():
     rows = torch.arange(0, T, 257, device=DEV)
     full = torch.cat([s[rows] for s in slices], dim=1).float().cpu()
     want = torch.logsumexp(full.double(), dim=1) - full.double()[torch.arange(len(rows)), t[rows].cpu()]
-    assert_parity(loss[rows].cpu().double(), want, torch.float32, "loss on sampled rows", scale=10)
+    assert_parity(loss[rows].cpu().double(), want, torch.float32, "loss on sampled rows")
     dl = 1.0 / T
     total = torch.zeros(T, dtype=torch.float64, device=DEV)
     for r, s in enumerate(slices):
