@@ -13,7 +13,12 @@ of cw_gemm_ksteps through the C ABI = one kernel launch.
 Prints ONE JSON line. `value` is TFLOP/s over the timed region (wall clock
 around K steps, synchronised on both sides). `roofline` prices the GEMM kernel
 against the MI355X dense bf16 MFMA peak with the average launch duration from
-HIP events on the launch stream. `aux` reports the bandwidth-bound kernels of
+HIP events on the launch stream over a SUSTAINED run (--sustained launches back
+to back, 10000 by default, more than a second: a short run finds the board below
+its power limit and the clock high; the figure from the K timed steps is
+reported beside it), together with the shader
+clock and the socket power read from the driver's sysfs files during that run.
+`aux` reports the bandwidth-bound kernels of
 the same path (LayerNorm2D, vocab-parallel CE: the third and fourth configurations)
 against the 8 TB/s HBM peak, on buffers rotated through > 512 MiB so that the
 256 MiB Infinity Cache cannot serve them. `cpu_baseline` times the reference's
@@ -31,6 +36,95 @@ HBM_PEAK_GBPS = 8000.0
 
 M, N, K, STEPS_K = 8192, 2048, 2048, 2
 GEMM_FLOP = 2 * M * N * K * STEPS_K
+
+
+class SmiSampler:
+    """Shader clock and socket power of card 0 from the amdgpu driver's sysfs files, sampled by a thread
+    while the caller runs its timed loop. The driver reports low-pass filtered values (they settle within
+    about a second), so the figures kept are those of the last 40 % of the sampled interval."""
+
+    def __init__(self, period_s=0.002):
+        import glob
+        self.period = period_s
+        dev = "/sys/class/drm/card0/device"
+        hw = sorted(glob.glob(dev + "/hwmon/hwmon*"))
+        self.power_path = hw[0] + "/power1_input" if hw and os.path.exists(hw[0] + "/power1_input") else None
+        self.cap_path = hw[0] + "/power1_cap" if hw and os.path.exists(hw[0] + "/power1_cap") else None
+        self.sclk_path = dev + "/pp_dpm_sclk" if os.path.exists(dev + "/pp_dpm_sclk") else None
+        self.samples = []
+        self._stop = False
+        self._thread = None
+
+    def available(self):
+        return self.power_path is not None and self.sclk_path is not None
+
+    def _read(self):
+        with open(self.power_path) as f:
+            watts = int(f.read()) / 1e6
+        mhz = None
+        with open(self.sclk_path) as f:
+            for line in f:
+                if line.rstrip().endswith("*"):  # the level the shader clock is at now
+                    mhz = float(line.split(":")[1].lower().replace("mhz", "").replace("*", "").strip())
+        return watts, mhz
+
+    def _run(self):
+        while not self._stop:
+            try:
+                w, m = self._read()
+                self.samples.append((time.perf_counter(), w, m))
+            except (OSError, ValueError, IndexError):
+                pass
+            time.sleep(self.period)
+
+    def __enter__(self):
+        if self.available():
+            import threading
+            self._thread = threading.Thread(target=self._run, daemon=True)
+            self._thread.start()
+        self.t0 = time.perf_counter()
+        return self
+
+    def __exit__(self, *exc):
+        self.t1 = time.perf_counter()
+        self._stop = True
+        if self._thread is not None:
+            self._thread.join()
+
+    def summary(self):
+        if not self.samples:
+            return None
+        lo = self.t0 + 0.6 * (self.t1 - self.t0)
+        tail = [s for s in self.samples if lo <= s[0] <= self.t1 and s[2] is not None]
+        if not tail:
+            return None
+        out = {"shader_clock_MHz": round(sum(s[2] for s in tail) / len(tail), 1),
+               "socket_power_W": round(sum(s[1] for s in tail) / len(tail), 1),
+               "samples": len(tail), "source": "sysfs pp_dpm_sclk / hwmon power1_input, last 40% of the run"}
+        if self.cap_path:
+            try:
+                with open(self.cap_path) as f:
+                    out["power_cap_W"] = int(f.read()) / 1e6
+            except (OSError, ValueError):
+                pass
+        return out
+
+
+def sustained_us(fn, launches):
+    """Average duration of fn() over `launches` back-to-back calls (events on the current stream), with the
+    clock and power the driver reports while they run."""
+    import torch
+    for _ in range(20):
+        fn()
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    with SmiSampler() as smi:
+        e0.record()
+        for _ in range(launches):
+            fn()
+        e1.record()
+        torch.cuda.synchronize()
+    return e0.elapsed_time(e1) * 1e3 / launches, smi.summary()
 
 
 def measured_traffic():
@@ -330,66 +424,176 @@ def bench_other_configs(device, sets):
     return out
 
 
+def _gloo_world_of_one():
+    """torch.distributed on gloo with one rank, as cubework/initialize.py:33-35 sets it up. Returns True when
+    the group exists (the raw all_reduce calls of the reference's CPU path then run on it)."""
+    import torch.distributed as dist
+    try:
+        if dist.is_initialized():
+            return True
+        import socket
+        s = socket.socket()
+        s.bind(("127.0.0.1", 0))
+        port = s.getsockname()[1]
+        s.close()
+        # gloo announces its connections on stdout; keep stdout for the one JSON line
+        sys.stdout.flush()
+        saved = os.dup(1)
+        os.dup2(2, 1)
+        try:
+            dist.init_process_group("gloo", init_method="tcp://127.0.0.1:%d" % port, rank=0, world_size=1)
+        finally:
+            sys.stdout.flush()
+            os.dup2(saved, 1)
+            os.close(saved)
+        return True
+    except Exception:  # the baseline still runs; the collectives are identities at world size 1
+        return False
+
+
+def _timed_passes(fn, budget_s, max_iters=300):
+    """One untimed call, one timed call to size the loop, then as many passes as fit the budget."""
+    fn()
+    t0 = time.perf_counter()
+    fn()
+    one = max(time.perf_counter() - t0, 1e-6)
+    iters = max(2, min(max_iters, int(budget_s / one)))
+    t0 = time.perf_counter()
+    for _ in range(iters):
+        fn()
+    return (time.perf_counter() - t0) / iters, iters
+
+
 def cpu_baseline():
-    """The reference's CPU path (torch on gloo, world size 1) for the same
-    workload, through the oracle's restatement of _SUMMA_AB.forward +
-    _SUMMAbias.forward + GeLU in the tensors' own dtype, on a bounded sample
-    of the rows (the k loop and the widths are the full ones)."""
+    """The reference's CPU path (torch on gloo, world size 1) on the GPU host's cores, restated by oracle/:
+    the headline workload (config 2: _SUMMA_AB.forward + _SUMMAbias.forward + GeLU in the tensors' own dtype)
+    and, under "other_configs", config 1 (fp32 F.linear forward + autograd backward), config 3 (LayerNorm2D
+    forward + backward) and config 4 (vocab-parallel cross-entropy forward + backward) with the all-reduce
+    calls the reference makes at world size 1. Each leg runs on a bounded sample: about 5-8 s of CPU work."""
     import torch
     import torch.distributed as dist
     import oracle
+    from oracle import cpu_path
 
-    inited = False
-    try:
-        if not dist.is_initialized():
-            import socket
-            s = socket.socket()
-            s.bind(("127.0.0.1", 0))
-            port = s.getsockname()[1]
-            s.close()
-            # gloo announces its connections on stdout; keep stdout for the one JSON line
-            sys.stdout.flush()
-            saved = os.dup(1)
-            os.dup2(2, 1)
-            try:
-                dist.init_process_group("gloo", init_method="tcp://127.0.0.1:%d" % port, rank=0, world_size=1)
-            finally:
-                sys.stdout.flush()
-                os.dup2(saved, 1)
-                os.close(saved)
-            inited = True
-    except Exception:  # the baseline still runs without the (unused at world size 1) group
-        inited = False
+    group_ok = _gloo_world_of_one()
     threads = torch.get_num_threads()
+    note = "os.cpu_count()=%d, torch threads=%d, gloo world of one %s" % (
+        os.cpu_count(), threads, "initialised" if group_ok else "NOT initialised (collectives skipped)")
 
-    def run(rows, iters):
+    # ---- config 2 (headline)
+    def run2(rows):
         A = [_seeded((rows, K), i, 1.0, torch.bfloat16) for i in range(STEPS_K)]
         B = [_seeded((K, N), 10 + i, 0.02, torch.bfloat16) for i in range(STEPS_K)]
         bias = _seeded((N,), 7, 0.02, torch.bfloat16)
-        f = lambda: torch.nn.functional.gelu(oracle.summa_ab_reference_dtype(A, B, bias), approximate="tanh")  # noqa: E731
-        f()
-        t0 = time.perf_counter()
-        for _ in range(iters):
-            f()
-        return (time.perf_counter() - t0) / iters
-
-    rows = 1024
-    t = run(rows, 1)
-    # grow the sample to the full row count if that stays within ~15 s of CPU work
-    per_row = t / rows
-    if per_row * M * 3 <= 15.0:
-        rows = M
-    else:
-        rows = max(256, min(M, int(15.0 / (3 * per_row)) // 256 * 256))
-    iters = max(2, min(300, int(10.0 / max(per_row * rows, 1e-6))))  # about 10 s of CPU work
-    t = run(rows, iters)
-    if inited:
-        dist.destroy_process_group()
+        return lambda: torch.nn.functional.gelu(oracle.summa_ab_reference_dtype(A, B, bias), approximate="tanh")
+    f = run2(1024)
+    f()
+    t0 = time.perf_counter()
+    f()
+    per_row = (time.perf_counter() - t0) / 1024
+    rows = M if per_row * M * 3 <= 8.0 else max(256, min(M, int(8.0 / (3 * per_row)) // 256 * 256))
+    t, iters = _timed_passes(run2(rows), 6.0)
     flop = 2.0 * rows * N * K * STEPS_K
-    return {"value": round(flop / t / 1e12, 4), "unit": "TFLOP/s", "cores": threads, "kind": "port",
+    head = {"value": round(flop / t / 1e12, 4), "unit": "TFLOP/s", "cores": threads, "kind": "port",
             "sample": "%d of %d rows, full K=%dx%d steps and N=%d, bf16 addmm per k-step + bias + GeLU(tanh) as "
-                      "parallel_2d/_operation.py:41-47,273 runs it on CPU tensors; %d timed passes, %.3f s each; "
-                      "os.cpu_count()=%d" % (rows, M, K, STEPS_K, N, iters, t, os.cpu_count())}
+                      "parallel_2d/_operation.py:41-47,273 runs it on CPU tensors; %d timed passes, %.3f s each; %s"
+                      % (rows, M, K, STEPS_K, N, iters, t, note)}
+    other = {}
+
+    # ---- config 1: Linear1D column-parallel, fp32, seed 0, forward + backward at full size
+    g = torch.Generator().manual_seed(0)
+    x1 = torch.randn((8, 512, 1024), generator=g)
+    w1 = (torch.rand((4096, 1024), generator=g) * 2 - 1) * (6.0 / 5120) ** 0.5   # xavier_uniform_, module/init.py:88-99
+    b1 = torch.zeros(4096)
+    dy1 = torch.randn((8, 512, 4096), generator=g)
+    t, iters = _timed_passes(lambda: cpu_path.linear1d_col_fwd_bwd(x1, w1, b1, dy1), 6.0)
+    flop1 = 3 * 2.0 * 4096 * 1024 * 4096
+    other["config1_linear1d_fp32_fwd_bwd"] = {
+        "value": round(flop1 / t / 1e12, 4), "unit": "TFLOP/s", "cores": threads, "kind": "port",
+        "sample": "full size: x [8,512,1024], W [4096,1024], F.linear forward + autograd backward "
+                  "(parallel_1d/module.py:263-278); %d timed passes, %.3f s each; %s" % (iters, t, note)}
+    del x1, w1, dy1
+
+    # ---- config 3: LayerNorm2D shard, bf16, forward + backward, H = 2048 (the peer's half is not there: the
+    # reference's arithmetic on the local shard is the same, its row sums would be all-reduced)
+    R3, C3 = 16384, 1024
+    x3 = _seeded((R3, C3), 100, 1.0, torch.bfloat16)
+    dy3 = _seeded((R3, C3), 200, 1.0, torch.bfloat16)
+    g3 = (torch.rand(C3, generator=torch.Generator().manual_seed(3)) * 0.2 + 0.9).to(torch.bfloat16)
+    b3 = _seeded((C3,), 4, 0.02, torch.bfloat16)
+    t, iters = _timed_passes(lambda: cpu_path.layernorm2d_fwd_bwd(x3, g3, b3, dy3, 2048, 1e-5, group_ok), 5.0)
+    bytes3 = (2 + 3) * R3 * C3 * 2   # forward reads x writes y; backward reads dy, x writes dx
+    other["config3_layernorm2d_bf16_fwd_bwd"] = {
+        "value": round(bytes3 / t / 1e9, 3), "unit": "GB/s", "cores": threads, "kind": "port",
+        "sample": "%d of 16384 rows x 1024 columns, forward + backward in bf16 as parallel_2d/module.py:142-171 and "
+                  "_operation.py:330-347 run on CPU tensors, the two backward all_reduce calls on the gloo group "
+                  "included; algorithmic bytes 5 x rows x 1024 x 2; %d timed passes, %.3f s each; %s"
+                  % (R3, iters, t, note)}
+    del x3, dy3
+
+    # ---- config 4: vocab-parallel cross-entropy, rank 1 of 4, forward + backward
+    T4, V4 = 8192, 12568
+    lg = _seeded((T4, V4), 300, 2.0, torch.bfloat16)
+    tg = torch.randint(0, 50272, (T4,), generator=torch.Generator().manual_seed(9))
+    dl = torch.full((T4,), 1.0 / 8192)
+    t, iters = _timed_passes(lambda: cpu_path.vpce1d_fwd_bwd(lg, tg, V4, dl, group_ok), 5.0)
+    bytes4 = T4 * V4 * 2 + T4 * V4 * 2 + T4 * V4 * 4   # forward reads the logits; backward reads them, writes fp32 grad
+    other["config4_vocab_parallel_ce_fwd_bwd"] = {
+        "value": round(bytes4 / t / 1e9, 3), "unit": "GB/s", "cores": threads, "kind": "port",
+        "sample": "%d of 8192 tokens x 12568 classes (rank 1 of 4), forward + backward as loss/loss_1d.py:14-79 runs "
+                  "on CPU tensors (fp32 copy of the bf16 logits, in place), the MAX / SUM / SUM all_reduce calls on "
+                  "the gloo group included; algorithmic bytes tokens x 12568 x (2 + 2 + 4); %d timed passes, %.3f s "
+                  "each; %s" % (T4, iters, t, note)}
+    if group_ok and dist.is_initialized():
+        dist.destroy_process_group()
+    head["other_configs"] = other
+    return head
+
+
+def mfma_rate_ceiling(lib, device):
+    """cw_diag_mfma_rate: the GEMM's matrix instruction issued back to back from registers, random operands of
+    the workload's magnitudes and all-zero operands, each for about half a second, with clock and power."""
+    import ctypes
+    import torch
+    iters = 20000
+    flop = lib.cw_diag_mfma_rate_flop(iters)
+    sink = torch.empty(65536, dtype=torch.float32, device=device)
+    stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+    out = {}
+    for name, zeros in (("random_operands", 0), ("zero_operands", 1)):
+        def call():
+            rc = lib.cw_diag_mfma_rate(iters, zeros, sink.data_ptr(), stream)
+            if rc != 0:
+                raise RuntimeError(lib.cw_last_error().decode())
+        us, smi = sustained_us(call, 60)
+        out[name] = {"TFLOPs": round(flop / us / 1e6, 1), "frac_of_peak": round(flop / us / 1e6 / MFMA_BF16_PEAK_TFLOPS, 4)}
+        if smi:
+            out[name].update({k: smi[k] for k in ("shader_clock_MHz", "socket_power_W")})
+    out["note"] = ("register-only loop of v_mfma_f32_32x32x16_bf16 on all 1024 SIMDs: what the board's power management "
+                   "leaves of the data-sheet rate for operands that toggle like the workload's")
+    return out
+
+
+def stream_ceiling(device):
+    """torch's own copy kernel over the sizes of the LayerNorm / cross-entropy workloads (one read and one write of
+    the buffer size), sources rotated through more than 512 MiB, replayed from a HIP graph like the aux figures:
+    what a plain streaming kernel of these sizes reaches on this GPU."""
+    import torch
+    out = {}
+    for mib, nbuf in ((32, 18), (64, 10), (196, 4)):
+        n = mib * (1 << 20) // 2
+        src = [torch.empty(n, device=device, dtype=torch.bfloat16).normal_() for _ in range(nbuf)]
+        dst = [torch.empty_like(src[0]) for _ in range(2)]
+        i = [0]
+
+        def copy():
+            i[0] += 1
+            dst[i[0] % 2].copy_(src[i[0] % nbuf])
+        us = graph_time_us(copy, 2 * nbuf)
+        out["copy_%dMiB" % mib] = {"us": round(us, 2), "bytes": 4 * n, "GBps": round(4 * n / us / 1e3, 1),
+                                   "frac": round(4 * n / us / 1e3 / HBM_PEAK_GBPS, 3)}
+        del src, dst
+    return out
 
 
 def main():
@@ -397,7 +601,15 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--sustained", type=int, default=10000,
+                    help="launches of the sustained run that roofline.achieved is taken from (0 = use the timed steps); "
+                         "the default runs for more than a second, past the window over which the board averages its "
+                         "power, so that clock and power have settled")
     ap.add_argument("--no-aux", action="store_true", help="skip the LayerNorm / CE kernels")
+    ap.add_argument("--stream-ceiling", action="store_true",
+                    help="instead of the benchmark: plain torch reads (max) and copies of 32, 64 and 196 MiB buffers, "
+                         "rotated through more than 512 MiB, for a kernel trace of what streaming kernels of the "
+                         "LayerNorm / cross-entropy sizes reach on this GPU")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run a plain 256 MiB device copy three times (the known-size kernel that hardware "
@@ -439,6 +651,14 @@ def main():
         torch.cuda.synchronize()
         return
 
+    if args.stream_ceiling:
+        print(json.dumps({"stream_ceiling": stream_ceiling(device)}))
+        return
+
+    # The bandwidth-bound kernels of the same path run first: the headline's warm-up and timed steps then find the
+    # chip as a training loop would, busy and at its working clock, not waking up from idle.
+    aux = None if args.no_aux else bench_bandwidth_kernels(device)
+
     n_sets = 3  # 3 x 80 MiB of operands rotate so that no step finds its inputs in the Infinity Cache
     sets, bias = make_gemm_inputs(n_sets, device)
     outs = [torch.empty((M, N), dtype=torch.bfloat16, device=device) for _ in range(n_sets)]
@@ -461,7 +681,12 @@ def main():
     torch.cuda.synchronize()
     t1 = time.perf_counter()
     ms_per_step = (t1 - t0) * 1e3 / args.steps
-    kernel_us = e0.elapsed_time(e1) * 1e3 / args.steps
+    steps_us = e0.elapsed_time(e1) * 1e3 / args.steps
+    # sustained: the same step, back to back for long enough that clock and power have settled
+    smi = None
+    kernel_us = steps_us
+    if args.sustained > 0:
+        kernel_us, smi = sustained_us(step, args.sustained)
     achieved = GEMM_FLOP / kernel_us / 1e6
 
     result = {
@@ -482,8 +707,23 @@ def main():
                    "layout": "NN", "flop_per_step": GEMM_FLOP, "operand_sets_rotated": n_sets, "device_arch": arch},
         "roofline": {"bound": "mfma", "achieved": round(achieved, 2), "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
                      "frac": round(achieved / MFMA_BF16_PEAK_TFLOPS, 4), "traffic": measured_traffic(),
-                     "kernel": "gemm_bf16_dma_kernel<NN, bias+gelu_tanh, 4 stages> (256x256x32 tiles)", "avg_launch_us": round(kernel_us, 2)},
+                     "traffic_source": "profiles/gemm_bf16_dma_kernel_linear2d_q2_counters.txt (committed counter runs of "
+                                       "this script, not measured in this run)",
+                     "kernel": "the launch cw_gemm_ksteps makes for this shape (gemm_bf16_dma_kernel, 256x256 tiles; "
+                               "name as the kernel trace of this command shows it)",
+                     "avg_launch_us": round(kernel_us, 2), "launches": args.sustained if args.sustained > 0 else args.steps,
+                     "timed_steps": {"avg_launch_us": round(steps_us, 2),
+                                     "frac": round(GEMM_FLOP / steps_us / 1e6 / MFMA_BF16_PEAK_TFLOPS, 4),
+                                     "note": "events around the K timed steps only (chip not yet at its sustained clock)"}},
     }
+    if smi is not None:
+        # 4096 matrix instructions of 32 cycles per SIMD and launch: the share of the launch's shader cycles in which
+        # the matrix pipe is busy, at the clock the driver reports
+        cycles = kernel_us * smi["shader_clock_MHz"]
+        smi["mfma_busy_frac"] = round(GEMM_FLOP / (256 * 4 * 1024.0) / cycles, 4) if cycles > 0 else None
+        smi["clock_x_busy_vs_2400MHz"] = round(smi["shader_clock_MHz"] / 2400.0 * smi["mfma_busy_frac"], 4)
+        result["roofline"]["sustained_clock_power"] = smi
+    result["roofline"]["mfma_rate_ceiling"] = mfma_rate_ceiling(lib, device)
     if args.calibrate_copy:
         src = torch.empty(256 << 20, dtype=torch.uint8, device=device).fill_(1)
         dst = torch.empty_like(src)
@@ -491,8 +731,8 @@ def main():
             dst.copy_(src)
         torch.cuda.synchronize()
         del src, dst
-    if not args.no_aux:
-        result["aux"] = bench_bandwidth_kernels(device)
+    if aux is not None:
+        result["aux"] = aux
         result["aux"]["hbm_peak_GBps"] = HBM_PEAK_GBPS
     if not args.no_aux:
         result["other_configs"] = bench_other_configs(device, sets)

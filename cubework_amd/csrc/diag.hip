@@ -1,0 +1,93 @@
+// Measurement aid: the rate at which this GPU sustains the block GEMM's matrix instruction when nothing else
+// is in the way. Every wavefront keeps 4 x 4 accumulator tiles (the register blocking of the ring kernel) and
+// eight operand fragments of seeded random bf16 values in registers and issues v_mfma_f32_32x32x16_bf16 back to
+// back: no global loads, no LDS, no barriers. With `zeros` the fragments are all zero (no switching activity in
+// the multipliers). The result says what the power management of the board leaves of the 2516.6 TFLOP/s that
+// the data sheet quotes at 2.4 GHz, for operands that toggle like the workload's; bench.py reports it beside
+// the GEMM kernel's own rate.
+#include "cw_common.h"
+#include "gemm_bf16_kernel.h"
+
+namespace cw {
+namespace {
+
+using gemm_bf16::bf16x8_t;
+using gemm_bf16::f32x16_t;
+
+__device__ __forceinline__ uint32_t mix(uint32_t x) {
+    x ^= x >> 15;
+    x *= 2246822519u;
+    x ^= x >> 13;
+    x *= 3266489917u;
+    x ^= x >> 16;
+    return x;
+}
+
+// a bf16 pair with the magnitudes of N(0, scale): sum of four uniform 16-bit numbers per value
+__device__ __forceinline__ uint32_t random_bf16_pair(uint32_t seed, float scale) {
+    uint32_t out = 0;
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+        const uint32_t x = mix(seed * 2u + h), y = mix(x + 0x9e3779b9u);
+        const float f = (float)((int)(x & 0xffff) + (int)(x >> 16) + (int)(y & 0xffff) + (int)(y >> 16) - 131070) * (scale / 37837.0f);
+        out |= (__float_as_uint(f) >> 16) << (16 * h);
+    }
+    return out;
+}
+
+__global__ __launch_bounds__(256) void mfma_rate_kernel(int iters, int zeros, float* __restrict__ sink) {
+    const uint32_t gid = blockIdx.x * 256u + threadIdx.x;
+    bf16x8_t a[4], b[4];
+#pragma unroll
+    for (int t = 0; t < 4; ++t) {
+        uint32_t wa[4], wb[4];
+#pragma unroll
+        for (int d = 0; d < 4; ++d) {
+            wa[d] = zeros ? 0u : random_bf16_pair(gid * 64u + t * 8u + d, 1.0f);
+            wb[d] = zeros ? 0u : random_bf16_pair(gid * 64u + 32u + t * 8u + d, 0.02f);
+        }
+        typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+        a[t] = __builtin_bit_cast(bf16x8_t, (u32x4){wa[0], wa[1], wa[2], wa[3]});
+        b[t] = __builtin_bit_cast(bf16x8_t, (u32x4){wb[0], wb[1], wb[2], wb[3]});
+    }
+    f32x16_t acc[4][4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+#pragma unroll
+            for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.0f;
+    for (int it = 0; it < iters; ++it) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+#pragma unroll
+            for (int j = 0; j < 4; ++j) acc[i][j] = gemm_bf16::mfma_32x32x16<bf16_t>(b[j], a[i], acc[i][j]);
+    }
+    float s = 0.0f;
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+#pragma unroll
+            for (int e = 0; e < 16; ++e) s += acc[i][j][e];
+    if (sink != nullptr) sink[gid] = s;  // keeps the products alive
+}
+
+}  // namespace
+}  // namespace cw
+
+using namespace cw;
+
+extern "C" int64_t cw_diag_mfma_rate_flop(int iters) {
+    // 1024 wavefronts x 16 instructions per trip x 32 x 32 x 16 x 2
+    return iters <= 0 ? 0 : (int64_t)iters * 1024 * 16 * 32768;
+}
+
+extern "C" int cw_diag_mfma_rate(int iters, int zeros, float* sink, void* stream) {
+    if (iters <= 0 || iters > (1 << 24)) return fail(CW_ERR_INVALID, "cw_diag_mfma_rate: iters=%d outside [1, 2^24]", iters);
+    if (const int drc = require_gfx950("cw_diag_mfma_rate"); drc != CW_OK) return drc;
+    hipStream_t s = (hipStream_t)stream;
+    // one workgroup of four wavefronts per compute unit, one wavefront per SIMD: 256 x 256 threads
+    hipLaunchKernelGGL(mfma_rate_kernel, dim3(256), dim3(256), 0, s, iters, zeros, sink);
+    return check_launch("mfma_rate_kernel");
+}

@@ -161,3 +161,40 @@ def test_colsum_and_activation_backward():
         g, s = oracle.act_bwd_colsum(kind, dy, pre)
         close(g, p.grad)
         close(s, p.grad.sum(0))
+
+
+def test_cpu_path_restatement_matches_torch_library_routines():
+    """oracle/cpu_path.py (what bench.py times as the reference's CPU path) against the library routines the
+    reference's tests use as their oracle: F.linear, F.layer_norm and F.cross_entropy with autograd."""
+    import torch.nn.functional as F
+    from oracle import cpu_path
+
+    g = torch.Generator().manual_seed(0)
+    x = torch.randn((24, 64), generator=g)
+    w = torch.randn((48, 64), generator=g) * 0.1
+    b = torch.randn((48,), generator=g)
+    dy = torch.randn((24, 48), generator=g)
+    y, dx, dw, db = cpu_path.linear1d_col_fwd_bwd(x, w, b, dy)
+    xr, wr, br = (t.clone().requires_grad_(True) for t in (x, w, b))
+    F.linear(xr, wr, br).backward(dy)
+    assert torch.allclose(y, F.linear(x, w, b)) and torch.allclose(dx, xr.grad) and torch.allclose(dw, wr.grad)
+    assert torch.allclose(db, br.grad)
+    # LayerNorm2D with the whole hidden size on the rank
+    xl = torch.randn((16, 96), generator=g)
+    gamma, beta = torch.rand((96,), generator=g) + 0.5, torch.randn((96,), generator=g)
+    dyl = torch.randn((16, 96), generator=g)
+    y, dx, dgam, dbet = cpu_path.layernorm2d_fwd_bwd(xl, gamma, beta, dyl, 96, 1e-5, False)
+    xr, gr, br = (t.clone().requires_grad_(True) for t in (xl, gamma, beta))
+    ref = F.layer_norm(xr, (96,), gr, br, 1e-5)
+    ref.backward(dyl)
+    for got, want in ((y, ref.detach()), (dx, xr.grad), (dgam, gr.grad), (dbet, br.grad)):
+        assert torch.allclose(got, want, atol=2e-5, rtol=1e-4)
+    # cross-entropy over two vocabulary slices: the slices' losses and gradients assemble F.cross_entropy's
+    logits = torch.randn((12, 40), generator=g) * 2
+    t = torch.randint(0, 40, (12,), generator=g)
+    dl = torch.rand((12,), generator=g) + 0.5
+    lr = logits.clone().requires_grad_(True)
+    ref = F.cross_entropy(lr, t, reduction="none")
+    ref.backward(dl)
+    loss, grad = cpu_path.vpce1d_fwd_bwd(logits, t, 0, dl, False)   # one slice holding the whole vocabulary
+    assert torch.allclose(loss, ref.detach(), atol=1e-5) and torch.allclose(grad, lr.grad, atol=1e-6)
