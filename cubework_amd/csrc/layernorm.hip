@@ -185,6 +185,8 @@ struct RowTile {
     static constexpr int V = elem<T>::kVec;
     raw16_t raw[NR][NCH];
 
+    // EXACT: the row is exactly NCH chunks wide, so no chunk needs a bounds check.
+    template <bool EXACT = false>
     __device__ __forceinline__ void load(const T* __restrict__ p, int64_t ld, int64_t row0, int64_t R, int64_t C,
                                          int lane) {
 #pragma unroll
@@ -192,6 +194,10 @@ struct RowTile {
             const int64_t row = (row0 + r < R) ? row0 + r : R - 1;
 #pragma unroll
             for (int j = 0; j < NCH; ++j) {
+                if constexpr (EXACT) {
+                    raw[r][j] = load_raw_stream(p + row * ld + ((int64_t)j * 64 + lane) * V);
+                    continue;
+                }
                 const bool ok = chunk_valid<T>(j, lane, C);
                 const int64_t c0 = ok ? ((int64_t)j * 64 + lane) * V : 0;
                 const raw16_t u = load_raw_stream(p + row * ld + c0);
@@ -251,7 +257,12 @@ __device__ __forceinline__ void tile_moments(const RowTile<T, NCH, NR>& t, int r
     s2 = wave_sum(a2);
 }
 
-template <typename T, int NCH, int NR>
+// EXACT (here and in the two kernels below): rows of exactly NCH chunks, and a grid with one tile per
+// wavefront, so a wavefront issues all its loads, works and exits: no trip loop, no per-chunk bounds
+// checks. On 16384 x 1024 bf16 that is the difference between 0.58 and 0.71 of the HBM peak for the
+// normalise kernel; wavefronts that loop read measurably slower at these sizes, however the loop is
+// pipelined.
+template <typename T, int NCH, int NR, bool EXACT>
 __global__ __launch_bounds__(kTileWaves * 64) void ln_stats_tile_kernel(int64_t R, int64_t C,
                                                                         const T* __restrict__ x, int64_t ld, int mode,
                                                                         const float* __restrict__ mean,
@@ -260,24 +271,46 @@ __global__ __launch_bounds__(kTileWaves * 64) void ln_stats_tile_kernel(int64_t 
     const int64_t wave = (int64_t)blockIdx.x * kTileWaves + (threadIdx.x >> 6);
     const int64_t step = (int64_t)gridDim.x * kTileWaves * NR;
     const bool centred = mode == CW_LN_TWO_PASS && mean != nullptr;
+    if constexpr (EXACT) {
+        // plain sums (the one-pass statistics and the first exchange of the two-pass flavour): no mean to fetch
+        if (!centred) {
+            const int64_t row0 = wave * NR;
+            if (row0 >= R) return;
+            RowTile<T, NCH, NR> t;
+            t.template load<true>(x, ld, row0, R, C, lane);
+#pragma unroll
+            for (int r = 0; r < NR; ++r) {
+                float s1, s2;
+                tile_moments(t, r, (int64_t)NCH * 64 * elem<T>::kVec, 0.0f, lane, s1, s2);
+                if (lane == 0 && row0 + r < R) {
+                    typedef float f32x2_t __attribute__((ext_vector_type(2)));
+                    const f32x2_t pair = {s1, mode == CW_LN_TWO_PASS ? 0.0f : s2};
+                    *reinterpret_cast<f32x2_t*>(stats + 2 * (row0 + r)) = pair;
+                }
+            }
+            return;
+        }
+    }
     for (int64_t row0 = wave * NR; row0 < R; row0 += step) {
         RowTile<T, NCH, NR> t;
-        t.load(x, ld, row0, R, C, lane);
+        t.template load<EXACT>(x, ld, row0, R, C, lane);
 #pragma unroll
         for (int r = 0; r < NR; ++r) {
             const int64_t row = row0 + r;
             const float mu = centred ? mean[row < R ? row : R - 1] : 0.0f;
             float s1, s2;
-            tile_moments(t, r, C, mu, lane, s1, s2);
+            tile_moments(t, r, EXACT ? (int64_t)NCH * 64 * elem<T>::kVec : C, mu, lane, s1, s2);
             if (lane == 0 && row < R) {
-                stats[2 * row] = s1;
-                stats[2 * row + 1] = (mode == CW_LN_TWO_PASS && mean == nullptr) ? 0.0f : s2;
+                typedef float f32x2_t __attribute__((ext_vector_type(2)));
+                const f32x2_t pair = {s1, (mode == CW_LN_TWO_PASS && mean == nullptr) ? 0.0f : s2};
+                *reinterpret_cast<f32x2_t*>(stats + 2 * row) = pair;  // one 8-byte store
             }
         }
+        if constexpr (EXACT) return;  // the grid has a tile for every wavefront
     }
 }
 
-template <typename T, int NCH, int NR, bool FUSED>
+template <typename T, int NCH, int NR, bool FUSED, bool EXACT>
 __global__ __launch_bounds__(kTileWaves * 64) void ln_normalize_tile_kernel(
     int64_t R, int64_t C, const T* __restrict__ x, int64_t ld, const float* __restrict__ stats, int mode, float inv_h,
     float eps, const T* __restrict__ gamma, const T* __restrict__ beta, T* __restrict__ y, int64_t ldy,
@@ -291,13 +324,18 @@ __global__ __launch_bounds__(kTileWaves * 64) void ln_normalize_tile_kernel(
     constexpr bool kHoldParams = !(sizeof(T) == 4 && NCH * NR >= 8);
     constexpr int NP = kHoldParams ? NCH : 1;
     raw16_t g_raw[NP], b_raw[NP];
-    if constexpr (kHoldParams) {
+    if constexpr (kHoldParams && !EXACT) {
         load_param_chunks<T, NCH>(gamma, C, lane, g_raw);
         load_param_chunks<T, NCH>(beta, C, lane, b_raw);
     }
+    if constexpr (EXACT) C = (int64_t)NCH * 64 * V;  // a compile-time width: chunk_valid() folds to true
     for (int64_t row0 = wave * NR; row0 < R; row0 += step) {
         RowTile<T, NCH, NR> t;
-        t.load(x, ld, row0, R, C, lane);
+        t.template load<EXACT>(x, ld, row0, R, C, lane);
+        if constexpr (kHoldParams && EXACT) {  // behind the row loads: the rows are what the wavefront waits for
+            load_param_chunks<T, NCH>(gamma, C, lane, g_raw);
+            load_param_chunks<T, NCH>(beta, C, lane, b_raw);
+        }
 #pragma unroll
         for (int r = 0; r < NR; ++r) {
             const int64_t row = row0 + r;
@@ -346,6 +384,7 @@ __global__ __launch_bounds__(kTileWaves * 64) void ln_normalize_tile_kernel(
                     store_raw_stream(y + row * ldy + ((int64_t)j * 64 + lane) * V, pack_raw(v, (const T*)nullptr));
             }
         }
+        if constexpr (EXACT) return;
     }
 }
 
@@ -484,7 +523,7 @@ __global__ __launch_bounds__(MAXW * 64) void ln_forward_split_kernel(
     }
 }
 
-template <typename T, int NCH, int NR>
+template <typename T, int NCH, int NR, bool EXACT>
 __global__ __launch_bounds__(kTileWaves * 64) void ln_bwd_dx_tile_kernel(
     int64_t R, int64_t C, const T* __restrict__ dY, int64_t ld_dy, const T* __restrict__ x, int64_t ld_x,
     const float* __restrict__ mean_rstd, const T* __restrict__ gamma, const float* __restrict__ row_sums, float inv_h,
@@ -494,11 +533,13 @@ __global__ __launch_bounds__(kTileWaves * 64) void ln_bwd_dx_tile_kernel(
     const int64_t wave = (int64_t)blockIdx.x * kTileWaves + (threadIdx.x >> 6);
     const int64_t step = (int64_t)gridDim.x * kTileWaves * NR;
     raw16_t g_raw[NCH];
-    load_param_chunks<T, NCH>(gamma, C, lane, g_raw);
+    if constexpr (!EXACT) load_param_chunks<T, NCH>(gamma, C, lane, g_raw);
+    if constexpr (EXACT) C = (int64_t)NCH * 64 * V;
     for (int64_t row0 = wave * NR; row0 < R; row0 += step) {
         RowTile<T, NCH, NR> tdy, tx;
-        tdy.load(dY, ld_dy, row0, R, C, lane);
-        tx.load(x, ld_x, row0, R, C, lane);
+        tdy.template load<EXACT>(dY, ld_dy, row0, R, C, lane);
+        tx.template load<EXACT>(x, ld_x, row0, R, C, lane);
+        if constexpr (EXACT) load_param_chunks<T, NCH>(gamma, C, lane, g_raw);
 #pragma unroll
         for (int r = 0; r < NR; ++r) {
             const int64_t row = row0 + r;
@@ -521,6 +562,7 @@ __global__ __launch_bounds__(kTileWaves * 64) void ln_bwd_dx_tile_kernel(
                     store_raw_stream(dx + row * ld_dx + ((int64_t)j * 64 + lane) * V, pack_raw(dy, (const T*)nullptr));
             }
         }
+        if constexpr (EXACT) return;
     }
 }
 
@@ -537,6 +579,29 @@ int dispatch_tile(int64_t nch, F&& f) {
     if (nch <= 2) return f(std::integral_constant<int, 2>{}, std::integral_constant<int, kRowsAt2Chunks>{});
     if (nch <= 4) return f(std::integral_constant<int, 4>{}, std::integral_constant<int, kRowsAt4Chunks>{});
     return f(std::integral_constant<int, 8>{}, std::integral_constant<int, 1>{});
+}
+
+// Calls f(NCH, NR) for rows of exactly `nch` (1, 2, 4 or 8) chunks with NR = max(1, LOADS / NCH) rows per
+// wavefront, LOADS being the 16-byte loads per lane and operand that the kernel wants in flight (measured
+// on 16384 x 1024 bf16, one tile per wavefront: 4 for the statistics, 8 for normalise, 2 for each of dx's
+// two operands).
+template <int LOADS, typename F>
+int dispatch_exact(int64_t nch, F&& f) {
+    if (nch == 1) return f(std::integral_constant<int, 1>{}, std::integral_constant<int, (LOADS >= 4 ? 4 : LOADS)>{});
+    if (nch == 2) return f(std::integral_constant<int, 2>{}, std::integral_constant<int, (LOADS / 2 >= 1 ? LOADS / 2 : 1)>{});
+    if (nch == 4) return f(std::integral_constant<int, 4>{}, std::integral_constant<int, (LOADS / 4 >= 1 ? LOADS / 4 : 1)>{});
+    return f(std::integral_constant<int, 8>{}, std::integral_constant<int, 1>{});
+}
+
+template <typename T>
+bool exact_chunks(int64_t C, int64_t nch) {
+    return (nch == 1 || nch == 2 || nch == 4 || nch == 8) && C == nch * 64 * elem<T>::kVec;
+}
+
+// One tile of nr rows per wavefront.
+int exact_grid(int64_t R, int nr) {
+    const int64_t rows_per_block = (int64_t)kTileWaves * nr;
+    return (int)((R + rows_per_block - 1) / rows_per_block);
 }
 
 int tile_grid(int64_t R, int nr) {
@@ -575,8 +640,7 @@ __global__ __launch_bounds__(NWAVES * 64) void ln_bwd_partials_kernel(
         tx.load(x, ld_x, row0, R, C, lane);
         tdy.zero_dead_rows(row0, R);  // a zero dY row adds nothing to the column sums
 #pragma unroll
-        for (int r = 0; r < NR; ++r) {
-            const int64_t row = row0 + r;
+        for (int r = 0; r < NR; ++r) {            const int64_t row = row0 + r;
             const int64_t row_c = row < R ? row : R - 1;
             const float mean = mean_rstd[2 * row_c];
             const float rstd = mean_rstd[2 * row_c + 1];
@@ -922,11 +986,19 @@ int stats_impl(int64_t R, int64_t C, const void* x, int64_t ld, int mode, const 
                hipStream_t s) {
     const int vec_ok = rows_vec_ok<T>(x, ld);
     const int64_t nch = row_chunks<T>(C);
+    if (vec_ok && exact_chunks<T>(C, nch) && R <= (int64_t)1 << 30) {
+        return dispatch_exact<4>(nch, [&](auto nch_c, auto nr_c) {
+            constexpr int NCH = decltype(nch_c)::value, NR = decltype(nr_c)::value;
+            hipLaunchKernelGGL((ln_stats_tile_kernel<T, NCH, NR, true>), dim3(exact_grid(R, NR)), dim3(kTileWaves * 64),
+                               0, s, R, C, (const T*)x, ld, mode, mean, stats);
+            return check_launch("ln_stats_tile_kernel");
+        });
+    }
     if (vec_ok && (C % elem<T>::kVec) == 0 && nch <= 8) {
         return dispatch_tile(nch, [&](auto nch_c, auto nr_c) {
             constexpr int NCH = decltype(nch_c)::value, NR = decltype(nr_c)::value;
-            hipLaunchKernelGGL((ln_stats_tile_kernel<T, NCH, NR>), dim3(tile_grid(R, NR)), dim3(kTileWaves * 64), 0,
-                               s, R, C, (const T*)x, ld, mode, mean, stats);
+            hipLaunchKernelGGL((ln_stats_tile_kernel<T, NCH, NR, false>), dim3(tile_grid(R, NR)), dim3(kTileWaves * 64),
+                               0, s, R, C, (const T*)x, ld, mode, mean, stats);
             return check_launch("ln_stats_tile_kernel");
         });
     }
@@ -953,10 +1025,19 @@ int normalize_impl(int64_t R, int64_t C, const void* x, int64_t ld, const float*
     const int vec_ok = rows_vec_ok<T>(x, ld) && rows_vec_ok<T>(y, ldy) && (gamma == nullptr || aligned16(gamma)) &&
                        (beta == nullptr || aligned16(beta));
     const int64_t nch = row_chunks<T>(C);
+    if (vec_ok && exact_chunks<T>(C, nch) && R <= (int64_t)1 << 30) {
+        return dispatch_exact<8>(nch, [&](auto nch_c, auto nr_c) {
+            constexpr int NCH = decltype(nch_c)::value, NR = decltype(nr_c)::value;
+            hipLaunchKernelGGL((ln_normalize_tile_kernel<T, NCH, NR, FUSED, true>), dim3(exact_grid(R, NR)),
+                               dim3(kTileWaves * 64), 0, s, R, C, (const T*)x, ld, stats, mode, 1.0f / (float)H, eps,
+                               (const T*)gamma, (const T*)beta, (T*)y, ldy, mean_rstd);
+            return check_launch("ln_normalize_tile_kernel");
+        });
+    }
     if (vec_ok && (C % elem<T>::kVec) == 0 && nch <= 8) {
         return dispatch_tile(nch, [&](auto nch_c, auto nr_c) {
             constexpr int NCH = decltype(nch_c)::value, NR = decltype(nr_c)::value;
-            hipLaunchKernelGGL((ln_normalize_tile_kernel<T, NCH, NR, FUSED>), dim3(tile_grid(R, NR)),
+            hipLaunchKernelGGL((ln_normalize_tile_kernel<T, NCH, NR, FUSED, false>), dim3(tile_grid(R, NR)),
                                dim3(kTileWaves * 64), 0, s, R, C, (const T*)x, ld, stats, mode, 1.0f / (float)H, eps,
                                (const T*)gamma, (const T*)beta, (T*)y, ldy, mean_rstd);
             return check_launch("ln_normalize_tile_kernel");
@@ -1160,11 +1241,20 @@ int bwd_dx_impl(int64_t R, int64_t C, const void* dY, int64_t ld_dy, const void*
                        (gamma == nullptr || aligned16(gamma));
     const int64_t nch = row_chunks<T>(C);
     // rows of more than 4 chunks are faster on the looping kernel (the 8-chunk tile needs 160-240 registers)
+    if (vec_ok && exact_chunks<T>(C, nch) && nch <= 4 && R <= (int64_t)1 << 30) {
+        return dispatch_exact<2>(nch, [&](auto nch_c, auto nr_c) {
+            constexpr int NCH = decltype(nch_c)::value, NR = decltype(nr_c)::value;
+            hipLaunchKernelGGL((ln_bwd_dx_tile_kernel<T, NCH, NR, true>), dim3(exact_grid(R, NR)), dim3(kTileWaves * 64),
+                               0, s, R, C, (const T*)dY, ld_dy, (const T*)x, ld_x, mean_rstd, (const T*)gamma, row_sums,
+                               1.0f / (float)H, (T*)dx, ld_dx);
+            return check_launch("ln_bwd_dx_tile_kernel");
+        });
+    }
     if (vec_ok && (C % elem<T>::kVec) == 0 && nch <= 4) {
         return dispatch_tile(nch, [&](auto nch_c, auto nr_c) {
             constexpr int NCH = decltype(nch_c)::value, NR = decltype(nr_c)::value;
-            hipLaunchKernelGGL((ln_bwd_dx_tile_kernel<T, NCH, NR>), dim3(tile_grid(R, NR)), dim3(kTileWaves * 64), 0,
-                               s, R, C, (const T*)dY, ld_dy, (const T*)x, ld_x, mean_rstd, (const T*)gamma, row_sums,
+            hipLaunchKernelGGL((ln_bwd_dx_tile_kernel<T, NCH, NR, false>), dim3(tile_grid(R, NR)), dim3(kTileWaves * 64),
+                               0, s, R, C, (const T*)dY, ld_dy, (const T*)x, ld_x, mean_rstd, (const T*)gamma, row_sums,
                                1.0f / (float)H, (T*)dx, ld_dx);
             return check_launch("ln_bwd_dx_tile_kernel");
         });
