@@ -14,7 +14,9 @@ namespace {
 
 constexpr int kCeBlock = 256;
 constexpr int kCeUnroll = 3;     // 16-byte loads in flight per thread, forward
-constexpr int kCeBwdUnroll = 6;  // backward (no dependent chain between the vectors)
+// Backward: one block of 16 wavefronts per row, every thread's share of the row requested at once. Measured on
+// 8192 x 12568 bf16 -> fp32 (8-byte loads, 16-byte stores): 256 threads per row 118 us, 512: 116, 1024: 107.
+constexpr int kCeBwdBlock = 1024;
 constexpr float kNegInf = -__builtin_huge_valf();
 
 // Running (max m, sum s of exp(x - m)) kept in the exp2 domain: m2 = m*log2(e).
@@ -230,74 +232,113 @@ __device__ __forceinline__ void grad_quad(raw8_t raw, int64_t i, int64_t tcol, f
     store_raw_stream(gr + i * 4, pack_raw(v, (const float*)nullptr));
 }
 
+// Per-row scalars of the backward: fetched after the row's first loads have been issued.
+struct CeRowScalars {
+    float m2, dl, scale;
+    int64_t tcol;
+};
+__device__ __forceinline__ CeRowScalars ce_row_scalars(int64_t row, int64_t V_cols, const int64_t* __restrict__ targets,
+                                                       int64_t vocab_start, const float* __restrict__ gmax,
+                                                       const float* __restrict__ gsum,
+                                                       const float* __restrict__ dloss_rows, float dloss_scale) {
+    CeRowScalars r;
+    r.m2 = gmax[row] * kLog2e;
+    r.dl = (dloss_rows != nullptr ? dloss_rows[row] : 1.0f) * dloss_scale;
+    r.scale = r.dl / gsum[row];
+    const int64_t t = targets[row];
+    const bool masked = (t < vocab_start) || (t >= vocab_start + V_cols);
+    r.tcol = masked ? -1 : (t - vocab_start);
+    return r;
+}
+
 template <typename T, typename G>
-__global__ __launch_bounds__(kCeBlock) void vpce_bwd_kernel(int64_t T_rows, int64_t V_cols,
-                                                            const T* __restrict__ logits, int64_t ld,
-                                                            const int64_t* __restrict__ targets, int64_t vocab_start,
-                                                            const float* __restrict__ gmax,
-                                                            const float* __restrict__ gsum,
-                                                            const float* __restrict__ dloss_rows, float dloss_scale,
-                                                            G* __restrict__ grad, int64_t ld_grad, int vec_ok) {
+__global__ __launch_bounds__(kCeBwdBlock) void vpce_bwd_kernel(int64_t T_rows, int64_t V_cols,
+                                                               const T* __restrict__ logits, int64_t ld,
+                                                               const int64_t* __restrict__ targets, int64_t vocab_start,
+                                                               const float* __restrict__ gmax,
+                                                               const float* __restrict__ gsum,
+                                                               const float* __restrict__ dloss_rows, float dloss_scale,
+                                                               G* __restrict__ grad, int64_t ld_grad, int vec_ok) {
     constexpr int V = elem<T>::kVec;
+    constexpr int B = kCeBwdBlock;
     const int tid = threadIdx.x;
     for (int64_t row = blockIdx.x; row < T_rows; row += gridDim.x) {
         const T* xr = logits + row * ld;
         G* gr = grad + row * ld_grad;
-        const float m2 = gmax[row] * kLog2e;
-        const float dl = (dloss_rows != nullptr ? dloss_rows[row] : 1.0f) * dloss_scale;
-        const float scale = dl / gsum[row];
-        const int64_t t = targets[row];
-        const bool masked = (t < vocab_start) || (t >= vocab_start + V_cols);
-        const int64_t tcol = masked ? -1 : (t - vocab_start);
-        bool done = false;
         if constexpr (sizeof(T) == 2 && std::is_same<G, float>::value) {
           if (vec_ok) {
-            done = true;
-            constexpr int U = 2 * kCeBwdUnroll;
+            // fp32 gradient of 16-bit logits: batches of U quads (8 bytes in, 16 out) per thread, all requested
+            // before the first is worked on; a position past the end of the row re-reads the last quad (no
+            // load under a branch) and stores nothing
+            constexpr int U = 4;
             const int64_t nq = V_cols / 4;
             const uint16_t* xb = reinterpret_cast<const uint16_t*>(xr);
             float* gf = reinterpret_cast<float*>(gr);
-            int64_t i = tid;
-            for (; i + (U - 1) * kCeBlock < nq; i += U * kCeBlock) {
+            CeRowScalars rs;
+            for (int64_t base = tid; base < nq; base += (int64_t)U * B) {
                 raw8_t raw[U];
 #pragma unroll
-                for (int u = 0; u < U; ++u)
-                    raw[u] = __builtin_nontemporal_load(reinterpret_cast<const raw8_t*>(xb + (i + u * kCeBlock) * 4));
+                for (int u = 0; u < U; ++u) {
+                    const int64_t i = base + (int64_t)u * B;
+                    raw[u] = __builtin_nontemporal_load(reinterpret_cast<const raw8_t*>(xb + (i < nq ? i : nq - 1) * 4));
+                }
+                if (base == tid) rs = ce_row_scalars(row, V_cols, targets, vocab_start, gmax, gsum, dloss_rows, dloss_scale);
 #pragma unroll
-                for (int u = 0; u < U; ++u) grad_quad<T>(raw[u], i + u * kCeBlock, tcol, m2, scale, dl, gf);
+                for (int u = 0; u < U; ++u) {
+                    const int64_t i = base + (int64_t)u * B;
+                    if (i < nq) grad_quad<T>(raw[u], i, rs.tcol, rs.m2, rs.scale, rs.dl, gf);
+                }
             }
-            for (; i < nq; i += kCeBlock)
-                grad_quad<T>(__builtin_nontemporal_load(reinterpret_cast<const raw8_t*>(xb + i * 4)), i, tcol, m2, scale, dl, gf);
-            for (int64_t c = nq * 4 + tid; c < V_cols; c += kCeBlock) {
-                float y = __builtin_amdgcn_exp2f(__builtin_fmaf(load_elem(xr + c), kLog2e, -m2)) * scale;
-                if (c == tcol) y -= dl;
-                store_elem(gr + c, y);
+            if (nq * 4 < V_cols) {
+                rs = ce_row_scalars(row, V_cols, targets, vocab_start, gmax, gsum, dloss_rows, dloss_scale);
+                for (int64_t c = nq * 4 + tid; c < V_cols; c += B) {
+                    float y = __builtin_amdgcn_exp2f(__builtin_fmaf(load_elem(xr + c), kLog2e, -rs.m2)) * rs.scale;
+                    if (c == rs.tcol) y -= rs.dl;
+                    store_elem(gr + c, y);
+                }
             }
+            continue;
           }
         }
-        if (done) continue;
         if (vec_ok) {
             const int64_t nvec = V_cols / V;
-            int64_t i = tid;
-            for (; i + (kCeBwdUnroll - 1) * kCeBlock < nvec; i += kCeBwdUnroll * kCeBlock) {
-                raw16_t raw[kCeBwdUnroll];
+            CeRowScalars rs;
+            if constexpr (sizeof(T) == 2) {
+                // 16-bit in, 16-bit out: one vector per thread and trip. Sixteen wavefronts per row and two rows
+                // per compute unit keep enough loads in flight; batching loads per thread measured slower here.
+                rs = ce_row_scalars(row, V_cols, targets, vocab_start, gmax, gsum, dloss_rows, dloss_scale);
+                for (int64_t i = tid; i < nvec; i += B)
+                    grad_vector<T, G, V>(load_raw_stream(xr + i * V), i, rs.tcol, rs.m2, rs.scale, rs.dl, gr);
+            } else {
+                constexpr int U = 4;  // 16-byte vectors per thread and batch
+                for (int64_t base = tid; base < nvec; base += (int64_t)U * B) {
+                    raw16_t raw[U];
 #pragma unroll
-                for (int u = 0; u < kCeBwdUnroll; ++u) raw[u] = load_raw_stream(xr + (i + u * kCeBlock) * V);
+                    for (int u = 0; u < U; ++u) {
+                        const int64_t i = base + (int64_t)u * B;
+                        raw[u] = load_raw_stream(xr + (i < nvec ? i : nvec - 1) * V);
+                    }
+                    if (base == tid) rs = ce_row_scalars(row, V_cols, targets, vocab_start, gmax, gsum, dloss_rows, dloss_scale);
 #pragma unroll
-                for (int u = 0; u < kCeBwdUnroll; ++u)
-                    grad_vector<T, G, V>(raw[u], i + u * kCeBlock, tcol, m2, scale, dl, gr);
+                    for (int u = 0; u < U; ++u) {
+                        const int64_t i = base + (int64_t)u * B;
+                        if (i < nvec) grad_vector<T, G, V>(raw[u], i, rs.tcol, rs.m2, rs.scale, rs.dl, gr);
+                    }
+                }
             }
-            for (; i < nvec; i += kCeBlock)
-                grad_vector<T, G, V>(load_raw_stream(xr + i * V), i, tcol, m2, scale, dl, gr);
-            for (int64_t c = nvec * V + tid; c < V_cols; c += kCeBlock) {
-                float y = __builtin_amdgcn_exp2f(__builtin_fmaf(load_elem(xr + c), kLog2e, -m2)) * scale;
-                if (c == tcol) y -= dl;
-                store_elem(gr + c, y);
+            if (nvec * V < V_cols) {
+                rs = ce_row_scalars(row, V_cols, targets, vocab_start, gmax, gsum, dloss_rows, dloss_scale);
+                for (int64_t c = nvec * V + tid; c < V_cols; c += B) {
+                    float y = __builtin_amdgcn_exp2f(__builtin_fmaf(load_elem(xr + c), kLog2e, -rs.m2)) * rs.scale;
+                    if (c == rs.tcol) y -= rs.dl;
+                    store_elem(gr + c, y);
+                }
             }
         } else {
-            for (int64_t c = tid; c < V_cols; c += kCeBlock) {
-                float y = __builtin_amdgcn_exp2f(__builtin_fmaf(load_elem(xr + c), kLog2e, -m2)) * scale;
-                if (c == tcol) y -= dl;
+            const CeRowScalars rs = ce_row_scalars(row, V_cols, targets, vocab_start, gmax, gsum, dloss_rows, dloss_scale);
+            for (int64_t c = tid; c < V_cols; c += B) {
+                float y = __builtin_amdgcn_exp2f(__builtin_fmaf(load_elem(xr + c), kLog2e, -rs.m2)) * rs.scale;
+                if (c == rs.tcol) y -= rs.dl;
                 store_elem(gr + c, y);
             }
         }
@@ -315,7 +356,7 @@ int bwd_impl(int64_t T_rows, int64_t V_cols, const void* logits, int64_t ld, con
              void* grad, int64_t ld_grad, hipStream_t s) {
     const int vec_ok = aligned16(logits) && (ld % elem<T>::kVec) == 0 && aligned16(grad) &&
                        (ld_grad % (16 / (int)sizeof(G))) == 0;
-    hipLaunchKernelGGL((vpce_bwd_kernel<T, G>), dim3(ce_grid(T_rows)), dim3(kCeBlock), 0, s, T_rows, V_cols,
+    hipLaunchKernelGGL((vpce_bwd_kernel<T, G>), dim3(ce_grid(T_rows)), dim3(kCeBwdBlock), 0, s, T_rows, V_cols,
                        (const T*)logits, ld, targets, vocab_start, gmax, gsum, dloss_rows, dloss_scale, (G*)grad,
                        ld_grad, vec_ok);
     return check_launch("vpce_bwd_kernel");
