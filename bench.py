@@ -376,7 +376,7 @@ def bench_other_configs(device, sets):
     nbytes = 3 * e_tok * 8 + live * e_dim * 2 + e_vloc * e_dim * 2
     out["vocab_embedding_bwd"] = {"us": round(us, 2), "GBps": round(nbytes / us / 1e3, 1), "bytes": nbytes,
                                   "frac": round(nbytes / us / 1e3 / HBM_PEAK_GBPS, 3),
-                                  "note": "three launches: token order (cw_embed_sort_ids), zero fill, per-row sums"}
+                                  "note": "two launches: token order (cw_embed_sort_ids), then per-row sums and zeros for the rows without tokens"}
     del tabs, dys_e
     # attention core of config 5: batch 4, 32 heads of 64, 2048 tokens, causal; FLOP counted on the
     # unmasked half only (4 b h s^2 d / 2 forward, 2.5 x that backward)

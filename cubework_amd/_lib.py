@@ -43,6 +43,8 @@ SIGNATURES = {
     "cw_embed_sort_workspace_bytes": (_i64, [_i64]),
     "cw_embed_sort_ids": (_int, [_i64, _ptr, _i64, _i64, _ptr, _ptr, _ptr, _i64, _ptr]),
     "cw_embed_bwd": (_int, [_i64, _i64, _ptr, _ptr, _i64, _i64, _i64, _ptr, _i64, _ptr, _i64, _int, _ptr]),
+    "cw_embed_bwd_ids_supported": (_int, [_i64, _i64, _ptr, _i64, _ptr, _i64, _int]),
+    "cw_embed_bwd_ids": (_int, [_i64, _i64, _ptr, _i64, _i64, _i64, _ptr, _i64, _ptr, _i64, _int, _ptr]),
     "cw_attn_fwd": (_int, [_i64, _i64, _i64, _i64, _ptr, _ptr, _ptr, _i64, _i64, _i64, _f32, _int, _ptr, _i64, _i64, _i64,
                            _ptr, _int, _ptr]),
     "cw_attn_bwd_workspace_bytes": (_i64, [_i64, _i64, _i64]),

@@ -47,14 +47,46 @@ __global__ __launch_bounds__(kEmbWaves * 64) void embed_fwd_kernel(int64_t T_row
     }
 }
 
+// Rows of the gradient that no token selects are written as zeros by the same launch that sums the others:
+// the first `zero_blocks` workgroups of the backward grid. A wavefront takes kZeroRows consecutive rows, sixteen
+// lanes per row; each group of sixteen finds its row's first position in the sorted ids with a 16-ary search
+// (probes of one step side by side, 4 dependent loads for 8192 tokens, any run lengths), and the rows that are
+// absent (or are skip_row, which the summing blocks leave alone) are then cleared by the whole wavefront.
+// Summing blocks write every column of a present row, so each row of the slice is written exactly once.
+constexpr int kZeroGroup = 16;
+constexpr int kZeroRows = 64 / kZeroGroup;
+
 template <typename T>
-__global__ __launch_bounds__(256) void zero_rows_kernel(int64_t R, int64_t E, T* __restrict__ p, int64_t ld, int vec_ok) {
+__device__ __forceinline__ void zero_absent_rows(int64_t wave_global, int lane, int T_rows, int64_t E,
+                                                 const int64_t* __restrict__ sorted_ids, int64_t vocab_start,
+                                                 int64_t V_loc, int64_t skip_row, T* __restrict__ d_weight, int64_t ldw,
+                                                 int vec_ok) {
     constexpr int V = elem<T>::kVec;
-    const int lane = threadIdx.x & 63;
-    const int64_t wave = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
-    const int64_t nwaves = (int64_t)gridDim.x * 4;
-    for (int64_t r = wave; r < R; r += nwaves) {
-        T* dst = p + r * ld;
+    const int grp = lane / kZeroGroup, g = lane % kZeroGroup;
+    const int64_t row0 = wave_global * kZeroRows;
+    if (row0 >= V_loc) return;
+    const int64_t row = row0 + grp;
+    const int64_t target = vocab_start + row;
+    int lo = 0, hi = row < V_loc ? T_rows : 0;  // the first position with sorted_ids >= target lies in [lo, hi]
+    while (__ballot(hi > lo) != 0ull) {
+        const int step = (hi - lo + kZeroGroup - 1) / kZeroGroup;
+        const int pos = lo + (g + 1) * step - 1;
+        const bool valid = hi > lo && pos < hi;
+        const bool less = valid && sorted_ids[valid ? pos : 0] < target;
+        const uint32_t mv = (uint32_t)(__ballot(valid) >> (grp * kZeroGroup)) & 0xffffu;
+        const uint32_t ml = (uint32_t)(__ballot(less) >> (grp * kZeroGroup)) & 0xffffu;
+        if (hi > lo) {
+            const int nless = __popc(ml);
+            lo += nless * step;                          // everything up to the last smaller probe is smaller
+            if (nless < __popc(mv)) hi = lo + step - 1;  // the next probe is not: the answer is at or before it
+        }
+    }
+    const bool present = row < V_loc && lo < T_rows && sorted_ids[lo < T_rows ? lo : 0] == target && row != skip_row;
+    const uint64_t mp = __ballot(present);
+#pragma unroll
+    for (int j = 0; j < kZeroRows; ++j) {
+        if (row0 + j >= V_loc || ((mp >> (j * kZeroGroup)) & 1ull)) continue;
+        T* dst = d_weight + (row0 + j) * ldw;
         if (vec_ok) {
             const int64_t nvec = E / V;
             for (int64_t c = lane; c < nvec; c += 64) store_raw_stream(dst + c * V, (raw16_t){0u, 0u, 0u, 0u});
@@ -63,6 +95,11 @@ __global__ __launch_bounds__(256) void zero_rows_kernel(int64_t R, int64_t E, T*
             for (int64_t c = lane; c < E; c += 64) store_elem(dst + c, 0.0f);
         }
     }
+}
+
+int zero_blocks_for(int64_t V_loc, int waves_per_block) {
+    const int64_t rows_per_block = (int64_t)kZeroRows * waves_per_block;
+    return (int)((V_loc + rows_per_block - 1) / rows_per_block);
 }
 
 // One block per position i of the sorted order. A run of fewer than kRunBlocks equal ids is summed by
@@ -82,12 +119,18 @@ __global__ __launch_bounds__(kRunWaves * 64) void embed_bwd_kernel(int64_t T_row
                                                                    const int64_t* __restrict__ order, int64_t vocab_start,
                                                                    int64_t V_loc, int64_t skip_row,
                                                                    const T* __restrict__ d_out, int64_t ldo,
-                                                                   T* __restrict__ d_weight, int64_t ldw) {
+                                                                   T* __restrict__ d_weight, int64_t ldw,
+                                                                   int zero_blocks) {
     constexpr int V = elem<T>::kVec;
     constexpr int kSlices = 16 / V;      // column slices held in registers at a time: 1024 columns
     constexpr int kTokens = 8 / kSlices;  // tokens of the run a wavefront loads together
     __shared__ float red[kRunWaves - 1][kSlices * V][64];
-    const int64_t i = blockIdx.x;
+    if ((int)blockIdx.x < zero_blocks) {
+        zero_absent_rows<T>((int64_t)blockIdx.x * kRunWaves + (threadIdx.x >> 6), threadIdx.x & 63, (int)T_rows, E, sorted_ids,
+                            vocab_start, V_loc, skip_row, d_weight, ldw, 1);
+        return;
+    }
+    const int64_t i = (int64_t)blockIdx.x - zero_blocks;
     const int64_t id = sorted_ids[i];
     // equal predecessors (k) and successors, as far as kRunBlocks - 1 each way: all loads are independent
     int k = 0, after = 0;
@@ -217,8 +260,14 @@ __global__ __launch_bounds__(256) void embed_bwd_generic_kernel(int64_t T_rows, 
                                                                 const int64_t* __restrict__ order, int64_t vocab_start,
                                                                 int64_t V_loc, int64_t skip_row,
                                                                 const T* __restrict__ d_out, int64_t ldo,
-                                                                T* __restrict__ d_weight, int64_t ldw) {
-    const int64_t i = blockIdx.x;
+                                                                T* __restrict__ d_weight, int64_t ldw, int zero_blocks,
+                                                                int w_vec) {
+    if ((int)blockIdx.x < zero_blocks) {
+        zero_absent_rows<T>((int64_t)blockIdx.x * 4 + (threadIdx.x >> 6), threadIdx.x & 63, (int)T_rows, E, sorted_ids,
+                            vocab_start, V_loc, skip_row, d_weight, ldw, w_vec);
+        return;
+    }
+    const int64_t i = (int64_t)blockIdx.x - zero_blocks;
     const int64_t id = sorted_ids[i];
     if (i > 0 && sorted_ids[i - 1] == id) return;
     const int64_t local = id - vocab_start;
@@ -229,6 +278,265 @@ __global__ __launch_bounds__(256) void embed_bwd_generic_kernel(int64_t T_rows, 
         float acc = 0.0f;
         for (int64_t r = 0; r < run; ++r) acc += load_elem(d_out + order[i + r] * ldo + c);
         store_elem(d_weight + local * ldw + c, acc);
+    }
+}
+
+// Backward straight from the unsorted ids, one launch, for batches of up to kDirMaxTokens tokens. A workgroup owns
+// kDirRows consecutive rows of the slice. It reads all ids (they stay in L2: every workgroup reads the same
+// 8 T bytes) and marks, per row, the tokens that select it in a bitmap in LDS. The rows that up to kDirHeavy
+// tokens select are dealt round-robin to the wavefronts, which sum a row's tokens in ascending token position
+// (what a stable sort by id would hand the sorted kernel), kDirBatch token rows in flight; the first batch of
+// loads is issued before any wavefront of the group starts on the zeros, so the reads do not queue behind
+// them in the compute unit's memory pipeline. The rows without tokens are then written as zeros, a fixed
+// share per wavefront. A row that more than kDirHeavy tokens select is left to the end and summed by all
+// wavefronts together, each over its contiguous range of token positions, partial sums added in wavefront
+// order. Fixed orders throughout: bit-reproducible, no global atomics. Every row of the slice is written
+// exactly once, so the zeros cost no pass of their own, and no token order has to be made first.
+#ifndef CW_DIR_WAVES
+#define CW_DIR_WAVES 8
+#define CW_DIR_ROWS 32
+#endif
+constexpr int kDirWaves = CW_DIR_WAVES;
+constexpr int kDirRows = CW_DIR_ROWS;
+constexpr int kDirRowsPerWave = kDirRows / kDirWaves;
+constexpr int kDirMaxTokens = 16384;
+constexpr int kDirHeavy = 8;
+constexpr int kDirBatch = 2;       // token rows a wavefront has in flight (twice that on the shared rows)
+constexpr int kDirIdsPerPass = 16;  // ids a thread has in flight
+static_assert(kDirRows <= 64 && kDirRows % kDirWaves == 0, "one lane per row of the group; whole rows per wavefront");
+
+template <typename T, int NV, int BATCH>
+__device__ __forceinline__ void dir_load_rows(const T* __restrict__ d_out, int64_t ldo, const int (&tok)[BATCH], int n,
+                                              const int64_t (&col)[NV], raw16_t (&raw)[BATCH][NV]) {
+#pragma unroll
+    for (int b = 0; b < BATCH; ++b) {
+#pragma unroll
+        for (int v = 0; v < NV; ++v) raw[b][v] = raw16_t{0u, 0u, 0u, 0u};
+        if (b < n) {
+#pragma unroll
+            for (int v = 0; v < NV; ++v) raw[b][v] = load_raw_stream(d_out + (int64_t)tok[b] * ldo + col[v]);
+        }
+    }
+}
+
+template <typename T, int NV, int BATCH>
+__device__ __forceinline__ void dir_accumulate(const raw16_t (&raw)[BATCH][NV], float (&acc)[NV][elem<T>::kVec]) {
+    constexpr int V = elem<T>::kVec;
+#pragma unroll
+    for (int b = 0; b < BATCH; ++b)
+#pragma unroll
+        for (int v = 0; v < NV; ++v) {
+            float x[V];
+            unpack_raw(raw[b][v], x, (const T*)nullptr);
+#pragma unroll
+            for (int e = 0; e < V; ++e) acc[v][e] += x[e];
+        }
+}
+
+// One round over 64 words of a row's bitmap held one per lane in `word`: the lowest marked token of each word
+// that has one, words in ascending order, goes to queue[0..n) (at most `want` of them) and is cleared in `word`.
+// Returns n. LDS operations of one wavefront execute in order, so the queue can be read back right after.
+__device__ __forceinline__ int dir_take_tokens(uint32_t& word, int wi, int want, uint16_t* queue) {
+    const uint64_t mask = __ballot(word != 0u);
+    const int rank = __builtin_amdgcn_mbcnt_hi((uint32_t)(mask >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t)mask, 0u));
+    if (word != 0u && rank < want) {
+        queue[rank] = (uint16_t)(wi * 32 + __builtin_ctz(word));
+        word &= word - 1u;
+    }
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    const int n = __popcll(mask);
+    return n < want ? n : want;
+}
+
+// acc += d_out rows of the tokens marked in words [w_lo, w_hi) of one row's bitmap, BATCH rows in flight.
+// The order is fixed by the bitmap alone: round by round the lowest marked token of every word, words ascending.
+template <typename T, int NV, int BATCH>
+__device__ __forceinline__ void dir_sum_tokens(const uint32_t* bm_row, int w_lo, int w_hi, int lane, uint16_t* queue,
+                                               const T* __restrict__ d_out, int64_t ldo, const int64_t (&col)[NV],
+                                               float (&acc)[NV][elem<T>::kVec]) {
+    for (int wb = w_lo; wb < w_hi; wb += 64) {
+        const int wi = wb + lane;
+        uint32_t word = wi < w_hi ? bm_row[wi] : 0u;
+        for (;;) {
+            const int n = dir_take_tokens(word, wi, 64, queue);
+            if (n == 0) break;
+            for (int i = 0; i < n; i += BATCH) {
+                int tok[BATCH];
+#pragma unroll
+                for (int b = 0; b < BATCH; ++b) tok[b] = __builtin_amdgcn_readfirstlane((int)queue[i + b < n ? i + b : i]);
+                raw16_t raw[BATCH][NV];
+                dir_load_rows<T, NV, BATCH>(d_out, ldo, tok, n - i, col, raw);
+                dir_accumulate<T, NV, BATCH>(raw, acc);
+            }
+            __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");  // the queue is rewritten by the next round
+        }
+    }
+}
+
+template <typename T, int NV>
+__device__ __forceinline__ void dir_columns(int64_t c0, int lane, int64_t E, int64_t (&col)[NV], float (&acc)[NV][elem<T>::kVec]) {
+    constexpr int V = elem<T>::kVec;
+#pragma unroll
+    for (int v = 0; v < NV; ++v) {
+        const int64_t cv = c0 + ((int64_t)v * 64 + lane) * V;
+        col[v] = cv < E ? cv : E - V;  // a position past the end re-reads the last vector and stores nothing
+#pragma unroll
+        for (int e = 0; e < V; ++e) acc[v][e] = 0.0f;
+    }
+}
+
+template <typename T, int NV>
+__device__ __forceinline__ void dir_store_columns(T* dst, int64_t c0, int lane, int64_t E, const int64_t (&col)[NV],
+                                                  const float (&acc)[NV][elem<T>::kVec]) {
+    constexpr int V = elem<T>::kVec;
+#pragma unroll
+    for (int v = 0; v < NV; ++v)
+        if (c0 + ((int64_t)v * 64 + lane) * V < E) store_raw_stream(dst + col[v], pack_raw(acc[v], (const T*)nullptr));
+}
+
+template <typename T>
+__global__ __launch_bounds__(kDirWaves * 64) void embed_bwd_direct_kernel(int T_rows, int64_t E, const int64_t* __restrict__ ids,
+                                                                          int64_t vocab_start, int64_t V_loc, int64_t skip_row,
+                                                                          const T* __restrict__ d_out, int64_t ldo,
+                                                                          T* __restrict__ d_weight, int64_t ldw) {
+    constexpr int V = elem<T>::kVec;
+    constexpr int NV = 4;   // column vectors per lane and pass of a row a wavefront sums alone
+    constexpr int NVH = 2;  // the same for a row all wavefronts share
+    constexpr int kThreads = kDirWaves * 64;
+    extern __shared__ uint32_t dir_bitmap[];  // [kDirRows][words]
+    __shared__ int cnt[kDirRows];
+    __shared__ float red[kDirWaves - 1][NVH * V][64];
+    __shared__ uint16_t dir_queue[kDirWaves][64];  // tokens a wavefront is about to load
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int words = (T_rows + 31) >> 5;
+    const int64_t r0 = (int64_t)blockIdx.x * kDirRows;
+    const uint64_t base = (uint64_t)vocab_start + (uint64_t)r0;
+    const uint64_t rows_here = (uint64_t)(V_loc - r0 < kDirRows ? V_loc - r0 : kDirRows);
+    // the first ids are on their way while the bitmap is cleared
+    int64_t idv[kDirIdsPerPass];
+#pragma unroll
+    for (int u = 0; u < kDirIdsPerPass; ++u) {
+        const int t = tid + u * kThreads;
+        idv[u] = T_rows > 0 ? ids[t < T_rows ? t : T_rows - 1] : 0;
+    }
+    for (int i = tid; i < kDirRows * words; i += kThreads) dir_bitmap[i] = 0u;
+    __syncthreads();
+    for (int t0 = 0; t0 < T_rows; t0 += kDirIdsPerPass * kThreads) {
+        if (t0 > 0) {
+#pragma unroll
+            for (int u = 0; u < kDirIdsPerPass; ++u) {
+                const int t = t0 + tid + u * kThreads;
+                idv[u] = ids[t < T_rows ? t : T_rows - 1];
+            }
+        }
+#pragma unroll
+        for (int u = 0; u < kDirIdsPerPass; ++u) {
+            const int t = t0 + tid + u * kThreads;
+            const uint64_t r = (uint64_t)idv[u] - base;
+            if (t < T_rows && r < rows_here) atomicOr(&dir_bitmap[(int)r * words + (t >> 5)], 1u << (t & 31));
+        }
+    }
+    __syncthreads();
+#pragma unroll
+    for (int q = 0; q < kDirRowsPerWave; ++q) {
+        const int j = wave * kDirRowsPerWave + q;
+        int c = 0;
+        for (int wi = lane; wi < words; wi += 64) c += __popc(dir_bitmap[j * words + wi]);
+        c = (int)wave_sum((float)c);  // at most kDirMaxTokens: exact
+        if (lane == 0) cnt[j] = (r0 + j != skip_row) ? c : 0;  // rows past the end of the slice have no tokens
+    }
+    __syncthreads();
+    const int my_cnt = lane < kDirRows ? cnt[lane] : 0;
+    uint64_t light = __ballot(my_cnt > 0 && my_cnt <= kDirHeavy);  // bit j: row j is summed by one wavefront
+    const uint64_t heavy = __ballot(my_cnt > kDirHeavy);
+    const uint64_t empty = __ballot(my_cnt == 0 && (uint64_t)lane < rows_here);
+    for (int k = 0; k < wave && light != 0ull; ++k) light &= light - 1;  // this wavefront's first: the wave-th set bit
+
+    // this wavefront's first row with tokens: the first batch of its loads goes out ahead of all zeros
+    uint16_t* queue = dir_queue[wave];
+    int64_t col[NV];
+    float acc[NV][V];
+    const int first_row = light != 0ull ? __builtin_ctzll(light) : -1;
+    int early[kDirBatch], n_early = 0;  // the tokens of that batch: out of the row's bitmap while its first pass runs
+#pragma unroll
+    for (int b = 0; b < kDirBatch; ++b) early[b] = 0;
+    {
+        raw16_t raw[kDirBatch][NV];
+        if (first_row >= 0) {
+            uint32_t* bm_row = dir_bitmap + first_row * words;
+            for (int wb = 0; wb < words && n_early == 0; wb += 64) {
+                const int wi = wb + lane;
+                uint32_t word = wi < words ? bm_row[wi] : 0u;
+                n_early = dir_take_tokens(word, wi, kDirBatch, queue);
+                if (wi < words) bm_row[wi] = word;
+            }
+#pragma unroll
+            for (int b = 0; b < kDirBatch; ++b) early[b] = __builtin_amdgcn_readfirstlane((int)queue[b < n_early ? b : 0]);
+            dir_columns<T, NV>(0, lane, E, col, acc);
+            dir_load_rows<T, NV, kDirBatch>(d_out, ldo, early, n_early, col, raw);
+        }
+        __builtin_amdgcn_s_barrier();  // no data passes here: it only keeps every wavefront's zeros behind the loads above
+
+        // zeros: the empty rows among this wavefront's kDirRowsPerWave
+#pragma unroll
+        for (int q = 0; q < kDirRowsPerWave; ++q) {
+            const int j = wave * kDirRowsPerWave + q;
+            if (!((empty >> j) & 1ull)) continue;
+            T* dst = d_weight + (r0 + j) * ldw;
+            for (int64_t c = (int64_t)lane * V; c < E; c += 64 * V) store_raw_stream(dst + c, raw16_t{0u, 0u, 0u, 0u});
+        }
+        if (first_row >= 0) dir_accumulate<T, NV, kDirBatch>(raw, acc);
+    }
+    // the rest of that row, then any further rows of this wavefront (kDirWaves set bits on each time)
+    for (bool first = true; light != 0ull; first = false) {
+        const int j = __builtin_ctzll(light);
+        T* dst = d_weight + (r0 + j) * ldw;
+        uint32_t* bm_row = dir_bitmap + j * words;
+        for (int64_t c0 = 0; c0 < E; c0 += (int64_t)64 * V * NV) {
+            if (!(first && c0 == 0)) dir_columns<T, NV>(c0, lane, E, col, acc);  // else: the sums of the first loads
+            dir_sum_tokens<T, NV, kDirBatch>(bm_row, 0, words, lane, queue, d_out, ldo, col, acc);
+            dir_store_columns<T, NV>(dst, c0, lane, E, col, acc);
+            if (first && c0 == 0) {  // further passes over the row's columns take all of its tokens
+#pragma unroll
+                for (int b = 0; b < kDirBatch; ++b)
+                    if (lane == b && b < n_early) atomicOr(&bm_row[early[b] >> 5], 1u << (early[b] & 31));
+                __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+            }
+        }
+        for (int k = 0; k < kDirWaves && light != 0ull; ++k) light &= light - 1;
+    }
+    // rows that many tokens select: every wavefront sums the tokens of its range of positions
+    const int words_per_wave = (words + kDirWaves - 1) / kDirWaves;
+    const int w_lo = wave * words_per_wave;
+    const int w_hi = w_lo + words_per_wave < words ? w_lo + words_per_wave : words;
+    for (uint64_t todo = heavy; todo != 0ull; todo &= todo - 1) {
+        const int j = __builtin_ctzll(todo);
+        T* dst = d_weight + (r0 + j) * ldw;
+        const uint32_t* bm_row = dir_bitmap + j * words;
+        for (int64_t c0 = 0; c0 < E; c0 += (int64_t)64 * V * NVH) {
+            int64_t colh[NVH];
+            float acch[NVH][V];
+            dir_columns<T, NVH>(c0, lane, E, colh, acch);
+            dir_sum_tokens<T, NVH, 2 * kDirBatch>(bm_row, w_lo, w_hi, lane, queue, d_out, ldo, colh, acch);
+            if (wave > 0) {
+#pragma unroll
+                for (int v = 0; v < NVH; ++v)
+#pragma unroll
+                    for (int e = 0; e < V; ++e) red[wave - 1][v * V + e][lane] = acch[v][e];
+            }
+            __syncthreads();
+            if (wave == 0) {
+#pragma unroll
+                for (int v = 0; v < NVH; ++v)
+#pragma unroll
+                    for (int w = 0; w < kDirWaves - 1; ++w)
+#pragma unroll
+                        for (int e = 0; e < V; ++e) acch[v][e] += red[w][v * V + e][lane];
+                dir_store_columns<T, NVH>(dst, c0, lane, E, colh, acch);
+            }
+            __syncthreads();
+        }
     }
 }
 
@@ -253,18 +561,37 @@ int bwd_impl(int64_t T_rows, int64_t E, const int64_t* sorted_ids, const int64_t
              int64_t V_loc, int64_t skip_row, const void* d_out, int64_t ldo, void* d_weight, int64_t ldw, hipStream_t s) {
     constexpr int V = elem<T>::kVec;
     const int w_vec = aligned16(d_weight) && ldw % V == 0;
-    hipLaunchKernelGGL(zero_rows_kernel<T>, dim3(rows_grid(V_loc, 4)), dim3(256), 0, s, V_loc, E, (T*)d_weight, ldw, w_vec);
-    int rc = check_launch("zero_rows_kernel");
-    if (rc != CW_OK || T_rows == 0) return rc;
-    const bool vec = w_vec && aligned16(d_out) && ldo % V == 0 && E % V == 0;
+    // one launch: the workgroups that clear the rows without tokens first (they carry most of the bytes), then one
+    // per position of the sorted order
+    const bool vec = w_vec && E % V == 0 && (T_rows == 0 || (aligned16(d_out) && ldo % V == 0));
     if (vec) {
-        hipLaunchKernelGGL(embed_bwd_kernel<T>, dim3((unsigned)T_rows), dim3(kRunWaves * 64), 0, s, T_rows, E, sorted_ids, order,
-                           vocab_start, V_loc, skip_row, (const T*)d_out, ldo, (T*)d_weight, ldw);
+        const int zb = zero_blocks_for(V_loc, kRunWaves);
+        hipLaunchKernelGGL(embed_bwd_kernel<T>, dim3((unsigned)(zb + T_rows)), dim3(kRunWaves * 64), 0, s, T_rows, E, sorted_ids,
+                           order, vocab_start, V_loc, skip_row, (const T*)d_out, ldo, (T*)d_weight, ldw, zb);
     } else {
-        hipLaunchKernelGGL(embed_bwd_generic_kernel<T>, dim3((unsigned)T_rows), dim3(256), 0, s, T_rows, E, sorted_ids, order,
-                           vocab_start, V_loc, skip_row, (const T*)d_out, ldo, (T*)d_weight, ldw);
+        const int zb = zero_blocks_for(V_loc, 4);
+        hipLaunchKernelGGL(embed_bwd_generic_kernel<T>, dim3((unsigned)(zb + T_rows)), dim3(256), 0, s, T_rows, E, sorted_ids,
+                           order, vocab_start, V_loc, skip_row, (const T*)d_out, ldo, (T*)d_weight, ldw, zb, w_vec);
     }
     return check_launch("embed_bwd_kernel");
+}
+
+bool direct_ok(int64_t T_rows, int64_t E, const void* d_out, int64_t ldo, const void* d_weight, int64_t ldw, int V) {
+    return T_rows <= kDirMaxTokens && E % V == 0 && aligned16(d_weight) && ldw % V == 0 &&
+           (T_rows == 0 || (aligned16(d_out) && ldo % V == 0));
+}
+
+template <typename T>
+int bwd_direct_impl(int64_t T_rows, int64_t E, const int64_t* ids, int64_t vocab_start, int64_t V_loc, int64_t skip_row,
+                    const void* d_out, int64_t ldo, void* d_weight, int64_t ldw, hipStream_t s) {
+    const int words = (int)((T_rows + 31) / 32);
+    const int lds = kDirRows * words * (int)sizeof(uint32_t);
+    if (const int rc = ensure_dynamic_lds((const void*)embed_bwd_direct_kernel<T>, kDirRows * (kDirMaxTokens / 32) * (int)sizeof(uint32_t),
+                                          "embed_bwd_direct_kernel"); rc != CW_OK) return rc;
+    const int64_t blocks = (V_loc + kDirRows - 1) / kDirRows;
+    hipLaunchKernelGGL(embed_bwd_direct_kernel<T>, dim3((unsigned)blocks), dim3(kDirWaves * 64), lds, s, (int)T_rows, E, ids,
+                       vocab_start, V_loc, skip_row, (const T*)d_out, ldo, (T*)d_weight, ldw);
+    return check_launch("embed_bwd_direct_kernel");
 }
 
 }  // namespace
@@ -293,7 +620,8 @@ extern "C" int cw_embed_bwd(int64_t T, int64_t E, const int64_t* sorted_ids, con
     if (T < 0 || E <= 0 || V_loc <= 0) return fail(CW_ERR_INVALID, "cw_embed_bwd: bad shape T=%lld E=%lld V_loc=%lld", (long long)T, (long long)E, (long long)V_loc);
     if (io_dtype != CW_BF16 && io_dtype != CW_F32 && io_dtype != CW_F16)
         return fail(CW_ERR_INVALID, "cw_embed_bwd: bad io_dtype %d", io_dtype);
-    if (T > INT32_MAX) return fail(CW_ERR_INVALID, "cw_embed_bwd: too many tokens");
+    if (T > INT32_MAX / 2 || V_loc > INT32_MAX / 2)
+        return fail(CW_ERR_INVALID, "cw_embed_bwd: more than 2^30 tokens or rows (the grid is one launch over both)");
     if (d_weight == nullptr || ldw < E) return fail(CW_ERR_INVALID, "cw_embed_bwd: d_weight is NULL or ldw < E");
     if (T > 0 && (sorted_ids == nullptr || order == nullptr || d_out == nullptr || ldo < E))
         return fail(CW_ERR_INVALID, "cw_embed_bwd: null pointer or leading dimension < E");
@@ -302,5 +630,33 @@ extern "C" int cw_embed_bwd(int64_t T, int64_t E, const int64_t* sorted_ids, con
     return with_elem_type(io_dtype, [&](auto* tag) {
         return bwd_impl<std::remove_pointer_t<decltype(tag)>>(T, E, sorted_ids, order, vocab_start, V_loc, skip_row, d_out,
                                                               ldo, d_weight, ldw, s);
+    });
+}
+
+extern "C" int cw_embed_bwd_ids_supported(int64_t T, int64_t E, const void* d_out, int64_t ldo, const void* d_weight,
+                                          int64_t ldw, int io_dtype) {
+    if (io_dtype != CW_BF16 && io_dtype != CW_F32 && io_dtype != CW_F16) return 0;
+    return direct_ok(T, E, d_out, ldo, d_weight, ldw, io_dtype == CW_F32 ? 4 : 8) ? 1 : 0;
+}
+
+extern "C" int cw_embed_bwd_ids(int64_t T, int64_t E, const int64_t* ids, int64_t vocab_start, int64_t V_loc,
+                                int64_t skip_row, const void* d_out, int64_t ldo, void* d_weight, int64_t ldw,
+                                int io_dtype, void* stream) {
+    if (T < 0 || E <= 0 || V_loc <= 0) return fail(CW_ERR_INVALID, "cw_embed_bwd_ids: bad shape T=%lld E=%lld V_loc=%lld", (long long)T, (long long)E, (long long)V_loc);
+    if (io_dtype != CW_BF16 && io_dtype != CW_F32 && io_dtype != CW_F16)
+        return fail(CW_ERR_INVALID, "cw_embed_bwd_ids: bad io_dtype %d", io_dtype);
+    if (V_loc > INT32_MAX / 2) return fail(CW_ERR_INVALID, "cw_embed_bwd_ids: more than 2^30 rows");
+    if (d_weight == nullptr || ldw < E) return fail(CW_ERR_INVALID, "cw_embed_bwd_ids: d_weight is NULL or ldw < E");
+    if (T > 0 && (ids == nullptr || d_out == nullptr || ldo < E))
+        return fail(CW_ERR_INVALID, "cw_embed_bwd_ids: null pointer or leading dimension < E");
+    if (!cw_embed_bwd_ids_supported(T, E, d_out, ldo, d_weight, ldw, io_dtype))
+        return fail(CW_ERR_UNSUPPORTED,
+                    "cw_embed_bwd_ids: needs T <= %d, 16-byte aligned rows and E a multiple of the 16-byte vector; "
+                    "use cw_embed_sort_ids + cw_embed_bwd", kDirMaxTokens);
+    if (const int drc = require_gfx950("cw_embed_bwd_ids"); drc != CW_OK) return drc;
+    hipStream_t s = (hipStream_t)stream;
+    return with_elem_type(io_dtype, [&](auto* tag) {
+        return bwd_direct_impl<std::remove_pointer_t<decltype(tag)>>(T, E, ids, vocab_start, V_loc, skip_row, d_out, ldo,
+                                                                     d_weight, ldw, s);
     });
 }

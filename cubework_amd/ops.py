@@ -519,15 +519,26 @@ def embedding_token_order(ids: torch.Tensor, num_rows: int, vocab_start: int = 0
 
 
 def embedding_bwd(ids: torch.Tensor, d_out: torch.Tensor, num_rows: int, vocab_start: int = 0,
-                  skip_row: int = -1) -> torch.Tensor:
-    """Gradient of embedding_fwd with respect to the [num_rows, E] weight slice. See cw_embed_bwd."""
+                  skip_row: int = -1, via_token_order: bool = False) -> torch.Tensor:
+    """Gradient of embedding_fwd with respect to the [num_rows, E] weight slice: one launch from the unsorted
+    ids where cw_embed_bwd_ids takes the shapes (up to 16384 tokens, 16-byte aligned rows), else (or with
+    via_token_order) the token order followed by cw_embed_bwd."""
     lib = _lib.load()
     _require_device(ids, d_out)
+    if ids.dtype != torch.int64:
+        raise TypeError("ids must be int64, got %s" % ids.dtype)
     g = _rows(d_out.reshape(-1, d_out.shape[-1]))
-    flat = ids.reshape(-1)
+    flat = ids.reshape(-1).contiguous()
     T, E = g.shape
-    sorted_ids, order = embedding_token_order(flat, num_rows, vocab_start)
+    if flat.numel() != T:
+        raise ValueError("ids select %d rows, d_out has %d" % (flat.numel(), T))
     dw = torch.empty((num_rows, E), dtype=g.dtype, device=g.device)
+    if not via_token_order and lib.cw_embed_bwd_ids_supported(T, E, _p(g), _ld(g), _p(dw), _ld(dw), _dtype_code(g)):
+        rc = lib.cw_embed_bwd_ids(T, E, _p(flat), int(vocab_start), num_rows, int(skip_row), _p(g), _ld(g), _p(dw),
+                                  _ld(dw), _dtype_code(g), _stream())
+        _lib.check(rc, "cw_embed_bwd_ids")
+        return dw
+    sorted_ids, order = embedding_token_order(flat, num_rows, vocab_start)
     rc = lib.cw_embed_bwd(T, E, _p(sorted_ids), _p(order), int(vocab_start), num_rows, int(skip_row), _p(g), _ld(g),
                           _p(dw), _ld(dw), _dtype_code(g), _stream())
     _lib.check(rc, "cw_embed_bwd")

@@ -318,7 +318,8 @@ int cw_embed_fwd(int64_t T, int64_t E, const int64_t* ids, int64_t vocab_start, 
  * once); rows without tokens, and row skip_row (F.embedding's padding_idx, -1 for none), are zero.
  * Autograd of the F.embedding call above. sorted_ids / order: the ids in ascending order and the
  * token position of each (a stable sort by the caller); runs of equal ids are summed in that order,
- * without atomics, so the result is bit-reproducible.
+ * without atomics, so the result is bit-reproducible. One launch: the rows without tokens are found by a
+ * search in sorted_ids and cleared by workgroups of the same grid. T, V_loc <= 2^30.
  */
 int cw_embed_bwd(int64_t T, int64_t E, const int64_t* sorted_ids, const int64_t* order,
                  int64_t vocab_start, int64_t V_loc, int64_t skip_row,
@@ -339,6 +340,24 @@ int64_t cw_embed_sort_workspace_bytes(int64_t T);
 int cw_embed_sort_ids(int64_t T, const int64_t* ids, int64_t vocab_start, int64_t V_loc,
                       int64_t* sorted_ids, int64_t* order, void* workspace, int64_t workspace_bytes,
                       void* stream);
+
+/*
+ * The same gradient as cw_embed_bwd straight from the unsorted ids, in one launch and one pass over the
+ * data: no token order is made first and the zeros of the rows without tokens are written by the launch
+ * that sums the others (every row of d_weight is written exactly once). Replaces the whole backward of
+ * the F.embedding call (parallel_1d/module.py:452, parallel_2d/module.py:353, parallel_3d/module.py:466)
+ * for a batch of up to 16384 tokens whose rows are 16-byte aligned (E a multiple of the 16-byte vector).
+ * A row's tokens are added in ascending token position, as after a stable sort; a row that more than 16
+ * tokens select is summed over 8 contiguous ranges of token positions whose partial sums are added in
+ * order. No atomics on global memory: bit-reproducible. cw_embed_bwd_ids_supported returns 1 when the
+ * shapes and pointers qualify; otherwise cw_embed_bwd_ids returns CW_ERR_UNSUPPORTED and the caller
+ * goes through cw_embed_sort_ids + cw_embed_bwd.
+ */
+int cw_embed_bwd_ids_supported(int64_t T, int64_t E, const void* d_out, int64_t ldo, const void* d_weight,
+                               int64_t ldw, int io_dtype);
+int cw_embed_bwd_ids(int64_t T, int64_t E, const int64_t* ids, int64_t vocab_start, int64_t V_loc,
+                     int64_t skip_row, const void* d_out, int64_t ldo, void* d_weight, int64_t ldw,
+                     int io_dtype, void* stream);
 
 /* ---- gradient-norm clipping ---------------------------------------------- */
 /*

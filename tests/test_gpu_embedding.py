@@ -1,5 +1,7 @@
-"""GPU parity of the vocab-parallel embedding (cw_embed_fwd / cw_embed_bwd through the C ABI): the lookup
-is a bit-exact copy with integer-exact masking; the gradient is an fp32 sum rounded once."""
+"""GPU parity of the vocab-parallel embedding (cw_embed_fwd, cw_embed_bwd_ids and cw_embed_sort_ids +
+cw_embed_bwd through the C ABI): the lookup is a bit-exact copy with integer-exact masking; the gradient
+is an fp32 sum rounded once. Every backward case runs both ways: in one launch from the unsorted ids
+(where the shapes qualify) and through the token order."""
 import pytest
 import torch
 
@@ -7,6 +9,7 @@ from tests.util import assert_parity, randn
 
 pytestmark = pytest.mark.gpu
 DEV = "cuda:0"
+both_paths = pytest.mark.parametrize("via_order", [False, True], ids=["from_ids", "token_order"])
 
 
 def _ids(shape, vocab, seed, hot=None):
@@ -20,7 +23,8 @@ def _ids(shape, vocab, seed, hot=None):
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32, torch.float16])
 @pytest.mark.parametrize("case", [(4, 37, 1000, 256, 250, 64), (2, 128, 50272, 12568, 12568, 2048),
                                   (1, 5, 64, 64, 0, 8), (3, 11, 300, 100, 100, 52), (1, 1, 16, 4, 12, 520)])
-def test_embedding_forward_backward_parity(case, dtype):
+@both_paths
+def test_embedding_forward_backward_parity(case, dtype, via_order):
     import oracle
     from cubework_amd import ops
 
@@ -39,8 +43,8 @@ def test_embedding_forward_backward_parity(case, dtype):
     d_out = randn((b, s, e), dtype, 6)
     for pad in (None, 1 if v_loc > 1 else 0):
         want_dw = oracle.vocab_embedding_bwd(ids, d_out, v_loc, start, pad)
-        got_dw = ops.embedding_bwd(ids.to(DEV), d_out.to(DEV), v_loc, start, -1 if pad is None else pad)
-        again = ops.embedding_bwd(ids.to(DEV), d_out.to(DEV), v_loc, start, -1 if pad is None else pad)
+        got_dw = ops.embedding_bwd(ids.to(DEV), d_out.to(DEV), v_loc, start, -1 if pad is None else pad, via_order)
+        again = ops.embedding_bwd(ids.to(DEV), d_out.to(DEV), v_loc, start, -1 if pad is None else pad, via_order)
         torch.cuda.synchronize()
         assert torch.equal(got_dw, again), "no atomics: bit-reproducible"
         assert_parity(got_dw, want_dw, dtype, "embedding d_weight %s pad=%s" % (case, pad))
@@ -53,7 +57,8 @@ def test_embedding_forward_backward_parity(case, dtype):
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32, torch.float16])
 @pytest.mark.parametrize("e", [520, 2048, 4104])
-def test_embedding_backward_every_run_length(e, dtype):
+@both_paths
+def test_embedding_backward_every_run_length(e, dtype, via_order):
     """Id j occurs j + 1 times (runs of 1 .. 45 tokens in the sorted order, shuffled over the batch): the
     short-run path, the shared path with its four column-sharing blocks and ragged last slices, and runs
     that end inside and at the edge of a wavefront's group of tokens all meet the oracle's sums."""
@@ -65,14 +70,15 @@ def test_embedding_backward_every_run_length(e, dtype):
     v_loc, start = 100, 0
     d_out = randn((ids.numel(), e), dtype, 7)
     want = oracle.vocab_embedding_bwd(ids, d_out, v_loc, start, None)
-    got = ops.embedding_bwd(ids.to(DEV), d_out.to(DEV), v_loc, start, -1)
+    got = ops.embedding_bwd(ids.to(DEV), d_out.to(DEV), v_loc, start, -1, via_order)
     torch.cuda.synchronize()
     assert_parity(got, want, dtype, "embedding d_weight, runs of 1..45, E=%d" % e)
     assert (got.cpu()[0:3] == 0).all() and (got.cpu()[4::2][:44] == 0).all(), "rows without tokens are exactly zero"
 
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32, torch.float16])
-def test_embedding_backward_one_id_thousands_of_times(dtype):
+@both_paths
+def test_embedding_backward_one_id_thousands_of_times(dtype, via_order):
     """Token frequencies of text: one id 3000 times among 5000 tokens (a run that every wavefront of the
     sharing blocks walks for many rounds), the rest spread over the table; compared in float64."""
     from cubework_amd import ops
@@ -83,8 +89,8 @@ def test_embedding_backward_one_id_thousands_of_times(dtype):
     e, v_loc = 1032, 400
     d_out = randn((5000, e), dtype, 8)
     want = torch.zeros((v_loc, e), dtype=torch.float64).index_add_(0, ids, d_out.double())
-    got = ops.embedding_bwd(ids.to(DEV), d_out.to(DEV), v_loc, 0, -1)
-    again = ops.embedding_bwd(ids.to(DEV), d_out.to(DEV), v_loc, 0, -1)
+    got = ops.embedding_bwd(ids.to(DEV), d_out.to(DEV), v_loc, 0, -1, via_order)
+    again = ops.embedding_bwd(ids.to(DEV), d_out.to(DEV), v_loc, 0, -1, via_order)
     torch.cuda.synchronize()
     assert torch.equal(got, again)
     # the longest run sums 3000 rows in fp32
@@ -179,3 +185,52 @@ def test_token_order_repeated_id():
     got_ids, got_order = ops.embedding_token_order(ids, 100, 0)
     assert torch.equal(got_ids, ids)
     assert torch.equal(got_order.cpu(), torch.arange(5000))
+
+
+@pytest.mark.parametrize("T", [0, 1, 16384])
+def test_embedding_backward_from_ids_edges(T):
+    """The one-launch backward on ids below, at and above the slice's edges, negative ids and the extremes
+    of int64 (none of which may select a row), on an empty batch (all zeros) and on the longest batch it
+    takes; the result equals the token-order path's bit for bit where no row has more than 16 tokens, and
+    float64 sums within the bar everywhere."""
+    from cubework_amd import ops
+
+    start, rows, e = 1000, 777, 264
+    g = torch.Generator().manual_seed(T + 1)
+    ids = torch.randint(start - 300, start + rows + 300, (T,), generator=g, dtype=torch.int64)
+    edges = torch.tensor([start - 1, start, start + rows - 1, start + rows, 0, -5, 2 ** 63 - 1, -2 ** 63], dtype=torch.int64)
+    n = min(T, edges.numel())
+    ids[:n] = edges[:n]
+    d_out = randn((T, e), torch.float32, 12)
+    got = ops.embedding_bwd(ids.to(DEV), d_out.to(DEV), rows, start, 5)
+    torch.cuda.synchronize()
+    local = ids - start
+    live = (ids >= start) & (ids < start + rows) & (local != 5)
+    want = torch.zeros((rows, e), dtype=torch.float64).index_add_(0, local[live], d_out.double()[live])
+    assert_parity(got, want, torch.float32, "embedding d_weight from ids, T=%d" % T)
+    assert (got[5] == 0).all()
+    if T <= 1:
+        via = ops.embedding_bwd(ids.to(DEV), d_out.to(DEV), rows, start, 5, via_token_order=True)
+        assert torch.equal(got, via)
+
+
+def test_embedding_backward_from_ids_refuses_what_it_cannot_take():
+    """More than 16384 tokens, or rows that are not 16-byte aligned: CW_ERR_UNSUPPORTED from the entry point
+    (nothing launched), and the wrapper goes through the token order instead."""
+    from cubework_amd import _lib, ops
+
+    lib = _lib.load()
+    T, e, rows = 16385, 64, 50
+    ids = torch.randint(0, rows, (T,), generator=torch.Generator().manual_seed(1)).to(DEV)
+    d_out = randn((T, e), torch.bfloat16, 2).to(DEV)
+    dw = torch.full((rows, e), 7.0, dtype=torch.bfloat16, device=DEV)
+    assert lib.cw_embed_bwd_ids_supported(T, e, d_out.data_ptr(), e, dw.data_ptr(), e, _lib.CW_BF16) == 0
+    rc = lib.cw_embed_bwd_ids(T, e, ids.data_ptr(), 0, rows, -1, d_out.data_ptr(), e, dw.data_ptr(), e, _lib.CW_BF16, None)
+    assert rc == -3  # CW_ERR_UNSUPPORTED
+    torch.cuda.synchronize()
+    assert (dw == 7.0).all(), "a refused call writes nothing"
+    got = ops.embedding_bwd(ids, d_out, rows)  # the wrapper's other path
+    want = torch.zeros((rows, e), dtype=torch.float64).index_add_(0, ids.cpu(), d_out.double().cpu())
+    assert_parity(got, want, torch.bfloat16, "embedding d_weight, 16385 tokens")
+    odd = d_out[:100, 1:]  # rows start 2 bytes off a 16-byte boundary
+    assert lib.cw_embed_bwd_ids_supported(100, e - 1, odd.data_ptr(), e, dw.data_ptr(), e, _lib.CW_BF16) == 0
