@@ -292,12 +292,8 @@ __global__ __launch_bounds__(256) void embed_bwd_generic_kernel(int64_t T_rows, 
 // wavefronts together, each over its contiguous range of token positions, partial sums added in wavefront
 // order. Fixed orders throughout: bit-reproducible, no global atomics. Every row of the slice is written
 // exactly once, so the zeros cost no pass of their own, and no token order has to be made first.
-#ifndef CW_DIR_WAVES
-#define CW_DIR_WAVES 8
-#define CW_DIR_ROWS 32
-#endif
-constexpr int kDirWaves = CW_DIR_WAVES;
-constexpr int kDirRows = CW_DIR_ROWS;
+constexpr int kDirWaves = 8;
+constexpr int kDirRows = 32;
 constexpr int kDirRowsPerWave = kDirRows / kDirWaves;
 constexpr int kDirMaxTokens = 16384;
 constexpr int kDirHeavy = 8;
@@ -421,6 +417,7 @@ __global__ __launch_bounds__(kDirWaves * 64) void embed_bwd_direct_kernel(int T_
         idv[u] = T_rows > 0 ? ids[t < T_rows ? t : T_rows - 1] : 0;
     }
     for (int i = tid; i < kDirRows * words; i += kThreads) dir_bitmap[i] = 0u;
+    if (tid < kDirRows) cnt[tid] = 0;
     __syncthreads();
     for (int t0 = 0; t0 < T_rows; t0 += kDirIdsPerPass * kThreads) {
         if (t0 > 0) {
@@ -434,20 +431,15 @@ __global__ __launch_bounds__(kDirWaves * 64) void embed_bwd_direct_kernel(int T_
         for (int u = 0; u < kDirIdsPerPass; ++u) {
             const int t = t0 + tid + u * kThreads;
             const uint64_t r = (uint64_t)idv[u] - base;
-            if (t < T_rows && r < rows_here) atomicOr(&dir_bitmap[(int)r * words + (t >> 5)], 1u << (t & 31));
+            if (t < T_rows && r < rows_here) {
+                atomicOr(&dir_bitmap[(int)r * words + (t >> 5)], 1u << (t & 31));
+                atomicAdd(&cnt[(int)r], 1);  // integer counts: the order of the additions does not matter
+            }
         }
     }
     __syncthreads();
-#pragma unroll
-    for (int q = 0; q < kDirRowsPerWave; ++q) {
-        const int j = wave * kDirRowsPerWave + q;
-        int c = 0;
-        for (int wi = lane; wi < words; wi += 64) c += __popc(dir_bitmap[j * words + wi]);
-        c = (int)wave_sum((float)c);  // at most kDirMaxTokens: exact
-        if (lane == 0) cnt[j] = (r0 + j != skip_row) ? c : 0;  // rows past the end of the slice have no tokens
-    }
-    __syncthreads();
-    const int my_cnt = lane < kDirRows ? cnt[lane] : 0;
+    int my_cnt = lane < kDirRows ? cnt[lane] : 0;
+    if (r0 + lane == skip_row) my_cnt = 0;  // its tokens are ignored: the row is written as zeros
     uint64_t light = __ballot(my_cnt > 0 && my_cnt <= kDirHeavy);  // bit j: row j is summed by one wavefront
     const uint64_t heavy = __ballot(my_cnt > kDirHeavy);
     const uint64_t empty = __ballot(my_cnt == 0 && (uint64_t)lane < rows_here);
@@ -465,10 +457,10 @@ __global__ __launch_bounds__(kDirWaves * 64) void embed_bwd_direct_kernel(int T_
         raw16_t raw[kDirBatch][NV];
         if (first_row >= 0) {
             uint32_t* bm_row = dir_bitmap + first_row * words;
-            for (int wb = 0; wb < words && n_early == 0; wb += 64) {
+            for (int wb = 0; wb < words && n_early < kDirBatch; wb += 64) {
                 const int wi = wb + lane;
                 uint32_t word = wi < words ? bm_row[wi] : 0u;
-                n_early = dir_take_tokens(word, wi, kDirBatch, queue);
+                n_early += dir_take_tokens(word, wi, kDirBatch - n_early, queue + n_early);
                 if (wi < words) bm_row[wi] = word;
             }
 #pragma unroll
@@ -477,18 +469,10 @@ __global__ __launch_bounds__(kDirWaves * 64) void embed_bwd_direct_kernel(int T_
             dir_load_rows<T, NV, kDirBatch>(d_out, ldo, early, n_early, col, raw);
         }
         __builtin_amdgcn_s_barrier();  // no data passes here: it only keeps every wavefront's zeros behind the loads above
-
-        // zeros: the empty rows among this wavefront's kDirRowsPerWave
-#pragma unroll
-        for (int q = 0; q < kDirRowsPerWave; ++q) {
-            const int j = wave * kDirRowsPerWave + q;
-            if (!((empty >> j) & 1ull)) continue;
-            T* dst = d_weight + (r0 + j) * ldw;
-            for (int64_t c = (int64_t)lane * V; c < E; c += 64 * V) store_raw_stream(dst + c, raw16_t{0u, 0u, 0u, 0u});
-        }
         if (first_row >= 0) dir_accumulate<T, NV, kDirBatch>(raw, acc);
     }
-    // the rest of that row, then any further rows of this wavefront (kDirWaves set bits on each time)
+    // the rest of that row, then any further rows of this wavefront (kDirWaves set bits on each time); the
+    // wavefronts without such rows are writing zeros meanwhile
     for (bool first = true; light != 0ull; first = false) {
         const int j = __builtin_ctzll(light);
         T* dst = d_weight + (r0 + j) * ldw;
@@ -505,6 +489,14 @@ __global__ __launch_bounds__(kDirWaves * 64) void embed_bwd_direct_kernel(int T_
             }
         }
         for (int k = 0; k < kDirWaves && light != 0ull; ++k) light &= light - 1;
+    }
+    // zeros: the empty rows among this wavefront's kDirRowsPerWave
+#pragma unroll
+    for (int q = 0; q < kDirRowsPerWave; ++q) {
+        const int j = wave * kDirRowsPerWave + q;
+        if (!((empty >> j) & 1ull)) continue;
+        T* dst = d_weight + (r0 + j) * ldw;
+        for (int64_t c = (int64_t)lane * V; c < E; c += 64 * V) store_raw_stream(dst + c, raw16_t{0u, 0u, 0u, 0u});
     }
     // rows that many tokens select: every wavefront sums the tokens of its range of positions
     const int words_per_wave = (words + kDirWaves - 1) / kDirWaves;
@@ -586,7 +578,7 @@ int bwd_direct_impl(int64_t T_rows, int64_t E, const int64_t* ids, int64_t vocab
                     const void* d_out, int64_t ldo, void* d_weight, int64_t ldw, hipStream_t s) {
     const int words = (int)((T_rows + 31) / 32);
     const int lds = kDirRows * words * (int)sizeof(uint32_t);
-    if (const int rc = ensure_dynamic_lds((const void*)embed_bwd_direct_kernel<T>, kDirRows * (kDirMaxTokens / 32) * (int)sizeof(uint32_t),
+    if (const int rc = ensure_dynamic_lds((const void*)embed_bwd_direct_kernel<T>, lds,
                                           "embed_bwd_direct_kernel"); rc != CW_OK) return rc;
     const int64_t blocks = (V_loc + kDirRows - 1) / kDirRows;
     hipLaunchKernelGGL(embed_bwd_direct_kernel<T>, dim3((unsigned)blocks), dim3(kDirWaves * 64), lds, s, (int)T_rows, E, ids,
