@@ -33,6 +33,7 @@ constexpr int kQT = 1;                    // 32-row query tiles per wavefront
 constexpr int kWaves = 8;                 // wavefronts per block
 constexpr int kThreads = kWaves * 64;
 constexpr int kQPerWave = 32 * kQT;
+constexpr float kLazy = 8.0f;             // log2 of the largest probability taken against a stale reference
 constexpr int kQPerBlock = kWaves * kQPerWave;
 
 struct AttnArgs {
@@ -69,7 +70,11 @@ __global__ __launch_bounds__(kThreads, NP == 1 ? 2 : 1) void attn_fwd_kernel(con
     const int b = bh / a.H, h = bh - b * a.H;
     const int qblk = a.n_qblocks - 1 - (int)(blockIdx.x / (unsigned)a.BH);
     const int q0 = qblk * kQPerBlock;
-    const int qw0 = q0 + wave * kQPerWave;
+    // Under the causal mask a wavefront's work grows with its query position, and wavefront w always runs on
+    // SIMD w % 4: half of the blocks deal the query tiles in reverse so that no SIMD collects the long ones
+    // (blocks 256 apart, which share a compute unit when the launch starts, differ in bit 8).
+    const int wq = (a.causal && (((blockIdx.x >> 8) ^ blockIdx.x) & 1)) ? kWaves - 1 - wave : wave;
+    const int qw0 = q0 + wq * kQPerWave;
 
     const uint16_t* qp = a.q + b * a.sb + h * a.sh;
     const uint16_t* kp = a.k + b * a.sb + h * a.sh;
@@ -93,7 +98,7 @@ __global__ __launch_bounds__(kThreads, NP == 1 ? 2 : 1) void attn_fwd_kernel(con
         for (int dt = 0; dt < 2 * NP; ++dt)
 #pragma unroll
             for (int e = 0; e < 16; ++e) oacc[qt][dt][e] = 0.0f;
-    float m_run[kQT], l_run[kQT];  // running maximum of scale*log2e*s; this lane's share of the running sum
+    float m_run[kQT], l_run[kQT];  // reference of the exponentials (scale*log2e*s units); this lane's share of the running sum
 #pragma unroll
     for (int qt = 0; qt < kQT; ++qt) {
         m_run[qt] = kNegBig;
@@ -176,11 +181,16 @@ __global__ __launch_bounds__(kThreads, NP == 1 ? 2 : 1) void attn_fwd_kernel(con
 #pragma unroll
                     for (int e = 1; e < 16; ++e) mx = fmaxf(mx, st[qt][e]);
                     mx = max_halves(mx);
-                    const float m_new = fmaxf(m_run[qt], mx * a.scale_log2e);
-                    const float m_use = (m_new == kNegBig) ? 0.0f : m_new;  // a row with no live key yet
-                    // rescale the running sum and O^T only when some row's maximum moved
-                    if (__builtin_amdgcn_ballot_w64(m_new != m_run[qt]) != 0) {
-                        const float alpha = __builtin_amdgcn_exp2f(m_run[qt] - m_use);
+                    // m_run is the reference the exponentials are taken against, not necessarily the maximum so
+                    // far: it moves (and the running sum and O^T are rescaled, 34 vector instructions) only
+                    // when some row's maximum exceeds it by more than kLazy, i.e. a probability would pass
+                    // 2^kLazy. With the true maximum as reference some row of the 32 moves in most tiles. The
+                    // quotient O / l does not depend on the reference, and bf16 / fp16 keep their relative
+                    // precision at 2^kLazy.
+                    const float mx_s = mx * a.scale_log2e;
+                    if (__builtin_amdgcn_ballot_w64(mx_s > m_run[qt] + kLazy) != 0) {
+                        const float m_new = fmaxf(m_run[qt], mx_s);
+                        const float alpha = __builtin_amdgcn_exp2f(m_run[qt] - ((m_new == kNegBig) ? 0.0f : m_new));
                         l_run[qt] *= alpha;
 #pragma unroll
                         for (int dt = 0; dt < 2 * NP; ++dt)
@@ -188,6 +198,7 @@ __global__ __launch_bounds__(kThreads, NP == 1 ? 2 : 1) void attn_fwd_kernel(con
                             for (int e = 0; e < 16; ++e) oacc[qt][dt][e] *= alpha;
                         m_run[qt] = m_new;
                     }
+                    const float m_use = (m_run[qt] == kNegBig) ? 0.0f : m_run[qt];  // a row with no live key yet
                     float p[16];
 #pragma unroll
                     for (int e = 0; e < 16; ++e)
@@ -211,7 +222,8 @@ __global__ __launch_bounds__(kThreads, NP == 1 ? 2 : 1) void attn_fwd_kernel(con
                 }
             };
             half_tile(std::integral_constant<int, 0>{});
-            half_tile(std::integral_constant<int, 1>{});
+            // the second 32 key rows of a tile that starts on the wavefront's diagonal are wholly masked
+            if (!a.causal || kv0 + 32 <= qw0 + kQPerWave - 1) half_tile(std::integral_constant<int, 1>{});
         }
         dma_wait<0>();  // the next tile has landed (a third stage and loads two tiles ahead gained nothing)
         __syncthreads();
