@@ -373,10 +373,10 @@ def bench_other_configs(device, sets):
         j[0] += 1
         ops.embedding_bwd(ids, dys_e[j[0] % 4], e_vloc, e_vloc)
     us = graph_time_us(emb_bwd, 8)
-    nbytes = 3 * e_tok * 8 + live * e_dim * 2 + e_vloc * e_dim * 2
+    nbytes = e_tok * 8 + live * e_dim * 2 + e_vloc * e_dim * 2
     out["vocab_embedding_bwd"] = {"us": round(us, 2), "GBps": round(nbytes / us / 1e3, 1), "bytes": nbytes,
                                   "frac": round(nbytes / us / 1e3 / HBM_PEAK_GBPS, 3),
-                                  "note": "two launches: token order (cw_embed_sort_ids), then per-row sums and zeros for the rows without tokens"}
+                                  "note": "one launch from the unsorted ids (cw_embed_bwd_ids): sums and the zeros of the rows without tokens"}
     del tabs, dys_e
     # attention core of config 5: batch 4, 32 heads of 64, 2048 tokens, causal; FLOP counted on the
     # unmasked half only (4 b h s^2 d / 2 forward, 2.5 x that backward)
@@ -575,9 +575,9 @@ def mfma_rate_ceiling(lib, device):
 
 
 def stream_ceiling(device):
-    """torch's own copy kernel over the sizes of the LayerNorm / cross-entropy workloads (one read and one write of
-    the buffer size), sources rotated through more than 512 MiB, replayed from a HIP graph like the aux figures:
-    what a plain streaming kernel of these sizes reaches on this GPU."""
+    """torch's own copy and fill kernels over the sizes of the LayerNorm / cross-entropy /
+    embedding workloads, buffers rotated through more than 512 MiB, replayed from a HIP graph like the aux figures:
+    what plain streaming kernels of these sizes reach on this GPU."""
     import torch
     out = {}
     for mib, nbuf in ((32, 18), (64, 10), (196, 4)):
@@ -592,6 +592,13 @@ def stream_ceiling(device):
         us = graph_time_us(copy, 2 * nbuf)
         out["copy_%dMiB" % mib] = {"us": round(us, 2), "bytes": 4 * n, "GBps": round(4 * n / us / 1e3, 1),
                                    "frac": round(4 * n / us / 1e3 / HBM_PEAK_GBPS, 3)}
+
+        def fill():
+            i[0] += 1
+            src[i[0] % nbuf].zero_()
+        us = graph_time_us(fill, 2 * nbuf)
+        out["fill_%dMiB" % mib] = {"us": round(us, 2), "bytes": 2 * n, "GBps": round(2 * n / us / 1e3, 1),
+                                   "frac": round(2 * n / us / 1e3 / HBM_PEAK_GBPS, 3)}
         del src, dst
     return out
 
@@ -607,7 +614,7 @@ def main():
                          "power, so that clock and power have settled")
     ap.add_argument("--no-aux", action="store_true", help="skip the LayerNorm / CE kernels")
     ap.add_argument("--stream-ceiling", action="store_true",
-                    help="instead of the benchmark: plain torch reads (max) and copies of 32, 64 and 196 MiB buffers, "
+                    help="instead of the benchmark: plain torch copies and fills of 32, 64 and 196 MiB buffers, "
                          "rotated through more than 512 MiB, for a kernel trace of what streaming kernels of the "
                          "LayerNorm / cross-entropy sizes reach on this GPU")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
@@ -657,11 +664,11 @@ def main():
 
     # The bandwidth-bound kernels of the same path run first: the headline's warm-up and timed steps then find the
     # chip as a training loop would, busy and at its working clock, not waking up from idle.
-    aux = None if args.no_aux else bench_bandwidth_kernels(device)
-
+    # (The headline's operands are made before them: seconds of host work during which the GPU would fall asleep.)
     n_sets = 3  # 3 x 80 MiB of operands rotate so that no step finds its inputs in the Infinity Cache
     sets, bias = make_gemm_inputs(n_sets, device)
     outs = [torch.empty((M, N), dtype=torch.bfloat16, device=device) for _ in range(n_sets)]
+    aux = None if args.no_aux else bench_bandwidth_kernels(device)
     it = [0]
 
     def step():
