@@ -285,10 +285,10 @@ __global__ __launch_bounds__(256) void embed_bwd_generic_kernel(int64_t T_rows, 
 // kDirRows consecutive rows of the slice. It reads all ids (they stay in L2: every workgroup reads the same
 // 8 T bytes) and marks, per row, the tokens that select it in a bitmap in LDS. The rows that up to kDirHeavy
 // tokens select are dealt round-robin to the wavefronts, which sum a row's tokens in ascending token position
-// (what a stable sort by id would hand the sorted kernel), kDirBatch token rows in flight; the first batch of
-// loads is issued before any wavefront of the group starts on the zeros, so the reads do not queue behind
-// them in the compute unit's memory pipeline. The rows without tokens are then written as zeros, a fixed
-// share per wavefront. A row that more than kDirHeavy tokens select is left to the end and summed by all
+// (what a stable sort by id would hand the sorted kernel), kDirBatch token rows in flight; the row of a row's
+// first token (known from the marking pass, an LDS minimum) is requested before any wavefront of the group
+// starts on the zeros, so the reads do not queue behind them in the compute unit's memory pipeline. The rows
+// without tokens are then written as zeros, a fixed share per wavefront. A row that more than kDirHeavy tokens select is left to the end and summed by all
 // wavefronts together, each over its contiguous range of token positions, partial sums added in wavefront
 // order. Fixed orders throughout: bit-reproducible, no global atomics. Every row of the slice is written
 // exactly once, so the zeros cost no pass of their own, and no token order has to be made first.
@@ -401,6 +401,7 @@ __global__ __launch_bounds__(kDirWaves * 64) void embed_bwd_direct_kernel(int T_
     constexpr int kThreads = kDirWaves * 64;
     extern __shared__ uint32_t dir_bitmap[];  // [kDirRows][words]
     __shared__ int cnt[kDirRows];
+    __shared__ int first_tok[kDirRows];  // lowest token position of each row
     __shared__ float red[kDirWaves - 1][NVH * V][64];
     __shared__ uint16_t dir_queue[kDirWaves][64];  // tokens a wavefront is about to load
     const int tid = threadIdx.x, lane = tid & 63;
@@ -417,7 +418,10 @@ __global__ __launch_bounds__(kDirWaves * 64) void embed_bwd_direct_kernel(int T_
         idv[u] = T_rows > 0 ? ids[t < T_rows ? t : T_rows - 1] : 0;
     }
     for (int i = tid; i < kDirRows * words; i += kThreads) dir_bitmap[i] = 0u;
-    if (tid < kDirRows) cnt[tid] = 0;
+    if (tid < kDirRows) {
+        cnt[tid] = 0;
+        first_tok[tid] = 0x7fffffff;
+    }
     __syncthreads();
     for (int t0 = 0; t0 < T_rows; t0 += kDirIdsPerPass * kThreads) {
         if (t0 > 0) {
@@ -433,7 +437,8 @@ __global__ __launch_bounds__(kDirWaves * 64) void embed_bwd_direct_kernel(int T_
             const uint64_t r = (uint64_t)idv[u] - base;
             if (t < T_rows && r < rows_here) {
                 atomicOr(&dir_bitmap[(int)r * words + (t >> 5)], 1u << (t & 31));
-                atomicAdd(&cnt[(int)r], 1);  // integer counts: the order of the additions does not matter
+                atomicAdd(&cnt[(int)r], 1);  // integer counts and minima: the order of the updates does not matter
+                atomicMin(&first_tok[(int)r], t);
             }
         }
     }
@@ -456,15 +461,13 @@ __global__ __launch_bounds__(kDirWaves * 64) void embed_bwd_direct_kernel(int T_
     {
         raw16_t raw[kDirBatch][NV];
         if (first_row >= 0) {
+            // the row's first token is known from the marking pass: its loads go out without a walk over the bitmap
+            // (most rows have that one token); it leaves the bitmap while the row's first pass runs
             uint32_t* bm_row = dir_bitmap + first_row * words;
-            for (int wb = 0; wb < words && n_early < kDirBatch; wb += 64) {
-                const int wi = wb + lane;
-                uint32_t word = wi < words ? bm_row[wi] : 0u;
-                n_early += dir_take_tokens(word, wi, kDirBatch - n_early, queue + n_early);
-                if (wi < words) bm_row[wi] = word;
-            }
-#pragma unroll
-            for (int b = 0; b < kDirBatch; ++b) early[b] = __builtin_amdgcn_readfirstlane((int)queue[b < n_early ? b : 0]);
+            early[0] = __builtin_amdgcn_readfirstlane(first_tok[first_row]);
+            n_early = 1;
+            if (lane == 0) atomicAnd(&bm_row[early[0] >> 5], ~(1u << (early[0] & 31)));
+            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
             dir_columns<T, NV>(0, lane, E, col, acc);
             dir_load_rows<T, NV, kDirBatch>(d_out, ldo, early, n_early, col, raw);
         }
