@@ -34,6 +34,7 @@ constexpr int kWaves = 8;                 // wavefronts per block
 constexpr int kThreads = kWaves * 64;
 constexpr int kQPerWave = 32 * kQT;
 constexpr float kLazy = 8.0f;             // log2 of the largest probability taken against a stale reference
+constexpr float kNoKey = -1.0e30f;        // reference of a row that has met no live key yet (finite on purpose)
 constexpr int kQPerBlock = kWaves * kQPerWave;
 
 struct AttnArgs {
@@ -98,10 +99,14 @@ __global__ __launch_bounds__(kThreads, NP == 1 ? 2 : 1) void attn_fwd_kernel(con
         for (int dt = 0; dt < 2 * NP; ++dt)
 #pragma unroll
             for (int e = 0; e < 16; ++e) oacc[qt][dt][e] = 0.0f;
-    float m_run[kQT], l_run[kQT];  // reference of the exponentials (scale*log2e*s units); this lane's share of the running sum
+    // reference of the exponentials (scale*log2e*s units), the raw score above which it moves, this lane's share
+    // of the running sum
+    float m_run[kQT], m_thr[kQT], l_run[kQT];
+    const float inv_scale_log2e = 1.0f / a.scale_log2e;
 #pragma unroll
     for (int qt = 0; qt < kQT; ++qt) {
-        m_run[qt] = kNegBig;
+        m_run[qt] = kNoKey;
+        m_thr[qt] = (kNoKey + kLazy) * inv_scale_log2e;
         l_run[qt] = 0.0f;
     }
 
@@ -134,13 +139,16 @@ __global__ __launch_bounds__(kThreads, NP == 1 ? 2 : 1) void attn_fwd_kernel(con
 #pragma unroll
         for (int kb = 0; kb < 4 * NP; ++kb) asm volatile("" : "+v"(qf[qt][kb]));
 
-    for (int t = 0; t < n_tiles; ++t) {
-        lds_char* ks = lds + (t & 1) * kStage;
+    // One tile of 64 key rows out of LDS stage STAGE (a compile-time constant, so that every fragment read is
+    // lane offset + immediate: no address arithmetic in the loop); the loop below alternates the two stages.
+    auto tile_step = [&](int t, auto stage_c) {
+        constexpr int STAGE = decltype(stage_c)::value;
+        lds_char* ks = lds + STAGE * kStage;
         lds_char* vs = ks + NP * kImage;
         const int kv0 = t * kTile;
         if (t + 1 < n_tiles) {
             // the other stage was last read in the previous trip, which ended with a barrier
-            load_stage(kv0 + kTile, lds_addr + ((t + 1) & 1) * kStage);
+            load_stage(kv0 + kTile, lds_addr + (1 - STAGE) * kStage);
         }
 
         const bool active = !a.causal || kv0 <= qw0 + kQPerWave - 1;
@@ -186,19 +194,22 @@ __global__ __launch_bounds__(kThreads, NP == 1 ? 2 : 1) void attn_fwd_kernel(con
                     // when some row's maximum exceeds it by more than kLazy, i.e. a probability would pass
                     // 2^kLazy. With the true maximum as reference some row of the 32 moves in most tiles. The
                     // quotient O / l does not depend on the reference, and bf16 / fp16 keep their relative
-                    // precision at 2^kLazy.
-                    const float mx_s = mx * a.scale_log2e;
-                    if (__builtin_amdgcn_ballot_w64(mx_s > m_run[qt] + kLazy) != 0) {
-                        const float m_new = fmaxf(m_run[qt], mx_s);
-                        const float alpha = __builtin_amdgcn_exp2f(m_run[qt] - ((m_new == kNegBig) ? 0.0f : m_new));
+                    // precision at 2^kLazy. The test is one compare against m_thr = (m_run + kLazy) / (scale
+                    // log2 e), in the units of the raw scores. A row without a live key so far has the finite
+                    // reference kNoKey: its maximum, once it has one, is always above the threshold, and until
+                    // then its scores are -inf and its probabilities exp2(-inf - kNoKey) = 0.
+                    if (__builtin_amdgcn_ballot_w64(mx > m_thr[qt]) != 0) {
+                        const float m_new = fmaxf(m_run[qt], mx * a.scale_log2e);
+                        const float alpha = __builtin_amdgcn_exp2f(m_run[qt] - m_new);
                         l_run[qt] *= alpha;
 #pragma unroll
                         for (int dt = 0; dt < 2 * NP; ++dt)
 #pragma unroll
                             for (int e = 0; e < 16; ++e) oacc[qt][dt][e] *= alpha;
                         m_run[qt] = m_new;
+                        m_thr[qt] = (m_new + kLazy) * inv_scale_log2e;
                     }
-                    const float m_use = (m_run[qt] == kNegBig) ? 0.0f : m_run[qt];  // a row with no live key yet
+                    const float m_use = m_run[qt];
                     float p[16];
 #pragma unroll
                     for (int e = 0; e < 16; ++e)
@@ -207,7 +218,7 @@ __global__ __launch_bounds__(kThreads, NP == 1 ? 2 : 1) void attn_fwd_kernel(con
                     // probabilities, the values the second product uses.
                     pb[qt][0] = pack_slots<E>(p, 0);
                     pb[qt][1] = pack_slots<E>(p, 1);
-                    l_run[qt] += sum_slots<E>(pb[qt][1], sum_slots<E>(pb[qt][0], 0.0f));
+                    l_run[qt] = sum_slots<E>(pb[qt][1], sum_slots<E>(pb[qt][0], l_run[qt]));
                 }
                 // O^T += V^T P^T over the 32 kv rows of this half tile
 #pragma unroll
@@ -227,6 +238,10 @@ __global__ __launch_bounds__(kThreads, NP == 1 ? 2 : 1) void attn_fwd_kernel(con
         }
         dma_wait<0>();  // the next tile has landed (a third stage and loads two tiles ahead gained nothing)
         __syncthreads();
+    };
+    for (int t = 0; t < n_tiles; t += 2) {
+        tile_step(t, std::integral_constant<int, 0>{});
+        if (t + 1 < n_tiles) tile_step(t + 1, std::integral_constant<int, 1>{});
     }
 
     // finish: combine the two halves' sums, normalise, store
