@@ -268,19 +268,27 @@ def bench_bandwidth_kernels(device):
     return out
 
 
-def event_time_us(fn, iters, warmup):
-    """Average duration of fn() per call from events on the current stream."""
+def event_time_us(fn, iters, warmup, min_ms=150.0):
+    """Average duration of fn() per call from events on the current stream. A first pass of `iters` calls is a
+    pilot; the figure comes from a second pass long enough (min_ms) for the clock to have settled - a burst of 30
+    launches right after host-side set-up still runs on a chip that is waking up."""
     import torch
+
+    def timed(n):
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(n):
+            fn()
+        e1.record()
+        torch.cuda.synchronize()
+        return e0.elapsed_time(e1) * 1e3 / n
+
     for _ in range(warmup):
         fn()
     torch.cuda.synchronize()
-    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-    e0.record()
-    for _ in range(iters):
-        fn()
-    e1.record()
-    torch.cuda.synchronize()
-    return e0.elapsed_time(e1) * 1e3 / iters
+    pilot = timed(iters)
+    n = int(min_ms * 1e3 / max(pilot, 1.0)) + 1
+    return timed(n) if n > iters else pilot
 
 
 def bench_other_configs(device, sets):

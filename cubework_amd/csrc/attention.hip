@@ -239,10 +239,12 @@ __global__ __launch_bounds__(kThreads, NP == 1 ? 2 : 1) void attn_fwd_kernel(con
         dma_wait<0>();  // the next tile has landed (a third stage and loads two tiles ahead gained nothing)
         __syncthreads();
     };
-    for (int t = 0; t < n_tiles; t += 2) {
+    int t = 0;
+    for (; t + 1 < n_tiles; t += 2) {
         tile_step(t, std::integral_constant<int, 0>{});
-        if (t + 1 < n_tiles) tile_step(t + 1, std::integral_constant<int, 1>{});
+        tile_step(t + 1, std::integral_constant<int, 1>{});
     }
+    if (t < n_tiles) tile_step(t, std::integral_constant<int, 0>{});
 
     // finish: combine the two halves' sums, normalise, store
 #pragma unroll
