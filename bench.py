@@ -161,7 +161,7 @@ def make_gemm_inputs(n_sets, device):
     return sets, bias
 
 
-def graph_time_us(fn, calls, replays=3):
+def graph_time_us(fn, calls, replays=3, min_ms=100.0):
     """Average duration of one fn() call when `calls` of them are replayed from
     a HIP graph: the host cost of the Python wrappers (tens of microseconds,
     more than these kernels run) stays outside the timed region, which is
@@ -180,13 +180,19 @@ def graph_time_us(fn, calls, replays=3):
             fn()
     graph.replay()
     torch.cuda.synchronize()
-    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-    e0.record()
-    for _ in range(replays):
-        graph.replay()
-    e1.record()
-    torch.cuda.synchronize()
-    return e0.elapsed_time(e1) * 1e3 / (replays * calls)
+
+    def timed(n):
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(n):
+            graph.replay()
+        e1.record()
+        torch.cuda.synchronize()
+        return e0.elapsed_time(e1) * 1e3 / (n * calls)
+
+    pilot = timed(replays)
+    n = int(min_ms * 1e3 / max(pilot * calls, 1.0)) + 1  # replays for min_ms of work: the rate the chip sustains
+    return timed(n) if n > replays else pilot
 
 
 def bench_bandwidth_kernels(device):
