@@ -152,14 +152,17 @@ __global__ __launch_bounds__(kThreads, 1) void attn_dq_kernel(const BwdArgs a) {
 #pragma unroll
     for (int kb = 0; kb < 4 * NP; ++kb) asm volatile("" : "+v"(qf[kb]), "+v"(dof[kb]));
 
-    for (int t = 0; t < n_tiles; ++t) {
-        lds_char* k_rows = lds + (t & 1) * kStage;
+    // One tile of 64 key rows out of LDS stage STAGE, a compile-time constant so that every fragment read is lane
+    // offset + immediate (no address arithmetic in the loop); the loop below alternates the two stages.
+    auto tile_step = [&](int t, auto stage_c) {
+        constexpr int STAGE = decltype(stage_c)::value;
+        lds_char* k_rows = lds + STAGE * kStage;
         lds_char* k_tr = k_rows + NP * kImage;
         lds_char* v_rows = k_rows + 2 * NP * kImage;
         const int kv0 = t * kTile;
         if (t + 1 < n_tiles) {
             // the other stage was last read in the previous trip, which ended with a barrier
-            load_stage(kv0 + kTile, lds_addr + ((t + 1) & 1) * kStage);
+            load_stage(kv0 + kTile, lds_addr + (1 - STAGE) * kStage);
         }
         const bool active = !a.causal || kv0 <= qw0 + kRowsPerWave - 1;
         if (active) {
@@ -200,10 +203,19 @@ __global__ __launch_bounds__(kThreads, 1) void attn_dq_kernel(const BwdArgs a) {
                 }
             };
             half_tile(std::integral_constant<int, 0>{});
-            half_tile(std::integral_constant<int, 1>{});
+            // the second 32 key rows of a tile that starts on the wavefront's diagonal are wholly masked
+            if (!a.causal || kv0 + 32 <= qw0 + kRowsPerWave - 1) half_tile(std::integral_constant<int, 1>{});
         }
         dma_wait<0>();
         __syncthreads();
+    };
+    {
+        int t = 0;
+        for (; t + 1 < n_tiles; t += 2) {
+            tile_step(t, std::integral_constant<int, 0>{});
+            tile_step(t + 1, std::integral_constant<int, 1>{});
+        }
+        if (t < n_tiles) tile_step(t, std::integral_constant<int, 0>{});
     }
     if (qi < S) {
         uint16_t* grow = a.dq + b * a.gb + (int64_t)qi * a.gs + h * a.gh;
@@ -307,8 +319,10 @@ __global__ __launch_bounds__(NW * 64, 1) void attn_dkdv_kernel(const BwdArgs a) 
 #pragma unroll
         for (int kb = 0; kb < 4 * NP; ++kb) asm volatile("" : "+v"(kf[kg][kb]), "+v"(vf[kg][kb]));  // arrived before the loop
 
-    for (int t = first_tile; t < n_tiles; ++t) {
-        lds_char* stg = lds + ((t - first_tile) & 1) * kDkdvStage;
+    // One tile of 64 query rows out of LDS stage STAGE (compile-time: fragment reads are lane offset + immediate)
+    auto tile_step = [&](int t, auto stage_c) {
+        constexpr int STAGE = decltype(stage_c)::value;
+        lds_char* stg = lds + STAGE * kDkdvStage;
         lds_char* q_rows = stg;
         lds_char* q_tr = stg + NP * kImage;
         lds_char* g_rows = stg + 2 * NP * kImage;
@@ -317,7 +331,7 @@ __global__ __launch_bounds__(NW * 64, 1) void attn_dkdv_kernel(const BwdArgs a) 
         const int q0 = t * kTile;
         if (t + 1 < n_tiles) {
             // the other stage was last read in the previous trip, which ended with a barrier
-            load_stage(q0 + kTile, lds_addr + ((t + 1 - first_tile) & 1) * kDkdvStage);
+            load_stage(q0 + kTile, lds_addr + (1 - STAGE) * kDkdvStage);
             load_stats(q0 + kTile);
         }
         // the wavefront's keys kw0 .. kw0 + kKeysPerWave - 1 see queries >= kw0 only
@@ -399,9 +413,17 @@ __global__ __launch_bounds__(NW * 64, 1) void attn_dkdv_kernel(const BwdArgs a) 
             q_tile(std::integral_constant<int, 0>{});
             q_tile(std::integral_constant<int, 1>{});
         }
-        if (t + 1 < n_tiles) store_stats(lds + ((t + 1 - first_tile) & 1) * kDkdvStage);
+        if (t + 1 < n_tiles) store_stats(lds + (1 - STAGE) * kDkdvStage);
         dma_wait<0>();
         __syncthreads();
+    };
+    {
+        int t = first_tile;
+        for (; t + 1 < n_tiles; t += 2) {
+            tile_step(t, std::integral_constant<int, 0>{});
+            tile_step(t + 1, std::integral_constant<int, 1>{});
+        }
+        if (t < n_tiles) tile_step(t, std::integral_constant<int, 0>{});
     }
 #pragma unroll
     for (int kg = 0; kg < KG; ++kg) {
