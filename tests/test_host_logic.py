@@ -166,3 +166,23 @@ def test_partition_batch():
     assert torch.equal(out["a"], x[2:])
     initialize("1d", 4)
     assert cube_nn.partition_batch(x) is x
+
+
+def test_bench_refuses_more_than_one_gpu_and_has_no_cpu_path():
+    """bench.py measures one rank's share on one GPU: `--gpus 2` (or a WORLD_SIZE above 1) ends with a message and
+    status 2 before anything touches a device, and on a host without a GPU the default invocation ends with
+    status 3 instead of timing a CPU stand-in."""
+    import os
+    import subprocess
+    import sys
+
+    bench = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "bench.py")
+    r = subprocess.run([sys.executable, bench, "--gpus", "2"], capture_output=True, text=True, timeout=120)
+    assert r.returncode == 2 and "ONE GPU" in r.stderr and r.stdout.strip() == ""
+    env_two = dict(os.environ, WORLD_SIZE="2")
+    r = subprocess.run([sys.executable, bench], capture_output=True, text=True, timeout=120, env=env_two)
+    assert r.returncode == 2
+    if not torch.cuda.is_available():
+        r = subprocess.run([sys.executable, bench, "--steps", "1", "--warmup", "0"], capture_output=True, text=True,
+                           timeout=300)
+        assert r.returncode == 3 and "no CPU fallback" in r.stderr and r.stdout.strip() == ""
