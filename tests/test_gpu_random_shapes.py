@@ -104,3 +104,55 @@ def test_random_layernorm(shape):
     assert_parity(dx, dx_ref, torch.bfloat16, "ln dx %s" % (shape,))
     assert_parity(dgam, dg_ref, torch.float32, "ln dgamma %s" % (shape,))
     assert_parity(dbet, db_ref, torch.float32, "ln dbeta %s" % (shape,))
+
+
+def _embedding_cases():
+    rng = random.Random(4242)
+    cases = []
+    for _ in range(14):
+        dtype_i = rng.randint(0, 2)
+        vec = 4 if dtype_i == 1 else 8
+        cases.append((rng.choice([1, 2, 31, 64, 65, 500, 2049, 8192, 16384]) if rng.random() < 0.5 else rng.randint(1, 16384),
+                      vec * rng.randint(1, 520), rng.randint(1, 3000), rng.randint(0, 5000), dtype_i,
+                      rng.choice(["uniform", "hot", "one_id", "zipf"]), rng.random() < 0.5))
+    return cases
+
+
+@pytest.mark.parametrize("case", _embedding_cases())
+def test_random_embedding_backward_from_ids(case):
+    """cw_embed_bwd_ids on drawn shapes and id distributions (uniform over a vocabulary wider than the slice, one hot
+    id for every third token, a single id for all tokens, Zipf-like frequencies), with and without a skipped row:
+    float64 sums within the dtype's bar, rows without tokens exactly zero, two calls bit-identical, and equal bit
+    for bit to the token-order path wherever no row has more than one token (where neither path adds anything)."""
+    from cubework_amd import ops
+
+    T, E, rows, start, dtype_i, dist, with_skip = case
+    dtype = [torch.bfloat16, torch.float32, torch.float16][dtype_i]
+    g = torch.Generator().manual_seed(T * 31 + E)
+    vocab = start + rows + 200
+    if dist == "one_id":
+        ids = torch.full((T,), start + rows // 2, dtype=torch.int64)
+    elif dist == "zipf":
+        u = torch.rand((T,), generator=g)
+        ids = (start - 50 + ((rows + 100) * u ** 3)).long().clamp(0, vocab - 1)
+    else:
+        ids = torch.randint(max(0, start - 100), vocab, (T,), generator=g)
+        if dist == "hot":
+            ids[::3] = start + min(7, rows - 1)
+    skip = min(3, rows - 1) if with_skip else -1
+    d_out = randn((T, E), dtype, T + 5)
+    got = ops.embedding_bwd(ids.to(DEV), d_out.to(DEV), rows, start, skip)
+    again = ops.embedding_bwd(ids.to(DEV), d_out.to(DEV), rows, start, skip)
+    torch.cuda.synchronize()
+    assert torch.equal(got, again), "fixed summation order: bit-reproducible"
+    local = ids - start
+    live = (local >= 0) & (local < rows) & (local != skip)
+    want = torch.zeros((rows, E), dtype=torch.float64).index_add_(0, local[live], d_out.double()[live])
+    assert_parity(got, want, dtype, "embedding d_weight from ids %s" % (case,))
+    untouched = torch.ones(rows, dtype=torch.bool)
+    untouched[local[live]] = False
+    assert (got.cpu()[untouched] == 0).all(), "rows without tokens (and the skipped row) are exactly zero"
+    counts = torch.bincount(local[live], minlength=rows)
+    if int(counts.max()) <= 1:
+        via = ops.embedding_bwd(ids.to(DEV), d_out.to(DEV), rows, start, skip, via_token_order=True)
+        assert torch.equal(got, via)
