@@ -282,7 +282,7 @@ __global__ __launch_bounds__(256) void embed_bwd_generic_kernel(int64_t T_rows, 
 }
 
 // Backward straight from the unsorted ids, one launch, for batches of up to kDirMaxTokens tokens. A workgroup owns
-// kDirRows consecutive rows of the slice. It reads all ids (they stay in L2: every workgroup reads the same
+// up to kDirRows rows of the slice, interleaved with the other workgroups' (row b, b + G, b + 2 G, ...). It reads all ids (they stay in L2: every workgroup reads the same
 // 8 T bytes) and marks, per row, the tokens that select it in a bitmap in LDS. The rows that up to kDirHeavy
 // tokens select are dealt round-robin to the wavefronts, which sum a row's tokens in ascending token position
 // (what a stable sort by id would hand the sorted kernel), kDirBatch token rows in flight; the row of a row's
@@ -394,7 +394,7 @@ template <typename T>
 __global__ __launch_bounds__(kDirWaves * 64) void embed_bwd_direct_kernel(int T_rows, int64_t E, const int64_t* __restrict__ ids,
                                                                           int64_t vocab_start, int64_t V_loc, int64_t skip_row,
                                                                           const T* __restrict__ d_out, int64_t ldo,
-                                                                          T* __restrict__ d_weight, int64_t ldw) {
+                                                                          T* __restrict__ d_weight, int64_t ldw, int log2_groups) {
     constexpr int V = elem<T>::kVec;
     constexpr int NV = 4;   // column vectors per lane and pass of a row a wavefront sums alone
     constexpr int NVH = 2;  // the same for a row all wavefronts share
@@ -407,9 +407,11 @@ __global__ __launch_bounds__(kDirWaves * 64) void embed_bwd_direct_kernel(int T_
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int words = (T_rows + 31) >> 5;
-    const int64_t r0 = (int64_t)blockIdx.x * kDirRows;
-    const uint64_t base = (uint64_t)vocab_start + (uint64_t)r0;
-    const uint64_t rows_here = (uint64_t)(V_loc - r0 < kDirRows ? V_loc - r0 : kDirRows);
+    // Row ownership is interleaved: workgroup b of G = 2^log2_groups owns rows b, b + G, b + 2 G, ... (at most
+    // kDirRows of them). Frequent tokens have neighbouring ids (the low ids of a BPE vocabulary): consecutive rows
+    // per workgroup would hand one workgroup most of the batch's tokens.
+    const uint64_t group_mask = ((uint64_t)1 << log2_groups) - 1;
+    auto row_of = [&](int j) { return (int64_t)blockIdx.x + ((int64_t)j << log2_groups); };
     // the first ids are on their way while the bitmap is cleared
     int64_t idv[kDirIdsPerPass];
 #pragma unroll
@@ -434,8 +436,9 @@ __global__ __launch_bounds__(kDirWaves * 64) void embed_bwd_direct_kernel(int T_
 #pragma unroll
         for (int u = 0; u < kDirIdsPerPass; ++u) {
             const int t = t0 + tid + u * kThreads;
-            const uint64_t r = (uint64_t)idv[u] - base;
-            if (t < T_rows && r < rows_here) {
+            const uint64_t local = (uint64_t)idv[u] - (uint64_t)vocab_start;  // below V_loc exactly for ids of the slice
+            const uint64_t r = local >> log2_groups;
+            if (t < T_rows && local < (uint64_t)V_loc && (local & group_mask) == (uint64_t)blockIdx.x) {
                 atomicOr(&dir_bitmap[(int)r * words + (t >> 5)], 1u << (t & 31));
                 atomicAdd(&cnt[(int)r], 1);  // integer counts and minima: the order of the updates does not matter
                 atomicMin(&first_tok[(int)r], t);
@@ -444,10 +447,10 @@ __global__ __launch_bounds__(kDirWaves * 64) void embed_bwd_direct_kernel(int T_
     }
     __syncthreads();
     int my_cnt = lane < kDirRows ? cnt[lane] : 0;
-    if (r0 + lane == skip_row) my_cnt = 0;  // its tokens are ignored: the row is written as zeros
+    if (row_of(lane) == skip_row) my_cnt = 0;  // its tokens are ignored: the row is written as zeros
     uint64_t light = __ballot(my_cnt > 0 && my_cnt <= kDirHeavy);  // bit j: row j is summed by one wavefront
     const uint64_t heavy = __ballot(my_cnt > kDirHeavy);
-    const uint64_t empty = __ballot(my_cnt == 0 && (uint64_t)lane < rows_here);
+    const uint64_t empty = __ballot(my_cnt == 0 && lane < kDirRows && row_of(lane) < V_loc);
     for (int k = 0; k < wave && light != 0ull; ++k) light &= light - 1;  // this wavefront's first: the wave-th set bit
 
     // this wavefront's first row with tokens: the first batch of its loads goes out ahead of all zeros
@@ -478,7 +481,7 @@ __global__ __launch_bounds__(kDirWaves * 64) void embed_bwd_direct_kernel(int T_
     // wavefronts without such rows are writing zeros meanwhile
     for (bool first = true; light != 0ull; first = false) {
         const int j = __builtin_ctzll(light);
-        T* dst = d_weight + (r0 + j) * ldw;
+        T* dst = d_weight + row_of(j) * ldw;
         uint32_t* bm_row = dir_bitmap + j * words;
         for (int64_t c0 = 0; c0 < E; c0 += (int64_t)64 * V * NV) {
             if (!(first && c0 == 0)) dir_columns<T, NV>(c0, lane, E, col, acc);  // else: the sums of the first loads
@@ -493,27 +496,20 @@ __global__ __launch_bounds__(kDirWaves * 64) void embed_bwd_direct_kernel(int T_
         }
         for (int k = 0; k < kDirWaves && light != 0ull; ++k) light &= light - 1;
     }
-    // zeros: the empty rows among this wavefront's kDirRowsPerWave
-#pragma unroll
-    for (int q = 0; q < kDirRowsPerWave; ++q) {
-        const int j = wave * kDirRowsPerWave + q;
-        if (!((empty >> j) & 1ull)) continue;
-        T* dst = d_weight + (r0 + j) * ldw;
-        for (int64_t c = (int64_t)lane * V; c < E; c += 64 * V) store_raw_stream(dst + c, raw16_t{0u, 0u, 0u, 0u});
-    }
-    // rows that many tokens select: every wavefront sums the tokens of its range of positions
+    // rows that many tokens select, before the zeros (the longest job of a workgroup goes first): every wavefront
+    // sums the tokens of its range of positions
     const int words_per_wave = (words + kDirWaves - 1) / kDirWaves;
     const int w_lo = wave * words_per_wave;
     const int w_hi = w_lo + words_per_wave < words ? w_lo + words_per_wave : words;
     for (uint64_t todo = heavy; todo != 0ull; todo &= todo - 1) {
         const int j = __builtin_ctzll(todo);
-        T* dst = d_weight + (r0 + j) * ldw;
+        T* dst = d_weight + row_of(j) * ldw;
         const uint32_t* bm_row = dir_bitmap + j * words;
         for (int64_t c0 = 0; c0 < E; c0 += (int64_t)64 * V * NVH) {
             int64_t colh[NVH];
             float acch[NVH][V];
             dir_columns<T, NVH>(c0, lane, E, colh, acch);
-            dir_sum_tokens<T, NVH, 2 * kDirBatch>(bm_row, w_lo, w_hi, lane, queue, d_out, ldo, colh, acch);
+            dir_sum_tokens<T, NVH, 4 * kDirBatch>(bm_row, w_lo, w_hi, lane, queue, d_out, ldo, colh, acch);
             if (wave > 0) {
 #pragma unroll
                 for (int v = 0; v < NVH; ++v)
@@ -532,6 +528,14 @@ __global__ __launch_bounds__(kDirWaves * 64) void embed_bwd_direct_kernel(int T_
             }
             __syncthreads();
         }
+    }
+    // zeros: the empty rows among this wavefront's kDirRowsPerWave
+#pragma unroll
+    for (int q = 0; q < kDirRowsPerWave; ++q) {
+        const int j = wave * kDirRowsPerWave + q;
+        if (!((empty >> j) & 1ull)) continue;
+        T* dst = d_weight + row_of(j) * ldw;
+        for (int64_t c = (int64_t)lane * V; c < E; c += 64 * V) store_raw_stream(dst + c, raw16_t{0u, 0u, 0u, 0u});
     }
 }
 
@@ -583,9 +587,11 @@ int bwd_direct_impl(int64_t T_rows, int64_t E, const int64_t* ids, int64_t vocab
     const int lds = kDirRows * words * (int)sizeof(uint32_t);
     if (const int rc = ensure_dynamic_lds((const void*)embed_bwd_direct_kernel<T>, lds,
                                           "embed_bwd_direct_kernel"); rc != CW_OK) return rc;
-    const int64_t blocks = (V_loc + kDirRows - 1) / kDirRows;
-    hipLaunchKernelGGL(embed_bwd_direct_kernel<T>, dim3((unsigned)blocks), dim3(kDirWaves * 64), lds, s, (int)T_rows, E, ids,
-                       vocab_start, V_loc, skip_row, (const T*)d_out, ldo, (T*)d_weight, ldw);
+    // a power of two of workgroups, each with between kDirRows / 2 + 1 and kDirRows interleaved rows
+    int log2_groups = 0;
+    while (((int64_t)kDirRows << log2_groups) < V_loc) ++log2_groups;
+    hipLaunchKernelGGL(embed_bwd_direct_kernel<T>, dim3(1u << log2_groups), dim3(kDirWaves * 64), lds, s, (int)T_rows, E, ids,
+                       vocab_start, V_loc, skip_row, (const T*)d_out, ldo, (T*)d_weight, ldw, log2_groups);
     return check_launch("embed_bwd_direct_kernel");
 }
 
