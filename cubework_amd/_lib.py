@@ -39,6 +39,8 @@ SIGNATURES = {
     "cw_multi_norm_partials": (_int, [_int, _pp, _ptr, _ptr, _ptr, _f32, _ptr, _ptr, _i64, _int, _ptr]),
     "cw_clip_coef": (_int, [_int, _ptr, _f32, _f32, _f32, _ptr, _ptr]),
     "cw_multi_scale": (_int, [_int, _pp, _ptr, _ptr, _int, _ptr]),
+    "cw_multi_norm_partial_count": (_i64, [_int, _ptr]),
+    "cw_clip_scale": (_int, [_int, _pp, _ptr, _int, _int, _ptr, _i64, _ptr, _f32, _f32, _f32, _ptr, _ptr]),
     "cw_embed_fwd": (_int, [_i64, _i64, _ptr, _i64, _i64, _ptr, _i64, _ptr, _i64, _int, _ptr]),
     "cw_embed_sort_workspace_bytes": (_i64, [_i64]),
     "cw_embed_sort_ids": (_int, [_i64, _ptr, _i64, _i64, _ptr, _ptr, _ptr, _i64, _ptr]),

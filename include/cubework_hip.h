@@ -370,9 +370,14 @@ int cw_embed_bwd_ids(int64_t T, int64_t E, const int64_t* ids, int64_t vocab_sta
  * (cubework/utils/clip_grad.py:31-46); group 1 = parameters tagged with NUM_PARTITIONS, whose sum
  * the caller all-reduces and divides by the tensor-parallel size (:48-49) before taking the root.
  * grads / numels / factors / groups are HOST arrays; all tensors share io_dtype and are contiguous.
- * Two deterministic stages through `workspace` (cw_multi_norm_workspace_bytes), no atomics.
+ * Two deterministic stages through `workspace` (cw_multi_norm_workspace_bytes), no atomics: the first leaves
+ * cw_multi_norm_partial_count (value, group) fp32 pairs at the start of `workspace`, the second combines them
+ * into out2. With out2 == NULL the second stage is left out and the pairs are the result, for cw_clip_scale
+ * (a caller with several dtypes gives each call the workspace address behind the previous call's pairs, so
+ * that all pairs are contiguous).
  */
 int64_t cw_multi_norm_workspace_bytes(int n_tensors, const int64_t* numels);
+int64_t cw_multi_norm_partial_count(int n_tensors, const int64_t* numels);
 int cw_multi_norm_partials(int n_tensors, const void* const* grads, const int64_t* numels,
                            const float* factors, const unsigned char* groups, float norm_type,
                            float* out2, void* workspace, int64_t workspace_bytes,
@@ -394,6 +399,18 @@ int cw_clip_coef(int n_sets, const float* sets, float tp_scale, float norm_type,
  */
 int cw_multi_scale(int n_tensors, void* const* grads, const int64_t* numels, const float* coef,
                    int io_dtype, void* stream);
+/*
+ * cw_clip_coef and cw_multi_scale in one launch (clip_grad.py:46-50,57-68): every workgroup of the scaling
+ * launch combines `sets` ([n_sets][2] finished results, as for cw_clip_coef; n_sets may be 0) and `partials`
+ * (n_partials unfinished (value, group) pairs left by cw_multi_norm_partials calls with out2 == NULL; may be 0)
+ * in one fixed order, takes the root and the clamp, and multiplies its share of the gradients; out2 receives
+ * (total norm, coefficient) as from cw_clip_coef. With partials, a clipping call that needs no exchange between
+ * ranks is two launches per dtype. out2 must not overlap sets or partials; a caller with several dtypes calls
+ * it once per dtype with the same sets / partials (out2 is rewritten with the same values).
+ */
+int cw_clip_scale(int n_tensors, void* const* grads, const int64_t* numels, int io_dtype, int n_sets,
+                  const float* sets, int64_t n_partials, const float* partials, float tp_scale,
+                  float norm_type, float max_norm, float* out2, void* stream);
 
 /* ---- attention core ------------------------------------------------------ */
 /*

@@ -145,3 +145,83 @@ def test_clip_grad_norm_nonfinite_gradients(norm_type, bad):
         p.grad = k
     with pytest.raises(RuntimeError):
         clip_grad_norm(ours, 1.0, norm_type, error_if_nonfinite=True)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("norm_type", [2.0, float("inf"), 3.0])
+def test_clip_scale_from_partials_equals_the_separate_launches(dtype, norm_type):
+    """cw_clip_scale on the unfinished block partials (two launches) against cw_multi_norm_partials with its
+    finalize, cw_clip_coef and cw_multi_scale (four launches): both add the partials in the same order, so the
+    norm, the coefficient and every scaled gradient agree to the bit. 70 tensors: two launches of the scaling."""
+    import ctypes as C
+    from cubework_amd import _lib, ops
+
+    lib = _lib.load()
+    shapes = [(300000,), (65536,), (7,), (1000, 33)] + [(129, 17)] * 66
+    a = [randn(s, dtype, 40 + i, std=0.3 + 0.05 * (i % 7)).to(DEV) for i, s in enumerate(shapes)]
+    b = [t.clone() for t in a]
+    n = len(a)
+    numels = (C.c_int64 * n)(*[t.numel() for t in a])
+    numels_p = C.cast(numels, C.c_void_p)
+    factors = (C.c_float * n)(*[float(1 + i % 3) for i in range(n)])
+    groups = (C.c_ubyte * n)(*[i % 2 for i in range(n)])
+    code = ops._dtype_code(a[0])
+    count = lib.cw_multi_norm_partial_count(n, numels_p)
+    assert count == 5 + 1 + 1 + 1 + 66
+    assert lib.cw_multi_norm_workspace_bytes(n, numels_p) == 8 * count
+    stream = ops._stream()
+
+    def tables(ts):
+        return (C.c_void_p * n)(*[t.data_ptr() for t in ts])
+
+    ws_a = torch.empty(2 * count, dtype=torch.float32, device=DEV)
+    sets = torch.empty(2, dtype=torch.float32, device=DEV)
+    out_a = torch.empty(2, dtype=torch.float32, device=DEV)
+    pa = tables(a)
+    assert lib.cw_multi_norm_partials(n, pa, numels_p, C.cast(factors, C.c_void_p), C.cast(groups, C.c_void_p), norm_type,
+                                      sets.data_ptr(), ws_a.data_ptr(), 8 * count, code, stream) == 0
+    assert lib.cw_clip_coef(1, sets.data_ptr(), 0.5, norm_type, 0.25, out_a.data_ptr(), stream) == 0
+    assert lib.cw_multi_scale(n, pa, numels_p, out_a[1:].data_ptr(), code, stream) == 0
+
+    ws_b = torch.full((2 * count,), float("nan"), dtype=torch.float32, device=DEV)
+    out_b = torch.empty(2, dtype=torch.float32, device=DEV)
+    pb = tables(b)
+    assert lib.cw_multi_norm_partials(n, pb, numels_p, C.cast(factors, C.c_void_p), C.cast(groups, C.c_void_p), norm_type,
+                                      None, ws_b.data_ptr(), 8 * count, code, stream) == 0
+    assert lib.cw_clip_scale(n, pb, numels_p, code, 0, None, count, ws_b.data_ptr(), 0.5, norm_type, 0.25,
+                             out_b.data_ptr(), stream) == 0
+    torch.cuda.synchronize()
+    assert torch.equal(ws_a, ws_b)
+    assert torch.equal(out_a, out_b), (out_a, out_b)
+    assert 0.0 < out_a[1].item() < 1.0
+    for x, y in zip(a, b):
+        assert torch.equal(x, y)
+
+    # finished sets and unfinished partials together: (sets + partials) of the same gradients count them twice
+    out_c = torch.empty(2, dtype=torch.float32, device=DEV)
+    assert lib.cw_clip_scale(0, None, None, code, 1, sets.data_ptr(), count, ws_b.data_ptr(), 0.5, norm_type, 1e9,
+                             out_c.data_ptr(), stream) == 0
+    torch.cuda.synchronize()
+    if norm_type == float("inf"):
+        assert out_c[0].item() == out_a[0].item()
+    else:
+        want = out_a[0].double().item() * 2.0 ** (1.0 / norm_type)
+        assert abs(out_c[0].item() - want) <= 1e-5 * want
+    assert out_c[1].item() == 1.0
+
+
+def test_clip_scale_argument_checks():
+    from cubework_amd import _lib
+
+    lib = _lib.load()
+    out = torch.empty(2, dtype=torch.float32, device=DEV)
+    assert lib.cw_clip_scale(0, None, None, 0, 65, None, 0, None, 1.0, 2.0, 1.0, out.data_ptr(), None) == -1
+    assert lib.cw_clip_scale(0, None, None, 0, 1, None, 0, None, 1.0, 2.0, 1.0, out.data_ptr(), None) == -1
+    assert lib.cw_clip_scale(0, None, None, 0, 0, None, 3, None, 1.0, 2.0, 1.0, out.data_ptr(), None) == -1
+    assert lib.cw_clip_scale(0, None, None, 0, 0, None, 0, None, 1.0, 2.0, 1.0, None, None) == -1
+    assert lib.cw_clip_scale(0, None, None, 0, 0, None, 0, None, 1.0, -2.0, 1.0, out.data_ptr(), None) == -1
+    assert lib.cw_clip_scale(0, None, None, 7, 0, None, 0, None, 1.0, 2.0, 1.0, out.data_ptr(), None) == -1
+    # no gradients at all: norm 0, coefficient 1
+    assert lib.cw_clip_scale(0, None, None, 0, 0, None, 0, None, 1.0, 2.0, 1.0, out.data_ptr(), None) == 0
+    torch.cuda.synchronize()
+    assert out.tolist() == [0.0, 1.0]
