@@ -226,7 +226,7 @@ __global__ __launch_bounds__(kThreads, 1) void attn_dq_kernel(const BwdArgs a) {
 
 // ---- dK, dV -----------------------------------------------------------------
 // LDS per stage: Q row images, Q transpose images, dO row images, dO transpose images (NP = head size / 64
-// panels of each), L*log2e and D of the 64 rows. NW wavefronts of 32 key rows: 8 at head size 64; 4 at 128,
+// panels of each), L*log2e and -D of the 64 rows. NW wavefronts of 32 key rows: 8 at head size 64; 4 at 128,
 // where a wavefront's accumulators and fragments need more than the 256 registers that 8 would leave it.
 template <int NP>
 constexpr int dkdv_stage_bytes() { return 4 * NP * kImage + 2 * kTile * 4; }
@@ -287,12 +287,12 @@ __global__ __launch_bounds__(NW * 64, 1) void attn_dkdv_kernel(const BwdArgs a) 
     TileDma<NW * 64> dma;
     dma.init(tid);
     const uint32_t lds_addr = (uint32_t)(uintptr_t)lds;
-    // threads 0..63: L of tile row tid (stored times log2e); 64..127: D of tile row tid - 64. Every thread
+    // threads 0..63: L of tile row tid (stored times log2e); 64..127: D of tile row tid - 64 (stored negated). Every thread
     // loads (no branch around the load: the value is not needed before the tile it belongs to is stored,
     // and a wait inside a branch would cover the tile prefetch issued just before); the rest discard.
     float stat = 0.0f;
     const float* statp = tid < kTile ? lsep : dltp;
-    const float stat_mul = tid < kTile ? kLog2e : 1.0f;
+    const float stat_mul = tid < kTile ? kLog2e : -1.0f;  // D is stored negated: it starts the dP accumulators
     auto load_stats = [&](int q0) {
         int row = q0 + (tid & (kTile - 1));
         row = row < S ? row : S - 1;
@@ -345,14 +345,20 @@ __global__ __launch_bounds__(NW * 64, 1) void attn_dkdv_kernel(const BwdArgs a) 
             const int hi = S - q0 - 4 * half;
             auto q_tile = [&](auto qt_c) {
                 constexpr int qt = decltype(qt_c)::value;
+                // the dP accumulators start at -D of their query rows (32 qt + 8 g + 4 half + {0..3}), so that the
+                // products leave dP - D
                 f32x16_t s_acc[KG], dp_acc[KG];
 #pragma unroll
-                for (int kg = 0; kg < KG; ++kg)
+                for (int kg = 0; kg < KG; ++kg) {
 #pragma unroll
-                    for (int e = 0; e < 16; ++e) {
-                        s_acc[kg][e] = 0.0f;
-                        dp_acc[kg][e] = 0.0f;
+                    for (int e = 0; e < 16; ++e) s_acc[kg][e] = 0.0f;
+#pragma unroll
+                    for (int g = 0; g < 4; ++g) {
+                        const f32x4_t dl = *(__attribute__((address_space(3))) const f32x4_t*)(stats + (kTile + 32 * qt + 8 * g) * 4);
+#pragma unroll
+                        for (int i = 0; i < 4; ++i) dp_acc[kg][4 * g + i] = dl[i];
                     }
+                }
 #pragma unroll
                 for (int kb = 0; kb < 4 * NP; ++kb) {
                     const bf16x8_t qa = read_rows<32 * qt>(q_rows + (kb >> 2) * kImage, ro, kb & 3);
@@ -369,14 +375,13 @@ __global__ __launch_bounds__(NW * 64, 1) void attn_dkdv_kernel(const BwdArgs a) 
                     float p[16], ds[16];
 #pragma unroll
                     for (int g = 0; g < 4; ++g) {
-                        // L*log2e and D of query rows 32 qt + 8 g + 4 half + {0..3}
+                        // L*log2e of query rows 32 qt + 8 g + 4 half + {0..3}
                         const f32x4_t l2 = *(__attribute__((address_space(3))) const f32x4_t*)(stats + (32 * qt + 8 * g) * 4);
-                        const f32x4_t dl = *(__attribute__((address_space(3))) const f32x4_t*)(stats + (kTile + 32 * qt + 8 * g) * 4);
 #pragma unroll
                         for (int i = 0; i < 4; ++i) {
                             const int e = 4 * g + i;
                             p[e] = __builtin_amdgcn_exp2f(__builtin_fmaf(s_acc[kg][e], a.scale_log2e, -l2[i]));
-                            ds[e] = p[e] * (dp_acc[kg][e] - dl[i]);
+                            ds[e] = p[e] * dp_acc[kg][e];
                         }
                     }
                     if (masked) {
