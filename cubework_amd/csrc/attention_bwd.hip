@@ -34,11 +34,13 @@ constexpr int kWaves = 8;
 constexpr int kThreads = kWaves * 64;
 constexpr int kRowsPerWave = 32;
 constexpr int kRowsPerBlock = kWaves * kRowsPerWave;
-// dK/dV kernel at head size 64: wavefronts per block and groups of 32 keys per wavefront. 4 x 2 (every LDS
-// operand read feeding two MFMAs, but one wavefront per SIMD: 510 registers) ran the kernel in 278 us against
-// 190 us for 8 x 1.
-constexpr int kDkdvWaves = 8, kDkdvGroups = 1;
-static_assert(kDkdvWaves * kDkdvGroups * kRowsPerWave == kRowsPerBlock, "the dK/dV kernel's key block equals the dQ kernel's query block");
+// dK/dV kernel: 4 wavefronts (128 keys) per workgroup. At head size 64 a wavefront needs 218 registers and two
+// workgroups share a compute unit (two wavefronts per SIMD, 2 x 65 KB of LDS): they run out of step, so that one's
+// MFMA groups overlap the other's vector work, where the 8 wavefronts of one workgroup met at a barrier per tile
+// and ran the same phase at the same time (302 -> 291 us for the whole backward at batch 4 x 32 heads x 2048
+// tokens). At head size 128 a wavefront needs more than 256 registers and a unit holds one workgroup. Two groups
+// of 32 keys per wavefront (every LDS operand read feeding two MFMAs, 510 registers) ran 278 us against 190 us.
+constexpr int kDkdvWaves = 4;
 
 struct BwdArgs {
     const uint16_t* q;
@@ -226,15 +228,14 @@ __global__ __launch_bounds__(kThreads, 1) void attn_dq_kernel(const BwdArgs a) {
 
 // ---- dK, dV -----------------------------------------------------------------
 // LDS per stage: Q row images, Q transpose images, dO row images, dO transpose images (NP = head size / 64
-// panels of each), L*log2e and -D of the 64 rows. NW wavefronts of 32 key rows: 8 at head size 64; 4 at 128,
-// where a wavefront's accumulators and fragments need more than the 256 registers that 8 would leave it.
+// panels of each), L*log2e and -D of the 64 rows. NW wavefronts of 32 key rows.
 template <int NP>
 constexpr int dkdv_stage_bytes() { return 4 * NP * kImage + 2 * kTile * 4; }
 
 // KG: groups of 32 key rows per wavefront. With two, every A operand read from LDS (Q, dO, their
 // transposes) feeds two MFMAs instead of one.
 template <int NP, int NW, int KG, typename E>
-__global__ __launch_bounds__(NW * 64, 1) void attn_dkdv_kernel(const BwdArgs a) {
+__global__ __launch_bounds__(NW * 64, NP == 1 ? 2 : 1) void attn_dkdv_kernel(const BwdArgs a) {
     constexpr int kKeysPerWave = KG * kRowsPerWave;
     constexpr int kDkdvStage = dkdv_stage_bytes<NP>();
     constexpr int kStatsAt = 4 * NP * kImage;
@@ -457,18 +458,19 @@ int launch_bwd(const BwdArgs& a, int64_t B, int64_t H, int64_t S, int64_t D, int
     else hipLaunchKernelGGL((attn_dq_kernel<2, E>), dim3((unsigned)(nblk * B * H)), dim3(kThreads), 0, s, a);
     rc = check_launch("attn_dq_kernel");
     if (rc != CW_OK) return rc;
+    // both head sizes: 4 wavefronts (128 keys) per workgroup
+    const int64_t nkv = (S + kDkdvWaves * kRowsPerWave - 1) / (kDkdvWaves * kRowsPerWave);
+    if (nkv * B * H > INT32_MAX) return fail(CW_ERR_INVALID, "cw_attn_bwd: S or B*H too large");
     if (D == 64) {
         constexpr int lds_bytes = 2 * dkdv_stage_bytes<1>();
-        auto kern = attn_dkdv_kernel<1, kDkdvWaves, kDkdvGroups, E>;
+        auto kern = attn_dkdv_kernel<1, kDkdvWaves, 1, E>;
         if (const int lrc = ensure_dynamic_lds((const void*)kern, (int)(lds_bytes), "attn_dkdv_kernel"); lrc != CW_OK) return lrc;
-        hipLaunchKernelGGL(kern, dim3((unsigned)(nblk * B * H)), dim3(kDkdvWaves * 64), lds_bytes, s, a);
+        hipLaunchKernelGGL(kern, dim3((unsigned)(nkv * B * H)), dim3(kDkdvWaves * 64), lds_bytes, s, a);
     } else {
         constexpr int lds_bytes = 2 * dkdv_stage_bytes<2>();
-        auto kern = attn_dkdv_kernel<2, 4, 1, E>;
-        const int64_t nkv = (S + 4 * kRowsPerWave - 1) / (4 * kRowsPerWave);
-        if (nkv * B * H > INT32_MAX) return fail(CW_ERR_INVALID, "cw_attn_bwd: S or B*H too large");
+        auto kern = attn_dkdv_kernel<2, kDkdvWaves, 1, E>;
         if (const int lrc = ensure_dynamic_lds((const void*)kern, (int)(lds_bytes), "attn_dkdv_kernel"); lrc != CW_OK) return lrc;
-        hipLaunchKernelGGL(kern, dim3((unsigned)(nkv * B * H)), dim3(4 * 64), lds_bytes, s, a);
+        hipLaunchKernelGGL(kern, dim3((unsigned)(nkv * B * H)), dim3(kDkdvWaves * 64), lds_bytes, s, a);
     }
     return check_launch("attn_dkdv_kernel");
 }
