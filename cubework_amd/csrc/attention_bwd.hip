@@ -8,10 +8,11 @@
 // which is what autograd derives for benchmark/opt/opt.py:84-117 of the
 // reference (scaled bmm, mask, softmax, bmm).
 //
-// Three kernels, no atomics (results are bit-reproducible):
-//   attn_delta_kernel : D_i.
+// Two kernels, no atomics (results are bit-reproducible):
 //   attn_dq_kernel    : a block owns 256 query rows (32 per wavefront, Q and dO
-//                       fragments in registers) and walks the K/V tiles; all
+//                       fragments in registers; D_i from them and the same rows
+//                       of O, also left in scratch for the second kernel) and
+//                       walks the K/V tiles; all
 //                       products are formed transposed (lane = query row), so
 //                       L_i and D_i are per-lane scalars.
 //   attn_dkdv_kernel  : a block owns 256 key rows (32 per wavefront, K and V
@@ -62,31 +63,6 @@ struct BwdArgs {
     int causal;
 };
 
-// ---- D_i = sum_d dO_id O_id : one group of LPR = head size / 8 lanes per (b, h, i) row -------------
-template <int LPR, typename E>
-__global__ __launch_bounds__(256) void attn_delta_kernel(const BwdArgs a) {
-    constexpr int kRows = 256 / LPR;
-    const int64_t row = (int64_t)blockIdx.x * kRows + (threadIdx.x / LPR);  // (bh, i) flattened
-    const int sub = threadIdx.x % LPR;
-    const int64_t total = (int64_t)a.BH * a.S;
-    const int64_t rc = row < total ? row : total - 1;
-    const int bh = (int)(rc / a.S);
-    const int i = (int)(rc - (int64_t)bh * a.S);
-    const int b = bh / a.H, h = bh - b * a.H;
-    const int64_t off = b * a.ob + (int64_t)i * a.os + h * a.oh + sub * 8;
-    float x[8], y[8];
-    unpack_raw(load_raw(a.o + off), x, (const E*)nullptr);
-    unpack_raw(load_raw(a.d_o + off), y, (const E*)nullptr);
-    float s = 0.0f;
-#pragma unroll
-    for (int e = 0; e < 8; ++e) s += x[e] * y[e];
-    s += dpp_move<kDppXor1>(s);
-    s += dpp_move<kDppXor2>(s);
-    s += dpp_move<kDppHalfMirror>(s);  // lanes 0..7 of a row of 16 lanes hold the sum of their 8
-    if (LPR == 16) s += dpp_move<kDppMirror>(s);  // lane l + lane 15 - l: both halves of the 16
-    if (sub == 0 && row < total) a.delta[row] = s;
-}
-
 // ---- dQ ---------------------------------------------------------------------
 // LDS per stage: K row images, K transpose images, V row images (NP = head size / 64 panels of each).
 template <int NP, typename E>
@@ -109,17 +85,28 @@ __global__ __launch_bounds__(kThreads, 1) void attn_dq_kernel(const BwdArgs a) {
     const int qi = qw0 + l32;
     const int qrow = qi < S ? qi : S - 1;
     bf16x8_t qf[4 * NP], dof[4 * NP];
+    // D of the lane's row, from the dO pieces it holds anyway and the same pieces of O: the two lanes of a row
+    // (half 0 and 1) add their parts. The dK/dV launch, which follows on the stream, reads it from a.delta.
+    float dlt_ld = 0.0f;
     {
         const uint16_t* p = a.q + b * a.sb + (int64_t)qrow * a.ss + h * a.sh + 8 * half;
         const uint16_t* g = a.d_o + b * a.ob + (int64_t)qrow * a.os + h * a.oh + 8 * half;
+        const uint16_t* o = a.o + b * a.ob + (int64_t)qrow * a.os + h * a.oh + 8 * half;
 #pragma unroll
         for (int kb = 0; kb < 4 * NP; ++kb) {
             qf[kb] = __builtin_bit_cast(bf16x8_t, load_raw(p + 16 * kb));
-            dof[kb] = __builtin_bit_cast(bf16x8_t, load_raw(g + 16 * kb));
+            const raw16_t graw = load_raw(g + 16 * kb);
+            dof[kb] = __builtin_bit_cast(bf16x8_t, graw);
+            float x[8], y[8];
+            unpack_raw(load_raw(o + 16 * kb), x, (const E*)nullptr);
+            unpack_raw(graw, y, (const E*)nullptr);
+#pragma unroll
+            for (int e = 0; e < 8; ++e) dlt_ld = __builtin_fmaf(x[e], y[e], dlt_ld);
         }
+        dlt_ld += __shfl_xor(dlt_ld, 32, 64);
+        if (half == 0 && qi < S) a.delta[(int64_t)bh * S + qi] = dlt_ld;
     }
     const float lse2_ld = a.lse[(int64_t)bh * S + qrow] * kLog2e;
-    const float dlt_ld = a.delta[(int64_t)bh * S + qrow];
     f32x16_t dq[2 * NP];
 #pragma unroll
     for (int dt = 0; dt < 2 * NP; ++dt)
@@ -449,15 +436,9 @@ __global__ __launch_bounds__(NW * 64, NP == 1 ? 2 : 1) void attn_dkdv_kernel(con
 // The three launches of the backward for element type E.
 template <typename E>
 int launch_bwd(const BwdArgs& a, int64_t B, int64_t H, int64_t S, int64_t D, int64_t nblk, hipStream_t s) {
-    const int64_t rows = B * H * S;
-    if (D == 64) hipLaunchKernelGGL((attn_delta_kernel<8, E>), dim3((unsigned)((rows + 31) / 32)), dim3(256), 0, s, a);
-    else hipLaunchKernelGGL((attn_delta_kernel<16, E>), dim3((unsigned)((rows + 15) / 16)), dim3(256), 0, s, a);
-    int rc = check_launch("attn_delta_kernel");
-    if (rc != CW_OK) return rc;
     if (D == 64) hipLaunchKernelGGL((attn_dq_kernel<1, E>), dim3((unsigned)(nblk * B * H)), dim3(kThreads), 0, s, a);
     else hipLaunchKernelGGL((attn_dq_kernel<2, E>), dim3((unsigned)(nblk * B * H)), dim3(kThreads), 0, s, a);
-    rc = check_launch("attn_dq_kernel");
-    if (rc != CW_OK) return rc;
+    if (const int rc = check_launch("attn_dq_kernel"); rc != CW_OK) return rc;
     // both head sizes: 4 wavefronts (128 keys) per workgroup
     const int64_t nkv = (S + kDkdvWaves * kRowsPerWave - 1) / (kDkdvWaves * kRowsPerWave);
     if (nkv * B * H > INT32_MAX) return fail(CW_ERR_INVALID, "cw_attn_bwd: S or B*H too large");
