@@ -149,6 +149,15 @@ static bool dma_kernel_enabled() {
     return enabled;
 }
 
+// CW_GEMM_IMPL=onelaunch keeps a product whose last round of tiles is mostly empty in one launch (A/B measurements).
+static bool strip_split_enabled() {
+    static const bool enabled = [] {
+        const char* v = std::getenv("CW_GEMM_IMPL");
+        return !(v != nullptr && std::strcmp(v, "onelaunch") == 0);
+    }();
+    return enabled;
+}
+
 static int staged_launch(const GemmArgs& a, int layout, int epilogue, bool big, bool exact, bool f16, hipStream_t s) {
     switch (layout) {
         case CW_NN: return f16 ? gemm_f16_launch_nn(a, epilogue, big, exact, s) : gemm_bf16_launch_nn(a, epilogue, big, exact, s);
@@ -203,7 +212,37 @@ int gemm_half_launch(const GemmArgs& args, int layout, int epilogue, bool f16, h
             args.lda < ((int64_t)1 << 23) && args.ldb < ((int64_t)1 << 23) && ((tiles128 >= 192 && (int64_t)args.K * args.n_steps < 12288) || !splits))
             return gemm_half_small_launch(args, layout, epilogue, f16, s);
     }
-    if (big && all_vec && ring_ok && edges_ok && (args.K % gemm_bf16::kBK) == 0) return dma_launch(args, layout, epilogue, f16, s);
+    if (big && all_vec && ring_ok && edges_ok && (args.K % gemm_bf16::kBK) == 0) {
+        // A last round of 256 x 256 tiles that is mostly empty (a vocabulary slice as N: 8192 x 12568 is 32 x 50 =
+        // 1600 tiles, 6.25 rounds of the 256 compute units): when the partial round is whole tile columns, at most
+        // 3/8 of a round, and those columns are at most one round of 128 x 128 tiles, they go to the small-tile
+        // kernel as a second launch and the rest is whole rounds.
+        const int64_t tiles_m = (args.M + 255) / 256, tiles_n = (args.N + 255) / 256;
+        const int64_t last_round = (tiles_m * tiles_n) % 256;
+        if (tiles_m * tiles_n > 256 && last_round > 0 && last_round <= 96 && last_round % tiles_m == 0 &&
+            strip_split_enabled()) {
+            const int64_t n0 = (tiles_n - last_round / tiles_m) * 256;  // columns of the whole rounds
+            const int64_t strip = args.N - n0;
+            const int64_t strip_tiles = ((args.M + 127) / 128) * ((strip + 127) / 128);
+            if (n0 >= 256 && strip >= 128 && strip_tiles <= 256 && (args.K % 64) == 0 && args.lda < ((int64_t)1 << 23) &&
+                args.ldb < ((int64_t)1 << 23)) {
+                GemmArgs head = args, tail = args;
+                head.N = (int)n0;
+                tail.N = (int)strip;
+                auto shift = [&](const void* p, int64_t elems) -> const void* {
+                    return p == nullptr ? nullptr : reinterpret_cast<const uint16_t*>(p) + elems;
+                };
+                for (int i = 0; i < args.n_steps; ++i) tail.B[i] = shift(args.B[i], layout == CW_NT ? n0 * args.ldb : n0);
+                for (int j = 0; j < args.n_addends; ++j) tail.addend[j] = shift(args.addend[j], n0);
+                tail.bias = shift(args.bias, n0);
+                tail.C = const_cast<void*>(shift(args.C, n0));
+                tail.preact = const_cast<void*>(shift(args.preact, n0));
+                if (const int rc = dma_launch(head, layout, epilogue, f16, s); rc != CW_OK) return rc;
+                return gemm_half_small_launch(tail, layout, epilogue, f16, s);
+            }
+        }
+        return dma_launch(args, layout, epilogue, f16, s);
+    }
     // A reduction length that is not a multiple of the k tile (a vocabulary slice as K: 12568 = 392 x 32 +
     // 24), with B stored [K, N]: the regular step covers the first K - K % 32 columns, one more step of 32
     // covers [K-32, K) with a copy of B's last 32 rows whose overlapping rows are zero. The copy (64 bytes
