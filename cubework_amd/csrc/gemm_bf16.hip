@@ -214,29 +214,44 @@ int gemm_half_launch(const GemmArgs& args, int layout, int epilogue, bool f16, h
     }
     if (big && all_vec && ring_ok && edges_ok && (args.K % gemm_bf16::kBK) == 0) {
         // A last round of 256 x 256 tiles that is mostly empty (a vocabulary slice as N: 8192 x 12568 is 32 x 50 =
-        // 1600 tiles, 6.25 rounds of the 256 compute units): when the partial round is whole tile columns, at most
-        // 3/8 of a round, and those columns are at most one round of 128 x 128 tiles, they go to the small-tile
-        // kernel as a second launch and the rest is whole rounds.
+        // 1600 tiles, 6.25 rounds of the 256 compute units): when the partial round is whole tile columns (or whole
+        // tile rows), at most 3/8 of a round, and that strip is at most one round of 128 x 128 tiles, it goes to the
+        // small-tile kernel as a second launch and the rest is whole rounds.
         const int64_t tiles_m = (args.M + 255) / 256, tiles_n = (args.N + 255) / 256;
         const int64_t last_round = (tiles_m * tiles_n) % 256;
-        if (tiles_m * tiles_n > 256 && last_round > 0 && last_round <= 96 && last_round % tiles_m == 0 &&
-            strip_split_enabled()) {
-            const int64_t n0 = (tiles_n - last_round / tiles_m) * 256;  // columns of the whole rounds
-            const int64_t strip = args.N - n0;
-            const int64_t strip_tiles = ((args.M + 127) / 128) * ((strip + 127) / 128);
-            if (n0 >= 256 && strip >= 128 && strip_tiles <= 256 && (args.K % 64) == 0 && args.lda < ((int64_t)1 << 23) &&
-                args.ldb < ((int64_t)1 << 23)) {
-                GemmArgs head = args, tail = args;
-                head.N = (int)n0;
-                tail.N = (int)strip;
-                auto shift = [&](const void* p, int64_t elems) -> const void* {
-                    return p == nullptr ? nullptr : reinterpret_cast<const uint16_t*>(p) + elems;
-                };
-                for (int i = 0; i < args.n_steps; ++i) tail.B[i] = shift(args.B[i], layout == CW_NT ? n0 * args.ldb : n0);
-                for (int j = 0; j < args.n_addends; ++j) tail.addend[j] = shift(args.addend[j], n0);
-                tail.bias = shift(args.bias, n0);
-                tail.C = const_cast<void*>(shift(args.C, n0));
-                tail.preact = const_cast<void*>(shift(args.preact, n0));
+        const bool small_ok = (args.K % 64) == 0 && args.lda < ((int64_t)1 << 23) && args.ldb < ((int64_t)1 << 23);
+        if (tiles_m * tiles_n > 256 && last_round > 0 && last_round <= 96 && small_ok && strip_split_enabled()) {
+            auto shift = [&](const void* p, int64_t elems) -> const void* {
+                return p == nullptr ? nullptr : reinterpret_cast<const uint16_t*>(p) + elems;
+            };
+            GemmArgs head = args, tail = args;
+            bool split = false;
+            if (last_round % tiles_m == 0) {  // whole tile columns
+                const int64_t n0 = (tiles_n - last_round / tiles_m) * 256, strip = args.N - n0;
+                if (n0 >= 256 && strip >= 128 && ((args.M + 127) / 128) * ((strip + 127) / 128) <= 256) {
+                    head.N = (int)n0;
+                    tail.N = (int)strip;
+                    for (int i = 0; i < args.n_steps; ++i) tail.B[i] = shift(args.B[i], layout == CW_NT ? n0 * args.ldb : n0);
+                    for (int k = 0; k < args.n_addends; ++k) tail.addend[k] = shift(args.addend[k], n0);
+                    tail.bias = shift(args.bias, n0);
+                    tail.C = const_cast<void*>(shift(args.C, n0));
+                    tail.preact = const_cast<void*>(shift(args.preact, n0));
+                    split = true;
+                }
+            }
+            if (!split && last_round % tiles_n == 0) {  // whole tile rows
+                const int64_t m0 = (tiles_m - last_round / tiles_n) * 256, strip = args.M - m0;
+                if (m0 >= 256 && strip >= 128 && ((strip + 127) / 128) * ((args.N + 127) / 128) <= 256) {
+                    head.M = (int)m0;
+                    tail.M = (int)strip;
+                    for (int i = 0; i < args.n_steps; ++i) tail.A[i] = shift(args.A[i], layout == CW_TN ? m0 : m0 * args.lda);
+                    for (int k = 0; k < args.n_addends; ++k) tail.addend[k] = shift(args.addend[k], m0 * args.ldadd);
+                    tail.C = const_cast<void*>(shift(args.C, m0 * args.ldc));
+                    tail.preact = const_cast<void*>(shift(args.preact, m0 * args.ldp));
+                    split = true;
+                }
+            }
+            if (split) {
                 if (const int rc = dma_launch(head, layout, epilogue, f16, s); rc != CW_OK) return rc;
                 return gemm_half_small_launch(tail, layout, epilogue, f16, s);
             }

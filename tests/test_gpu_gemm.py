@@ -101,12 +101,13 @@ def test_bf16_vocab_slice_classifier_shape():
 
 
 @pytest.mark.parametrize("layout", LAYOUTS)
-@pytest.mark.parametrize("shape", [(4096, 4376, 128), (4096, 4608, 64), (4100, 4480, 192)])
+@pytest.mark.parametrize("shape", [(4096, 4376, 128), (4096, 4608, 64), (4100, 4480, 192), (8472, 2048, 128)])
 def test_bf16_mostly_empty_last_round_goes_to_small_tiles(layout, shape):
     """16 or 17 x 18 tiles of 256 x 256 are one round of the 256 compute units plus 32 or 50 tiles: when the
     remainder is whole tile columns (the first two shapes: 280 and 512 columns) they are a second launch of the
     128 x 128 tile kernel, with their share of the bias, the addend and the pre-activation copy; the third shape's
-    remainder (17 x 18 = 306 = 256 + 50, not a multiple of 17) stays in the one launch."""
+    remainder (17 x 18 = 306 = 256 + 50, not a multiple of 17) stays in the one launch; the fourth is 34 x 8 tiles,
+    whose last 16 are two tile rows (280 rows)."""
     M, N, K = shape
     _run(layout, M, N, K, 2, torch.bfloat16, act="gelu_tanh", n_add=1, preact=True, seed=11)
 
