@@ -35,6 +35,12 @@ def test_f16_ragged_around_aligned_core(layout):
     _run(layout, 4100, 2056, 136, 2, F16, act="gelu_erf", seed=5)   # guarded 256x256 tiles
 
 
+@pytest.mark.parametrize("layout", LAYOUTS)
+def test_f16_mostly_empty_last_round_goes_to_small_tiles(layout):
+    _run(layout, 4096, 4376, 128, 2, F16, act="gelu_tanh", n_add=1, preact=True, seed=11)   # 280 columns peeled
+    _run(layout, 8472, 2048, 64, 1, F16, act="relu", seed=12)                               # 280 rows peeled
+
+
 @pytest.mark.parametrize("layout", ["NN", "TN"])
 def test_f16_ragged_reduction_length(layout):
     _run(layout, 4096, 8192, 344, 1, F16, act="relu", n_add=1, preact=True, seed=7)
