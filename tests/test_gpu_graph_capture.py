@@ -10,7 +10,7 @@ pytestmark = pytest.mark.gpu
 DEV = "cuda:0"
 
 
-def _pipeline(x, w1, b1, w2, gamma, beta, targets, ids, table_rows):
+def _pipeline(x, w1, b1, w2, gamma, beta, targets, ids, table_rows, wide_w, clip_params):
     from cubework_amd import ops
 
     h = ops.gemm_ksteps("NN", [x], [w1], b1, "gelu_tanh")                      # LDS-ring kernel
@@ -23,7 +23,18 @@ def _pipeline(x, w1, b1, w2, gamma, beta, targets, ids, table_rows):
     dw = ops.embedding_bwd(ids, y, table_rows, 0)
     qkv = ops.gemm_ksteps("NN", [y], [w1[:, :768].contiguous()])               # 4 heads of 64: q, k, v side by side
     att = ops.attention_core(qkv.view(4, -1, 768), 4)
-    return h, y, small, loss, grad, dw, att
+    # attention backward (two launches, the first leaves D for the second in scratch)
+    t4 = qkv.view(4, -1, 4, 192)
+    q, k, v = t4[..., :64], t4[..., 64:128], t4[..., 128:]
+    o, lse = ops.attn_fwd(q, k, v, want_lse=True)
+    g = torch.empty_like(t4)
+    ops.attn_bwd(q, k, v, o, att, lse, g[..., :64], g[..., 64:128], g[..., 128:])
+    # 16 x 18 tiles of 256 x 256: the last 32 go to the small-tile kernel as a second launch
+    wide = ops.gemm_ksteps("NN", [x], [wide_w], None, "relu")
+    # gradient clipping (norm stage + scaling stage; a coefficient of 1 keeps the replays idempotent)
+    from cubework_amd.clip_grad import clip_grad_norm
+    norm = clip_grad_norm(clip_params, 1e30)
+    return h, y, small, loss, grad, dw, att, g, wide, norm.reshape(1)
 
 
 def test_entry_points_replay_from_a_graph():
@@ -36,7 +47,13 @@ def test_entry_points_replay_from_a_graph():
     beta = randn((H,), torch.bfloat16, 5, std=0.1).to(DEV)
     targets = torch.randint(0, V, (T,), generator=torch.Generator().manual_seed(6)).to(DEV)
     ids = torch.randint(0, 300, (T,), generator=torch.Generator().manual_seed(7)).to(DEV)
-    args = (x, w1, b1, w2, gamma, beta, targets, ids, 300)
+    wide_w = randn((H, 4376), torch.bfloat16, 8, std=0.03).to(DEV)
+    clip_params = []
+    for i, shape in enumerate([(70000,), (300, 7), (65536,)]):
+        p = torch.nn.Parameter(torch.zeros(shape, dtype=torch.bfloat16, device=DEV))
+        p.grad = randn(shape, torch.bfloat16, 20 + i).to(DEV)
+        clip_params.append(p)
+    args = (x, w1, b1, w2, gamma, beta, targets, ids, 300, wide_w, clip_params)
 
     eager = [t.clone() for t in _pipeline(*args)]
     torch.cuda.synchronize()
@@ -54,7 +71,8 @@ def test_entry_points_replay_from_a_graph():
             t.fill_(float("nan")) if t.is_floating_point() else t.zero_()
         graph.replay()
         torch.cuda.synchronize()
-        for name, got, want in zip(("gemm", "layernorm", "split-k gemm", "loss", "logits grad", "embedding grad", "attention"),
+        for name, got, want in zip(("gemm", "layernorm", "split-k gemm", "loss", "logits grad", "embedding grad", "attention",
+                                    "attention grad", "two-launch gemm", "gradient norm"),
                                    outs, eager):
             assert torch.equal(got, want), "%s differs on replay %d" % (name, replay)
         # the program's own eager work between replays
