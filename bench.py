@@ -198,8 +198,11 @@ def graph_time_us(fn, calls, replays=3, min_ms=100.0):
 def bench_bandwidth_kernels(device):
     """LayerNorm2D (config 3) and vocab-parallel CE (config 4) kernels: algorithmic
     bytes per launch / average launch duration. Each call below is one C-ABI
-    entry point (cw_ln_bwd_partials launches its partials kernel and a small
-    finalize kernel); the launches are replayed from a HIP graph."""
+    entry point; the launches are replayed from a HIP graph. The LayerNorm2D
+    backward is timed as the layers run it: cw_ln_bwd_partials_open (one launch,
+    leaves the column sums as partial rows) and cw_ln_bwd_dx_close (one launch
+    whose leading workgroups finish them); cw_ln_bwd_partials with its own
+    finalize launch is kept beside them as ln_bwd_partials_two_launches."""
     import torch
     from cubework_amd import ops
 
@@ -214,7 +217,8 @@ def bench_bandwidth_kernels(device):
     peer = _seeded((R, C), 5, 1.0, torch.bfloat16).to(device)
     stats = ops.ln_partial_stats(xs[0]) + ops.ln_partial_stats(peer)
     _, mr = ops.ln_normalize(xs[0], stats, H, 1e-5, gamma, beta)
-    rs = ops.ln_bwd_partials(dys[0], xs[0], mr, gamma)[0] * 2
+    rs, pending = ops.ln_bwd_partials_open(dys[0], xs[0], mr, gamma)
+    rs = rs * 2
     mr_whole = ops.ln_forward_fused(xs[0], 1e-5, gamma, beta)[1]  # the same rows taken as whole (H = 1024)
     i = [0]
 
@@ -225,8 +229,12 @@ def bench_bandwidth_kernels(device):
     cases = [
         ("ln_partial_stats", 33554432 + 131072, lambda: ops.ln_partial_stats(rot(xs))),
         ("ln_normalize", 2 * 33554432 + 2 * 131072 + 4096, lambda: ops.ln_normalize(rot(xs), stats, H, 1e-5, gamma, beta)),
-        ("ln_bwd_partials", 2 * 33554432 + 2 * 131072 + 8192, lambda: ops.ln_bwd_partials(rot(dys), xs[i[0] % nb], mr, gamma)),
-        ("ln_bwd_dx", 3 * 33554432 + 2 * 131072 + 2048, lambda: ops.ln_bwd_dx(rot(dys), xs[i[0] % nb], mr, rs, H, gamma)),
+        ("ln_bwd_partials", 2 * 33554432 + 2 * 131072 + 8192,
+         lambda: ops.ln_bwd_partials_open(rot(dys), xs[i[0] % nb], mr, gamma)),
+        ("ln_bwd_dx", 3 * 33554432 + 2 * 131072 + 2048 + 8192,
+         lambda: ops.ln_bwd_dx_close(rot(dys), xs[i[0] % nb], mr, rs, H, pending, gamma)),
+        ("ln_bwd_partials_two_launches", 2 * 33554432 + 2 * 131072 + 8192,
+         lambda: ops.ln_bwd_partials(rot(dys), xs[i[0] % nb], mr, gamma)),
         # rows complete on the rank (tensor-parallel size 1): partials + dx in one pass, dy and x read once
         ("ln_backward_fused", 3 * 33554432 + 2 * 131072 + 8192,
          lambda: ops.ln_backward_fused(rot(dys), xs[i[0] % nb], mr_whole, gamma)),

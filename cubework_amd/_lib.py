@@ -66,6 +66,9 @@ SIGNATURES = {
     "cw_ln_backward_fused": (_int, [_i64, _i64, _ptr, _i64, _ptr, _i64, _ptr, _ptr, _ptr, _ptr, _i64, _ptr, _ptr, _ptr, _i64,
                                     _int, _ptr]),
     "cw_ln_bwd_dx": (_int, [_i64, _i64, _ptr, _i64, _ptr, _i64, _ptr, _ptr, _ptr, _i64, _ptr, _i64, _int, _ptr]),
+    "cw_ln_bwd_partials_open": (_int, [_i64, _i64, _ptr, _i64, _ptr, _i64, _ptr, _ptr, _ptr, _ptr, _i64, _ptr, _int, _ptr]),
+    "cw_ln_bwd_dx_close": (_int, [_i64, _i64, _ptr, _i64, _ptr, _i64, _ptr, _ptr, _ptr, _i64, _ptr, _i64, _ptr, _i64, _ptr,
+                                  _ptr, _int, _ptr]),
     "cw_vpce_fwd_local": (_int, [_i64, _i64, _ptr, _i64, _ptr, _i64, _ptr, _ptr, _ptr, _ptr, _int, _ptr]),
     "cw_vpce_finalize": (_int, [_i64, _int, _ptr, _ptr, _ptr, _ptr, _ptr, _ptr, _ptr, _ptr]),
     "cw_diag_mfma_rate_flop": (_i64, [_int]),

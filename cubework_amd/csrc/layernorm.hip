@@ -528,11 +528,16 @@ template <typename T, int NCH, int NR, bool EXACT>
 __global__ __launch_bounds__(kTileWaves * 64) void ln_bwd_dx_tile_kernel(
     int64_t R, int64_t C, const T* __restrict__ dY, int64_t ld_dy, const T* __restrict__ x, int64_t ld_x,
     const float* __restrict__ mean_rstd, const T* __restrict__ gamma, const float* __restrict__ row_sums, float inv_h,
-    T* __restrict__ dx, int64_t ld_dx) {
+    T* __restrict__ dx, int64_t ld_dx, const FinishCols fin) {
     constexpr int V = elem<T>::kVec;
+    if (fin.blocks > 0 && (int)blockIdx.x < fin.blocks) {  // the leading workgroups finish the column sums
+        __shared__ float fin_red[kTileWaves * 64];
+        finish_cols_block<kTileWaves * 64>(fin, (int)blockIdx.x, fin_red);
+        return;
+    }
     const int lane = threadIdx.x & 63;
-    const int64_t wave = (int64_t)blockIdx.x * kTileWaves + (threadIdx.x >> 6);
-    const int64_t step = (int64_t)gridDim.x * kTileWaves * NR;
+    const int64_t wave = (int64_t)((int)blockIdx.x - fin.blocks) * kTileWaves + (threadIdx.x >> 6);
+    const int64_t step = (int64_t)((int)gridDim.x - fin.blocks) * kTileWaves * NR;
     raw16_t g_raw[NCH];
     if constexpr (!EXACT) load_param_chunks<T, NCH>(gamma, C, lane, g_raw);
     if constexpr (EXACT) C = (int64_t)NCH * 64 * V;
@@ -902,11 +907,17 @@ __global__ __launch_bounds__(kLnBlock) void ln_bwd_dx_kernel(int64_t R, int64_t 
                                                              const float* __restrict__ mean_rstd,
                                                              const T* __restrict__ gamma,
                                                              const float* __restrict__ row_sums, float inv_h,
-                                                             T* __restrict__ dx, int64_t ld_dx, int vec_ok) {
+                                                             T* __restrict__ dx, int64_t ld_dx, int vec_ok,
+                                                             const FinishCols fin) {
     constexpr int V = elem<T>::kVec;
+    if (fin.blocks > 0 && (int)blockIdx.x < fin.blocks) {  // the leading workgroups finish the column sums
+        __shared__ float fin_red[kLnBlock];
+        finish_cols_block<kLnBlock>(fin, (int)blockIdx.x, fin_red);
+        return;
+    }
     const int lane = threadIdx.x & 63;
-    const int64_t wave = (int64_t)blockIdx.x * (kLnBlock / 64) + (threadIdx.x >> 6);
-    const int64_t nwaves = (int64_t)gridDim.x * (kLnBlock / 64);
+    const int64_t wave = (int64_t)((int)blockIdx.x - fin.blocks) * (kLnBlock / 64) + (threadIdx.x >> 6);
+    const int64_t nwaves = (int64_t)((int)gridDim.x - fin.blocks) * (kLnBlock / 64);
     for (int64_t row = wave; row < R; row += nwaves) {
         const float mean = mean_rstd[2 * row];
         const float rstd = mean_rstd[2 * row + 1];
@@ -1179,10 +1190,12 @@ template <typename T>
 int bwd_partials_impl(int64_t R, int64_t C, const void* dY, int64_t ld_dy, const void* x, int64_t ld_x,
                       const float* mean_rstd, const void* gamma, float* row_sums, float* dgamma, float* dbeta,
                       void* workspace, int64_t workspace_bytes, hipStream_t s, void* dx = nullptr, int64_t ld_dx = 0,
-                      bool* dx_done = nullptr) {
+                      bool* dx_done = nullptr, int64_t* open_parts = nullptr) {
+    // open_parts: the column partials are left in the workspace, their count is reported, and whoever launches next
+    // on the stream adds them up (bwd_dx_impl with a FinishCols)
     constexpr int V = elem<T>::kVec;
     if (dx_done != nullptr) *dx_done = false;
-    const int want_cols = (dgamma != nullptr || dbeta != nullptr) ? 1 : 0;
+    const int want_cols = (dgamma != nullptr || dbeta != nullptr || open_parts != nullptr) ? 1 : 0;
     const bool vec = rows_vec_ok<T>(dY, ld_dy) && rows_vec_ok<T>(x, ld_x) && (gamma == nullptr || aligned16(gamma)) &&
                      (C % V) == 0;
     const int64_t nch = (C + 64 * V - 1) / (64 * V);
@@ -1231,6 +1244,10 @@ int bwd_partials_impl(int64_t R, int64_t C, const void* dY, int64_t ld_dy, const
             if (rc != CW_OK) return rc;
         }
     }
+    if (open_parts != nullptr) {
+        *open_parts = nparts;
+        return rc;
+    }
     if (want_cols) {
         // ws is [nparts][2][C]: dgamma partials are rows 2p, dbeta partials rows 2p+1.
         rc = finalize_col_partials((const float*)workspace, nparts, 2 * C, 2, C, dgamma, dbeta, s);
@@ -1241,32 +1258,34 @@ int bwd_partials_impl(int64_t R, int64_t C, const void* dY, int64_t ld_dy, const
 template <typename T>
 int bwd_dx_impl(int64_t R, int64_t C, const void* dY, int64_t ld_dy, const void* x, int64_t ld_x,
                 const float* mean_rstd, const void* gamma, const float* row_sums, int64_t H, void* dx, int64_t ld_dx,
-                hipStream_t s) {
+                hipStream_t s, const FinishCols* finish = nullptr) {
     const int vec_ok = rows_vec_ok<T>(dY, ld_dy) && rows_vec_ok<T>(x, ld_x) && rows_vec_ok<T>(dx, ld_dx) &&
                        (gamma == nullptr || aligned16(gamma));
+    const FinishCols fin = finish != nullptr ? *finish : FinishCols{};
+    const unsigned fb = (unsigned)fin.blocks;
     const int64_t nch = row_chunks<T>(C);
     // rows of more than 4 chunks are faster on the looping kernel (the 8-chunk tile needs 160-240 registers)
     if (vec_ok && exact_chunks<T>(C, nch) && nch <= 4 && R <= (int64_t)1 << 30) {
         return dispatch_exact<2>(nch, [&](auto nch_c, auto nr_c) {
             constexpr int NCH = decltype(nch_c)::value, NR = decltype(nr_c)::value;
-            hipLaunchKernelGGL((ln_bwd_dx_tile_kernel<T, NCH, NR, true>), dim3(exact_grid(R, NR)), dim3(kTileWaves * 64),
+            hipLaunchKernelGGL((ln_bwd_dx_tile_kernel<T, NCH, NR, true>), dim3(exact_grid(R, NR) + fb), dim3(kTileWaves * 64),
                                0, s, R, C, (const T*)dY, ld_dy, (const T*)x, ld_x, mean_rstd, (const T*)gamma, row_sums,
-                               1.0f / (float)H, (T*)dx, ld_dx);
+                               1.0f / (float)H, (T*)dx, ld_dx, fin);
             return check_launch("ln_bwd_dx_tile_kernel");
         });
     }
     if (vec_ok && (C % elem<T>::kVec) == 0 && nch <= 4) {
         return dispatch_tile(nch, [&](auto nch_c, auto nr_c) {
             constexpr int NCH = decltype(nch_c)::value, NR = decltype(nr_c)::value;
-            hipLaunchKernelGGL((ln_bwd_dx_tile_kernel<T, NCH, NR, false>), dim3(tile_grid(R, NR)), dim3(kTileWaves * 64),
+            hipLaunchKernelGGL((ln_bwd_dx_tile_kernel<T, NCH, NR, false>), dim3(tile_grid(R, NR) + fb), dim3(kTileWaves * 64),
                                0, s, R, C, (const T*)dY, ld_dy, (const T*)x, ld_x, mean_rstd, (const T*)gamma, row_sums,
-                               1.0f / (float)H, (T*)dx, ld_dx);
+                               1.0f / (float)H, (T*)dx, ld_dx, fin);
             return check_launch("ln_bwd_dx_tile_kernel");
         });
     }
-    hipLaunchKernelGGL(ln_bwd_dx_kernel<T>, dim3(ln_grid(R)), dim3(kLnBlock), 0, s, R, C, (const T*)dY, ld_dy,
+    hipLaunchKernelGGL(ln_bwd_dx_kernel<T>, dim3(ln_grid(R) + fb), dim3(kLnBlock), 0, s, R, C, (const T*)dY, ld_dy,
                        (const T*)x, ld_x, mean_rstd, (const T*)gamma, row_sums, 1.0f / (float)H, (T*)dx, ld_dx,
-                       vec_ok);
+                       vec_ok, fin);
     return check_launch("ln_bwd_dx_kernel");
 }
 
@@ -1411,5 +1430,59 @@ extern "C" int cw_ln_bwd_dx(int64_t R, int64_t C, const void* dY, int64_t ld_dy,
     return with_elem_type(io_dtype, [&](auto* tag) {
         return bwd_dx_impl<std::remove_pointer_t<decltype(tag)>>(R, C, dY, ld_dy, x, ld_x, mean_rstd, gamma, row_sums, H, dx,
                                                                  ld_dx, s);
+    });
+}
+
+extern "C" int cw_ln_bwd_partials_open(int64_t R, int64_t C, const void* dY, int64_t ld_dy, const void* x, int64_t ld_x,
+                                       const float* mean_rstd, const void* gamma, float* row_sums, void* workspace,
+                                       int64_t workspace_bytes, int64_t* n_parts, int io_dtype, void* stream) {
+    int rc = check_rc("cw_ln_bwd_partials_open", R, C, io_dtype);
+    if (rc != CW_OK) return rc;
+    if (n_parts == nullptr) return fail(CW_ERR_INVALID, "cw_ln_bwd_partials_open: n_parts is NULL");
+    *n_parts = 0;
+    if (R == 0) return CW_OK;
+    if (dY == nullptr || x == nullptr || mean_rstd == nullptr || row_sums == nullptr || workspace == nullptr || ld_dy < C ||
+        ld_x < C)
+        return fail(CW_ERR_INVALID, "cw_ln_bwd_partials_open: null pointer or leading dimension < C");
+    if (const int drc = require_gfx950("cw_ln_bwd_partials_open"); drc != CW_OK) return drc;
+    hipStream_t s = (hipStream_t)stream;
+    return with_elem_type(io_dtype, [&](auto* tag) {
+        return bwd_partials_impl<std::remove_pointer_t<decltype(tag)>>(R, C, dY, ld_dy, x, ld_x, mean_rstd, gamma, row_sums,
+                                                                       nullptr, nullptr, workspace, workspace_bytes, s,
+                                                                       nullptr, 0, nullptr, n_parts);
+    });
+}
+
+extern "C" int cw_ln_bwd_dx_close(int64_t R, int64_t C, const void* dY, int64_t ld_dy, const void* x, int64_t ld_x,
+                                  const float* mean_rstd, const void* gamma, const float* row_sums, int64_t H, void* dx,
+                                  int64_t ld_dx, const void* workspace, int64_t n_parts, float* dgamma, float* dbeta,
+                                  int io_dtype, void* stream) {
+    int rc = check_rc("cw_ln_bwd_dx_close", R, C, io_dtype);
+    if (rc != CW_OK) return rc;
+    if (H < C) return fail(CW_ERR_INVALID, "cw_ln_bwd_dx_close: hidden size H=%lld smaller than local C=%lld", (long long)H, (long long)C);
+    if (dgamma == nullptr || dbeta == nullptr) return fail(CW_ERR_INVALID, "cw_ln_bwd_dx_close: dgamma and dbeta are both needed");
+    if (n_parts < 0 || n_parts > (1 << 20) || (n_parts > 0 && workspace == nullptr) || C > ((int64_t)1 << 30))
+        return fail(CW_ERR_INVALID, "cw_ln_bwd_dx_close: bad partial count %lld, NULL workspace or C too large", (long long)n_parts);
+    if (const int drc = require_gfx950("cw_ln_bwd_dx_close"); drc != CW_OK) return drc;
+    hipStream_t s = (hipStream_t)stream;
+    if (R == 0 || n_parts == 0) {
+        // no rows: the column sums are zero (the finalize kernel over zero partial rows writes them)
+        rc = finalize_col_partials(nullptr, 0, 2 * C, 2, C, dgamma, dbeta, s);
+        if (rc != CW_OK || R == 0) return rc;
+    }
+    if (dY == nullptr || x == nullptr || mean_rstd == nullptr || row_sums == nullptr || dx == nullptr || ld_dy < C ||
+        ld_x < C || ld_dx < C)
+        return fail(CW_ERR_INVALID, "cw_ln_bwd_dx_close: null pointer or leading dimension < C");
+    FinishCols fin;
+    fin.ws = (const float*)workspace;
+    fin.nparts = n_parts;
+    fin.part_stride = 2 * C;
+    fin.C = C;
+    fin.out0 = dgamma;
+    fin.out1 = dbeta;
+    fin.blocks = n_parts > 0 ? 2 * (int)((C + 63) / 64) : 0;
+    return with_elem_type(io_dtype, [&](auto* tag) {
+        return bwd_dx_impl<std::remove_pointer_t<decltype(tag)>>(R, C, dY, ld_dy, x, ld_x, mean_rstd, gamma, row_sums, H, dx,
+                                                                 ld_dx, s, &fin);
     });
 }

@@ -52,6 +52,52 @@ __device__ __forceinline__ void block_flat_reduce(const float (&acc)[NREG], floa
     }
 }
 
+// The column finalize as the leading workgroups of another launch: the first `blocks` workgroups of a kernel that
+// was handed a FinishCols add the partial rows (out_k[c] = sum_p ws[p*part_stride + k*C + c], k < 2) and return, the
+// others do the kernel's own work with their index shifted. blocks = 2 * ceil(C / 64); 0 = nothing to finish.
+struct FinishCols {
+    const float* ws;
+    int64_t nparts, part_stride, C;
+    float* out0;
+    float* out1;
+    int blocks;
+};
+
+// Workgroup `block` (< f.blocks) of THREADS threads: 64 columns of one of the two sets. The THREADS / 64 groups
+// of 64 threads split the partial rows, 16 independent loads in flight each, and are combined in index order.
+// red: THREADS floats of LDS. Must be reached by every thread of the workgroup.
+template <int THREADS>
+__device__ __forceinline__ void finish_cols_block(const FinishCols& f, int block, float* red) {
+    constexpr int G = THREADS / 64;
+    const int lane = threadIdx.x & 63, grp = threadIdx.x >> 6;
+    const int col_blocks = f.blocks / 2;
+    const int k = block / col_blocks;
+    const int64_t c = (int64_t)(block - k * col_blocks) * 64 + lane;
+    float acc = 0.0f;
+    if (c < f.C) {
+        const float* base = f.ws + (int64_t)k * f.C + c;
+        for (int64_t p = grp; p < f.nparts; p += 16 * G) {
+            float v[16];
+#pragma unroll
+            for (int u = 0; u < 16; ++u) {
+                const int64_t q = p + u * G;
+                v[u] = base[(q < f.nparts ? q : f.nparts - 1) * f.part_stride];
+            }
+#pragma unroll
+            for (int u = 0; u < 16; ++u) acc += (p + u * G < f.nparts) ? v[u] : 0.0f;
+        }
+    }
+    red[grp * 64 + lane] = acc;
+    __syncthreads();
+    if (grp == 0 && c < f.C) {
+        float total = red[lane];
+#pragma unroll
+        for (int g = 1; g < G; ++g) total += red[g * 64 + lane];
+        float* out = (k == 0) ? f.out0 : f.out1;
+        if (out != nullptr) out[c] = total;
+    }
+}
+
 // out_k[c] = sum_p ws[p*part_stride + k*C + c], k < nsets (nsets is 1 or 2;
 // out1 is ignored when nsets == 1). Enqueued on `s`.
 int finalize_col_partials(const float* ws, int64_t nparts, int64_t part_stride, int nsets, int64_t C, float* out0,

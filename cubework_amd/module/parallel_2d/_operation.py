@@ -218,9 +218,11 @@ class _Layernorm2D(torch.autograd.Function):
             if row_mode.world_size == 1:
                 input_grad, dgamma, dbeta = ops.ln_backward_fused(output_grad, x, mean_rstd, gamma)
             else:
-                row_sums, dgamma, dbeta = ops.ln_bwd_partials(output_grad, x, mean_rstd, gamma)
+                # the dx launch also finishes the column sums that the first launch leaves as partial rows
+                row_sums, pending = ops.ln_bwd_partials_open(output_grad, x, mean_rstd, gamma)
                 row_sums = all_reduce(row_sums, row_mode)
-                input_grad = ops.ln_bwd_dx(output_grad, x, mean_rstd, row_sums, hidden_size, gamma)
+                input_grad, dgamma, dbeta = ops.ln_bwd_dx_close(output_grad, x, mean_rstd, row_sums, hidden_size, pending,
+                                                                gamma)
             weight_grad = reduce_scatter(dgamma, -1, col_mode).to(w_dtype)
             bias_grad = reduce_scatter(dbeta, -1, col_mode).to(b_dtype)
         return input_grad, weight_grad, bias_grad, None, None, None, None

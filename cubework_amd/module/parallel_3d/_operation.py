@@ -201,9 +201,10 @@ class _Layernorm3D(torch.autograd.Function):
             if out_mode.world_size == 1:
                 input_grad, dgamma, dbeta = ops.ln_backward_fused(output_grad, x, mean_rstd, weight)
             else:
-                row_sums, dgamma, dbeta = ops.ln_bwd_partials(output_grad, x, mean_rstd, weight)
+                # the dx launch also finishes the column sums that the first launch leaves as partial rows
+                row_sums, pending = ops.ln_bwd_partials_open(output_grad, x, mean_rstd, weight)
                 row_sums = all_reduce(row_sums, out_mode)
-                input_grad = ops.ln_bwd_dx(output_grad, x, mean_rstd, row_sums, hidden, weight)
+                input_grad, dgamma, dbeta = ops.ln_bwd_dx_close(output_grad, x, mean_rstd, row_sums, hidden, pending, weight)
             weight_grad = all_reduce(dgamma, ixw_mode).to(w_dtype)
             bias_grad = all_reduce(dbeta, ixw_mode).to(b_dtype)
         return input_grad, weight_grad, bias_grad, None, None, None, None, None, None

@@ -303,6 +303,48 @@ def ln_bwd_dx(dy: torch.Tensor, x: torch.Tensor, mean_rstd: torch.Tensor, row_su
     return dx.reshape(shape)
 
 
+def ln_bwd_partials_open(dy: torch.Tensor, x: torch.Tensor, mean_rstd: torch.Tensor,
+                         gamma: Optional[torch.Tensor] = None):
+    """Row sums [R,2] fp32 now, the parameter gradients later: returns (row_sums, pending), where `pending`
+    goes to ln_bwd_dx_close after the row sums have been summed over the ranks. See cw_ln_bwd_partials_open."""
+    lib = _lib.load()
+    dy, x = _rows(dy), _rows(x)
+    _require_device(dy, x, mean_rstd, gamma)
+    if dy.shape != x.shape or dy.dtype != x.dtype:
+        raise ValueError("dy and x must agree in shape and dtype")
+    R, C = x.shape
+    gamma = None if gamma is None else gamma.to(x.dtype).contiguous()
+    row_sums = torch.empty((R, 2), dtype=torch.float32, device=x.device)
+    ws = _workspace(R, C, x.device)
+    n_parts = ctypes.c_int64(0)
+    rc = lib.cw_ln_bwd_partials_open(R, C, _p(dy), _ld(dy), _p(x), _ld(x), _p(mean_rstd), _p(gamma), _p(row_sums), _p(ws),
+                                     ws.numel(), ctypes.cast(ctypes.byref(n_parts), ctypes.c_void_p), _dtype_code(x),
+                                     _stream())
+    _lib.check(rc, "cw_ln_bwd_partials_open")
+    return row_sums, (ws, n_parts.value)
+
+
+def ln_bwd_dx_close(dy: torch.Tensor, x: torch.Tensor, mean_rstd: torch.Tensor, row_sums: torch.Tensor, hidden: int,
+                    pending, gamma: Optional[torch.Tensor] = None):
+    """(dx, dgamma [C] fp32, dbeta [C] fp32): ln_bwd_dx whose launch also finishes the column sums that
+    ln_bwd_partials_open left pending. See cw_ln_bwd_dx_close."""
+    lib = _lib.load()
+    shape = x.shape
+    dy, x = _rows(dy), _rows(x)
+    _require_device(dy, x, mean_rstd, row_sums, gamma)
+    R, C = x.shape
+    ws, n_parts = pending
+    gamma = None if gamma is None else gamma.to(x.dtype).contiguous()
+    row_sums = row_sums.reshape(R, 2).to(torch.float32).contiguous()
+    dx = torch.empty((R, C), dtype=x.dtype, device=x.device)
+    dgamma = torch.empty(C, dtype=torch.float32, device=x.device)
+    dbeta = torch.empty(C, dtype=torch.float32, device=x.device)
+    rc = lib.cw_ln_bwd_dx_close(R, C, _p(dy), _ld(dy), _p(x), _ld(x), _p(mean_rstd), _p(gamma), _p(row_sums), hidden,
+                                _p(dx), _ld(dx), _p(ws), n_parts, _p(dgamma), _p(dbeta), _dtype_code(x), _stream())
+    _lib.check(rc, "cw_ln_bwd_dx_close")
+    return dx.reshape(shape), dgamma, dbeta
+
+
 def ln_backward_fused(dy: torch.Tensor, x: torch.Tensor, mean_rstd: torch.Tensor,
                       gamma: Optional[torch.Tensor] = None, want_param_grads: bool = True):
     """Backward of LayerNorm over rows this rank holds whole: (dx, dgamma [C] fp32 or None, dbeta [C] fp32

@@ -247,6 +247,22 @@ int cw_ln_bwd_dx(int64_t R, int64_t C, const void* dY, int64_t ld_dy,
                  const void* x, int64_t ld_x, const float* mean_rstd, const void* gamma,
                  const float* row_sums, int64_t H, void* dx, int64_t ld_dx,
                  int io_dtype, void* stream);
+/*
+ * cw_ln_bwd_partials and cw_ln_bwd_dx with the column finalize moved from a launch of its own (the second launch of
+ * cw_ln_bwd_partials, 3 - 5 us between the two kernels) into the dx launch: cw_ln_bwd_partials_open writes row_sums
+ * and leaves *n_parts unfinished column partial rows in `workspace` (sized by cw_ln_bwd_workspace_bytes; *n_parts
+ * is a host value, set before the call returns); the caller all-reduces row_sums as before
+ * (parallel_2d/_operation.py:335,339) and cw_ln_bwd_dx_close writes dx and, from its leading workgroups, dgamma and
+ * dbeta (fp32 [C]) out of those rows, which must still be in `workspace`. Same arithmetic as the pair above; the
+ * column sums are added in a fixed order (bit-reproducible) that differs from cw_ln_bwd_partials' in the last bits.
+ */
+int cw_ln_bwd_partials_open(int64_t R, int64_t C, const void* dY, int64_t ld_dy, const void* x, int64_t ld_x,
+                            const float* mean_rstd, const void* gamma, float* row_sums, void* workspace,
+                            int64_t workspace_bytes, int64_t* n_parts, int io_dtype, void* stream);
+int cw_ln_bwd_dx_close(int64_t R, int64_t C, const void* dY, int64_t ld_dy, const void* x, int64_t ld_x,
+                       const float* mean_rstd, const void* gamma, const float* row_sums, int64_t H, void* dx,
+                       int64_t ld_dx, const void* workspace, int64_t n_parts, float* dgamma, float* dbeta,
+                       int io_dtype, void* stream);
 
 /*
  * cw_ln_bwd_partials + cw_ln_bwd_dx with H = C in one pass over dY and x, for rows that are complete on

@@ -276,3 +276,58 @@ def test_ln_strided_rows(case, dtype):
            (rs_w, f32), (dg_w, f32), (db_w, f32), (dx_w, dtype)]
     for name, a, (w, dt) in zip(names, got, exp):
         assert_parity(a, w.reshape(a.shape), dt, "strided " + name)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32, torch.float16])
+@pytest.mark.parametrize("shape", [(16384, 1024), (8192, 2048), (4096, 4096), (300, 1000), (5, 24), (1, 8), (2048, 8200),
+                                   (777, 520)])
+def test_backward_with_the_column_finalize_in_the_dx_launch(dtype, shape):
+    """cw_ln_bwd_partials_open + cw_ln_bwd_dx_close against cw_ln_bwd_partials + cw_ln_bwd_dx on every kernel
+    family (whole-row tiles, exact tiles, rows split over wavefronts, looping kernels, ragged rows): row sums
+    and dx to the bit (the same kernels compute them), the column sums to fp32 rounding of a sum over the
+    partial rows (they are added in another fixed order) and against float64; twice in a row to the bit."""
+    import oracle
+    from cubework_amd import ops
+
+    R, C = shape
+    x = randn((R, C), dtype, 61).to(DEV)
+    dy = randn((R, C), dtype, 62).to(DEV)
+    gamma = rand_uniform((C,), dtype, 63, 0.9, 1.1).to(DEV)
+    _, mr = ops.ln_forward_fused(x, 1e-5, gamma, torch.zeros_like(gamma))
+    rs, dg, db = ops.ln_bwd_partials(dy, x, mr, gamma)
+    dx = ops.ln_bwd_dx(dy, x, mr, rs, C, gamma)
+    rs2, pending = ops.ln_bwd_partials_open(dy, x, mr, gamma)
+    dx2, dg2, db2 = ops.ln_bwd_dx_close(dy, x, mr, rs2, C, pending, gamma)
+    rs3, pending3 = ops.ln_bwd_partials_open(dy, x, mr, gamma)
+    dx3, dg3, db3 = ops.ln_bwd_dx_close(dy, x, mr, rs3, C, pending3, gamma)
+    torch.cuda.synchronize()
+    assert torch.equal(rs, rs2) and torch.equal(dx, dx2)
+    assert torch.equal(dg2, dg3) and torch.equal(db2, db3) and torch.equal(dx2, dx3)
+    with oracle.precision(torch.float64):
+        _, dg_w, db_w = oracle.ln_backward_full(dy.cpu(), x.cpu(), mr.cpu(), gamma.cpu())
+    assert_parity(dg2, dg_w, torch.float32, "dgamma from the dx launch")
+    assert_parity(db2, db_w, torch.float32, "dbeta from the dx launch")
+    assert_parity(dg2, dg.double().cpu(), torch.float32, "dgamma against the two-launch path")
+    assert_parity(db2, db.double().cpu(), torch.float32, "dbeta against the two-launch path")
+
+
+def test_dx_close_argument_checks_and_no_rows():
+    import ctypes as C
+    from cubework_amd import _lib
+
+    lib = _lib.load()
+    n = C.c_int64(-1)
+    out = torch.full((2, 8), float("nan"), dtype=torch.float32, device=DEV)
+    assert lib.cw_ln_bwd_partials_open(4, 8, None, 8, None, 8, None, None, None, None, 0, None, 0, None) == -1     # n_parts NULL
+    assert lib.cw_ln_bwd_partials_open(4, 8, None, 8, None, 8, None, None, None, None, 0, C.cast(C.byref(n), C.c_void_p), 0, None) == -1
+    assert n.value == 0
+    assert lib.cw_ln_bwd_dx_close(4, 8, None, 8, None, 8, None, None, None, 8, None, 8, None, 0, None, None, 0, None) == -1   # no dgamma
+    assert lib.cw_ln_bwd_dx_close(4, 8, None, 8, None, 8, None, None, None, 8, None, 8, None, 3, out[0].data_ptr(),
+                                  out[1].data_ptr(), 0, None) == -1                                                        # partials without workspace
+    assert lib.cw_ln_bwd_dx_close(4, 8, None, 8, None, 8, None, None, None, 4, None, 8, None, 0, out[0].data_ptr(),
+                                  out[1].data_ptr(), 0, None) == -1                                                        # H < C
+    # no rows: zero column sums, nothing else touched
+    assert lib.cw_ln_bwd_dx_close(0, 8, None, 8, None, 8, None, None, None, 8, None, 8, None, 0, out[0].data_ptr(),
+                                  out[1].data_ptr(), 0, None) == 0
+    torch.cuda.synchronize()
+    assert torch.equal(out, torch.zeros_like(out))
