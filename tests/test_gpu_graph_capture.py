@@ -34,7 +34,11 @@ def _pipeline(x, w1, b1, w2, gamma, beta, targets, ids, table_rows, wide_w, clip
     # gradient clipping (norm stage + scaling stage; a coefficient of 1 keeps the replays idempotent)
     from cubework_amd.clip_grad import clip_grad_norm
     norm = clip_grad_norm(clip_params, 1e30)
-    return h, y, small, loss, grad, dw, att, g, wide, norm.reshape(1)
+    # LayerNorm backward of a row-split layer: the dx launch finishes the first launch's column sums
+    _, mr = ops.ln_forward_fused(h, 1e-5, gamma, beta)
+    rs, pending = ops.ln_bwd_partials_open(x, h, mr, gamma)
+    ln_dx, ln_dg, ln_db = ops.ln_bwd_dx_close(x, h, mr, rs, h.shape[-1], pending, gamma)
+    return h, y, small, loss, grad, dw, att, g, wide, norm.reshape(1), ln_dx, ln_dg, ln_db
 
 
 def test_entry_points_replay_from_a_graph():
@@ -72,7 +76,8 @@ def test_entry_points_replay_from_a_graph():
         graph.replay()
         torch.cuda.synchronize()
         for name, got, want in zip(("gemm", "layernorm", "split-k gemm", "loss", "logits grad", "embedding grad", "attention",
-                                    "attention grad", "two-launch gemm", "gradient norm"),
+                                    "attention grad", "two-launch gemm", "gradient norm", "layernorm dx", "layernorm dgamma",
+                                    "layernorm dbeta"),
                                    outs, eager):
             assert torch.equal(got, want), "%s differs on replay %d" % (name, replay)
         # the program's own eager work between replays
