@@ -1038,12 +1038,13 @@ int normalize_impl(int64_t R, int64_t C, const void* x, int64_t ld, const float*
                        (beta == nullptr || aligned16(beta));
     const int64_t nch = row_chunks<T>(C);
     if (vec_ok && exact_chunks<T>(C, nch) && R <= (int64_t)1 << 30) {
-        // rows per wavefront: 8 loads per lane in flight, except that the fused kernel (which cannot store a row
-        // before its statistics are complete) is faster with two rows of two chunks than with four (16384 x 1024
-        // bf16: 12.4 against 14.6 us; four-chunk rows are best at two rows either way)
+        // rows per wavefront, by measurement (one tile per wavefront, 16-bit rows): four rows of one chunk (12.8 us
+        // on 32768 x 512 against 14.8 with two and 14.5 with eight), two rows of two chunks (16384 x 1024: 11.9
+        // against 12.8 us with four; fused 12.4 against 14.6), two rows of four chunks (8192 x 2048 fused: 13.6
+        // against 15.5 us with one)
         return dispatch_exact<8>(nch, [&](auto nch_c, auto nr_c) {
             constexpr int NCH = decltype(nch_c)::value;
-            constexpr int NR = (FUSED && NCH == 2) ? 2 : decltype(nr_c)::value;
+            constexpr int NR = NCH == 2 ? 2 : decltype(nr_c)::value;
             hipLaunchKernelGGL((ln_normalize_tile_kernel<T, NCH, NR, FUSED, true>), dim3(exact_grid(R, NR)),
                                dim3(kTileWaves * 64), 0, s, R, C, (const T*)x, ld, stats, mode, 1.0f / (float)H, eps,
                                (const T*)gamma, (const T*)beta, (T*)y, ldy, mean_rstd);
