@@ -574,7 +574,8 @@ def cpu_baseline():
 
 def mfma_rate_ceiling(lib, device):
     """cw_diag_mfma_rate: the GEMM's matrix instruction issued back to back from registers, random operands of
-    the workload's magnitudes and all-zero operands, each for about half a second, with clock and power."""
+    the workload's magnitudes, all-zero operands, and random operands read from LDS at the ring kernel's rate,
+    each for about half a second, with clock and power."""
     import ctypes
     import torch
     iters = 20000
@@ -582,9 +583,9 @@ def mfma_rate_ceiling(lib, device):
     sink = torch.empty(65536, dtype=torch.float32, device=device)
     stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
     out = {}
-    for name, zeros in (("random_operands", 0), ("zero_operands", 1)):
+    for name, mode in (("random_operands", 0), ("zero_operands", 1), ("random_operands_read_from_lds", 2)):
         def call():
-            rc = lib.cw_diag_mfma_rate(iters, zeros, sink.data_ptr(), stream)
+            rc = lib.cw_diag_mfma_rate(iters, mode, sink.data_ptr(), stream)
             if rc != 0:
                 raise RuntimeError(lib.cw_last_error().decode())
         us, smi = sustained_us(call, 60)
@@ -592,7 +593,8 @@ def mfma_rate_ceiling(lib, device):
         if smi:
             out[name].update({k: smi[k] for k in ("shader_clock_MHz", "socket_power_W")})
     out["note"] = ("register-only loop of v_mfma_f32_32x32x16_bf16 on all 1024 SIMDs: what the board's power management "
-                   "leaves of the data-sheet rate for operands that toggle like the workload's")
+                   "leaves of the data-sheet rate for operands that toggle like the workload's; read_from_lds: the same "
+                   "loop with the ring kernel's fragment reads from LDS (8 KB per 16 MFMAs), no global loads")
     return out
 
 

@@ -1,10 +1,13 @@
 // Measurement aid: the rate at which this GPU sustains the block GEMM's matrix instruction when nothing else
 // is in the way. Every wavefront keeps 4 x 4 accumulator tiles (the register blocking of the ring kernel) and
 // eight operand fragments of seeded random bf16 values in registers and issues v_mfma_f32_32x32x16_bf16 back to
-// back: no global loads, no LDS, no barriers. With `zeros` the fragments are all zero (no switching activity in
-// the multipliers). The result says what the power management of the board leaves of the 2516.6 TFLOP/s that
-// the data sheet quotes at 2.4 GHz, for operands that toggle like the workload's; bench.py reports it beside
-// the GEMM kernel's own rate.
+// back: no global loads, no LDS, no barriers. With mode 1 the fragments are all zero (no switching activity in
+// the multipliers). With mode 2 the eight fragments of every trip are read from LDS (64 KB of the same random
+// values, 16-byte reads, the next trip's fragments requested before the current trip's MFMAs), which is the
+// LDS traffic of the ring kernel's k loop: 8 KB per wavefront and 16 MFMAs. The result says what the power
+// management of the board leaves of the 2516.6 TFLOP/s that the data sheet quotes at 2.4 GHz, for operands that
+// toggle like the workload's, and what it leaves a kernel that also has to fetch them from LDS; bench.py reports
+// both beside the GEMM kernel's own rate.
 #include "cw_common.h"
 #include "gemm_bf16_kernel.h"
 
@@ -35,8 +38,12 @@ __device__ __forceinline__ uint32_t random_bf16_pair(uint32_t seed, float scale)
     return out;
 }
 
+template <bool LDS>
 __global__ __launch_bounds__(256) void mfma_rate_kernel(int iters, int zeros, float* __restrict__ sink) {
+    __shared__ __attribute__((aligned(16))) uint32_t frag_lds[LDS ? 16384 : 4];  // 64 fragments of 1 KB
     const uint32_t gid = blockIdx.x * 256u + threadIdx.x;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
     bf16x8_t a[4], b[4];
 #pragma unroll
     for (int t = 0; t < 4; ++t) {
@@ -46,9 +53,17 @@ __global__ __launch_bounds__(256) void mfma_rate_kernel(int iters, int zeros, fl
             wa[d] = zeros ? 0u : random_bf16_pair(gid * 64u + t * 8u + d, 1.0f);
             wb[d] = zeros ? 0u : random_bf16_pair(gid * 64u + 32u + t * 8u + d, 0.02f);
         }
-        typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
         a[t] = __builtin_bit_cast(bf16x8_t, (u32x4){wa[0], wa[1], wa[2], wa[3]});
         b[t] = __builtin_bit_cast(bf16x8_t, (u32x4){wb[0], wb[1], wb[2], wb[3]});
+    }
+    if constexpr (LDS) {
+        // fragment f of the block's 64: lanes' 16-byte pieces side by side, A fragments (magnitude 1) in the even
+        // slots, B fragments (0.02) in the odd ones
+        for (int i = threadIdx.x; i < 16384; i += 256) {
+            const int f = i >> 8;
+            frag_lds[i] = random_bf16_pair(blockIdx.x * 16384u + (uint32_t)i, (f & 1) ? 0.02f : 1.0f);
+        }
+        __syncthreads();
     }
     f32x16_t acc[4][4];
 #pragma unroll
@@ -57,11 +72,34 @@ __global__ __launch_bounds__(256) void mfma_rate_kernel(int iters, int zeros, fl
         for (int j = 0; j < 4; ++j)
 #pragma unroll
             for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.0f;
+    auto frag = [&](int slot) {  // slot < 64
+        return *reinterpret_cast<const bf16x8_t*>(reinterpret_cast<const char*>(frag_lds) + slot * 1024 + lane * 16);
+    };
     for (int it = 0; it < iters; ++it) {
+        bf16x8_t an[4], bn[4];
+        if constexpr (LDS) {
+            // the next trip's fragments: the wavefront walks its 16 slots (8 A, 8 B) two trips round
+            const int base = wave * 16 + ((it & 1) << 3);
+#pragma unroll
+            for (int t = 0; t < 4; ++t) {
+                an[t] = frag(base + 2 * t);
+                bn[t] = frag(base + 2 * t + 1);
+            }
+        }
 #pragma unroll
         for (int i = 0; i < 4; ++i)
 #pragma unroll
-            for (int j = 0; j < 4; ++j) acc[i][j] = gemm_bf16::mfma_32x32x16<bf16_t>(b[j], a[i], acc[i][j]);
+            for (int j = 0; j < 4; ++j) {
+                const int js = (i & 1) ? 3 - j : j;
+                acc[i][js] = gemm_bf16::mfma_32x32x16<bf16_t>(b[js], a[i], acc[i][js]);
+            }
+        if constexpr (LDS) {
+#pragma unroll
+            for (int t = 0; t < 4; ++t) {
+                a[t] = an[t];
+                b[t] = bn[t];
+            }
+        }
     }
     float s = 0.0f;
 #pragma unroll
@@ -83,11 +121,13 @@ extern "C" int64_t cw_diag_mfma_rate_flop(int iters) {
     return iters <= 0 ? 0 : (int64_t)iters * 1024 * 16 * 32768;
 }
 
-extern "C" int cw_diag_mfma_rate(int iters, int zeros, float* sink, void* stream) {
+extern "C" int cw_diag_mfma_rate(int iters, int mode, float* sink, void* stream) {
+    if (mode < 0 || mode > 2) return fail(CW_ERR_INVALID, "cw_diag_mfma_rate: mode %d outside [0, 2]", mode);
     if (iters <= 0 || iters > (1 << 24)) return fail(CW_ERR_INVALID, "cw_diag_mfma_rate: iters=%d outside [1, 2^24]", iters);
     if (const int drc = require_gfx950("cw_diag_mfma_rate"); drc != CW_OK) return drc;
     hipStream_t s = (hipStream_t)stream;
     // one workgroup of four wavefronts per compute unit, one wavefront per SIMD: 256 x 256 threads
-    hipLaunchKernelGGL(mfma_rate_kernel, dim3(256), dim3(256), 0, s, iters, zeros, sink);
+    if (mode == 2) hipLaunchKernelGGL(mfma_rate_kernel<true>, dim3(256), dim3(256), 0, s, iters, 0, sink);
+    else hipLaunchKernelGGL(mfma_rate_kernel<false>, dim3(256), dim3(256), 0, s, iters, mode, sink);
     return check_launch("mfma_rate_kernel");
 }

@@ -471,13 +471,15 @@ int cw_attn_bwd(int64_t B, int64_t H, int64_t S, int64_t D,
 /*
  * The block GEMM's matrix instruction (v_mfma_f32_32x32x16_bf16, 16 accumulator tiles per wavefront, one
  * wavefront per SIMD on every compute unit) issued back to back from registers for `iters` trips: no memory
- * traffic, no LDS, no barriers. Operand fragments are seeded random bf16 values with the workload's
- * magnitudes (zeros != 0: all zero). No counterpart in the reference; bench.py times it to report what the
- * board's power management leaves of the data-sheet MFMA rate, next to the GEMM kernel's own rate.
+ * traffic, no LDS, no barriers. mode 0: operand fragments are seeded random bf16 values with the workload's
+ * magnitudes; mode 1: all zero; mode 2: the random fragments of every trip are read from LDS (8 KB per wavefront
+ * and 16 MFMAs, the fragment traffic of the ring kernel's k loop; still no global loads). No counterpart in the
+ * reference; bench.py times it to report what the board's power management leaves of the data-sheet MFMA rate,
+ * with and without the LDS reads, next to the GEMM kernel's own rate.
  * cw_diag_mfma_rate_flop(iters) is the FLOP count of one call. sink: NULL or 65536 floats.
  */
 int64_t cw_diag_mfma_rate_flop(int iters);
-int cw_diag_mfma_rate(int iters, int zeros, float* sink, void* stream);
+int cw_diag_mfma_rate(int iters, int mode, float* sink, void* stream);
 
 #ifdef __cplusplus
 }
