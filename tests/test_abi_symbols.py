@@ -89,6 +89,11 @@ def test_scratch_sizes_and_refusals_of_the_later_entry_points():
     assert lib.cw_clip_coef(1, None, 1.0, 2.0, 1.0, None, None) == -1
     assert lib.cw_multi_norm_partial_count(3, C.cast(numels, C.c_void_p)) == 1 + 1 + 2
     assert lib.cw_multi_norm_partial_count(0, None) == 0
+    # measurement aid: modes 0 (random operands), 1 (zeros), 2 (random operands read from LDS)
+    assert lib.cw_diag_mfma_rate(0, 0, None, None) == -1
+    assert lib.cw_diag_mfma_rate(10, 3, None, None) == -1
+    assert b"mode" in lib.cw_last_error()
+    assert lib.cw_diag_mfma_rate_flop(2) == 2 * 1024 * 16 * 32768
     assert lib.cw_clip_scale(0, None, None, BF16, 1, None, 0, None, 1.0, 2.0, 1.0, None, None) == -1
     # attention: head sizes other than 64 / 128 and fp32 are refused before any launch
     assert lib.cw_attn_bwd_workspace_bytes(4, 32, 2048) == 4 * 32 * 2048 * 4
