@@ -56,3 +56,24 @@ def test_colsum_padded_rows():
     with oracle.precision(torch.float64):
         want = oracle.colsum(view.cpu())
     assert_parity(ops.colsum(view), want, torch.float32, "padded colsum")
+
+
+def test_mfma_rate_diagnostic_runs_in_every_mode():
+    """cw_diag_mfma_rate (the measurement aid behind bench.py's MFMA ceilings): zero operands leave zero sums;
+    random operands, from registers or read from LDS, leave finite non-zero ones, the same on every call."""
+    from cubework_amd import _lib
+
+    lib = _lib.load()
+    sink = torch.full((65536,), float("nan"), dtype=torch.float32, device=DEV)
+    assert lib.cw_diag_mfma_rate(3, 1, sink.data_ptr(), None) == 0
+    torch.cuda.synchronize()
+    assert torch.equal(sink, torch.zeros_like(sink))
+    for mode in (0, 2):
+        runs = []
+        for _ in range(2):
+            sink.fill_(float("nan"))
+            assert lib.cw_diag_mfma_rate(4, mode, sink.data_ptr(), None) == 0
+            torch.cuda.synchronize()
+            runs.append(sink.clone())
+        assert torch.isfinite(runs[0]).all() and (runs[0] != 0).any()
+        assert torch.equal(runs[0], runs[1])
