@@ -194,6 +194,7 @@ __global__ __launch_bounds__(kClipThreads) void clip_only_kernel(const ClipArgs 
 // one tensor, one batch per thread (measured on 100 MB of bf16 gradients: 35.0 us against 40.9 us with 128 KB
 // per workgroup in four batches).
 constexpr int kScaleBatch = 8;
+constexpr int kFusedPairsMax = 2048;  // pairs that every workgroup of the fused scaling launch may read
 constexpr int kScaleChunkBytes = kScaleBatch * kClipThreads * 16;  // one batch per thread: 32 KB per workgroup
 
 template <typename T, bool FUSED>
@@ -378,6 +379,15 @@ int scale_impl(const char* who, int n_tensors, void* const* grads, const int64_t
     if (const int drc = require_gfx950(who); drc != CW_OK) return drc;
     hipStream_t s = (hipStream_t)stream;
     const ClipArgs none = {};
+    // Every workgroup of the fused scaling launch reads all pairs: fine for a few thousand (16 KB from L2 beside the
+    // 64 KB it moves), quadratic beyond. More pairs than that (the gradients of a billion parameters leave 16384) are
+    // combined by one launch of their own first, and the scaling launch reads the coefficient it leaves in out2.
+    if (clip != nullptr && clip->n_partials > kFusedPairsMax) {
+        hipLaunchKernelGGL(clip_only_kernel, dim3(1), dim3(kClipThreads), 0, s, *clip);
+        if (const int rc = check_launch("clip_only_kernel"); rc != CW_OK) return rc;
+        coef = clip->out2 + 1;
+        clip = nullptr;
+    }
     int done = 0, launches = 0;
     while (done < n_tensors) {
         TensorBatch b;

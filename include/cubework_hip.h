@@ -421,7 +421,8 @@ int cw_multi_scale(int n_tensors, void* const* grads, const int64_t* numels, con
  * (n_partials unfinished (value, group) pairs left by cw_multi_norm_partials calls with out2 == NULL; may be 0)
  * in one fixed order, takes the root and the clamp, and multiplies its share of the gradients; out2 receives
  * (total norm, coefficient) as from cw_clip_coef. With partials, a clipping call that needs no exchange between
- * ranks is two launches per dtype. out2 must not overlap sets or partials; a caller with several dtypes calls
+ * ranks is two launches per dtype (three beyond 2048 pairs, i.e. 134 M elements: every workgroup of the scaling launch
+ * reads all pairs, so more of them are combined by one launch of their own first). out2 must not overlap sets or partials; a caller with several dtypes calls
  * it once per dtype with the same sets / partials (out2 is rewritten with the same values).
  */
 int cw_clip_scale(int n_tensors, void* const* grads, const int64_t* numels, int io_dtype, int n_sets,

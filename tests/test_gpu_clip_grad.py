@@ -225,3 +225,40 @@ def test_clip_scale_argument_checks():
     assert lib.cw_clip_scale(0, None, None, 0, 0, None, 0, None, 1.0, 2.0, 1.0, out.data_ptr(), None) == 0
     torch.cuda.synchronize()
     assert out.tolist() == [0.0, 1.0]
+
+
+def test_clip_scale_with_more_pairs_than_a_workgroup_should_read():
+    """Beyond 2048 block partials (here 2100 chunks of 65536 elements plus two small tensors) cw_clip_scale combines
+    them with one launch of their own instead of in every workgroup of the scaling launch; the results still equal
+    those of cw_multi_norm_partials with its finalize, cw_clip_coef and cw_multi_scale to the bit."""
+    import ctypes as C
+    from cubework_amd import _lib, ops
+
+    lib = _lib.load()
+    shapes = [(2100 * 65536,), (1000, 33), (7,)]
+    a = [randn(s, torch.bfloat16, 70 + i, std=0.01).to(DEV) for i, s in enumerate(shapes)]
+    b = [t.clone() for t in a]
+    n = len(a)
+    numels = (C.c_int64 * n)(*[t.numel() for t in a])
+    numels_p = C.cast(numels, C.c_void_p)
+    code = ops._dtype_code(a[0])
+    count = lib.cw_multi_norm_partial_count(n, numels_p)
+    assert count == 2100 + 1 + 1
+    stream = ops._stream()
+    ws = torch.empty(2 * count, dtype=torch.float32, device=DEV)
+    sets = torch.empty(2, dtype=torch.float32, device=DEV)
+    out_a = torch.empty(2, dtype=torch.float32, device=DEV)
+    out_b = torch.empty(2, dtype=torch.float32, device=DEV)
+    pa = (C.c_void_p * n)(*[t.data_ptr() for t in a])
+    pb = (C.c_void_p * n)(*[t.data_ptr() for t in b])
+    assert lib.cw_multi_norm_partials(n, pa, numels_p, None, None, 2.0, sets.data_ptr(), ws.data_ptr(), 8 * count, code, stream) == 0
+    assert lib.cw_clip_coef(1, sets.data_ptr(), 1.0, 2.0, 1.0, out_a.data_ptr(), stream) == 0
+    assert lib.cw_multi_scale(n, pa, numels_p, out_a[1:].data_ptr(), code, stream) == 0
+    assert lib.cw_multi_norm_partials(n, pb, numels_p, None, None, 2.0, None, ws.data_ptr(), 8 * count, code, stream) == 0
+    assert lib.cw_clip_scale(n, pb, numels_p, code, 0, None, count, ws.data_ptr(), 1.0, 2.0, 1.0, out_b.data_ptr(), stream) == 0
+    torch.cuda.synchronize()
+    assert torch.equal(out_a, out_b), (out_a, out_b)
+    want = (2100 * 65536 + 33000 + 7) ** 0.5 * 0.01
+    assert abs(out_a[0].item() - want) < 0.02 * want and 0.0 < out_a[1].item() < 1.0
+    for x, y in zip(a, b):
+        assert torch.equal(x, y)
