@@ -26,6 +26,16 @@ def pytest_collection_modifyitems(config, items):
             item.add_marker(skip)
 
 
+@pytest.fixture(autouse=True)
+def single_rank_by_default(request):
+    """Every GPU test starts from a world of one rank, whatever the test before it set up (the tests that play one
+    rank of a grid call initialize(...) themselves)."""
+    if "gpu" in request.keywords:
+        from cubework_amd.distributed import initialize
+        initialize(None, 1)
+    yield
+
+
 @pytest.fixture
 def oracle64():
     """The oracle evaluates its formulas in float64 for the duration of the test."""
