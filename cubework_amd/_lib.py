@@ -18,6 +18,7 @@ CW_EPI_NONE, CW_EPI_BIAS, CW_EPI_BIAS_GELU_TANH, CW_EPI_BIAS_GELU_ERF, CW_EPI_BI
 CW_ACT_NONE, CW_ACT_GELU_TANH, CW_ACT_GELU_ERF, CW_ACT_RELU = 0, 2, 3, 4
 CW_LN_ONE_PASS, CW_LN_TWO_PASS = 0, 1
 CW_MAX_KSTEPS, CW_MAX_ADDENDS = 16, 8
+CW_ERR_INVALID, CW_ERR_ALIGNMENT, CW_ERR_UNSUPPORTED, CW_ERR_LAUNCH, CW_ERR_DEVICE = -1, -2, -3, -4, -5
 
 _i64 = ctypes.c_int64
 _int = ctypes.c_int

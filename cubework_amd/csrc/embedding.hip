@@ -580,11 +580,15 @@ int bwd_impl(int64_t T_rows, int64_t E, const int64_t* sorted_ids, const int64_t
 // faster path; measured on a 50272-row bf16 slice: T = 16384, E = 512: 81 against 66 us, E = 1024: 86 against 76,
 // E = 2048: 96 against 98; T = 8192, E = 512: 32 against 35 (up to 8192 tokens two workgroups share a compute unit,
 // beyond that the token bitmaps leave room for one).
+bool direct_possible(int64_t T_rows, int64_t E, const void* d_out, int64_t ldo, const void* d_weight, int64_t ldw, int V) {
+    return T_rows <= kDirMaxTokens && E % V == 0 && aligned16(d_weight) && ldw % V == 0 &&
+           (T_rows == 0 || (aligned16(d_out) && ldo % V == 0));
+}
+
 bool direct_ok(int64_t T_rows, int64_t E, const void* d_out, int64_t ldo, const void* d_weight, int64_t ldw, int V) {
     const int64_t row_bytes = E * (16 / V);
     const bool pays = T_rows <= (T_rows <= 8192 ? 8 : 4) * row_bytes;
-    return T_rows <= kDirMaxTokens && pays && E % V == 0 && aligned16(d_weight) && ldw % V == 0 &&
-           (T_rows == 0 || (aligned16(d_out) && ldo % V == 0));
+    return pays && direct_possible(T_rows, E, d_out, ldo, d_weight, ldw, V);
 }
 
 template <typename T>
@@ -657,7 +661,7 @@ extern "C" int cw_embed_bwd_ids(int64_t T, int64_t E, const int64_t* ids, int64_
     if (d_weight == nullptr || ldw < E) return fail(CW_ERR_INVALID, "cw_embed_bwd_ids: d_weight is NULL or ldw < E");
     if (T > 0 && (ids == nullptr || d_out == nullptr || ldo < E))
         return fail(CW_ERR_INVALID, "cw_embed_bwd_ids: null pointer or leading dimension < E");
-    if (!cw_embed_bwd_ids_supported(T, E, d_out, ldo, d_weight, ldw, io_dtype))
+    if (!direct_possible(T, E, d_out, ldo, d_weight, ldw, io_dtype == CW_F32 ? 4 : 8))
         return fail(CW_ERR_UNSUPPORTED,
                     "cw_embed_bwd_ids: needs T <= %d, 16-byte aligned rows and E a multiple of the 16-byte vector; "
                     "use cw_embed_sort_ids + cw_embed_bwd", kDirMaxTokens);

@@ -561,10 +561,11 @@ def embedding_token_order(ids: torch.Tensor, num_rows: int, vocab_start: int = 0
 
 
 def embedding_bwd(ids: torch.Tensor, d_out: torch.Tensor, num_rows: int, vocab_start: int = 0,
-                  skip_row: int = -1, via_token_order: bool = False) -> torch.Tensor:
+                  skip_row: int = -1, via_token_order: Optional[bool] = None) -> torch.Tensor:
     """Gradient of embedding_fwd with respect to the [num_rows, E] weight slice: one launch from the unsorted
-    ids where cw_embed_bwd_ids takes the shapes (up to 16384 tokens, 16-byte aligned rows), else (or with
-    via_token_order) the token order followed by cw_embed_bwd."""
+    ids where cw_embed_bwd_ids_supported says that it pays (up to 16384 tokens, 16-byte aligned rows, rows not
+    much smaller than the batch's ids), else the token order followed by cw_embed_bwd. via_token_order = True /
+    False asks for one path (False: the one launch wherever it is possible at all)."""
     lib = _lib.load()
     _require_device(ids, d_out)
     if ids.dtype != torch.int64:
@@ -575,11 +576,16 @@ def embedding_bwd(ids: torch.Tensor, d_out: torch.Tensor, num_rows: int, vocab_s
     if flat.numel() != T:
         raise ValueError("ids select %d rows, d_out has %d" % (flat.numel(), T))
     dw = torch.empty((num_rows, E), dtype=g.dtype, device=g.device)
-    if not via_token_order and lib.cw_embed_bwd_ids_supported(T, E, _p(g), _ld(g), _p(dw), _ld(dw), _dtype_code(g)):
+    if via_token_order is None:
+        direct = bool(lib.cw_embed_bwd_ids_supported(T, E, _p(g), _ld(g), _p(dw), _ld(dw), _dtype_code(g)))
+    else:
+        direct = not via_token_order
+    if direct:
         rc = lib.cw_embed_bwd_ids(T, E, _p(flat), int(vocab_start), num_rows, int(skip_row), _p(g), _ld(g), _p(dw),
                                   _ld(dw), _dtype_code(g), _stream())
-        _lib.check(rc, "cw_embed_bwd_ids")
-        return dw
+        if rc != _lib.CW_ERR_UNSUPPORTED:
+            _lib.check(rc, "cw_embed_bwd_ids")
+            return dw
     sorted_ids, order = embedding_token_order(flat, num_rows, vocab_start)
     rc = lib.cw_embed_bwd(T, E, _p(sorted_ids), _p(order), int(vocab_start), num_rows, int(skip_row), _p(g), _ld(g),
                           _p(dw), _ld(dw), _dtype_code(g), _stream())

@@ -367,9 +367,11 @@ int cw_embed_sort_ids(int64_t T, const int64_t* ids, int64_t vocab_start, int64_
  * tokens select is summed over 8 contiguous ranges of token positions whose partial sums are added in
  * order. No atomics on global memory: bit-reproducible. A row that n tokens select is summed by one
  * workgroup at about 70 ns per token, so a batch dominated by one id is better served by the token order,
- * which shares a long run among several workgroups. cw_embed_bwd_ids_supported returns 1 when the
- * shapes and pointers qualify; otherwise cw_embed_bwd_ids returns CW_ERR_UNSUPPORTED and the caller
- * goes through cw_embed_sort_ids + cw_embed_bwd.
+ * which shares a long run among several workgroups. Every workgroup scans all T ids for its 32 rows, so the
+ * launch pays while a row is not much smaller than T / 4 bytes: cw_embed_bwd_ids_supported returns 1 when the
+ * shapes and pointers qualify and T <= 8 row sizes in bytes (4 beyond 8192 tokens); cw_embed_bwd_ids itself
+ * refuses only what it cannot do (CW_ERR_UNSUPPORTED: more than 16384 tokens, unaligned rows), and the caller
+ * then goes through cw_embed_sort_ids + cw_embed_bwd.
  */
 int cw_embed_bwd_ids_supported(int64_t T, int64_t E, const void* d_out, int64_t ldo, const void* d_weight,
                                int64_t ldw, int io_dtype);

@@ -202,7 +202,7 @@ def test_embedding_backward_from_ids_edges(T):
     n = min(T, edges.numel())
     ids[:n] = edges[:n]
     d_out = randn((T, e), torch.float32, 12)
-    got = ops.embedding_bwd(ids.to(DEV), d_out.to(DEV), rows, start, 5)
+    got = ops.embedding_bwd(ids.to(DEV), d_out.to(DEV), rows, start, 5, via_token_order=False)
     torch.cuda.synchronize()
     local = ids - start
     live = (ids >= start) & (ids < start + rows) & (local != 5)
@@ -234,3 +234,33 @@ def test_embedding_backward_from_ids_refuses_what_it_cannot_take():
     assert_parity(got, want, torch.bfloat16, "embedding d_weight, 16385 tokens")
     odd = d_out[:100, 1:]  # rows start 2 bytes off a 16-byte boundary
     assert lib.cw_embed_bwd_ids_supported(100, e - 1, odd.data_ptr(), e, dw.data_ptr(), e, _lib.CW_BF16) == 0
+
+
+def test_embedding_backward_from_ids_is_offered_only_where_it_pays():
+    """Every workgroup of the one-launch kernel scans all ids, so for rows much smaller than the batch's ids
+    cw_embed_bwd_ids_supported says no (the wrapper then takes the token order); the entry point itself still
+    serves such a call, with the same sums."""
+    from cubework_amd import _lib, ops
+
+    lib = _lib.load()
+    BF16 = _lib.CW_BF16
+    dummy = torch.empty(16, dtype=torch.bfloat16, device=DEV)
+    p = dummy.data_ptr()
+    assert lib.cw_embed_bwd_ids_supported(8192, 2048, p, 2048, p, 2048, BF16) == 1    # the benchmark's shape
+    assert lib.cw_embed_bwd_ids_supported(16384, 2048, p, 2048, p, 2048, BF16) == 1
+    assert lib.cw_embed_bwd_ids_supported(16384, 1024, p, 1024, p, 1024, BF16) == 0   # 4 row sizes = 8192 < 16384
+    assert lib.cw_embed_bwd_ids_supported(8192, 512, p, 512, p, 512, BF16) == 1       # 8 row sizes up to 8192 tokens
+    assert lib.cw_embed_bwd_ids_supported(8192, 256, p, 256, p, 256, BF16) == 0
+    assert lib.cw_embed_bwd_ids_supported(8192, 256, p, 256, p, 256, _lib.CW_F32) == 1
+    T, e, rows = 4096, 64, 3000
+    ids = torch.randint(0, rows, (T,), generator=torch.Generator().manual_seed(3)).to(DEV)
+    d_out = randn((T, e), torch.bfloat16, 4).to(DEV)
+    assert lib.cw_embed_bwd_ids_supported(T, e, d_out.data_ptr(), e, p, e, BF16) == 0
+    auto = ops.embedding_bwd(ids, d_out, rows)
+    forced = ops.embedding_bwd(ids, d_out, rows, via_token_order=False)
+    order = ops.embedding_bwd(ids, d_out, rows, via_token_order=True)
+    torch.cuda.synchronize()
+    assert torch.equal(auto, order)
+    want = torch.zeros((rows, e), dtype=torch.float64).index_add_(0, ids.cpu(), d_out.double().cpu())
+    assert_parity(forced, want, torch.bfloat16, "one launch where it does not pay")
+    assert_parity(auto, want, torch.bfloat16, "token order chosen by the wrapper")

@@ -141,8 +141,8 @@ def test_random_embedding_backward_from_ids(case):
             ids[::3] = start + min(7, rows - 1)
     skip = min(3, rows - 1) if with_skip else -1
     d_out = randn((T, E), dtype, T + 5)
-    got = ops.embedding_bwd(ids.to(DEV), d_out.to(DEV), rows, start, skip)
-    again = ops.embedding_bwd(ids.to(DEV), d_out.to(DEV), rows, start, skip)
+    got = ops.embedding_bwd(ids.to(DEV), d_out.to(DEV), rows, start, skip, via_token_order=False)
+    again = ops.embedding_bwd(ids.to(DEV), d_out.to(DEV), rows, start, skip, via_token_order=False)
     torch.cuda.synchronize()
     assert torch.equal(got, again), "fixed summation order: bit-reproducible"
     local = ids - start
