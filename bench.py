@@ -43,9 +43,11 @@ class SmiSampler:
     while the caller runs its timed loop. The driver reports low-pass filtered values (they settle within
     about a second), so the figures kept are those of the last 40 % of the sampled interval."""
 
-    def __init__(self, period_s=0.002):
+    def __init__(self, period_s=0.002, metrics=None):
         import glob
         self.period = period_s
+        self.metrics = metrics if metrics is not None and metrics.handle is not None else None
+        self.tables = []   # distinct gpu_metrics tables seen during the run (one reading every 50 ms)
         dev = "/sys/class/drm/card0/device"
         hw = sorted(glob.glob(dev + "/hwmon/hwmon*"))
         self.power_path = hw[0] + "/power1_input" if hw and os.path.exists(hw[0] + "/power1_input") else None
@@ -56,9 +58,11 @@ class SmiSampler:
         self._thread = None
 
     def available(self):
-        return self.power_path is not None and self.sclk_path is not None
+        return (self.power_path is not None and self.sclk_path is not None) or self.metrics is not None
 
     def _read(self):
+        if self.power_path is None or self.sclk_path is None:
+            raise OSError("no sysfs power / clock files")
         with open(self.power_path) as f:
             watts = int(f.read()) / 1e6
         mhz = None
@@ -69,12 +73,18 @@ class SmiSampler:
         return watts, mhz
 
     def _run(self):
+        next_table = 0.0
         while not self._stop:
             try:
                 w, m = self._read()
                 self.samples.append((time.perf_counter(), w, m))
             except (OSError, ValueError, IndexError):
                 pass
+            if self.metrics is not None and time.perf_counter() >= next_table:
+                tab = self.metrics.read()
+                if tab is not None and (not self.tables or tab["firmware_timestamp"] != self.tables[-1]["firmware_timestamp"]):
+                    self.tables.append(tab)
+                next_table = time.perf_counter() + 0.05
             time.sleep(self.period)
 
     def __enter__(self):
@@ -110,21 +120,110 @@ class SmiSampler:
         return out
 
 
+class GpuMetrics:
+    """The driver's gpu_metrics table of GPU 0 through ROCm's amdsmi binding (shipped under /opt/rocm): the
+    socket energy accumulator (15.259 uJ units), the firmware's own timestamp (10 ns units) and its residency
+    counters of the limiters (package power, PROCHOT, socket / regulator / HBM temperature: one count per
+    millisecond in which the limiter held the clock down). The firmware refreshes the table about once a second,
+    so only differences between two DISTINCT tables mean anything, and only tables whose whole period lies inside
+    the interval of interest describe it. Everything is optional: without the binding the fields are left out."""
+
+    FIELDS = ("energy_accumulator", "firmware_timestamp", "accumulation_counter", "ppt_residency_acc",
+              "prochot_residency_acc", "socket_thm_residency_acc", "vr_thm_residency_acc", "hbm_thm_residency_acc")
+    LIMITERS = (("package_power_ppt", "ppt_residency_acc"), ("prochot", "prochot_residency_acc"),
+                ("socket_thermal", "socket_thm_residency_acc"), ("regulator_thermal", "vr_thm_residency_acc"),
+                ("hbm_thermal", "hbm_thm_residency_acc"))
+    REFRESH_S = 1.0
+
+    def __init__(self):
+        self.handle = None
+        try:
+            if "/opt/rocm/share/amd_smi" not in sys.path:
+                sys.path.append("/opt/rocm/share/amd_smi")
+            import amdsmi
+            self.amdsmi = amdsmi
+            amdsmi.amdsmi_init()
+            self.handle = amdsmi.amdsmi_get_processor_handles()[0]
+            if self.read() is None:
+                self.handle = None
+        except Exception:  # no binding, no permission, another table revision
+            self.handle = None
+
+    def read(self):
+        if self.handle is None:
+            return None
+        try:
+            m = self.amdsmi.amdsmi_get_gpu_metrics_info(self.handle)
+        except Exception:
+            return None
+        out = {k: m.get(k) for k in self.FIELDS}
+        if not all(isinstance(out[k], int) for k in ("energy_accumulator", "firmware_timestamp")):
+            return None
+        out["t"] = time.perf_counter()
+        out["xcd_clocks_MHz"] = m.get("current_gfxclks")
+        return out
+
+    @classmethod
+    def window(cls, tables, t0, t1, launch_us=None):
+        """tables: distinct readings (by firmware timestamp) taken while a kernel ran back to back from host time
+        t0 to t1 (each is seen within 50 ms of its refresh). Uses the first and the last table refreshed inside
+        the run, after a margin for the clock to settle: average socket power from the energy counter over the firmware's own clock, the share of the
+        firmware's samples in which each limiter was active, and, given the launch duration, energy per launch."""
+        inside = [m for m in tables if t0 + 0.4 <= m["t"] <= t1]
+        if len(inside) < 2:
+            return {"note": "the run was too short for two refreshes of the firmware's table (about one a second)"}
+        a, b = inside[0], inside[-1]
+        dt = (b["firmware_timestamp"] - a["firmware_timestamp"]) * 1e-8
+        if dt <= 0:
+            return None
+        watts = (b["energy_accumulator"] - a["energy_accumulator"]) * 15.259e-6 / dt
+        out = {"socket_power_W_from_energy_counter": round(watts, 1), "window_s": round(dt, 3), "tables": len(inside)}
+        if launch_us:
+            out["energy_mJ_per_launch"] = round(watts * launch_us * 1e-3, 2)
+        n = (b["accumulation_counter"] - a["accumulation_counter"]) if isinstance(a.get("accumulation_counter"), int) else 0
+        if n > 0:
+            out["limiter_residency"] = {name: round((b[key] - a[key]) / n, 4) for name, key in cls.LIMITERS
+                                        if isinstance(a.get(key), int) and isinstance(b.get(key), int)}
+        if b.get("xcd_clocks_MHz"):
+            clk = [c for c in b["xcd_clocks_MHz"] if isinstance(c, int)]
+            if clk:
+                out["xcd_clocks_MHz"] = clk
+        return out
+
+
+_GPU_METRICS = None
+
+
+def gpu_metrics():
+    global _GPU_METRICS
+    if _GPU_METRICS is None:
+        _GPU_METRICS = GpuMetrics()
+    return _GPU_METRICS
+
+
 def sustained_us(fn, launches):
     """Average duration of fn() over `launches` back-to-back calls (events on the current stream), with the
-    clock and power the driver reports while they run."""
+    clock and power the driver reports while they run and, when the run is long enough for the firmware's
+    table to refresh twice inside it, the socket energy counter and the limiters' residencies."""
     import torch
     for _ in range(20):
         fn()
     torch.cuda.synchronize()
     e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-    with SmiSampler() as smi:
+    with SmiSampler(metrics=gpu_metrics()) as smi:
         e0.record()
         for _ in range(launches):
             fn()
         e1.record()
         torch.cuda.synchronize()
-    return e0.elapsed_time(e1) * 1e3 / launches, smi.summary()
+    us = e0.elapsed_time(e1) * 1e3 / launches
+    summary = smi.summary()
+    if smi.tables:
+        w = GpuMetrics.window(smi.tables, smi.t0, smi.t1, us)
+        if w is not None:
+            summary = dict(summary or {})
+            summary["gpu_metrics"] = w
+    return us, summary
 
 
 def measured_traffic():
@@ -305,6 +404,81 @@ def event_time_us(fn, iters, warmup, min_ms=150.0):
     return timed(n) if n > iters else pilot
 
 
+class AbiCallTimer:
+    """Stands in for the loaded library during one instrumented pass: every C-ABI compute call is bracketed by two
+    events on the launch stream, so that each entry point's device time inside a composite step (the OPT-shaped
+    block) can be told apart. The events stretch the step; the step's own time is measured without them."""
+
+    # entry point -> (what the call's work is priced in, function of the call's arguments giving FLOP or bytes)
+    @staticmethod
+    def _es(code):
+        return 4 if code == 1 else 2
+
+    def __init__(self, lib):
+        self._lib = lib
+        self.records = []   # (name, shape text, kind, work, ev0, ev1)
+
+    def _work(self, name, a):
+        es = self._es
+        if name in ("cw_gemm_ksteps_ws", "cw_gemm_ksteps"):
+            lay, m, n, k, steps = a[0], a[1], a[2], a[3], a[4]
+            return ("%s %dx%dx%d" % ("NN NT TN".split()[lay], m, n, k * max(steps, 1)), "flop", 2.0 * m * n * k * steps)
+        if name == "cw_attn_fwd":
+            b, h, s, d, causal = a[0], a[1], a[2], a[3], a[11]
+            return ("b%d h%d s%d d%d" % (b, h, s, d), "flop", 4.0 * b * h * s * s * d / (2 if causal else 1))
+        if name == "cw_attn_bwd":
+            b, h, s, d, causal = a[0], a[1], a[2], a[3], a[17]
+            return ("b%d h%d s%d d%d" % (b, h, s, d), "flop", 10.0 * b * h * s * s * d / (2 if causal else 1))
+        if name == "cw_ln_forward_fused":
+            return ("%dx%d" % (a[0], a[1]), "bytes", 2.0 * a[0] * a[1] * es(a[11]))
+        if name == "cw_ln_backward_fused":
+            return ("%dx%d" % (a[0], a[1]), "bytes", 3.0 * a[0] * a[1] * es(a[15]))
+        if name == "cw_colsum":
+            return ("%dx%d" % (a[0], a[1]), "bytes", 1.0 * a[0] * a[1] * es(a[7]))
+        if name == "cw_act_bwd_colsum":
+            return ("%dx%d" % (a[1], a[2]), "bytes", 3.0 * a[1] * a[2] * es(a[12]))
+        return ("", None, 0.0)
+
+    def __getattr__(self, name):
+        fn = getattr(self._lib, name)
+        if not name.startswith("cw_") or name.endswith("_bytes") or name.endswith("_supported") or name in (
+                "cw_version", "cw_device_arch", "cw_last_error"):
+            return fn
+
+        def timed(*args):
+            import torch
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            rc = fn(*args)
+            e1.record()
+            shape, kind, work = self._work(name, args)
+            self.records.append((name, shape, kind, work, e0, e1))
+            return rc
+        return timed
+
+    def table(self, passes, step_us):
+        """Per (entry point, shape): calls per step, device time per step, share of the step, and the fraction of
+        the call's own roofline (dense bf16 MFMA peak for FLOP, 8 TB/s for bytes)."""
+        rows = {}
+        for name, shape, kind, work, e0, e1 in self.records:
+            r = rows.setdefault((name, shape), {"entry_point": name, "shape": shape, "calls": 0, "us": 0.0, "kind": kind, "work": work})
+            r["calls"] += 1
+            r["us"] += e0.elapsed_time(e1) * 1e3
+        out = []
+        for r in sorted(rows.values(), key=lambda r: -r["us"]):
+            calls = r["calls"] / passes
+            us = r["us"] / passes
+            row = {"entry_point": r["entry_point"], "shape": r["shape"], "calls_per_step": round(calls, 2),
+                   "us_per_step": round(us, 1), "share_of_step": round(us / step_us, 4)}
+            per_call = us / max(calls, 1e-9)
+            if r["kind"] == "flop":
+                row["frac_of_mfma_peak"] = round(r["work"] / per_call / 1e6 / MFMA_BF16_PEAK_TFLOPS, 4)
+            elif r["kind"] == "bytes":
+                row["frac_of_hbm_peak"] = round(r["work"] / per_call / 1e3 / HBM_PEAK_GBPS, 4)
+            out.append(row)
+        return out
+
+
 def bench_other_configs(device, sets):
     """The other GEMM orientations at config 2's FLOP count (the backward products of the same layer),
     config 1's fp32 forward GEMM, and one OPT-1.3B-shaped block (config 5) forward+backward."""
@@ -336,6 +510,42 @@ def bench_other_configs(device, sets):
     us = event_time_us(tn, 50, 10)
     out["gemm_tn_dW_splitk"] = {"us": round(us, 2), "TFLOPs": round(GEMM_FLOP / us / 1e6, 1),
                                 "frac": round(GEMM_FLOP / us / 1e6 / MFMA_BF16_PEAK_TFLOPS, 4)}
+    # Vendor anchor, outside the product path: torch.matmul (hipBLASLt) beside cw_gemm_ksteps on the same operands,
+    # without bias or activation on either side - config 2's product with its two k-steps concatenated
+    # ([8192,4096] x [4096,2048], operands rotated like the headline's) and one 8192^3 product.
+    cat_sets = [(torch.cat(a, dim=1), torch.cat(b, dim=0)) for a, b in sets]
+    o_cat = torch.empty((M, N), dtype=torch.bfloat16, device=device)
+    c_ = [0]
+
+    def rot_cat():
+        c_[0] += 1
+        return cat_sets[c_[0] % n_sets]
+    anchor = {}
+    for name, fn in (("cw_gemm_ksteps", lambda: ops.gemm_ksteps("NN", *[[t] for t in rot_cat()], out=o_cat)),
+                     ("torch_matmul", lambda: torch.matmul(*rot_cat(), out=o_cat))):
+        us = event_time_us(fn, 50, 10)
+        anchor[name] = {"us": round(us, 2), "TFLOPs": round(GEMM_FLOP / us / 1e6, 1),
+                        "frac": round(GEMM_FLOP / us / 1e6 / MFMA_BF16_PEAK_TFLOPS, 4)}
+    out["vendor_anchor_config2_concatenated_8192x2048x4096"] = anchor
+    del cat_sets, o_cat
+    big = [(_seeded((8192, 8192), 60 + 2 * j_, 1.0, torch.bfloat16).to(device),
+            _seeded((8192, 8192), 61 + 2 * j_, 0.02, torch.bfloat16).to(device)) for j_ in range(2)]
+    o_big = torch.empty((8192, 8192), dtype=torch.bfloat16, device=device)
+    flop_big = 2.0 * 8192 ** 3
+
+    def rot_big():
+        c_[0] += 1
+        return big[c_[0] % 2]
+    anchor = {}
+    for name, fn in (("cw_gemm_ksteps", lambda: ops.gemm_ksteps("NN", *[[t] for t in rot_big()], out=o_big)),
+                     ("torch_matmul", lambda: torch.matmul(*rot_big(), out=o_big))):
+        us = event_time_us(fn, 10, 3)
+        anchor[name] = {"us": round(us, 2), "TFLOPs": round(flop_big / us / 1e6, 1),
+                        "frac": round(flop_big / us / 1e6 / MFMA_BF16_PEAK_TFLOPS, 4)}
+    anchor["note"] = ("torch.matmul is the vendor library (hipBLASLt) on the same bf16 operands in the same process: a "
+                      "comparison line only, nothing on the product path calls it")
+    out["vendor_anchor_8192x8192x8192"] = anchor
+    del big, o_big
     # config 2's product with float16 operands (what a plain torch.autocast hands the GEMM-type operators):
     # the same kernel with the other MFMA opcode and conversion
     a16 = [t.to(torch.float16) for t in sets[0][0]]
@@ -430,6 +640,24 @@ def bench_other_configs(device, sets):
         y = blk(xb)
         y.backward(dyb)
     us = event_time_us(block_step, 10, 3)
+    # where the step's time goes: the same step with every C-ABI call bracketed by events (instrumented passes,
+    # not the timed ones); what is left is torch's own kernels between the calls (gradient accumulation at the
+    # residual forks, dtype casts of the parameter gradients, zero_grad)
+    from cubework_amd import _lib as _cw_lib
+    real_lib = _cw_lib.load()
+    timer = AbiCallTimer(real_lib)
+    passes = 5
+    _cw_lib._lib = timer
+    try:
+        for _ in range(passes):
+            block_step()
+        torch.cuda.synchronize()
+    finally:
+        _cw_lib._lib = real_lib
+    per_kernel = timer.table(passes, us)
+    in_calls = sum(r["us_per_step"] for r in per_kernel)
+    per_kernel.append({"entry_point": "(torch kernels and gaps between the calls)", "shape": "", "calls_per_step": None,
+                       "us_per_step": round(us - in_calls, 1), "share_of_step": round((us - in_calls) / us, 4)})
     # gradient-norm clipping over the block's 12 parameter gradients (one read for the norm, read + write
     # for the scaling)
     from cubework_amd.clip_grad import clip_grad_norm
@@ -442,7 +670,10 @@ def bench_other_configs(device, sets):
     lin_flop = 3 * 2.0 * 8192 * 2048 * (6144 + 2048 + 8192 + 8192)
     out["opt_block_fwd_bwd"] = {"ms": round(us / 1e3, 3), "linear_flop": lin_flop,
                                 "linear_TFLOPs_if_all_time_were_linears": round(lin_flop / us / 1e6, 1),
-                                "note": "four Linear2D, two LayerNorm2D and the fused attention core (cw_attn_fwd / cw_attn_bwd), tp=1"}
+                                "note": "four Linear2D, two LayerNorm2D and the fused attention core (cw_attn_fwd / cw_attn_bwd), tp=1",
+                                "per_kernel": per_kernel,
+                                "per_kernel_source": "events around every C-ABI call during %d instrumented passes of the same "
+                                                     "step in this run; the last row is the step's time minus their sum" % passes}
     return out
 
 
@@ -572,12 +803,14 @@ def cpu_baseline():
     return head
 
 
-def mfma_rate_ceiling(lib, device):
-    """cw_diag_mfma_rate: the GEMM's matrix instruction issued back to back from registers, random operands of
-    the workload's magnitudes, all-zero operands, and random operands read from LDS at the ring kernel's rate,
-    each for about half a second, with clock and power."""
+def mfma_rate_ceiling(device, seconds=0.4):
+    """cw_diag_mfma_rate (measurement library): the GEMM's matrix instruction issued back to back from registers,
+    random operands of the workload's magnitudes, all-zero operands, and random operands read from LDS at the ring
+    kernel's rate, each for `seconds`, with clock and power (and, for runs of 3 s and more, the energy counter)."""
     import ctypes
     import torch
+    from cubework_amd import _diag
+    lib = _diag.load()
     iters = 20000
     flop = lib.cw_diag_mfma_rate_flop(iters)
     sink = torch.empty(65536, dtype=torch.float32, device=device)
@@ -588,13 +821,85 @@ def mfma_rate_ceiling(lib, device):
             rc = lib.cw_diag_mfma_rate(iters, mode, sink.data_ptr(), stream)
             if rc != 0:
                 raise RuntimeError(lib.cw_last_error().decode())
-        us, smi = sustained_us(call, 60)
+        us, smi = sustained_us(call, max(10, int(seconds * 1e6 / 6000)))
         out[name] = {"TFLOPs": round(flop / us / 1e6, 1), "frac_of_peak": round(flop / us / 1e6 / MFMA_BF16_PEAK_TFLOPS, 4)}
         if smi:
-            out[name].update({k: smi[k] for k in ("shader_clock_MHz", "socket_power_W")})
+            out[name].update({k: smi[k] for k in ("shader_clock_MHz", "socket_power_W", "gpu_metrics") if k in smi})
+            gm = out[name].get("gpu_metrics")
+            if gm and "socket_power_W_from_energy_counter" in gm:
+                gm.pop("energy_mJ_per_launch", None)
+                gm["pJ_per_FLOP"] = round(gm["socket_power_W_from_energy_counter"] / (flop / us / 1e6), 4)
     out["note"] = ("register-only loop of v_mfma_f32_32x32x16_bf16 on all 1024 SIMDs: what the board's power management "
                    "leaves of the data-sheet rate for operands that toggle like the workload's; read_from_lds: the same "
                    "loop with the ring kernel's fragment reads from LDS (8 KB per 16 MFMAs), no global loads")
+    return out
+
+
+def energy_table(device, sets, bias, outs, seconds):
+    """Where a launch of the headline GEMM spends its energy: the ring kernel whole and with one part taken out
+    (cw_diag_gemm_part of the measurement library: the same kernel source, parts 1-3 not computing anything
+    meaningful), each run back to back for `seconds`, priced by the socket's energy counter (average power over
+    whole refresh periods of the firmware's table inside the run x the event-timed launch duration). At the power
+    cap time = energy / power, so the joules are what the microseconds are made of."""
+    import ctypes
+    import torch
+    from cubework_amd import _diag
+    lib = _diag.load()
+    stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+    tabs = []
+    for A, B in sets:
+        tabs.append(((ctypes.c_void_p * STEPS_K)(*[t.data_ptr() for t in A]),
+                     (ctypes.c_void_p * STEPS_K)(*[t.data_ptr() for t in B])))
+    it = [0]
+
+    def make(part, rotate):
+        def call():
+            k = it[0] % len(sets) if rotate else 0
+            it[0] += 1
+            ta, tb = tabs[k]
+            rc = lib.cw_diag_gemm_part(part, M, N, K, STEPS_K, ta, K, tb, N, bias.data_ptr(), outs[k].data_ptr(), N, stream)
+            if rc != 0:
+                raise RuntimeError(lib.cw_last_error().decode())
+        return call
+
+    runs = {}
+    for name, part, rotate in (("whole_kernel_operands_from_hbm", 0, True), ("whole_kernel_operands_cache_resident", 0, False),
+                               ("no_operand_loads_in_the_k_loop", 1, False), ("no_lds_fragment_reads_in_the_k_loop", 3, False),
+                               ("no_epilogue", 2, False)):
+        fn = make(part, rotate)
+        pilot, _ = sustained_us(fn, 2000)
+        us, smi = sustained_us(fn, int(seconds * 1e6 / pilot) + 1)
+        row = {"us_per_launch": round(us, 2)}
+        if smi:
+            row.update({k: smi[k] for k in ("shader_clock_MHz", "socket_power_W") if k in smi})
+            gm = smi.get("gpu_metrics") or {}
+            for k in ("socket_power_W_from_energy_counter", "energy_mJ_per_launch", "limiter_residency", "window_s"):
+                if k in gm:
+                    row[k] = gm[k]
+        runs[name] = row
+    ceil = mfma_rate_ceiling(device, seconds)
+    out = {"runs": runs, "matrix_instruction_loops": ceil, "flop_per_launch": GEMM_FLOP}
+
+    def mj(name):
+        return runs[name].get("energy_mJ_per_launch")
+    pj = {k: (ceil[k].get("gpu_metrics") or {}).get("pJ_per_FLOP") for k in ("random_operands", "random_operands_read_from_lds", "zero_operands")}
+    if all(mj(k) is not None for k in runs) and pj["random_operands"]:
+        whole, cached = mj("whole_kernel_operands_from_hbm"), mj("whole_kernel_operands_cache_resident")
+        parts = {
+            "matrix_instructions": round(pj["random_operands"] * GEMM_FLOP * 1e-9, 2),
+            "lds_fragment_reads": round(cached - mj("no_lds_fragment_reads_in_the_k_loop"), 2),
+            "operand_loads_l2_to_lds": round(cached - mj("no_operand_loads_in_the_k_loop"), 2),
+            "hbm_and_fabric_instead_of_cache": round(whole - cached, 2),
+            "epilogue_bias_gelu_store": round(cached - mj("no_epilogue"), 2),
+        }
+        parts["rest_launch_gap_prologue_barriers_waits"] = round(whole - sum(parts.values()), 2)
+        out["energy_mJ_per_launch"] = {"whole_kernel": whole, **parts}
+        if pj["random_operands_read_from_lds"]:
+            out["energy_mJ_per_launch"]["cross_check_lds_reads_from_the_matrix_loops"] = round(
+                (pj["random_operands_read_from_lds"] - pj["random_operands"]) * GEMM_FLOP * 1e-9, 2)
+        out["note"] = ("each part = whole kernel minus the kernel without that part (cache-resident operands), the matrix "
+                       "instructions priced by the register-only loop on random operands; the parts overlap in time, so "
+                       "the differences are attributions, and the rest is what no ablation removes")
     return out
 
 
@@ -632,16 +937,22 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
-    ap.add_argument("--sustained", type=int, default=10000,
+    ap.add_argument("--sustained", type=int, default=30000,
                     help="launches of the sustained run that roofline.achieved is taken from (0 = use the timed steps); "
-                         "the default runs for more than a second, past the window over which the board averages its "
-                         "power, so that clock and power have settled")
+                         "the default runs for about 3.5 s: past the window over which the board averages its power, "
+                         "and long enough for the firmware's metrics table (energy counter, limiter residencies: one "
+                         "refresh a second) to refresh at least twice inside the run")
     ap.add_argument("--no-aux", action="store_true", help="skip the LayerNorm / CE kernels")
     ap.add_argument("--stream-ceiling", action="store_true",
                     help="instead of the benchmark: plain torch copies and fills of 32, 64 and 196 MiB buffers, "
                          "rotated through more than 512 MiB, for a kernel trace of what streaming kernels of the "
                          "LayerNorm / cross-entropy sizes reach on this GPU")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
+    ap.add_argument("--energy-table", type=float, default=0.0, metavar="SECONDS",
+                    help="instead of the benchmark: run the headline GEMM kernel whole and with one part taken out "
+                         "(operand loads, LDS fragment reads, epilogue), and the register-only matrix instruction "
+                         "loops, each for SECONDS (4 or more, for the firmware's energy counter), and print where a "
+                         "launch's energy goes")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run a plain 256 MiB device copy three times (the known-size kernel that hardware "
                          "counter runs of this script are scaled by)")
@@ -694,6 +1005,9 @@ def main():
     n_sets = 5
     sets, bias = make_gemm_inputs(n_sets, device)
     outs = [torch.empty((M, N), dtype=torch.bfloat16, device=device) for _ in range(n_sets)]
+    if args.energy_table > 0:
+        print(json.dumps({"energy_table": energy_table(device, sets, bias, outs, args.energy_table)}))
+        return
     aux = None if args.no_aux else bench_bandwidth_kernels(device)
     it = [0]
 
@@ -754,14 +1068,15 @@ def main():
                                      "frac": round(GEMM_FLOP / steps_us / 1e6 / MFMA_BF16_PEAK_TFLOPS, 4),
                                      "note": "HIP events around the K timed steps only, which follow the sustained run"}},
     }
-    if smi is not None:
+    if smi is not None and smi.get("shader_clock_MHz"):
         # 4096 matrix instructions of 32 cycles per SIMD and launch: the share of the launch's shader cycles in which
         # the matrix pipe is busy, at the clock the driver reports
         cycles = kernel_us * smi["shader_clock_MHz"]
         smi["mfma_busy_frac"] = round(GEMM_FLOP / (256 * 4 * 1024.0) / cycles, 4) if cycles > 0 else None
         smi["clock_x_busy_vs_2400MHz"] = round(smi["shader_clock_MHz"] / 2400.0 * smi["mfma_busy_frac"], 4)
+    if smi is not None:
         result["roofline"]["sustained_clock_power"] = smi
-    result["roofline"]["mfma_rate_ceiling"] = mfma_rate_ceiling(lib, device)
+    result["roofline"]["mfma_rate_ceiling"] = mfma_rate_ceiling(device)
     if args.calibrate_copy:
         src = torch.empty(256 << 20, dtype=torch.uint8, device=device).fill_(1)
         dst = torch.empty_like(src)

@@ -54,26 +54,24 @@ SIGNATURES = {
     "cw_attn_bwd": (_int, [_i64, _i64, _i64, _i64, _ptr, _ptr, _ptr, _i64, _i64, _i64, _ptr, _ptr, _i64, _i64, _i64, _ptr,
                            _f32, _int, _ptr, _ptr, _ptr, _i64, _i64, _i64, _ptr, _i64, _int, _ptr]),
     "cw_colsum_workspace_bytes": (_i64, [_i64, _i64]),
-    "cw_colsum": (_int, [_i64, _i64, _ptr, _i64, _ptr, _ptr, _i64, _int, _ptr]),
+    "cw_colsum": (_int, [_i64, _i64, _ptr, _i64, _ptr, _int, _ptr, _i64, _int, _ptr]),
     "cw_colsum_static_max_bytes": (_i64, []),
-    "cw_colsum_static": (_int, [_i64, _i64, _ptr, _i64, _ptr, _int, _ptr]),
-    "cw_act_bwd_colsum": (_int, [_int, _i64, _i64, _ptr, _i64, _ptr, _i64, _ptr, _i64, _ptr, _ptr, _i64, _int, _ptr]),
+    "cw_colsum_static": (_int, [_i64, _i64, _ptr, _i64, _ptr, _int, _int, _ptr]),
+    "cw_act_bwd_colsum": (_int, [_int, _i64, _i64, _ptr, _i64, _ptr, _i64, _ptr, _i64, _ptr, _int, _ptr, _i64, _int, _ptr]),
     "cw_ln_partial_stats": (_int, [_i64, _i64, _ptr, _i64, _int, _ptr, _ptr, _int, _ptr]),
     "cw_ln_normalize": (_int, [_i64, _i64, _ptr, _i64, _ptr, _int, _i64, _f32, _ptr, _ptr, _ptr, _i64, _ptr, _int,
                                _ptr]),
     "cw_ln_forward_fused": (_int, [_i64, _i64, _ptr, _i64, _int, _f32, _ptr, _ptr, _ptr, _i64, _ptr, _int, _ptr]),
-    "cw_ln_bwd_partials": (_int, [_i64, _i64, _ptr, _i64, _ptr, _i64, _ptr, _ptr, _ptr, _ptr, _ptr, _ptr, _i64, _int,
+    "cw_ln_bwd_partials": (_int, [_i64, _i64, _ptr, _i64, _ptr, _i64, _ptr, _ptr, _ptr, _ptr, _ptr, _int, _ptr, _i64, _int,
                                   _ptr]),
-    "cw_ln_backward_fused": (_int, [_i64, _i64, _ptr, _i64, _ptr, _i64, _ptr, _ptr, _ptr, _ptr, _i64, _ptr, _ptr, _ptr, _i64,
-                                    _int, _ptr]),
+    "cw_ln_backward_fused": (_int, [_i64, _i64, _ptr, _i64, _ptr, _i64, _ptr, _ptr, _ptr, _ptr, _i64, _ptr, _ptr, _int, _ptr,
+                                    _i64, _int, _ptr]),
     "cw_ln_bwd_dx": (_int, [_i64, _i64, _ptr, _i64, _ptr, _i64, _ptr, _ptr, _ptr, _i64, _ptr, _i64, _int, _ptr]),
     "cw_ln_bwd_partials_open": (_int, [_i64, _i64, _ptr, _i64, _ptr, _i64, _ptr, _ptr, _ptr, _ptr, _i64, _ptr, _int, _ptr]),
     "cw_ln_bwd_dx_close": (_int, [_i64, _i64, _ptr, _i64, _ptr, _i64, _ptr, _ptr, _ptr, _i64, _ptr, _i64, _ptr, _i64, _ptr,
-                                  _ptr, _int, _ptr]),
+                                  _ptr, _int, _int, _ptr]),
     "cw_vpce_fwd_local": (_int, [_i64, _i64, _ptr, _i64, _ptr, _i64, _ptr, _ptr, _ptr, _ptr, _int, _ptr]),
     "cw_vpce_finalize": (_int, [_i64, _int, _ptr, _ptr, _ptr, _ptr, _ptr, _ptr, _ptr, _ptr]),
-    "cw_diag_mfma_rate_flop": (_i64, [_int]),
-    "cw_diag_mfma_rate": (_int, [_int, _int, _ptr, _ptr]),
     "cw_vpce_bwd": (_int, [_i64, _i64, _ptr, _i64, _ptr, _i64, _ptr, _ptr, _ptr, _f32, _ptr, _i64, _int, _int, _ptr]),
 }
 

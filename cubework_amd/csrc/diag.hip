@@ -1,4 +1,4 @@
-// Measurement aid: the rate at which this GPU sustains the block GEMM's matrix instruction when nothing else
+// Measurement aid (libcubework_diag.so, loaded by bench.py only): the rate at which this GPU sustains the block GEMM's matrix instruction when nothing else
 // is in the way. Every wavefront keeps 4 x 4 accumulator tiles (the register blocking of the ring kernel) and
 // eight operand fragments of seeded random bf16 values in registers and issues v_mfma_f32_32x32x16_bf16 back to
 // back: no global loads, no LDS, no barriers. With mode 1 the fragments are all zero (no switching activity in

@@ -284,8 +284,9 @@ __global__ __launch_bounds__(256) void embed_bwd_generic_kernel(int64_t T_rows, 
 // Backward straight from the unsorted ids, one launch, for batches of up to kDirMaxTokens tokens. A workgroup owns
 // up to kDirRows rows of the slice, interleaved with the other workgroups' (row b, b + G, b + 2 G, ...). It reads all ids (they stay in L2: every workgroup reads the same
 // 8 T bytes) and marks, per row, the tokens that select it in a bitmap in LDS. The rows that up to kDirHeavy
-// tokens select are dealt round-robin to the wavefronts, which sum a row's tokens in ascending token position
-// (what a stable sort by id would hand the sorted kernel), kDirBatch token rows in flight; the row of a row's
+// tokens select are dealt round-robin to the wavefronts, which sum a row's tokens round by round, the lowest
+// remaining token of every 32-token word of its bitmap, words ascending (ascending token position - what a stable
+// sort by id would hand the sorted kernel - when no two of the row's tokens share a word), kDirBatch token rows in flight; the row of a row's
 // first token (known from the marking pass, an LDS minimum) is requested before any wavefront of the group
 // starts on the zeros, so the reads do not queue behind them in the compute unit's memory pipeline. The rows
 // without tokens are then written as zeros, a fixed share per wavefront. A row that more than kDirHeavy tokens select is left to the end and summed by all

@@ -103,8 +103,8 @@ __global__ __launch_bounds__(256) void colsum_generic_kernel(int64_t M, int64_t 
 constexpr int kFinGroups = 16;
 __global__ __launch_bounds__(kFinGroups * 64) void finalize_cols_kernel(const float* __restrict__ ws, int64_t nparts,
                                                                         int64_t part_stride, int64_t C,
-                                                                        float* __restrict__ out0,
-                                                                        float* __restrict__ out1) {
+                                                                        void* __restrict__ out0,
+                                                                        void* __restrict__ out1, int out_dtype) {
     __shared__ float red[kFinGroups][64];
     const int lane = threadIdx.x & 63;
     const int grp = threadIdx.x >> 6;
@@ -132,8 +132,8 @@ __global__ __launch_bounds__(kFinGroups * 64) void finalize_cols_kernel(const fl
         float total = red[0][lane];
 #pragma unroll
         for (int g = 1; g < kFinGroups; ++g) total += red[g][lane];
-        float* out = (k == 0) ? out0 : out1;
-        if (out != nullptr) out[c] = total;
+        void* out = (k == 0) ? out0 : out1;
+        if (out != nullptr) store_col_total(out, c, total, out_dtype);
     }
 }
 
@@ -156,7 +156,8 @@ void colsum_plan(int64_t M, int64_t N, int V, bool vec, int64_t& slabs, int64_t&
 
 template <typename T, int MODE>
 int colsum_impl(int64_t M, int64_t N, const void* dY, int64_t ld_dy, const void* pre, int64_t ld_pre, void* dPre,
-                int64_t ld_dpre, int act, float* out, void* workspace, int64_t workspace_bytes, hipStream_t s) {
+                int64_t ld_dpre, int act, void* out, int out_dtype, void* workspace, int64_t workspace_bytes,
+                hipStream_t s) {
     constexpr int V = elem<T>::kVec;
     const int want_sum = out != nullptr ? 1 : 0;
     bool vec = aligned16(dY) && (ld_dy % V) == 0 && (N % V) == 0;
@@ -188,15 +189,15 @@ int colsum_impl(int64_t M, int64_t N, const void* dY, int64_t ld_dy, const void*
     }
     int rc = check_launch("colsum kernel");
     if (rc != CW_OK || !want_sum) return rc;
-    return finalize_col_partials((const float*)workspace, slabs, N, 1, N, out, nullptr, s);
+    return finalize_col_partials((const float*)workspace, slabs, N, 1, N, out, nullptr, out_dtype, s);
 }
 
 }  // namespace
 
-int finalize_col_partials(const float* ws, int64_t nparts, int64_t part_stride, int nsets, int64_t C, float* out0,
-                          float* out1, hipStream_t s) {
+int finalize_col_partials(const float* ws, int64_t nparts, int64_t part_stride, int nsets, int64_t C, void* out0,
+                          void* out1, int out_dtype, hipStream_t s) {
     hipLaunchKernelGGL(finalize_cols_kernel, dim3((unsigned)((C + 63) / 64), (unsigned)nsets), dim3(kFinGroups * 64), 0, s, ws,
-                       nparts, part_stride, C, out0, out1);
+                       nparts, part_stride, C, out0, out1, out_dtype);
     return check_launch("finalize_cols_kernel");
 }
 
@@ -213,24 +214,34 @@ std::atomic<void*> g_scratch_ptr[kMaxDevices];
 std::mutex g_scratch_mutex;
 }  // namespace
 
-// Device address of this GPU's copy of `scratch` (nullptr + error text on failure).
-static void* static_scratch_ptr() {
+// Device address of this GPU's copy of `scratch` (nullptr + error text, *rc set, on failure). The first call on a
+// device looks the address up; a stream that is being captured is not the place for that (the lookup may load the
+// code object), so such a first call is refused and records nothing.
+static void* static_scratch_ptr(hipStream_t s, int* rc) {
     int dev = -1;
     if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) {
         (void)hipGetLastError();
-        fail(CW_ERR_DEVICE, "cw_colsum_static: no current HIP device (or device index above %d)", kMaxDevices - 1);
+        *rc = fail(CW_ERR_DEVICE, "cw_colsum_static: no current HIP device (or device index above %d)", kMaxDevices - 1);
         return nullptr;
     }
     void* p = g_scratch_ptr[dev].load(std::memory_order_acquire);
     if (p != nullptr) return p;
+    hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
+    if (hipStreamIsCapturing(s, &capturing) != hipSuccess) (void)hipGetLastError();
+    if (capturing != hipStreamCaptureStatusNone) {
+        *rc = fail(CW_ERR_UNSUPPORTED,
+                   "cw_colsum_static: the first call on a device looks up the scratch array's address and must be made "
+                   "outside a stream capture; call it once before capturing");
+        return nullptr;
+    }
     std::lock_guard<std::mutex> lock(g_scratch_mutex);
     p = g_scratch_ptr[dev].load(std::memory_order_acquire);
     if (p != nullptr) return p;
     const hipError_t e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
     if (e != hipSuccess || p == nullptr) {
         (void)hipGetLastError();
-        fail(CW_ERR_DEVICE, "cw_colsum_static: hipGetSymbolAddress(scratch) failed on device %d: %s", dev,
-             hipGetErrorString(e));
+        *rc = fail(CW_ERR_DEVICE, "cw_colsum_static: hipGetSymbolAddress(scratch) failed on device %d: %s", dev,
+                   hipGetErrorString(e));
         return nullptr;
     }
     g_scratch_ptr[dev].store(p, std::memory_order_release);
@@ -263,36 +274,38 @@ extern "C" int64_t cw_colsum_workspace_bytes(int64_t M, int64_t N) {
     return a > b ? a : b;
 }
 
-extern "C" int cw_colsum(int64_t M, int64_t N, const void* dY, int64_t ld, float* out, void* workspace,
+extern "C" int cw_colsum(int64_t M, int64_t N, const void* dY, int64_t ld, void* out, int out_dtype, void* workspace,
                          int64_t workspace_bytes, int io_dtype, void* stream) {
     if (M < 0 || N <= 0) return fail(CW_ERR_INVALID, "cw_colsum: bad shape M=%lld N=%lld", (long long)M, (long long)N);
     if (io_dtype != CW_BF16 && io_dtype != CW_F32 && io_dtype != CW_F16)
         return fail(CW_ERR_INVALID, "cw_colsum: bad io_dtype %d", io_dtype);
     if (out == nullptr) return fail(CW_ERR_INVALID, "cw_colsum: out is NULL");
+    if (!col_out_dtype_ok(out_dtype)) return fail(CW_ERR_INVALID, "cw_colsum: bad out_dtype %d", out_dtype);
     if (const int drc = require_gfx950("cw_colsum"); drc != CW_OK) return drc;
     hipStream_t s = (hipStream_t)stream;
-    if (M == 0) return finalize_col_partials(nullptr, 0, N, 1, N, out, nullptr, s);  // zero fill
+    if (M == 0) return finalize_col_partials(nullptr, 0, N, 1, N, out, nullptr, out_dtype, s);  // zero fill
     if (dY == nullptr || workspace == nullptr || ld < N)
         return fail(CW_ERR_INVALID, "cw_colsum: null pointer or ld < N");
     if (io_dtype == CW_F16)
-        return colsum_impl<f16_t, 0>(M, N, dY, ld, nullptr, 0, nullptr, 0, 0, out, workspace, workspace_bytes, s);
+        return colsum_impl<f16_t, 0>(M, N, dY, ld, nullptr, 0, nullptr, 0, 0, out, out_dtype, workspace, workspace_bytes, s);
     return io_dtype == CW_BF16
-               ? colsum_impl<bf16_t, 0>(M, N, dY, ld, nullptr, 0, nullptr, 0, 0, out, workspace, workspace_bytes, s)
-               : colsum_impl<float, 0>(M, N, dY, ld, nullptr, 0, nullptr, 0, 0, out, workspace, workspace_bytes, s);
+               ? colsum_impl<bf16_t, 0>(M, N, dY, ld, nullptr, 0, nullptr, 0, 0, out, out_dtype, workspace, workspace_bytes, s)
+               : colsum_impl<float, 0>(M, N, dY, ld, nullptr, 0, nullptr, 0, 0, out, out_dtype, workspace, workspace_bytes, s);
 }
 
 extern "C" int64_t cw_colsum_static_max_bytes(void) { return kStaticScratchBytes; }
 
-extern "C" int cw_colsum_static(int64_t M, int64_t N, const void* dY, int64_t ld, float* out, int io_dtype,
-                                void* stream) {
+extern "C" int cw_colsum_static(int64_t M, int64_t N, const void* dY, int64_t ld, void* out, int out_dtype,
+                                int io_dtype, void* stream) {
     if (M < 0 || N <= 0)
         return fail(CW_ERR_INVALID, "cw_colsum_static: bad shape M=%lld N=%lld", (long long)M, (long long)N);
     if (io_dtype != CW_BF16 && io_dtype != CW_F32 && io_dtype != CW_F16)
         return fail(CW_ERR_INVALID, "cw_colsum_static: bad io_dtype %d", io_dtype);
     if (out == nullptr) return fail(CW_ERR_INVALID, "cw_colsum_static: out is NULL");
+    if (!col_out_dtype_ok(out_dtype)) return fail(CW_ERR_INVALID, "cw_colsum_static: bad out_dtype %d", out_dtype);
     if (const int drc = require_gfx950("cw_colsum_static"); drc != CW_OK) return drc;
     hipStream_t s = (hipStream_t)stream;
-    if (M == 0) return finalize_col_partials(nullptr, 0, N, 1, N, out, nullptr, s);  // zero fill
+    if (M == 0) return finalize_col_partials(nullptr, 0, N, 1, N, out, nullptr, out_dtype, s);  // zero fill
     if (dY == nullptr || ld < N) return fail(CW_ERR_INVALID, "cw_colsum_static: null pointer or ld < N");
     const int64_t need = with_elem_type(io_dtype, [&](auto* tag) -> int {
         using T = std::remove_pointer_t<decltype(tag)>;
@@ -304,14 +317,16 @@ extern "C" int cw_colsum_static(int64_t M, int64_t N, const void* dY, int64_t ld
                     "cw_colsum_static: [%lld, %lld] needs more than the %lld bytes of the library's static scratch "
                     "(16-byte aligned operands: N <= 1048576; others: ceil(M/64) * N <= 1048576); use cw_colsum",
                     (long long)M, (long long)N, (long long)kStaticScratchBytes);
-    void* ws = static_scratch_ptr();  // the device address, never the array's name
-    if (ws == nullptr) return CW_ERR_DEVICE;
-    return cw_colsum(M, N, dY, ld, out, ws, kStaticScratchBytes, io_dtype, stream);
+    int prc = CW_ERR_DEVICE;
+    void* ws = static_scratch_ptr(s, &prc);  // the device address, never the array's name
+    if (ws == nullptr) return prc;
+    return cw_colsum(M, N, dY, ld, out, out_dtype, ws, kStaticScratchBytes, io_dtype, stream);
 }
 
 extern "C" int cw_act_bwd_colsum(int activation, int64_t M, int64_t N, const void* dY, int64_t ld_dy,
-                                 const void* preact, int64_t ld_pre, void* dPre, int64_t ld_dpre, float* dbias,
-                                 void* workspace, int64_t workspace_bytes, int io_dtype, void* stream) {
+                                 const void* preact, int64_t ld_pre, void* dPre, int64_t ld_dpre, void* dbias,
+                                 int dbias_dtype, void* workspace, int64_t workspace_bytes, int io_dtype,
+                                 void* stream) {
     if (M < 0 || N <= 0)
         return fail(CW_ERR_INVALID, "cw_act_bwd_colsum: bad shape M=%lld N=%lld", (long long)M, (long long)N);
     if (io_dtype != CW_BF16 && io_dtype != CW_F32 && io_dtype != CW_F16)
@@ -319,21 +334,23 @@ extern "C" int cw_act_bwd_colsum(int activation, int64_t M, int64_t N, const voi
     if (activation != CW_ACT_NONE && activation != CW_ACT_GELU_TANH && activation != CW_ACT_GELU_ERF &&
         activation != CW_ACT_RELU)
         return fail(CW_ERR_INVALID, "cw_act_bwd_colsum: bad activation %d", activation);
+    if (dbias != nullptr && !col_out_dtype_ok(dbias_dtype))
+        return fail(CW_ERR_INVALID, "cw_act_bwd_colsum: bad dbias_dtype %d", dbias_dtype);
     if (const int drc = require_gfx950("cw_act_bwd_colsum"); drc != CW_OK) return drc;
     hipStream_t s = (hipStream_t)stream;
     if (M == 0) {
         if (dbias == nullptr) return CW_OK;
-        return finalize_col_partials(nullptr, 0, N, 1, N, dbias, nullptr, s);  // zero fill
+        return finalize_col_partials(nullptr, 0, N, 1, N, dbias, nullptr, dbias_dtype, s);  // zero fill
     }
     if (dY == nullptr || preact == nullptr || dPre == nullptr || ld_dy < N || ld_pre < N || ld_dpre < N)
         return fail(CW_ERR_INVALID, "cw_act_bwd_colsum: null pointer or leading dimension < N");
     if (dbias != nullptr && workspace == nullptr)
         return fail(CW_ERR_INVALID, "cw_act_bwd_colsum: workspace is NULL");
     if (io_dtype == CW_F16)
-        return colsum_impl<f16_t, 1>(M, N, dY, ld_dy, preact, ld_pre, dPre, ld_dpre, activation, dbias, workspace,
-                                     workspace_bytes, s);
+        return colsum_impl<f16_t, 1>(M, N, dY, ld_dy, preact, ld_pre, dPre, ld_dpre, activation, dbias, dbias_dtype,
+                                     workspace, workspace_bytes, s);
     return io_dtype == CW_BF16 ? colsum_impl<bf16_t, 1>(M, N, dY, ld_dy, preact, ld_pre, dPre, ld_dpre, activation, dbias,
-                                                        workspace, workspace_bytes, s)
+                                                        dbias_dtype, workspace, workspace_bytes, s)
                                : colsum_impl<float, 1>(M, N, dY, ld_dy, preact, ld_pre, dPre, ld_dpre, activation, dbias,
-                                                       workspace, workspace_bytes, s);
+                                                       dbias_dtype, workspace, workspace_bytes, s);
 }

@@ -116,7 +116,12 @@ struct FragReader {
 // SPLIT: blockIdx.y selects one of gridDim.y equal slices of every step's k
 // range; the block writes its fp32 partial tile to args.partial and
 // splitk_reduce_kernel finishes the sum and the epilogue.
-template <bool TRANS_A, bool TRANS_B, int EPI, int NS, bool SPLIT, typename E>
+// ABL: 0 in every instantiation of the library. The measurement library instantiates the same kernel with one
+// part taken out, to price that part (time and energy per launch against the whole kernel; the results of such
+// a launch are meaningless): 1 = the k loop issues no operand loads (the ring's stages are filled once, in the
+// prologue, and re-used), 2 = no epilogue (nothing is stored), 3 = the k loop reads no fragments from LDS (the
+// first tile's stay in the registers).
+template <bool TRANS_A, bool TRANS_B, int EPI, int NS, bool SPLIT, typename E, int ABL = 0>
 __global__ __launch_bounds__(kThreads) void gemm_bf16_dma_kernel(const RingArgs args) {
     extern __shared__ __attribute__((aligned(16))) uint16_t lds[];
     lds_char* lds_base = (lds_char*)lds;
@@ -224,7 +229,7 @@ __global__ __launch_bounds__(kThreads) void gemm_bf16_dma_kernel(const RingArgs 
 
     // prologue: tiles 0..NS-3 in flight, plus the A part of tile NS-2 (its B part
     // is issued by the first loop iteration, like every later tile's)
-    for (int p = 0; p < NS - 2; ++p) {
+    for (int p = 0; p < (ABL == 1 ? NS : NS - 2); ++p) {
         const uint32_t st = lds_addr0 + is_stage * kStageBytes;
         gemm_bf16::static_for<4>([&](auto I) {
             dma_one<TRANS_A, I.value>(is_a, lda_bytes, is_k0, a_even, a_odd, st, wave);
@@ -232,13 +237,14 @@ __global__ __launch_bounds__(kThreads) void gemm_bf16_dma_kernel(const RingArgs 
         });
         issue_advance();
     }
-    {
+    if constexpr (ABL != 1) {
         const uint32_t st = lds_addr0 + is_stage * kStageBytes;
         gemm_bf16::static_for<4>([&](auto I) {
             dma_one<TRANS_A, I.value>(is_a, lda_bytes, is_k0, a_even, a_odd, st, wave);
         });
     }
-    dma_wait<kDmaPerTile*(NS - 3) + 4>();
+    if constexpr (ABL == 1) dma_wait<0>();
+    else dma_wait<kDmaPerTile*(NS - 3) + 4>();
     __builtin_amdgcn_s_barrier();
     asm volatile("" ::: "memory");
 
@@ -247,6 +253,10 @@ __global__ __launch_bounds__(kThreads) void gemm_bf16_dma_kernel(const RingArgs 
     gemm_bf16::static_for<4>([&](auto t) {
         af[0][t.value] = fa.template read<t.value, 0>(lds_base);
         bfr[0][t.value] = fb.template read<t.value, 0>(lds_base + kOperBytes);
+        if constexpr (ABL == 3) {
+            af[1][t.value] = fa.template read<t.value, 1>(lds_base);
+            bfr[1][t.value] = fb.template read<t.value, 1>(lds_base + kOperBytes);
+        }
     });
 
     for (int kt = 0; kt < KT; ++kt) {
@@ -268,9 +278,9 @@ __global__ __launch_bounds__(kThreads) void gemm_bf16_dma_kernel(const RingArgs 
                     // (measurably less power than row by row, where every fourth changes both)
                     constexpr int JS = (I & 1) ? 3 - J : J;
                     acc[I][JS] = gemm_bf16::mfma_32x32x16<E>(bfr[0][JS], af[0][I], acc[I][JS]);
-                    if constexpr (Q < 4) af[1][Q] = fa.template read<Q, 1>(sa);
-                    else if constexpr (Q < 8) bfr[1][Q - 4] = fb.template read<Q - 4, 1>(sb);
-                    else if constexpr ((Q & 1) == 0) dma_one<TRANS_B, (Q - 8) / 2>(is_b, ldb_bytes, is_k0, b_even, b_odd, st + kOperBytes, wave);
+                    if constexpr (Q < 4) { if constexpr (ABL != 3) af[1][Q] = fa.template read<Q, 1>(sa); }
+                    else if constexpr (Q < 8) { if constexpr (ABL != 3) bfr[1][Q - 4] = fb.template read<Q - 4, 1>(sb); }
+                    else if constexpr ((Q & 1) == 0 && ABL != 1) dma_one<TRANS_B, (Q - 8) / 2>(is_b, ldb_bytes, is_k0, b_even, b_odd, st + kOperBytes, wave);
                     CW_PIN();
                 });
             });
@@ -290,9 +300,9 @@ __global__ __launch_bounds__(kThreads) void gemm_bf16_dma_kernel(const RingArgs 
                     constexpr int I = i.value, J = j.value, Q = I * 4 + J;
                     constexpr int JS = (I & 1) ? 3 - J : J;
                     acc[I][JS] = gemm_bf16::mfma_32x32x16<E>(bfr[1][JS], af[1][I], acc[I][JS]);
-                    if constexpr (Q < 8 && (Q & 1) == 0) dma_one<TRANS_A, Q / 2>(is_a, lda_bytes, is_k0, a_even, a_odd, st, wave);
-                    else if constexpr (Q >= 8 && Q < 12) af[0][Q - 8] = fa.template read<Q - 8, 0>(na);
-                    else if constexpr (Q >= 12) bfr[0][Q - 12] = fb.template read<Q - 12, 0>(nb);
+                    if constexpr (Q < 8 && (Q & 1) == 0) { if constexpr (ABL != 1) dma_one<TRANS_A, Q / 2>(is_a, lda_bytes, is_k0, a_even, a_odd, st, wave); }
+                    else if constexpr (Q >= 8 && Q < 12) { if constexpr (ABL != 3) af[0][Q - 8] = fa.template read<Q - 8, 0>(na); }
+                    else if constexpr (Q >= 12) { if constexpr (ABL != 3) bfr[0][Q - 12] = fb.template read<Q - 12, 0>(nb); }
                     CW_PIN();
                 });
             });
@@ -318,6 +328,9 @@ __global__ __launch_bounds__(kThreads) void gemm_bf16_dma_kernel(const RingArgs 
                     u.w = __float_as_uint(acc[i][j][4 * g + 3]);
                     *reinterpret_cast<raw16_t*>(part + (int64_t)i * 32 * N + j * 32 + 8 * g) = u;
                 }
+    } else if constexpr (ABL == 2) {
+        // never true for a launch that got this far: keeps the products alive without storing them
+        if (args.n_steps < 0) gemm_bf16::gemm_epilogue_slabs<EPI, E>(acc, args, bias_raw, lds, m0, n0, wm, wn, lane, tid);
     } else {
         gemm_bf16::gemm_epilogue_slabs<EPI, E>(acc, args, bias_raw, lds, m0, n0, wm, wn, lane, tid);
     }

@@ -1189,9 +1189,9 @@ constexpr int64_t kGenericSlabRows = 64;
 // kernel chosen wrote dx or the caller still has to run the dx kernel.
 template <typename T>
 int bwd_partials_impl(int64_t R, int64_t C, const void* dY, int64_t ld_dy, const void* x, int64_t ld_x,
-                      const float* mean_rstd, const void* gamma, float* row_sums, float* dgamma, float* dbeta,
-                      void* workspace, int64_t workspace_bytes, hipStream_t s, void* dx = nullptr, int64_t ld_dx = 0,
-                      bool* dx_done = nullptr, int64_t* open_parts = nullptr) {
+                      const float* mean_rstd, const void* gamma, float* row_sums, void* dgamma, void* dbeta,
+                      int param_dtype, void* workspace, int64_t workspace_bytes, hipStream_t s, void* dx = nullptr,
+                      int64_t ld_dx = 0, bool* dx_done = nullptr, int64_t* open_parts = nullptr) {
     // open_parts: the column partials are left in the workspace, their count is reported, and whoever launches next
     // on the stream adds them up (bwd_dx_impl with a FinishCols)
     constexpr int V = elem<T>::kVec;
@@ -1251,7 +1251,7 @@ int bwd_partials_impl(int64_t R, int64_t C, const void* dY, int64_t ld_dy, const
     }
     if (want_cols) {
         // ws is [nparts][2][C]: dgamma partials are rows 2p, dbeta partials rows 2p+1.
-        rc = finalize_col_partials((const float*)workspace, nparts, 2 * C, 2, C, dgamma, dbeta, s);
+        rc = finalize_col_partials((const float*)workspace, nparts, 2 * C, 2, C, dgamma, dbeta, param_dtype, s);
     }
     return rc;
 }
@@ -1360,11 +1360,13 @@ extern "C" int cw_ln_forward_fused(int64_t R, int64_t C, const void* x, int64_t 
 }
 
 extern "C" int cw_ln_bwd_partials(int64_t R, int64_t C, const void* dY, int64_t ld_dy, const void* x, int64_t ld_x,
-                                  const float* mean_rstd, const void* gamma, float* row_sums, float* dgamma,
-                                  float* dbeta, void* workspace, int64_t workspace_bytes, int io_dtype,
+                                  const float* mean_rstd, const void* gamma, float* row_sums, void* dgamma,
+                                  void* dbeta, int param_dtype, void* workspace, int64_t workspace_bytes, int io_dtype,
                                   void* stream) {
     int rc = check_rc("cw_ln_bwd_partials", R, C, io_dtype);
     if (rc != CW_OK) return rc;
+    if (dgamma != nullptr && !col_out_dtype_ok(param_dtype))
+        return fail(CW_ERR_INVALID, "cw_ln_bwd_partials: bad param_dtype %d", param_dtype);
     if ((dgamma == nullptr) != (dbeta == nullptr))
         return fail(CW_ERR_INVALID, "cw_ln_bwd_partials: dgamma and dbeta must both be given or both be NULL");
     if (R == 0) return CW_OK;
@@ -1375,7 +1377,8 @@ extern "C" int cw_ln_bwd_partials(int64_t R, int64_t C, const void* dY, int64_t 
     hipStream_t s = (hipStream_t)stream;
     return with_elem_type(io_dtype, [&](auto* tag) {
         return bwd_partials_impl<std::remove_pointer_t<decltype(tag)>>(R, C, dY, ld_dy, x, ld_x, mean_rstd, gamma, row_sums,
-                                                                       dgamma, dbeta, workspace, workspace_bytes, s);
+                                                                       dgamma, dbeta, param_dtype, workspace,
+                                                                       workspace_bytes, s);
     });
 }
 
@@ -1384,10 +1387,11 @@ namespace {
 template <typename T>
 int backward_fused_impl(int64_t R, int64_t C, const void* dY, int64_t ld_dy, const void* x, int64_t ld_x,
                         const float* mean_rstd, const void* gamma, float* row_sums, void* dx, int64_t ld_dx,
-                        float* dgamma, float* dbeta, void* workspace, int64_t workspace_bytes, hipStream_t s) {
+                        void* dgamma, void* dbeta, int param_dtype, void* workspace, int64_t workspace_bytes,
+                        hipStream_t s) {
     bool dx_done = false;
-    int rc = bwd_partials_impl<T>(R, C, dY, ld_dy, x, ld_x, mean_rstd, gamma, row_sums, dgamma, dbeta, workspace,
-                                  workspace_bytes, s, dx, ld_dx, &dx_done);
+    int rc = bwd_partials_impl<T>(R, C, dY, ld_dy, x, ld_x, mean_rstd, gamma, row_sums, dgamma, dbeta, param_dtype,
+                                  workspace, workspace_bytes, s, dx, ld_dx, &dx_done);
     if (rc != CW_OK || dx_done) return rc;
     return bwd_dx_impl<T>(R, C, dY, ld_dy, x, ld_x, mean_rstd, gamma, row_sums, C, dx, ld_dx, s);
 }
@@ -1396,10 +1400,12 @@ int backward_fused_impl(int64_t R, int64_t C, const void* dY, int64_t ld_dy, con
 
 extern "C" int cw_ln_backward_fused(int64_t R, int64_t C, const void* dY, int64_t ld_dy, const void* x, int64_t ld_x,
                                     const float* mean_rstd, const void* gamma, float* row_sums, void* dx,
-                                    int64_t ld_dx, float* dgamma, float* dbeta, void* workspace,
+                                    int64_t ld_dx, void* dgamma, void* dbeta, int param_dtype, void* workspace,
                                     int64_t workspace_bytes, int io_dtype, void* stream) {
     int rc = check_rc("cw_ln_backward_fused", R, C, io_dtype);
     if (rc != CW_OK) return rc;
+    if (dgamma != nullptr && !col_out_dtype_ok(param_dtype))
+        return fail(CW_ERR_INVALID, "cw_ln_backward_fused: bad param_dtype %d", param_dtype);
     if ((dgamma == nullptr) != (dbeta == nullptr))
         return fail(CW_ERR_INVALID, "cw_ln_backward_fused: dgamma and dbeta must both be given or both be NULL");
     if (R == 0) return CW_OK;
@@ -1411,8 +1417,8 @@ extern "C" int cw_ln_backward_fused(int64_t R, int64_t C, const void* dY, int64_
     hipStream_t s = (hipStream_t)stream;
     return with_elem_type(io_dtype, [&](auto* tag) {
         return backward_fused_impl<std::remove_pointer_t<decltype(tag)>>(R, C, dY, ld_dy, x, ld_x, mean_rstd, gamma, row_sums,
-                                                                         dx, ld_dx, dgamma, dbeta, workspace,
-                                                                         workspace_bytes, s);
+                                                                         dx, ld_dx, dgamma, dbeta, param_dtype,
+                                                                         workspace, workspace_bytes, s);
     });
 }
 
@@ -1449,17 +1455,18 @@ extern "C" int cw_ln_bwd_partials_open(int64_t R, int64_t C, const void* dY, int
     hipStream_t s = (hipStream_t)stream;
     return with_elem_type(io_dtype, [&](auto* tag) {
         return bwd_partials_impl<std::remove_pointer_t<decltype(tag)>>(R, C, dY, ld_dy, x, ld_x, mean_rstd, gamma, row_sums,
-                                                                       nullptr, nullptr, workspace, workspace_bytes, s,
-                                                                       nullptr, 0, nullptr, n_parts);
+                                                                       nullptr, nullptr, CW_F32, workspace,
+                                                                       workspace_bytes, s, nullptr, 0, nullptr, n_parts);
     });
 }
 
 extern "C" int cw_ln_bwd_dx_close(int64_t R, int64_t C, const void* dY, int64_t ld_dy, const void* x, int64_t ld_x,
                                   const float* mean_rstd, const void* gamma, const float* row_sums, int64_t H, void* dx,
-                                  int64_t ld_dx, const void* workspace, int64_t n_parts, float* dgamma, float* dbeta,
-                                  int io_dtype, void* stream) {
+                                  int64_t ld_dx, const void* workspace, int64_t n_parts, void* dgamma, void* dbeta,
+                                  int param_dtype, int io_dtype, void* stream) {
     int rc = check_rc("cw_ln_bwd_dx_close", R, C, io_dtype);
     if (rc != CW_OK) return rc;
+    if (!col_out_dtype_ok(param_dtype)) return fail(CW_ERR_INVALID, "cw_ln_bwd_dx_close: bad param_dtype %d", param_dtype);
     if (H < C) return fail(CW_ERR_INVALID, "cw_ln_bwd_dx_close: hidden size H=%lld smaller than local C=%lld", (long long)H, (long long)C);
     if (dgamma == nullptr || dbeta == nullptr) return fail(CW_ERR_INVALID, "cw_ln_bwd_dx_close: dgamma and dbeta are both needed");
     if (n_parts < 0 || n_parts > (1 << 20) || (n_parts > 0 && workspace == nullptr) || C > ((int64_t)1 << 30))
@@ -1468,7 +1475,7 @@ extern "C" int cw_ln_bwd_dx_close(int64_t R, int64_t C, const void* dY, int64_t 
     hipStream_t s = (hipStream_t)stream;
     if (R == 0 || n_parts == 0) {
         // no rows: the column sums are zero (the finalize kernel over zero partial rows writes them)
-        rc = finalize_col_partials(nullptr, 0, 2 * C, 2, C, dgamma, dbeta, s);
+        rc = finalize_col_partials(nullptr, 0, 2 * C, 2, C, dgamma, dbeta, param_dtype, s);
         if (rc != CW_OK || R == 0) return rc;
     }
     if (dY == nullptr || x == nullptr || mean_rstd == nullptr || row_sums == nullptr || dx == nullptr || ld_dy < C ||
@@ -1481,6 +1488,7 @@ extern "C" int cw_ln_bwd_dx_close(int64_t R, int64_t C, const void* dY, int64_t 
     fin.C = C;
     fin.out0 = dgamma;
     fin.out1 = dbeta;
+    fin.out_dtype = param_dtype;
     fin.blocks = n_parts > 0 ? 2 * (int)((C + 63) / 64) : 0;
     return with_elem_type(io_dtype, [&](auto* tag) {
         return bwd_dx_impl<std::remove_pointer_t<decltype(tag)>>(R, C, dY, ld_dy, x, ld_x, mean_rstd, gamma, row_sums, H, dx,

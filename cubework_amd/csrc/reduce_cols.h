@@ -58,10 +58,18 @@ __device__ __forceinline__ void block_flat_reduce(const float (&acc)[NREG], floa
 struct FinishCols {
     const float* ws;
     int64_t nparts, part_stride, C;
-    float* out0;
-    float* out1;
+    void* out0;
+    void* out1;
     int blocks;
+    int out_dtype;  // CW_F32 / CW_BF16 / CW_F16: the type the totals are stored in (rounded once, to nearest even)
 };
+
+// One finished column total into an output vector of the given element type.
+__device__ __forceinline__ void store_col_total(void* out, int64_t c, float total, int out_dtype) {
+    if (out_dtype == CW_F32) reinterpret_cast<float*>(out)[c] = total;
+    else if (out_dtype == CW_BF16) store_elem(reinterpret_cast<bf16_t*>(out) + c, total);
+    else store_elem(reinterpret_cast<f16_t*>(out) + c, total);
+}
 
 // Workgroup `block` (< f.blocks) of THREADS threads: 64 columns of one of the two sets. The THREADS / 64 groups
 // of 64 threads split the partial rows, 16 independent loads in flight each, and are combined in index order.
@@ -93,15 +101,17 @@ __device__ __forceinline__ void finish_cols_block(const FinishCols& f, int block
         float total = red[lane];
 #pragma unroll
         for (int g = 1; g < G; ++g) total += red[g * 64 + lane];
-        float* out = (k == 0) ? f.out0 : f.out1;
-        if (out != nullptr) out[c] = total;
+        void* out = (k == 0) ? f.out0 : f.out1;
+        if (out != nullptr) store_col_total(out, c, total, f.out_dtype);
     }
 }
 
 // out_k[c] = sum_p ws[p*part_stride + k*C + c], k < nsets (nsets is 1 or 2;
-// out1 is ignored when nsets == 1). Enqueued on `s`.
-int finalize_col_partials(const float* ws, int64_t nparts, int64_t part_stride, int nsets, int64_t C, float* out0,
-                          float* out1, hipStream_t s);
+// out1 is ignored when nsets == 1), stored as out_dtype. Enqueued on `s`.
+int finalize_col_partials(const float* ws, int64_t nparts, int64_t part_stride, int nsets, int64_t C, void* out0,
+                          void* out1, int out_dtype, hipStream_t s);
+
+inline bool col_out_dtype_ok(int dt) { return dt == CW_F32 || dt == CW_BF16 || dt == CW_F16; }
 
 // Scratch bounds of the two users, combined by cw_colsum_workspace_bytes.
 int64_t colsum_workspace_bytes(int64_t M, int64_t N);

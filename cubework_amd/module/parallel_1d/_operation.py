@@ -49,12 +49,12 @@ class _LinearNT(torch.autograd.Function):
         dbias = None
         with torch.no_grad():
             if activation is not None:
-                g, dbias = ops.act_bwd_colsum(activation, g, pre, want_dbias=has_bias)
+                g, dbias = ops.act_bwd_colsum(activation, g, pre, want_dbias=has_bias, out_dtype=bias_dtype)
             elif has_bias:
-                dbias = ops.colsum(g)
+                dbias = ops.colsum(g, out_dtype=bias_dtype)   # fp32 sums stored in the parameter's dtype: no cast launch
             dx = ops.gemm_ksteps("NN", [g], [weight]).reshape(in_shape) if ctx.needs_input_grad[0] else None
             dw = ops.gemm_ksteps("TN", [g], [x2]) if ctx.needs_input_grad[1] else None
-        return dx, dw, None if dbias is None else dbias.to(bias_dtype), None
+        return dx, dw, dbias, None
 
 
 def linear_nt(input_: Tensor, weight: Tensor, bias: Optional[Tensor] = None,

@@ -109,7 +109,7 @@ class _BiasAdd(torch.autograd.Function):
 
     @staticmethod
     def backward(ctx, grad):
-        return grad, ops.colsum(grad.reshape(-1, grad.shape[-1])).to(ctx.bias_dtype)
+        return grad, ops.colsum(grad.reshape(-1, grad.shape[-1]), out_dtype=ctx.bias_dtype)
 
 
 class Linear1D(nn.Module):

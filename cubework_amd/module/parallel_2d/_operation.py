@@ -33,15 +33,19 @@ class _SUMMA_AB(torch.autograd.Function):
 
     @staticmethod
     @gemm_fwd()
-    def forward(ctx, A, B, bias, summa_dim, out_shape, row_parallel_mode, col_parallel_mode, activation):
+    def forward(ctx, A, B, bias, summa_dim, out_shape, row_parallel_mode, col_parallel_mode, activation, residual=None):
         assert A.shape[-1] == B.shape[-2], "Invalid shapes: A={}, B={} for AB.".format(A.shape, B.shape)
+        if residual is not None and activation is not None:
+            raise ValueError("a residual addend and a fused activation cannot be combined: the addend would be "
+                             "added before the activation")
         A2, B2 = _flat(A), _flat(B)
         A_steps = [broadcast(A2, row_parallel_mode.rank_by_idx(i), row_parallel_mode) for i in range(summa_dim)]
         B_steps = [broadcast(B2, col_parallel_mode.rank_by_idx(i), col_parallel_mode) for i in range(summa_dim)]
         bias_full = None if bias is None else all_gather(bias, -1, col_parallel_mode)
         # ReLU needs no separate pre-activation: its derivative [pre > 0] is [out > 0], so the output serves
         need_pre = activation is not None and activation != "relu"
-        res = ops.gemm_ksteps("NN", A_steps, B_steps, bias_full, activation, want_preact=need_pre)
+        addends = () if residual is None else (residual.reshape(-1, out_shape[-1]),)
+        res = ops.gemm_ksteps("NN", A_steps, B_steps, bias_full, activation, addends=addends, want_preact=need_pre)
         out, pre = res if need_pre else (res, None)
         if activation == "relu":
             pre = out
@@ -57,30 +61,34 @@ class _SUMMA_AB(torch.autograd.Function):
         summa_dim, row_mode, col_mode, activation, has_bias, bias_dtype, A_shape, B_shape = ctx.meta
         g = _flat(output_grad)
         bias_grad = None
+        # with nobody to sum the column sums with, they are stored in the parameter's dtype at once (no cast launch);
+        # across ranks the fp32 sums are reduced first and rounded once afterwards
+        sum_dtype = bias_dtype if has_bias and col_mode.world_size == 1 else None
         with torch.no_grad():
             if activation is not None:
-                g, dbias = ops.act_bwd_colsum(activation, g, pre, want_dbias=has_bias)
+                g, dbias = ops.act_bwd_colsum(activation, g, pre, want_dbias=has_bias, out_dtype=sum_dtype)
             elif has_bias:
-                dbias = ops.colsum(g)
+                dbias = ops.colsum(g, out_dtype=sum_dtype)
             if has_bias:
                 bias_grad = reduce_scatter(dbias, -1, col_mode).to(bias_dtype)
             g = g.reshape(output_grad.shape)
             A_grad = summa_ABT(g, B, summa_dim, A_shape, row_mode, col_mode) if ctx.needs_input_grad[0] else None
             B_grad = summa_ATB(A, g, summa_dim, B_shape, row_mode, col_mode) if ctx.needs_input_grad[1] else None
-        return A_grad, B_grad, bias_grad, None, None, None, None, None
+        residual_grad = output_grad if len(ctx.needs_input_grad) > 8 and ctx.needs_input_grad[8] else None
+        return A_grad, B_grad, bias_grad, None, None, None, None, None, residual_grad
 
 
 def summa_AB(A: Tensor, B: Tensor, summa_dim: int, out_shape: Tuple[int, ...], row_parallel_mode: ParallelMode,
              col_parallel_mode: ParallelMode) -> Tensor:
     """Reference signature (_operation.py:83-91)."""
-    return _SUMMA_AB.apply(A, B, None, summa_dim, out_shape, row_parallel_mode, col_parallel_mode, None)
+    return _SUMMA_AB.apply(A, B, None, summa_dim, out_shape, row_parallel_mode, col_parallel_mode, None, None)
 
 
 def summa_AB_bias_act(A: Tensor, B: Tensor, bias: Optional[Tensor], summa_dim: int, out_shape: Tuple[int, ...],
                       row_parallel_mode: ParallelMode, col_parallel_mode: ParallelMode,
-                      activation: Optional[str] = None) -> Tensor:
-    """summa_AB + add_bias_2d (+ activation) in one kernel."""
-    return _SUMMA_AB.apply(A, B, bias, summa_dim, out_shape, row_parallel_mode, col_parallel_mode, activation)
+                      activation: Optional[str] = None, residual: Optional[Tensor] = None) -> Tensor:
+    """summa_AB + add_bias_2d (+ activation, or + a residual of the output's shape) in one kernel."""
+    return _SUMMA_AB.apply(A, B, bias, summa_dim, out_shape, row_parallel_mode, col_parallel_mode, activation, residual)
 
 
 class _SUMMA_ABT(torch.autograd.Function):
@@ -179,7 +187,7 @@ class _SUMMAbias(torch.autograd.Function):
         col_mode, skipped, bias_dtype = ctx.meta
         if skipped:
             return None, reduce_scatter(output_grad, -1, col_mode), None, None, None
-        dbias = ops.colsum(_flat(output_grad))
+        dbias = ops.colsum(_flat(output_grad), out_dtype=bias_dtype if col_mode.world_size == 1 else None)
         return output_grad, reduce_scatter(dbias, -1, col_mode).to(bias_dtype), None, None, None
 
 
@@ -214,15 +222,17 @@ class _Layernorm2D(torch.autograd.Function):
     def backward(ctx, output_grad):
         x, gamma, mean_rstd = ctx.saved_tensors
         hidden_size, row_mode, col_mode, w_dtype, b_dtype = ctx.meta
+        # dgamma / dbeta: fp32 sums, stored in the parameters' dtype at once where no reduce-scatter follows
+        pd = w_dtype if col_mode.world_size == 1 and w_dtype == b_dtype else None
         with torch.no_grad():
             if row_mode.world_size == 1:
-                input_grad, dgamma, dbeta = ops.ln_backward_fused(output_grad, x, mean_rstd, gamma)
+                input_grad, dgamma, dbeta = ops.ln_backward_fused(output_grad, x, mean_rstd, gamma, param_dtype=pd)
             else:
                 # the dx launch also finishes the column sums that the first launch leaves as partial rows
                 row_sums, pending = ops.ln_bwd_partials_open(output_grad, x, mean_rstd, gamma)
                 row_sums = all_reduce(row_sums, row_mode)
                 input_grad, dgamma, dbeta = ops.ln_bwd_dx_close(output_grad, x, mean_rstd, row_sums, hidden_size, pending,
-                                                                gamma)
+                                                                gamma, param_dtype=pd)
             weight_grad = reduce_scatter(dgamma, -1, col_mode).to(w_dtype)
             bias_grad = reduce_scatter(dbeta, -1, col_mode).to(b_dtype)
         return input_grad, weight_grad, bias_grad, None, None, None, None
@@ -259,7 +269,8 @@ class _Classifier2D(torch.autograd.Function):
             A_grad = ops.gemm_ksteps("NN", [g], [B_temp]).reshape(A_shape)
             B_grad = ops.gemm_ksteps("TN", [g], [A2])
             B_grad = reduce_scatter(B_grad, -1, col_mode).reshape(B_shape)
-            bias_grad = all_reduce(ops.colsum(g), col_mode).to(bias_dtype) if use_bias else None
+            sum_dtype = bias_dtype if use_bias and col_mode.world_size == 1 else None
+            bias_grad = all_reduce(ops.colsum(g, out_dtype=sum_dtype), col_mode).to(bias_dtype) if use_bias else None
         return A_grad, B_grad, bias_grad, None, None, None, None
 
 

@@ -60,10 +60,12 @@ class _Linear3D(torch.autograd.Function):
             g = all_gather(output_grad, 0, out_mode)
             g2 = _flat(g)
             bias_grad = None
+            # fp32 column sums, stored in the parameter's dtype at once when nobody else adds to them
+            sum_dtype = bias_dtype if use_bias and w_mode.world_size == 1 else None
             if activation is not None:
-                g2, dbias = ops.act_bwd_colsum(activation, g2, pre, want_dbias=use_bias)
+                g2, dbias = ops.act_bwd_colsum(activation, g2, pre, want_dbias=use_bias, out_dtype=sum_dtype)
             elif use_bias:
-                dbias = ops.colsum(g2)
+                dbias = ops.colsum(g2, out_dtype=sum_dtype)
             if use_bias:
                 bias_grad = all_reduce(dbias, w_mode).to(bias_dtype)
             weight_grad = ops.gemm_ksteps("TN", [_flat(x)], [g2])
@@ -110,7 +112,8 @@ class _Classifier3D(torch.autograd.Function):
                 weight_grad = None
             bias_grad = None
             if use_bias:
-                bias_grad = all_reduce(all_reduce(ops.colsum(g2), in_mode), w_mode).to(bias_dtype)
+                sum_dtype = bias_dtype if in_mode.world_size == 1 and w_mode.world_size == 1 else None
+                bias_grad = all_reduce(all_reduce(ops.colsum(g2, out_dtype=sum_dtype), in_mode), w_mode).to(bias_dtype)
             input_grad = ops.gemm_ksteps("NN", [g2], [w]).reshape(input_.shape)
         return input_grad, weight_grad, bias_grad, None, None, None
 
@@ -159,7 +162,8 @@ class _VocabParallelClassifier3D(torch.autograd.Function):
                 weight_grad = ops.gemm_ksteps("TN", [_flat(x)], [g2])             # [in, classes]
                 weight_grad = reduce_scatter(weight_grad.transpose(0, 1), 0, w_mode)
                 input_grad = ops.gemm_ksteps("NT", [g2], [w]).reshape(x.shape)
-            bias_grad = all_reduce(ops.colsum(g2), w_mode).to(bias_dtype) if use_bias else None
+            sum_dtype = bias_dtype if use_bias and w_mode.world_size == 1 else None
+            bias_grad = all_reduce(ops.colsum(g2, out_dtype=sum_dtype), w_mode).to(bias_dtype) if use_bias else None
             input_grad = reduce_scatter(input_grad, 0, in_mode)
         return input_grad, weight_grad, bias_grad, None, None, None
 
@@ -197,14 +201,16 @@ class _Layernorm3D(torch.autograd.Function):
     def backward(ctx, output_grad):
         x, weight, mean_rstd = ctx.saved_tensors
         hidden, out_mode, ixw_mode, w_dtype, b_dtype = ctx.meta
+        pd = w_dtype if ixw_mode.world_size == 1 and w_dtype == b_dtype else None
         with torch.no_grad():
             if out_mode.world_size == 1:
-                input_grad, dgamma, dbeta = ops.ln_backward_fused(output_grad, x, mean_rstd, weight)
+                input_grad, dgamma, dbeta = ops.ln_backward_fused(output_grad, x, mean_rstd, weight, param_dtype=pd)
             else:
                 # the dx launch also finishes the column sums that the first launch leaves as partial rows
                 row_sums, pending = ops.ln_bwd_partials_open(output_grad, x, mean_rstd, weight)
                 row_sums = all_reduce(row_sums, out_mode)
-                input_grad, dgamma, dbeta = ops.ln_bwd_dx_close(output_grad, x, mean_rstd, row_sums, hidden, pending, weight)
+                input_grad, dgamma, dbeta = ops.ln_bwd_dx_close(output_grad, x, mean_rstd, row_sums, hidden, pending, weight,
+                                                                param_dtype=pd)
             weight_grad = all_reduce(dgamma, ixw_mode).to(w_dtype)
             bias_grad = all_reduce(dbeta, ixw_mode).to(b_dtype)
         return input_grad, weight_grad, bias_grad, None, None, None, None, None, None

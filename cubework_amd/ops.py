@@ -172,22 +172,36 @@ def _workspace(M: int, N: int, device) -> torch.Tensor:
     return torch.empty(max(nbytes, 16), dtype=torch.uint8, device=device)
 
 
-def colsum(dy: torch.Tensor) -> torch.Tensor:
-    """fp32 column sums of a [M,N] tensor (bias gradient)."""
+def _out_dtype(out_dtype: Optional[torch.dtype]) -> torch.dtype:
+    """dtype of column-sum results: fp32 unless the caller names the parameter's dtype (the sums are always
+    accumulated in fp32 and rounded once on the way out)."""
+    out_dtype = out_dtype or torch.float32
+    if out_dtype not in (torch.float32, torch.bfloat16, torch.float16):
+        raise TypeError("column sums are stored as float32, bfloat16 or float16, not %s" % out_dtype)
+    return out_dtype
+
+
+_TORCH_CODE = {torch.float32: CW_F32, torch.bfloat16: CW_BF16, torch.float16: CW_F16}
+
+
+def colsum(dy: torch.Tensor, out_dtype: Optional[torch.dtype] = None) -> torch.Tensor:
+    """Column sums of a [M,N] tensor (bias gradient): fp32 sums, stored as out_dtype (default float32)."""
     lib = _lib.load()
     dy = _rows(dy)
     _require_device(dy)
     M, N = dy.shape
-    out = torch.empty(N, dtype=torch.float32, device=dy.device)
+    out_dtype = _out_dtype(out_dtype)
+    out = torch.empty(N, dtype=out_dtype, device=dy.device)
     ws = _workspace(M, N, dy.device)
-    rc = lib.cw_colsum(M, N, _p(dy), _ld(dy), _p(out), _p(ws), ws.numel(), _dtype_code(dy), _stream())
+    rc = lib.cw_colsum(M, N, _p(dy), _ld(dy), _p(out), _TORCH_CODE[out_dtype], _p(ws), ws.numel(), _dtype_code(dy),
+                       _stream())
     _lib.check(rc, "cw_colsum")
     return out
 
 
-def act_bwd_colsum(activation: Optional[str], dy: torch.Tensor, preact: torch.Tensor,
-                   want_dbias: bool = True) -> Tuple[torch.Tensor, Optional[torch.Tensor]]:
-    """dPre = dy * act'(preact) and (optionally) its fp32 column sums."""
+def act_bwd_colsum(activation: Optional[str], dy: torch.Tensor, preact: torch.Tensor, want_dbias: bool = True,
+                   out_dtype: Optional[torch.dtype] = None) -> Tuple[torch.Tensor, Optional[torch.Tensor]]:
+    """dPre = dy * act'(preact) and (optionally) its column sums (fp32 sums stored as out_dtype, default float32)."""
     lib = _lib.load()
     dy, preact = _rows(dy), _rows(preact)
     _require_device(dy, preact)
@@ -195,10 +209,11 @@ def act_bwd_colsum(activation: Optional[str], dy: torch.Tensor, preact: torch.Te
         raise ValueError("dy and preact must agree in shape and dtype")
     M, N = dy.shape
     dpre = torch.empty((M, N), dtype=dy.dtype, device=dy.device)
-    dbias = torch.empty(N, dtype=torch.float32, device=dy.device) if want_dbias else None
+    out_dtype = _out_dtype(out_dtype)
+    dbias = torch.empty(N, dtype=out_dtype, device=dy.device) if want_dbias else None
     ws = _workspace(M, N, dy.device) if want_dbias else None
     rc = lib.cw_act_bwd_colsum(ACTIVATIONS[activation], M, N, _p(dy), _ld(dy), _p(preact), _ld(preact), _p(dpre),
-                               _ld(dpre), _p(dbias), _p(ws), ws.numel() if ws is not None else 0,
+                               _ld(dpre), _p(dbias), _TORCH_CODE[out_dtype], _p(ws), ws.numel() if ws is not None else 0,
                                _dtype_code(dy), _stream())
     _lib.check(rc, "cw_act_bwd_colsum")
     return dpre, dbias
@@ -265,8 +280,10 @@ def ln_forward_fused(x: torch.Tensor, eps: float, gamma: Optional[torch.Tensor] 
 
 
 def ln_bwd_partials(dy: torch.Tensor, x: torch.Tensor, mean_rstd: torch.Tensor,
-                    gamma: Optional[torch.Tensor] = None, want_param_grads: bool = True):
-    """Returns (row_sums [R,2] fp32, dgamma [C] fp32 or None, dbeta [C] fp32 or None)."""
+                    gamma: Optional[torch.Tensor] = None, want_param_grads: bool = True,
+                    param_dtype: Optional[torch.dtype] = None):
+    """Returns (row_sums [R,2] fp32, dgamma [C] or None, dbeta [C] or None); the parameter gradients are fp32
+    sums stored as param_dtype (default float32)."""
     lib = _lib.load()
     dy, x = _rows(dy), _rows(x)
     _require_device(dy, x, mean_rstd, gamma)
@@ -276,13 +293,14 @@ def ln_bwd_partials(dy: torch.Tensor, x: torch.Tensor, mean_rstd: torch.Tensor,
     gamma = None if gamma is None else gamma.to(x.dtype).contiguous()
     row_sums = torch.empty((R, 2), dtype=torch.float32, device=x.device)
     dgamma = dbeta = ws = None
+    param_dtype = _out_dtype(param_dtype)
     if want_param_grads:
-        dgamma = torch.empty(C, dtype=torch.float32, device=x.device)
-        dbeta = torch.empty(C, dtype=torch.float32, device=x.device)
+        dgamma = torch.empty(C, dtype=param_dtype, device=x.device)
+        dbeta = torch.empty(C, dtype=param_dtype, device=x.device)
         ws = _workspace(R, C, x.device)
     rc = lib.cw_ln_bwd_partials(R, C, _p(dy), _ld(dy), _p(x), _ld(x), _p(mean_rstd), _p(gamma), _p(row_sums),
-                                _p(dgamma), _p(dbeta), _p(ws), ws.numel() if ws is not None else 0, _dtype_code(x),
-                                _stream())
+                                _p(dgamma), _p(dbeta), _TORCH_CODE[param_dtype], _p(ws),
+                                ws.numel() if ws is not None else 0, _dtype_code(x), _stream())
     _lib.check(rc, "cw_ln_bwd_partials")
     return row_sums, dgamma, dbeta
 
@@ -325,9 +343,9 @@ def ln_bwd_partials_open(dy: torch.Tensor, x: torch.Tensor, mean_rstd: torch.Ten
 
 
 def ln_bwd_dx_close(dy: torch.Tensor, x: torch.Tensor, mean_rstd: torch.Tensor, row_sums: torch.Tensor, hidden: int,
-                    pending, gamma: Optional[torch.Tensor] = None):
-    """(dx, dgamma [C] fp32, dbeta [C] fp32): ln_bwd_dx whose launch also finishes the column sums that
-    ln_bwd_partials_open left pending. See cw_ln_bwd_dx_close."""
+                    pending, gamma: Optional[torch.Tensor] = None, param_dtype: Optional[torch.dtype] = None):
+    """(dx, dgamma [C], dbeta [C]): ln_bwd_dx whose launch also finishes the column sums that
+    ln_bwd_partials_open left pending (stored as param_dtype, default float32). See cw_ln_bwd_dx_close."""
     lib = _lib.load()
     shape = x.shape
     dy, x = _rows(dy), _rows(x)
@@ -337,18 +355,22 @@ def ln_bwd_dx_close(dy: torch.Tensor, x: torch.Tensor, mean_rstd: torch.Tensor, 
     gamma = None if gamma is None else gamma.to(x.dtype).contiguous()
     row_sums = row_sums.reshape(R, 2).to(torch.float32).contiguous()
     dx = torch.empty((R, C), dtype=x.dtype, device=x.device)
-    dgamma = torch.empty(C, dtype=torch.float32, device=x.device)
-    dbeta = torch.empty(C, dtype=torch.float32, device=x.device)
+    param_dtype = _out_dtype(param_dtype)
+    dgamma = torch.empty(C, dtype=param_dtype, device=x.device)
+    dbeta = torch.empty(C, dtype=param_dtype, device=x.device)
     rc = lib.cw_ln_bwd_dx_close(R, C, _p(dy), _ld(dy), _p(x), _ld(x), _p(mean_rstd), _p(gamma), _p(row_sums), hidden,
-                                _p(dx), _ld(dx), _p(ws), n_parts, _p(dgamma), _p(dbeta), _dtype_code(x), _stream())
+                                _p(dx), _ld(dx), _p(ws), n_parts, _p(dgamma), _p(dbeta), _TORCH_CODE[param_dtype],
+                                _dtype_code(x), _stream())
     _lib.check(rc, "cw_ln_bwd_dx_close")
     return dx.reshape(shape), dgamma, dbeta
 
 
 def ln_backward_fused(dy: torch.Tensor, x: torch.Tensor, mean_rstd: torch.Tensor,
-                      gamma: Optional[torch.Tensor] = None, want_param_grads: bool = True):
-    """Backward of LayerNorm over rows this rank holds whole: (dx, dgamma [C] fp32 or None, dbeta [C] fp32
-    or None) in one pass over dy and x. See cw_ln_backward_fused."""
+                      gamma: Optional[torch.Tensor] = None, want_param_grads: bool = True,
+                      param_dtype: Optional[torch.dtype] = None):
+    """Backward of LayerNorm over rows this rank holds whole: (dx, dgamma [C] or None, dbeta [C] or None) in
+    one pass over dy and x; the parameter gradients are fp32 sums stored as param_dtype (default float32).
+    See cw_ln_backward_fused."""
     lib = _lib.load()
     shape = x.shape
     dy, x = _rows(dy), _rows(x)
@@ -360,13 +382,14 @@ def ln_backward_fused(dy: torch.Tensor, x: torch.Tensor, mean_rstd: torch.Tensor
     row_sums = torch.empty((R, 2), dtype=torch.float32, device=x.device)
     dx = torch.empty((R, C), dtype=x.dtype, device=x.device)
     dgamma = dbeta = ws = None
+    param_dtype = _out_dtype(param_dtype)
     if want_param_grads:
-        dgamma = torch.empty(C, dtype=torch.float32, device=x.device)
-        dbeta = torch.empty(C, dtype=torch.float32, device=x.device)
+        dgamma = torch.empty(C, dtype=param_dtype, device=x.device)
+        dbeta = torch.empty(C, dtype=param_dtype, device=x.device)
         ws = _workspace(R, C, x.device)
     rc = lib.cw_ln_backward_fused(R, C, _p(dy), _ld(dy), _p(x), _ld(x), _p(mean_rstd), _p(gamma), _p(row_sums), _p(dx),
-                                  _ld(dx), _p(dgamma), _p(dbeta), _p(ws), ws.numel() if ws is not None else 0,
-                                  _dtype_code(x), _stream())
+                                  _ld(dx), _p(dgamma), _p(dbeta), _TORCH_CODE[param_dtype], _p(ws),
+                                  ws.numel() if ws is not None else 0, _dtype_code(x), _stream())
     _lib.check(rc, "cw_ln_backward_fused")
     return dx.reshape(shape), dgamma, dbeta
 
@@ -529,10 +552,10 @@ def embedding_fwd(ids: torch.Tensor, weight: torch.Tensor, vocab_start: int = 0)
     others; ids of any shape, result ids.shape + (E,). See cw_embed_fwd."""
     lib = _lib.load()
     _require_device(ids, weight)
-    if ids.dtype != torch.int64:
-        raise TypeError("ids must be int64")
+    if ids.dtype not in (torch.int64, torch.int32):
+        raise TypeError("ids must be int64 or int32 (what F.embedding takes), got %s" % ids.dtype)
     w = _rows(weight)
-    flat = ids.reshape(-1).contiguous()
+    flat = ids.reshape(-1).to(torch.int64).contiguous()   # a no-op for int64 ids
     T, (V_loc, E) = flat.numel(), w.shape
     out = torch.empty((T, E), dtype=w.dtype, device=w.device)
     rc = lib.cw_embed_fwd(T, E, _p(flat), int(vocab_start), V_loc, _p(w), _ld(w), _p(out), _ld(out), _dtype_code(w),
@@ -568,10 +591,10 @@ def embedding_bwd(ids: torch.Tensor, d_out: torch.Tensor, num_rows: int, vocab_s
     False asks for one path (False: the one launch wherever it is possible at all)."""
     lib = _lib.load()
     _require_device(ids, d_out)
-    if ids.dtype != torch.int64:
-        raise TypeError("ids must be int64, got %s" % ids.dtype)
+    if ids.dtype not in (torch.int64, torch.int32):
+        raise TypeError("ids must be int64 or int32 (what F.embedding takes), got %s" % ids.dtype)
     g = _rows(d_out.reshape(-1, d_out.shape[-1]))
-    flat = ids.reshape(-1).contiguous()
+    flat = ids.reshape(-1).to(torch.int64).contiguous()   # a no-op for int64 ids
     T, E = g.shape
     if flat.numel() != T:
         raise ValueError("ids select %d rows, d_out has %d" % (flat.numel(), T))

@@ -19,6 +19,7 @@ import torch.nn.functional as F
 
 from . import module as cube_nn
 from . import ops
+from .module.parallel_2d import Linear2D
 
 
 class OPTBlock(nn.Module):
@@ -46,17 +47,24 @@ class OPTBlock(nn.Module):
         o = F.scaled_dot_product_attention(q, k, v, is_causal=True)
         return o.transpose(1, 2).reshape(b, s, self.heads * self.head_dim)
 
+    @staticmethod
+    def _linear_plus(layer, inp: torch.Tensor, residual: torch.Tensor) -> torch.Tensor:
+        """residual + layer(inp) (benchmark/opt/opt.py:184,206): in the GEMM's epilogue where the layer offers it
+        (Linear2D's `residual` option), as a separate addition elsewhere."""
+        inner = getattr(layer, "linear", layer)
+        if isinstance(inner, Linear2D) and inner.activation is None and not inner.skip_bias_add:
+            return layer(inp, residual=residual)
+        return residual + layer(inp)
+
     def forward(self, x: torch.Tensor) -> torch.Tensor:
         h = self.self_attn_layer_norm(x)
-        h = self.out_proj(self._attention_core(self.qkv_proj(h)))
-        x = x + h
+        x = self._linear_plus(self.out_proj, self._attention_core(self.qkv_proj(h)), x)
         shape = x.shape
         r = x.reshape(-1, shape[-1])
         h = self.fc1(self.final_layer_norm(r))
         if not self.fuse_activation:
             h = _ACT[self.activation](h)
-        h = self.fc2(h)
-        return (r + h).view(shape)
+        return self._linear_plus(self.fc2, h, r).view(shape)
 
 
 _ACT = {"relu": F.relu, "gelu": F.gelu, "gelu_erf": F.gelu, "gelu_tanh": lambda t: F.gelu(t, approximate="tanh")}

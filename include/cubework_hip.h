@@ -153,13 +153,16 @@ int cw_gemm_ksteps_ws(int layout, int64_t M, int64_t N, int64_t K, int n_steps,
 int64_t cw_colsum_workspace_bytes(int64_t M, int64_t N);
 
 /*
- * out[N] (fp32) = sum over rows of dY[M,N].
+ * out[N] = sum over rows of dY[M,N], accumulated in fp32 and stored as out_dtype
+ * (CW_F32, or CW_BF16 / CW_F16 rounded once to nearest even: the parameter's own
+ * type, so that no cast launch follows, as the reference's sum in the tensors'
+ * dtype leaves none).
  * Replaces torch.sum(output_grad, dim=reduce_dim) in _SUMMAbias.backward
  * (parallel_2d/_operation.py:285-286), _Classifier2D.backward (:414),
  * _Linear3D.backward (parallel_3d/_operation.py:59). Two deterministic stages
  * through `workspace` (no atomics).
  */
-int cw_colsum(int64_t M, int64_t N, const void* dY, int64_t ld, float* out,
+int cw_colsum(int64_t M, int64_t N, const void* dY, int64_t ld, void* out, int out_dtype,
               void* workspace, int64_t workspace_bytes, int io_dtype, void* stream);
 
 /*
@@ -171,22 +174,25 @@ int cw_colsum(int64_t M, int64_t N, const void* dY, int64_t ld, float* out,
  * not fit are refused with CW_ERR_UNSUPPORTED: with 16-byte aligned dY and ld, N % (16 / element size)
  * == 0 the limit is N <= 1048576, otherwise ceil(M / 64) * N <= 1048576. Calls on one GPU share the array:
  * calls that may overlap on the device (two streams, two threads) race; calls on one stream do not. The
- * first call on a device looks the array's address up (hipGetSymbolAddress): make it outside a capture.
+ * first call on a device looks the array's address up (hipGetSymbolAddress): make it outside a capture (a first
+ * call on a capturing stream is refused with CW_ERR_UNSUPPORTED and records nothing).
  * No hipMalloc / hipFree / allocating library routine on any call.
  */
 int64_t cw_colsum_static_max_bytes(void);
-int cw_colsum_static(int64_t M, int64_t N, const void* dY, int64_t ld, float* out, int io_dtype, void* stream);
+int cw_colsum_static(int64_t M, int64_t N, const void* dY, int64_t ld, void* out, int out_dtype, int io_dtype,
+                     void* stream);
 
 /*
- * dPre[M,N] = dY * act'(preact); optionally dbias[N] (fp32) = column sums of
- * dPre (dbias may be NULL, then workspace may be NULL). Backward of the fused
+ * dPre[M,N] = dY * act'(preact); optionally dbias[N] = column sums of dPre, fp32
+ * sums stored as dbias_dtype like cw_colsum's (dbias may be NULL, then workspace
+ * may be NULL and dbias_dtype is ignored). Backward of the fused
  * activation epilogue of cw_gemm_ksteps; the reference runs it as autograd of
  * nn.functional.gelu / nn.ReLU (benchmark/gpt2/gpt2.py:117, benchmark/opt/opt.py:200)
  * followed by _SUMMAbias.backward.
  */
 int cw_act_bwd_colsum(int activation, int64_t M, int64_t N,
                       const void* dY, int64_t ld_dy, const void* preact, int64_t ld_pre,
-                      void* dPre, int64_t ld_dpre, float* dbias,
+                      void* dPre, int64_t ld_dpre, void* dbias, int dbias_dtype,
                       void* workspace, int64_t workspace_bytes, int io_dtype, void* stream);
 
 /* ---- LayerNorm ---------------------------------------------------------- */
@@ -227,7 +233,8 @@ int cw_ln_forward_fused(int64_t R, int64_t C, const void* x, int64_t ld, int mod
 /*
  * Backward partials. With g = dY * gamma and xhat = (x - mean) * rstd:
  *   row_sums[r] = (sum_c g, sum_c g*xhat)                 (fp32 [R,2])
- *   dgamma[c]   = sum_r dY*xhat, dbeta[c] = sum_r dY      (fp32 [C] each, optional)
+ *   dgamma[c]   = sum_r dY*xhat, dbeta[c] = sum_r dY      ([C] each, optional; fp32 sums stored as
+ *                                                          param_dtype: CW_F32, CW_BF16 or CW_F16)
  * Replaces _Layernorm_2D.backward sums (parallel_2d/_operation.py:334,338), the
  * autograd of torch.addcmul (parallel_2d/module.py:170) and the bias_grad /
  * weight_grad sums of _Layernorm3D.backward (parallel_3d/_operation.py:294-301).
@@ -235,7 +242,7 @@ int cw_ln_forward_fused(int64_t R, int64_t C, const void* x, int64_t ld, int mod
  */
 int cw_ln_bwd_partials(int64_t R, int64_t C, const void* dY, int64_t ld_dy,
                        const void* x, int64_t ld_x, const float* mean_rstd, const void* gamma,
-                       float* row_sums, float* dgamma, float* dbeta,
+                       float* row_sums, void* dgamma, void* dbeta, int param_dtype,
                        void* workspace, int64_t workspace_bytes, int io_dtype, void* stream);
 
 /*
@@ -253,7 +260,7 @@ int cw_ln_bwd_dx(int64_t R, int64_t C, const void* dY, int64_t ld_dy,
  * and leaves *n_parts unfinished column partial rows in `workspace` (sized by cw_ln_bwd_workspace_bytes; *n_parts
  * is a host value, set before the call returns); the caller all-reduces row_sums as before
  * (parallel_2d/_operation.py:335,339) and cw_ln_bwd_dx_close writes dx and, from its leading workgroups, dgamma and
- * dbeta (fp32 [C]) out of those rows, which must still be in `workspace`. Same arithmetic as the pair above; the
+ * dbeta ([C], stored as param_dtype) out of those rows, which must still be in `workspace`. Same arithmetic as the pair above; the
  * column sums are added in a fixed order (bit-reproducible) that differs from cw_ln_bwd_partials' in the last bits.
  */
 int cw_ln_bwd_partials_open(int64_t R, int64_t C, const void* dY, int64_t ld_dy, const void* x, int64_t ld_x,
@@ -261,8 +268,8 @@ int cw_ln_bwd_partials_open(int64_t R, int64_t C, const void* dY, int64_t ld_dy,
                             int64_t workspace_bytes, int64_t* n_parts, int io_dtype, void* stream);
 int cw_ln_bwd_dx_close(int64_t R, int64_t C, const void* dY, int64_t ld_dy, const void* x, int64_t ld_x,
                        const float* mean_rstd, const void* gamma, const float* row_sums, int64_t H, void* dx,
-                       int64_t ld_dx, const void* workspace, int64_t n_parts, float* dgamma, float* dbeta,
-                       int io_dtype, void* stream);
+                       int64_t ld_dx, const void* workspace, int64_t n_parts, void* dgamma, void* dbeta,
+                       int param_dtype, int io_dtype, void* stream);
 
 /*
  * cw_ln_bwd_partials + cw_ln_bwd_dx with H = C in one pass over dY and x, for rows that are complete on
@@ -273,7 +280,7 @@ int cw_ln_bwd_dx_close(int64_t R, int64_t C, const void* dY, int64_t ld_dy, cons
  */
 int cw_ln_backward_fused(int64_t R, int64_t C, const void* dY, int64_t ld_dy,
                          const void* x, int64_t ld_x, const float* mean_rstd, const void* gamma,
-                         float* row_sums, void* dx, int64_t ld_dx, float* dgamma, float* dbeta,
+                         float* row_sums, void* dx, int64_t ld_dx, void* dgamma, void* dbeta, int param_dtype,
                          void* workspace, int64_t workspace_bytes, int io_dtype, void* stream);
 
 /* ---- vocab-parallel cross-entropy -------------------------------------- */
@@ -363,9 +370,14 @@ int cw_embed_sort_ids(int64_t T, const int64_t* ids, int64_t vocab_start, int64_
  * that sums the others (every row of d_weight is written exactly once). Replaces the whole backward of
  * the F.embedding call (parallel_1d/module.py:452, parallel_2d/module.py:353, parallel_3d/module.py:466)
  * for a batch of up to 16384 tokens whose rows are 16-byte aligned (E a multiple of the 16-byte vector).
- * A row's tokens are added in ascending token position, as after a stable sort; a row that more than 16
- * tokens select is summed over 8 contiguous ranges of token positions whose partial sums are added in
- * order. No atomics on global memory: bit-reproducible. A row that n tokens select is summed by one
+ * A row's tokens are added in an order that the ids and the shape alone fix (the same bits on every call):
+ * the row's token positions are walked in blocks of 32, round by round the lowest remaining token of every
+ * block, blocks ascending (a workgroup's first row per wavefront takes its lowest token ahead of the walk).
+ * That is ascending token position (the order of cw_embed_sort_ids + cw_embed_bwd, hence the same bits) when
+ * no two of the row's tokens share a block of 32 positions, and another fixed order, equal up to fp32
+ * reassociation, when some do. A row that more than 8 tokens select is summed over 8 contiguous ranges of
+ * token positions (the same walk inside each) whose partial sums are added in order. No atomics on global
+ * memory: bit-reproducible. A row that n tokens select is summed by one
  * workgroup at about 70 ns per token, so a batch dominated by one id is better served by the token order,
  * which shares a long run among several workgroups. Every workgroup scans all T ids for its 32 rows, so the
  * launch pays while a row is not much smaller than T / 4 bytes: cw_embed_bwd_ids_supported returns 1 when the
@@ -469,20 +481,6 @@ int cw_attn_bwd(int64_t B, int64_t H, int64_t S, int64_t D,
                 void* dq, void* dk, void* dv,
                 int64_t grad_stride_b, int64_t grad_stride_s, int64_t grad_stride_h,
                 void* workspace, int64_t workspace_bytes, int io_dtype, void* stream);
-
-/* ---- measurement aid ------------------------------------------------------- */
-/*
- * The block GEMM's matrix instruction (v_mfma_f32_32x32x16_bf16, 16 accumulator tiles per wavefront, one
- * wavefront per SIMD on every compute unit) issued back to back from registers for `iters` trips: no memory
- * traffic, no LDS, no barriers. mode 0: operand fragments are seeded random bf16 values with the workload's
- * magnitudes; mode 1: all zero; mode 2: the random fragments of every trip are read from LDS (8 KB per wavefront
- * and 16 MFMAs, the fragment traffic of the ring kernel's k loop; still no global loads). No counterpart in the
- * reference; bench.py times it to report what the board's power management leaves of the data-sheet MFMA rate,
- * with and without the LDS reads, next to the GEMM kernel's own rate.
- * cw_diag_mfma_rate_flop(iters) is the FLOP count of one call. sink: NULL or 65536 floats.
- */
-int64_t cw_diag_mfma_rate_flop(int iters);
-int cw_diag_mfma_rate(int iters, int mode, float* sink, void* stream);
 
 #ifdef __cplusplus
 }

@@ -89,11 +89,6 @@ def test_scratch_sizes_and_refusals_of_the_later_entry_points():
     assert lib.cw_clip_coef(1, None, 1.0, 2.0, 1.0, None, None) == -1
     assert lib.cw_multi_norm_partial_count(3, C.cast(numels, C.c_void_p)) == 1 + 1 + 2
     assert lib.cw_multi_norm_partial_count(0, None) == 0
-    # measurement aid: modes 0 (random operands), 1 (zeros), 2 (random operands read from LDS)
-    assert lib.cw_diag_mfma_rate(0, 0, None, None) == -1
-    assert lib.cw_diag_mfma_rate(10, 3, None, None) == -1
-    assert b"mode" in lib.cw_last_error()
-    assert lib.cw_diag_mfma_rate_flop(2) == 2 * 1024 * 16 * 32768
     assert lib.cw_clip_scale(0, None, None, BF16, 1, None, 0, None, 1.0, 2.0, 1.0, None, None) == -1
     # attention: head sizes other than 64 / 128 and fp32 are refused before any launch
     assert lib.cw_attn_bwd_workspace_bytes(4, 32, 2048) == 4 * 32 * 2048 * 4
@@ -103,7 +98,7 @@ def test_scratch_sizes_and_refusals_of_the_later_entry_points():
     args[3], args[17] = 64, F32
     assert lib.cw_attn_fwd(*args) == -3
     # fused LayerNorm backward: the two column outputs come together
-    assert lib.cw_ln_backward_fused(4, 8, None, 8, None, 8, None, None, None, None, 8, None, C.c_void_p(16), None, 0, BF16, None) == -1
+    assert lib.cw_ln_backward_fused(4, 8, None, 8, None, 8, None, None, None, None, 8, None, C.c_void_p(16), F32, None, 0, BF16, None) == -1
     assert b"both" in lib.cw_last_error()
 
 
@@ -119,11 +114,33 @@ def test_no_usable_device_is_reported_as_such():
         pytest.skip("a GPU is visible: the refusal path needs a machine without one")
     lib = _lib.load()
     p = C.c_void_p(256)
-    assert lib.cw_colsum(8, 8, p, 8, p, p, 1 << 20, _lib.CW_F32, None) == -5
+    assert lib.cw_colsum(8, 8, p, 8, p, _lib.CW_F32, p, 1 << 20, _lib.CW_F32, None) == -5
     assert b"device" in lib.cw_last_error().lower()
-    assert lib.cw_colsum_static(8, 8, p, 8, p, _lib.CW_F32, None) == -5
+    assert lib.cw_colsum_static(8, 8, p, 8, p, _lib.CW_F32, _lib.CW_F32, None) == -5
     assert lib.cw_ln_partial_stats(4, 8, p, 8, _lib.CW_LN_ONE_PASS, None, p, _lib.CW_BF16, None) == -5
     tab = (C.c_void_p * 1)(256)
     assert lib.cw_gemm_ksteps(_lib.CW_NN, 8, 8, 8, 1, tab, 8, tab, 8, None, 0, p, 8, None, 0, None, 0, 0, _lib.CW_BF16, None) == -5
     assert lib.cw_vpce_finalize(4, 1, p, p, p, p, p, p, p, None) == -5
     assert lib.cw_device_arch() == b""
+
+
+def test_measurement_library_is_separate_from_the_boundary():
+    """The measurement aids bench.py uses (MFMA rate loop, the ring kernel with one part taken out) live in a
+    library of their own: the product library exports none of them, and their host-side checks work without a
+    device."""
+    from cubework_amd import _diag, _lib
+    if not os.path.exists(_lib.LIB_PATH) or not os.path.exists(_diag.LIB_PATH):
+        pytest.skip("libraries not built yet")
+    product = ctypes.CDLL(_lib.LIB_PATH)
+    for name in _diag.SIGNATURES:
+        if name.startswith("cw_diag"):
+            assert not hasattr(product, name), name
+    diag = _diag.load()
+    assert diag.cw_diag_mfma_rate(0, 0, None, None) == -1
+    assert diag.cw_diag_mfma_rate(10, 3, None, None) == -1
+    assert b"mode" in diag.cw_last_error()
+    assert diag.cw_diag_mfma_rate_flop(2) == 2 * 1024 * 16 * 32768
+    assert diag.cw_diag_gemm_part(7, 8192, 2048, 2048, 2, None, 2048, None, 2048, None, None, 2048, None) == -1
+    tab = (ctypes.c_void_p * 2)(256, 256)
+    p = ctypes.c_void_p(256)
+    assert diag.cw_diag_gemm_part(1, 8192, 2000, 2048, 2, tab, 2048, tab, 2048, p, p, 2048, None) == -3

@@ -191,8 +191,8 @@ def test_token_order_repeated_id():
 def test_embedding_backward_from_ids_edges(T):
     """The one-launch backward on ids below, at and above the slice's edges, negative ids and the extremes
     of int64 (none of which may select a row), on an empty batch (all zeros) and on the longest batch it
-    takes; the result equals the token-order path's bit for bit where no row has more than 16 tokens, and
-    float64 sums within the bar everywhere."""
+    takes; float64 sums within the bar everywhere (bit equality with the token-order path is the subject of
+    test_embedding_backward_from_ids_order_of_addition)."""
     from cubework_amd import ops
 
     start, rows, e = 1000, 777, 264
@@ -212,6 +212,45 @@ def test_embedding_backward_from_ids_edges(T):
     if T <= 1:
         via = ops.embedding_bwd(ids.to(DEV), d_out.to(DEV), rows, start, 5, via_token_order=True)
         assert torch.equal(got, via)
+
+
+def test_embedding_backward_from_ids_order_of_addition():
+    """The one-launch backward walks a row's token positions in blocks of 32, round by round the lowest remaining
+    token of every block. Rows whose tokens (2 to 8 of them) all sit in different blocks are therefore added in
+    ascending token position and equal the token-order path bit for bit; a row with two tokens in one block and
+    later ones ({0, 1, 40}, {64, 70, 75, 130, 131}) may be added in another fixed order: the same bits on every
+    call, equal to the token-order path only up to fp32 reassociation - bit equality with it is waived there,
+    by design."""
+    from cubework_amd import ops
+
+    rows, e, T = 64, 264, 512
+    d_out = randn((T, e), torch.float32, 21)
+    # (a) tokens of each row in distinct 32-blocks: row r gets tokens r%32 + 32*k for k < 2 + r % 7
+    ids = torch.full((T,), rows + 5, dtype=torch.int64)   # outside the slice
+    for r in range(20):
+        for k in range(2 + r % 7):
+            ids[(r % 32) + 32 * k + (0 if r < 32 else 1)] = r
+    a = ops.embedding_bwd(ids.to(DEV), d_out.to(DEV), rows, 0, -1, via_token_order=False)
+    b = ops.embedding_bwd(ids.to(DEV), d_out.to(DEV), rows, 0, -1, via_token_order=True)
+    assert torch.equal(a, b)
+    # (b) {0, 1, 40} and friends: two tokens in one block plus later ones
+    ids = torch.full((T,), rows + 5, dtype=torch.int64)
+    ids[[0, 1, 40]] = 3
+    ids[[64, 70, 75, 130, 131]] = 9
+    a1 = ops.embedding_bwd(ids.to(DEV), d_out.to(DEV), rows, 0, -1, via_token_order=False)
+    a2 = ops.embedding_bwd(ids.to(DEV), d_out.to(DEV), rows, 0, -1, via_token_order=False)
+    b = ops.embedding_bwd(ids.to(DEV), d_out.to(DEV), rows, 0, -1, via_token_order=True)
+    assert torch.equal(a1, a2)                                            # a fixed order
+    untouched = torch.ones(rows, dtype=torch.bool)
+    untouched[[3, 9]] = False
+    assert torch.equal(a1[untouched], b[untouched])                       # every other row: the same bits
+    assert_parity(a1, b, torch.float32, "one launch against the token order, tokens sharing a block")
+    want = torch.zeros((rows, e), dtype=torch.float64).index_add_(0, ids[ids < rows], d_out.double()[ids < rows])
+    assert_parity(a1, want, torch.float32, "embedding d_weight from ids, tokens sharing a block")
+    # int32 ids, which F.embedding also takes, give the same result
+    assert torch.equal(ops.embedding_bwd(ids.int().to(DEV), d_out.to(DEV), rows, 0, -1, via_token_order=False), a1)
+    w = randn((rows, e), torch.float32, 22).to(DEV)
+    assert torch.equal(ops.embedding_fwd(ids.int().to(DEV), w, 0), ops.embedding_fwd(ids.to(DEV), w, 0))
 
 
 def test_embedding_backward_from_ids_refuses_what_it_cannot_take():

@@ -59,11 +59,12 @@ def test_colsum_padded_rows():
 
 
 def test_mfma_rate_diagnostic_runs_in_every_mode():
-    """cw_diag_mfma_rate (the measurement aid behind bench.py's MFMA ceilings): zero operands leave zero sums;
-    random operands, from registers or read from LDS, leave finite non-zero ones, the same on every call."""
-    from cubework_amd import _lib
+    """cw_diag_mfma_rate (the measurement aid behind bench.py's MFMA ceilings, in the measurement library): zero
+    operands leave zero sums; random operands, from registers or read from LDS, leave finite non-zero ones, the
+    same on every call."""
+    from cubework_amd import _diag
 
-    lib = _lib.load()
+    lib = _diag.load()
     sink = torch.full((65536,), float("nan"), dtype=torch.float32, device=DEV)
     assert lib.cw_diag_mfma_rate(3, 1, sink.data_ptr(), None) == 0
     torch.cuda.synchronize()
@@ -77,3 +78,27 @@ def test_mfma_rate_diagnostic_runs_in_every_mode():
             runs.append(sink.clone())
         assert torch.isfinite(runs[0]).all() and (runs[0] != 0).any()
         assert torch.equal(runs[0], runs[1])
+
+
+def test_gemm_part_diagnostic_whole_kernel_matches_the_library():
+    """cw_diag_gemm_part with part 0 is the library's ring kernel for the benchmark's shape: bit-equal to
+    cw_gemm_ksteps; parts 1 to 3 (no operand loads / no epilogue / no LDS reads in the k loop) run and return."""
+    import ctypes
+    from cubework_amd import _diag, ops
+
+    lib = _diag.load()
+    M, N, K = 8192, 2048, 512   # 256 tiles: the shape class the library gives to this kernel
+    A = [randn((M, K), torch.bfloat16, 40 + i).to(DEV) for i in range(2)]
+    B = [randn((K, N), torch.bfloat16, 50 + i, 0.05).to(DEV) for i in range(2)]
+    bias = randn((N,), torch.bfloat16, 60, 0.1).to(DEV)
+    want = ops.gemm_ksteps("NN", A, B, bias, "gelu_tanh")
+    ta = (ctypes.c_void_p * 2)(*[t.data_ptr() for t in A])
+    tb = (ctypes.c_void_p * 2)(*[t.data_ptr() for t in B])
+    out = torch.empty_like(want)
+    stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+    assert lib.cw_diag_gemm_part(0, M, N, K, 2, ta, K, tb, N, bias.data_ptr(), out.data_ptr(), N, stream) == 0
+    torch.cuda.synchronize()
+    assert torch.equal(out, want)
+    for part in (1, 2, 3):
+        assert lib.cw_diag_gemm_part(part, M, N, K, 2, ta, K, tb, N, bias.data_ptr(), out.data_ptr(), N, stream) == 0
+    torch.cuda.synchronize()

@@ -81,17 +81,20 @@ def test_opt_block_full_size_operator_by_operator(activation):
     for n in names:
         mod = getattr(blk, n)
 
-        def fwd(m, args, out, n=n):
+        def fwd(m, args, kwargs, out, n=n):
             cap[n]["in"], cap[n]["out"] = args[0].detach(), out.detach()
+            res = kwargs.get("residual")   # out_proj and fc2 add the residual stream in their epilogue
+            cap[n]["residual"] = None if res is None else res.detach()
 
         def bwd(m, gin, gout, n=n):
             cap[n]["d_in"], cap[n]["d_out"] = gin[0].detach(), gout[0].detach()
-        hooks += [mod.register_forward_hook(fwd), mod.register_full_backward_hook(bwd)]
+        hooks += [mod.register_forward_hook(fwd, with_kwargs=True), mod.register_full_backward_hook(bwd)]
     y = blk(x)
     y.backward(dy)
     torch.cuda.synchronize()
     for h in hooks:
         h.remove()
+    assert cap["out_proj"]["residual"] is not None and cap["fc2"]["residual"] is not None  # both ride the epilogue
     params = dict(blk.named_parameters())
 
     def prm(prefix, leaf):
@@ -132,6 +135,8 @@ def test_opt_block_full_size_operator_by_operator(activation):
         Wd, bd = W.detach().double().cpu(), b.detach().double().cpu()
         xin = _rows(c["in"], rows).requires_grad_(True)
         pre = xin @ Wd + bd
+        if c["residual"] is not None:
+            pre = pre + _rows(c["residual"], rows)
         out_rows = _rows(c["out"], rows)
         if n == "fc1":
             if activation == "relu":

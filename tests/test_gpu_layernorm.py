@@ -221,6 +221,39 @@ def test_ln_baseline_shape_properties():
     assert ((dx * xh).sum(dim=1).abs() / scale).max().item() < 1e-2
 
 
+def test_ln_baseline_shape_sampled_rows_against_the_float64_oracle():
+    """The benchmark's LayerNorm2D shard at exactly its size (16384 x 1024 bf16 of H = 2048, gamma ~ U(0.9, 1.1),
+    beta ~ N(0, 0.02), peer statistics from a second seeded half): 64 sampled rows of cw_ln_normalize's output and
+    saved (mean, rstd) and of cw_ln_bwd_dx_close's dx against the oracle's formulas in float64, evaluated from the
+    same inputs the kernels were given (the global statistics / row sums the GPU run produced, as a rank receives
+    them after the all-reduce); dgamma / dbeta of the open/close pair in full (16384 rows reduced)."""
+    import oracle
+    from cubework_amd import ops
+
+    R, C, H, eps = 16384, 1024, 2048, 1e-5
+    x, dy, gamma, beta = _inputs(R, C, torch.bfloat16, 0)
+    peer = randn((R, C), torch.bfloat16, 7)
+    xd, dyd, gd, bd, pd = (t.to(DEV) for t in (x, dy, gamma, beta, peer))
+    stats = ops.ln_partial_stats(xd) + ops.ln_partial_stats(pd)
+    y, mr = ops.ln_normalize(xd, stats, H, eps, gd, bd)
+    rs_local, pending = ops.ln_bwd_partials_open(dyd, xd, mr, gd)
+    rs = rs_local * 1.75          # stands in for the all-reduced row sums: any values exercise the dx formula
+    dx, dgamma, dbeta = ops.ln_bwd_dx_close(dyd, xd, mr, rs, H, pending, gd)
+    g = torch.Generator().manual_seed(3)
+    rows = torch.cat([torch.tensor([0, 1, 63, 64, R - 1]), torch.randint(0, R, (59,), generator=g)])
+    with oracle.precision(torch.float64):
+        st = stats.cpu()[rows]
+        want_y, want_mr = oracle.ln2d_normalize(x[rows], st, H, eps, gamma, beta)
+        assert_parity(mr.cpu()[rows], want_mr, torch.float32, "mean / rstd, 64 rows of 16384 x 1024")
+        assert_parity(y.cpu()[rows], _rounded(want_y, torch.bfloat16), torch.bfloat16, "ln_normalize, 64 rows of 16384 x 1024")
+        want_rs, want_dg, want_db = oracle.ln2d_backward_partials(dy, x, mr.cpu(), gamma)
+        assert_parity(rs_local, want_rs, torch.float32, "row sums (all 16384 rows)")
+        assert_parity(dgamma, want_dg, torch.float32, "dgamma (16384 rows reduced)")
+        assert_parity(dbeta, want_db, torch.float32, "dbeta (16384 rows reduced)")
+        want_dx = oracle.ln2d_backward_dx(dy[rows], x[rows], mr.cpu()[rows], rs.cpu()[rows], H, gamma)
+        assert_parity(dx.cpu()[rows], _rounded(want_dx, torch.bfloat16), torch.bfloat16, "ln_bwd_dx_close, 64 rows of 16384 x 1024")
+
+
 def test_ln_empty_and_errors():
     from cubework_amd import ops, _lib
 
@@ -321,13 +354,13 @@ def test_dx_close_argument_checks_and_no_rows():
     assert lib.cw_ln_bwd_partials_open(4, 8, None, 8, None, 8, None, None, None, None, 0, None, 0, None) == -1     # n_parts NULL
     assert lib.cw_ln_bwd_partials_open(4, 8, None, 8, None, 8, None, None, None, None, 0, C.cast(C.byref(n), C.c_void_p), 0, None) == -1
     assert n.value == 0
-    assert lib.cw_ln_bwd_dx_close(4, 8, None, 8, None, 8, None, None, None, 8, None, 8, None, 0, None, None, 0, None) == -1   # no dgamma
+    assert lib.cw_ln_bwd_dx_close(4, 8, None, 8, None, 8, None, None, None, 8, None, 8, None, 0, None, None, 1, 0, None) == -1   # no dgamma
     assert lib.cw_ln_bwd_dx_close(4, 8, None, 8, None, 8, None, None, None, 8, None, 8, None, 3, out[0].data_ptr(),
-                                  out[1].data_ptr(), 0, None) == -1                                                        # partials without workspace
+                                  out[1].data_ptr(), 1, 0, None) == -1                                                        # partials without workspace
     assert lib.cw_ln_bwd_dx_close(4, 8, None, 8, None, 8, None, None, None, 4, None, 8, None, 0, out[0].data_ptr(),
-                                  out[1].data_ptr(), 0, None) == -1                                                        # H < C
+                                  out[1].data_ptr(), 1, 0, None) == -1                                                        # H < C
     # no rows: zero column sums, nothing else touched
     assert lib.cw_ln_bwd_dx_close(0, 8, None, 8, None, 8, None, None, None, 8, None, 8, None, 0, out[0].data_ptr(),
-                                  out[1].data_ptr(), 0, None) == 0
+                                  out[1].data_ptr(), 1, 0, None) == 0
     torch.cuda.synchronize()
     assert torch.equal(out, torch.zeros_like(out))

@@ -83,6 +83,67 @@ def test_linear2d_fused_activation(act):
     assert_parity(layer.bias.grad, b.grad, torch.bfloat16, "dbias")
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+def test_linear2d_residual_addend(dtype):
+    """Linear2D's additive `residual` option: residual + x W + b in the GEMM's epilogue, the residual's
+    gradient being the output's; the bias gradient arrives in the parameter's dtype (fp32 sums rounded once)."""
+    from cubework_amd.distributed import initialize
+    from cubework_amd.module.parallel_2d import Linear2D
+
+    initialize("2d", 1)
+    layer = Linear2D(128, 256).to(dtype).to(DEV)
+    x = _leaf(randn((3, 40, 128), dtype, 0).to(DEV))
+    res = _leaf(randn((3, 40, 256), dtype, 2).to(DEV))
+    dy = randn((3, 40, 256), dtype, 1).to(DEV)
+    y = layer(x, residual=res)
+    y.backward(dy)
+    xr, rr = _leaf(x.detach().double().cpu()), _leaf(res.detach().double().cpu())
+    w = _leaf(layer.weight.detach().double().cpu())
+    b = _leaf(layer.bias.detach().double().cpu())
+    ref = rr + xr @ w + b
+    ref.backward(dy.double().cpu())
+    assert_parity(y, ref.detach(), dtype, "residual forward")
+    assert_parity(x.grad, xr.grad, dtype, "dX")
+    assert torch.equal(res.grad, dy)
+    assert_parity(layer.weight.grad, w.grad, dtype, "dW")
+    assert layer.bias.grad.dtype == dtype
+    assert_parity(layer.bias.grad, b.grad, dtype, "dbias")
+    with pytest.raises(ValueError):
+        Linear2D(128, 256, activation="relu").to(dtype).to(DEV)(x, residual=res)
+    with pytest.raises(AssertionError):
+        layer(x, residual=res[:, :, :128])
+
+
+@pytest.mark.parametrize("out_dtype", [torch.bfloat16, torch.float16])
+def test_column_sums_stored_in_the_parameter_dtype(out_dtype):
+    """The finalize stage stores its fp32 totals as bf16 / fp16 when asked: the same bits as the fp32 result
+    cast afterwards (one rounding to nearest even), for every entry point with column sums."""
+    from cubework_amd import ops
+
+    io = out_dtype
+    dy = randn((700, 520), io, 3).to(DEV)
+    pre = randn((700, 520), io, 4).to(DEV)
+    assert torch.equal(ops.colsum(dy, out_dtype=out_dtype), ops.colsum(dy).to(out_dtype))
+    _, want = ops.act_bwd_colsum("gelu_tanh", dy, pre)
+    _, got = ops.act_bwd_colsum("gelu_tanh", dy, pre, out_dtype=out_dtype)
+    assert got.dtype == out_dtype and torch.equal(got, want.to(out_dtype))
+    x = randn((700, 520), io, 5).to(DEV)
+    gamma = randn((520,), io, 6).to(DEV)
+    _, mr = ops.ln_forward_fused(x, 1e-5, gamma, None)
+    dx0, dg0, db0 = ops.ln_backward_fused(dy, x, mr, gamma)
+    dx1, dg1, db1 = ops.ln_backward_fused(dy, x, mr, gamma, param_dtype=out_dtype)
+    assert torch.equal(dx0, dx1) and torch.equal(dg1, dg0.to(out_dtype)) and torch.equal(db1, db0.to(out_dtype))
+    rs0, dg0, db0 = ops.ln_bwd_partials(dy, x, mr, gamma)
+    rs1, dg1, db1 = ops.ln_bwd_partials(dy, x, mr, gamma, param_dtype=out_dtype)
+    assert torch.equal(rs0, rs1) and torch.equal(dg1, dg0.to(out_dtype)) and torch.equal(db1, db0.to(out_dtype))
+    rs, pending = ops.ln_bwd_partials_open(dy, x, mr, gamma)
+    _, dg0, db0 = ops.ln_bwd_dx_close(dy, x, mr, rs, 520, pending, gamma)
+    _, dg1, db1 = ops.ln_bwd_dx_close(dy, x, mr, rs, 520, pending, gamma, param_dtype=out_dtype)
+    assert torch.equal(dg1, dg0.to(out_dtype)) and torch.equal(db1, db0.to(out_dtype))
+    with pytest.raises(TypeError):
+        ops.colsum(dy, out_dtype=torch.float64)
+
+
 def test_skip_bias_add_and_errors():
     from cubework_amd.distributed import initialize
     from cubework_amd.module.parallel_1d import Linear1D_Col, Linear1D_Row

@@ -167,6 +167,35 @@ def test_vpce_baseline_shape_properties():
     assert (total.abs() / dl).max().item() < 1e-4
 
 
+def test_vpce_baseline_shape_sampled_rows_against_the_float64_oracle():
+    """The benchmark's cross-entropy workload at exactly its size (8192 tokens x 12568 classes of 50272, rank 1 of
+    4, bf16 logits ~ N(0, 2), dloss = 1/8192): 64 sampled rows of the bf16 and of the fp32 gradient against the
+    oracle's formula in float64, evaluated with the global (max, sum) the GPU forward produced (what the rank is
+    handed after the all-reduce), and the local forward statistics of those rows (mask / gathered logit / max
+    bit-exact)."""
+    import oracle
+    from cubework_amd import ops
+
+    T, V, p, r = 8192, 12568, 4, 1
+    t = _targets(T, V * p, 1)
+    slices = [randn((T, V), torch.bfloat16, 10 + k, std=2.0) for k in range(p)]
+    dev_slices = [s.to(DEV) for s in slices]
+    stats = [ops.vpce_fwd_local(s, t.to(DEV), k * V) for k, s in enumerate(dev_slices)]
+    loss, gmax, gsum = ops.vpce_finalize(*(torch.stack([st[k] for st in stats]) for k in range(4)))
+    g = torch.Generator().manual_seed(4)
+    rows = torch.cat([torch.tensor([0, 1, 255, 256, T - 1]), torch.randint(0, T, (59,), generator=g)])
+    dl = torch.full((T,), 1.0 / T)
+    with oracle.precision(torch.float64):
+        want = oracle.vpce_fwd_local(slices[r][rows], t[rows], r * V)
+        got = [st.cpu()[rows] for st in stats[r]]
+        assert torch.equal(got[3], want[3]) and torch.equal(got[2], want[2].float()) and torch.equal(got[0], want[0].float())
+        assert_parity(got[1], want[1], torch.float32, "sum exp, 64 rows of 8192 x 12568")
+        want_g = oracle.vpce_bwd(slices[r][rows], t[rows], r * V, gmax.cpu()[rows], gsum.cpu()[rows], dl[rows])
+        for gd in (torch.bfloat16, torch.float32):
+            grad = ops.vpce_bwd(dev_slices[r], t.to(DEV), r * V, gmax, gsum, None, 1.0 / T, grad_dtype=gd)
+            assert_parity(grad.cpu()[rows], want_g, gd, "vpce_bwd %s grad, 64 rows of 8192 x 12568" % str(gd).split(".")[-1])
+
+
 def test_vpce_empty():
     from cubework_amd import ops
 
