@@ -18,7 +18,7 @@ LIB_PATH = os.path.join(HERE, "libcubework_hip.so")
 
 SOURCES = ["gemm_bf16_tn.hip", "gemm_f16_tn.hip", "gemm_bf16_nn.hip", "gemm_f16_nn.hip", "gemm_bf16_nt.hip", "gemm_f16_nt.hip",  # slowest first
            "gemm_bf16_dma_nn.hip", "gemm_bf16_dma_nt.hip", "gemm_bf16_dma_tn.hip", "gemm_f16_dma_nn.hip", "gemm_f16_dma_nt.hip", "gemm_f16_dma_tn.hip",
-           "cw_runtime.hip", "cw_api.hip", "gemm_bf16.hip", "gemm_half_small.hip", "gemm_f32.hip", "epilogue.hip", "layernorm.hip", "vpce.hip", "attention.hip", "attention_bwd.hip", "embedding.hip", "embed_sort.hip", "clip_grad.hip"]
+           "cw_runtime.hip", "cw_api.hip", "gemm_plan.hip", "gemm_bf16.hip", "gemm_half_small.hip", "gemm_f32.hip", "epilogue.hip", "layernorm.hip", "vpce.hip", "attention.hip", "attention_bwd.hip", "embedding.hip", "embed_sort.hip", "clip_grad.hip"]
 # the measurement library: its own kernels plus the runtime services (error text, device check), nothing else
 DIAG_SOURCES = ["diag_gemm.hip", "diag.hip"]
 DIAG_LIB_PATH = os.path.join(HERE, "libcubework_diag.so")

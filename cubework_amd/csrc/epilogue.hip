@@ -8,16 +8,14 @@
 #include <type_traits>
 
 #include "cw_common.h"
+#include "gemm_plan.h"
 #include "reduce_cols.h"
 
 namespace cw {
 
 namespace {
 
-constexpr int kColWaves = 4;   // wavefronts per block on the vector path, each on its own rows
-constexpr int kColUnroll = 4;  // rows in flight per wavefront
-constexpr int64_t kColBlocks = 1024;  // blocks aimed at (4 resident per compute unit)
-constexpr int64_t kGenericSlabRows = 64;
+constexpr int64_t kGenericSlabRows = kColGenericSlabRows;  // rows per slab of the element-wise kernel (gemm_plan.h)
 
 // MODE 0: column sums of dY. MODE 1: dPre = dY * ACT'(pre), column sums of dPre.
 template <typename T, int MODE, int ACT>
@@ -135,23 +133,6 @@ __global__ __launch_bounds__(kFinGroups * 64) void finalize_cols_kernel(const fl
         void* out = (k == 0) ? out0 : out1;
         if (out != nullptr) store_col_total(out, c, total, out_dtype);
     }
-}
-
-// Row slabs of an [M,N] operand with V elements per 16 bytes: one partial row of N sums per slab.
-void colsum_plan(int64_t M, int64_t N, int V, bool vec, int64_t& slabs, int64_t& rows_per_slab) {
-    if (!vec) {
-        rows_per_slab = kGenericSlabRows;
-        slabs = (M + rows_per_slab - 1) / rows_per_slab;
-        return;
-    }
-    const int64_t coltiles = (N + 64 * V - 1) / (64 * V);
-    slabs = kColBlocks / coltiles;
-    const int64_t max_slabs = (M + kColWaves * kColUnroll - 1) / (kColWaves * kColUnroll);
-    if (slabs > max_slabs) slabs = max_slabs;
-    if (slabs > 512) slabs = 512;  // the bound cw_colsum_workspace_bytes promises
-    if (slabs < 1) slabs = 1;
-    rows_per_slab = (M + slabs - 1) / slabs;
-    slabs = (M + rows_per_slab - 1) / rows_per_slab;
 }
 
 template <typename T, int MODE>

@@ -14,6 +14,7 @@
 #include <cstring>
 
 #include "gemm_bf16_kernel.h"
+#include "gemm_plan.h"
 
 namespace cw {
 
@@ -34,16 +35,6 @@ int gemm_f16_dma_split_launch_nt(const GemmArgs& args, int slices, hipStream_t s
 int gemm_f16_dma_split_launch_tn(const GemmArgs& args, int slices, hipStream_t s);
 
 int gemm_half_small_launch(const GemmArgs& args, int layout, int epilogue, bool f16, hipStream_t s);
-
-int gemm_bf16_split_slices(int64_t M, int64_t N, int64_t K, int n_steps) {
-    if (M <= 0 || N <= 0 || K <= 0 || n_steps <= 0 || n_steps > kRingMaxSteps) return 1;
-    if ((M % 256) != 0 || (N % 256) != 0 || (K % 64) != 0) return 1;
-    const int64_t tiles = (M / 256) * (N / 256);
-    if (tiles >= 128 || K * n_steps < 2048) return 1;  // enough tiles already, or a short reduction
-    int slices = 8;
-    while (slices > 1 && (tiles * slices > 256 || (K % (64 * slices)) != 0 || K / slices < 256)) slices >>= 1;
-    return slices;
-}
 
 namespace {
 
@@ -134,13 +125,6 @@ __global__ __launch_bounds__(256) void ktail_rows_kernel(const uint16_t* __restr
     *reinterpret_cast<raw16_t*>(out + (int64_t)r * ld + c) = v;
 }
 
-int64_t gemm_bf16_ktail_workspace_bytes(int layout, int64_t M, int64_t N, int64_t K, int n_steps) {
-    if (layout == CW_NT || n_steps != 1 || K < 64 || (K % 32) == 0 || (K % 8) != 0) return 0;
-    const int64_t tiles = ((M + 255) / 256) * ((N + 255) / 256);
-    if (tiles < 128 || M < 256 || N < 256 || (N % 8) != 0) return 0;
-    return 32 * N * (int64_t)sizeof(uint16_t);
-}
-
 static bool dma_kernel_enabled() {
     static const bool enabled = [] {
         const char* v = std::getenv("CW_GEMM_IMPL");
@@ -181,118 +165,38 @@ static int dma_launch(const GemmArgs& a, int layout, int epilogue, bool f16, hip
 }
 
 // f16: the operands, bias, addends and outputs are IEEE half instead of bfloat16; everything else is shared.
+// The choice of kernel and the cuts are gemm_half_plan's (gemm_plan.hip); this function only launches.
 int gemm_half_launch(const GemmArgs& args, int layout, int epilogue, bool f16, hipStream_t s) {
-    // the unguarded kernels address operands with 32-bit byte offsets
-    const int64_t max_dim = args.M > args.N ? (args.M > args.K ? args.M : args.K) : (args.N > args.K ? args.N : args.K);
-    const bool fits32 = (max_dim + 64) * (args.lda > args.ldb ? args.lda : args.ldb) * 2 < ((int64_t)1 << 32);
-    const bool all_vec = fits32 && args.vec_a && args.vec_b && args.vec_c && (args.preact == nullptr || args.vec_p) &&
-                         (args.bias == nullptr || args.vec_bias) && (args.n_addends == 0 || args.vec_add);
-    const int64_t tiles256 = (int64_t)((args.M + 255) / 256) * ((args.N + 255) / 256);
-    const bool big = tiles256 >= 128;
-    const int tile = big ? 256 : 128;
-    const bool exact = all_vec && (args.M % tile) == 0 && (args.N % tile) == 0 && (args.K % gemm_bf16::kBK) == 0;
-    const bool ring_ok = args.n_steps > 0 && args.n_steps <= kRingMaxSteps && args.n_addends <= kRingMaxAddends &&
-                         dma_kernel_enabled();
-    // The LDS-DMA kernel takes M and N that are not tile multiples (its last tiles overlap their
-    // neighbours): a vocabulary slice of 12568 columns is 50 tiles instead of 49.1. What it needs is one
-    // full tile in each direction and 16-byte steps wherever a tile origin moves along a contiguous
-    // dimension (N always: the output and a [K, N] operand; M for a [K, M] operand).
-    const bool edges_ok = args.M >= 256 && args.N >= 256 && (args.N % 8) == 0 && (layout != CW_TN || (args.M % 8) == 0);
-    // Fewer than 160 tiles of 256 x 256 (at 128 .. 159 of them the large tiles leave 40 % of the compute units
-    // idle, and four times as many small tiles fill them): the ring kernel with 128 x 128 tiles, unless a long
-    // reduction over few tiles is better served by splitting k (below; measured on 2048 x 2048 outputs: the
-    // small tiles win up to a reduction length of 8192, the split from 16384).
-    const int slices = gemm_bf16_split_slices(args.M, args.N, args.K, args.n_steps);
-    {
-        const int64_t tiles128 = (int64_t)((args.M + 127) / 128) * ((args.N + 127) / 128);
-        const bool splits = slices > 1 && args.workspace != nullptr && aligned16(args.workspace) &&
-                            args.workspace_bytes >= (int64_t)slices * args.M * args.N * (int64_t)sizeof(float);
-        if (tiles256 < 160 && all_vec && ring_ok && args.M >= 128 && args.N >= 128 && (args.N % 8) == 0 &&
-            (layout != CW_TN || (args.M % 8) == 0) && args.K >= 64 && (args.K % 64) == 0 &&
-            args.lda < ((int64_t)1 << 23) && args.ldb < ((int64_t)1 << 23) && ((tiles128 >= 192 && (int64_t)args.K * args.n_steps < 12288) || !splits))
-            return gemm_half_small_launch(args, layout, epilogue, f16, s);
-    }
-    if (big && all_vec && ring_ok && edges_ok && (args.K % gemm_bf16::kBK) == 0) {
-        // A last round of 256 x 256 tiles that is mostly empty (a vocabulary slice as N: 8192 x 12568 is 32 x 50 =
-        // 1600 tiles, 6.25 rounds of the 256 compute units): when the partial round is whole tile columns (or whole
-        // tile rows), at most 3/8 of a round, and that strip is at most one round of 128 x 128 tiles, it goes to the
-        // small-tile kernel as a second launch and the rest is whole rounds.
-        const int64_t tiles_m = (args.M + 255) / 256, tiles_n = (args.N + 255) / 256;
-        const int64_t last_round = (tiles_m * tiles_n) % 256;
-        const bool small_ok = (args.K % 64) == 0 && args.lda < ((int64_t)1 << 23) && args.ldb < ((int64_t)1 << 23);
-        if (tiles_m * tiles_n > 256 && last_round > 0 && last_round <= 96 && small_ok && strip_split_enabled()) {
-            auto shift = [&](const void* p, int64_t elems) -> const void* {
-                return p == nullptr ? nullptr : reinterpret_cast<const uint16_t*>(p) + elems;
-            };
-            GemmArgs head = args, tail = args;
-            bool split = false;
-            if (last_round % tiles_m == 0) {  // whole tile columns
-                const int64_t n0 = (tiles_n - last_round / tiles_m) * 256, strip = args.N - n0;
-                if (n0 >= 256 && strip >= 128 && ((args.M + 127) / 128) * ((strip + 127) / 128) <= 256) {
-                    head.N = (int)n0;
-                    tail.N = (int)strip;
-                    for (int i = 0; i < args.n_steps; ++i) tail.B[i] = shift(args.B[i], layout == CW_NT ? n0 * args.ldb : n0);
-                    for (int k = 0; k < args.n_addends; ++k) tail.addend[k] = shift(args.addend[k], n0);
-                    tail.bias = shift(args.bias, n0);
-                    tail.C = const_cast<void*>(shift(args.C, n0));
-                    tail.preact = const_cast<void*>(shift(args.preact, n0));
-                    split = true;
-                }
-            }
-            if (!split && last_round % tiles_n == 0) {  // whole tile rows
-                const int64_t m0 = (tiles_m - last_round / tiles_n) * 256, strip = args.M - m0;
-                if (m0 >= 256 && strip >= 128 && ((strip + 127) / 128) * ((args.N + 127) / 128) <= 256) {
-                    head.M = (int)m0;
-                    tail.M = (int)strip;
-                    for (int i = 0; i < args.n_steps; ++i) tail.A[i] = shift(args.A[i], layout == CW_TN ? m0 : m0 * args.lda);
-                    for (int k = 0; k < args.n_addends; ++k) tail.addend[k] = shift(args.addend[k], m0 * args.ldadd);
-                    tail.C = const_cast<void*>(shift(args.C, m0 * args.ldc));
-                    tail.preact = const_cast<void*>(shift(args.preact, m0 * args.ldp));
-                    split = true;
-                }
-            }
-            if (split) {
-                if (const int rc = dma_launch(head, layout, epilogue, f16, s); rc != CW_OK) return rc;
-                return gemm_half_small_launch(tail, layout, epilogue, f16, s);
-            }
+    const GemmPlan plan = gemm_half_plan(args, layout, dma_kernel_enabled(), strip_split_enabled());
+    switch (plan.route) {
+        case kRouteSmallRing: return gemm_half_small_launch(plan.head, layout, epilogue, f16, s);
+        case kRouteRing: return dma_launch(plan.head, layout, epilogue, f16, s);
+        case kRouteRingThenSmall: {
+            if (const int rc = dma_launch(plan.head, layout, epilogue, f16, s); rc != CW_OK) return rc;
+            return gemm_half_small_launch(plan.tail, layout, epilogue, f16, s);
         }
-        return dma_launch(args, layout, epilogue, f16, s);
-    }
-    // A reduction length that is not a multiple of the k tile (a vocabulary slice as K: 12568 = 392 x 32 +
-    // 24), with B stored [K, N]: the regular step covers the first K - K % 32 columns, one more step of 32
-    // covers [K-32, K) with a copy of B's last 32 rows whose overlapping rows are zero. The copy (64 bytes
-    // per column) lives in the caller's scratch and has B's row pitch, which the steps share.
-    if (big && all_vec && ring_ok && edges_ok && layout != CW_NT && args.n_steps == 1 && args.K >= 64 &&
-        (args.K % 32) != 0 && (args.K % 8) == 0 && args.workspace != nullptr && aligned16(args.workspace) &&
-        args.workspace_bytes >= 32 * args.ldb * (int64_t)sizeof(uint16_t)) {
-        const int kr = args.K % 32;
-        uint16_t* tail_b = reinterpret_cast<uint16_t*>(args.workspace);
-        const int vecs = 32 * (args.N / 8);
-        hipLaunchKernelGGL(ktail_rows_kernel, dim3((vecs + 255) / 256), dim3(256), 0, s,
-                           reinterpret_cast<const uint16_t*>(args.B[0]), args.ldb, (int64_t)args.K, args.N, 32 - kr, tail_b);
-        int rc = check_launch("ktail_rows_kernel");
-        if (rc != CW_OK) return rc;
-        // A's part of the step: columns (NN, A is [M, K]) or rows (TN, A is [K, M]) K-32 .. K-1, in place
-        const uint16_t* a0 = reinterpret_cast<const uint16_t*>(args.A[0]);
-        const void* tail_a = layout == CW_TN ? a0 + (int64_t)(args.K - 32) * args.lda : a0 + (args.K - 32);
-        GemmArgs main_part = args;
-        main_part.K = args.K - kr;
-        return dma_launch(main_part, layout, epilogue, f16, s, tail_a, tail_b);
-    }
-    if (slices > 1 && all_vec && args.n_addends <= kRingMaxAddends && dma_kernel_enabled() &&
-        args.workspace != nullptr && aligned16(args.workspace) &&
-        args.workspace_bytes >= (int64_t)slices * args.M * args.N * (int64_t)sizeof(float)) {
-        int rc;
-        switch (layout) {
-            case CW_NN: rc = f16 ? gemm_f16_dma_split_launch_nn(args, slices, s) : gemm_bf16_dma_split_launch_nn(args, slices, s); break;
-            case CW_NT: rc = f16 ? gemm_f16_dma_split_launch_nt(args, slices, s) : gemm_bf16_dma_split_launch_nt(args, slices, s); break;
-            case CW_TN: rc = f16 ? gemm_f16_dma_split_launch_tn(args, slices, s) : gemm_bf16_dma_split_launch_tn(args, slices, s); break;
-            default: return fail(CW_ERR_INVALID, "cw_gemm_ksteps: bad layout %d", layout);
+        case kRouteRingKTail: {
+            uint16_t* tail_b = reinterpret_cast<uint16_t*>(args.workspace);
+            const int vecs = 32 * (args.N / 8);
+            hipLaunchKernelGGL(ktail_rows_kernel, dim3((vecs + 255) / 256), dim3(256), 0, s,
+                               reinterpret_cast<const uint16_t*>(args.B[0]), args.ldb, (int64_t)args.K, args.N,
+                               plan.ktail_zero_rows, tail_b);
+            if (const int rc = check_launch("ktail_rows_kernel"); rc != CW_OK) return rc;
+            return dma_launch(plan.head, layout, epilogue, f16, s, plan.ktail_a, tail_b);
         }
-        if (rc != CW_OK) return rc;
-        return f16 ? splitk_reduce<f16_t>(args, slices, epilogue, s) : splitk_reduce<bf16_t>(args, slices, epilogue, s);
+        case kRouteSplitK: {
+            int rc;
+            switch (layout) {
+                case CW_NN: rc = f16 ? gemm_f16_dma_split_launch_nn(args, plan.slices, s) : gemm_bf16_dma_split_launch_nn(args, plan.slices, s); break;
+                case CW_NT: rc = f16 ? gemm_f16_dma_split_launch_nt(args, plan.slices, s) : gemm_bf16_dma_split_launch_nt(args, plan.slices, s); break;
+                case CW_TN: rc = f16 ? gemm_f16_dma_split_launch_tn(args, plan.slices, s) : gemm_bf16_dma_split_launch_tn(args, plan.slices, s); break;
+                default: return fail(CW_ERR_INVALID, "cw_gemm_ksteps: bad layout %d", layout);
+            }
+            if (rc != CW_OK) return rc;
+            return f16 ? splitk_reduce<f16_t>(args, plan.slices, epilogue, s) : splitk_reduce<bf16_t>(args, plan.slices, epilogue, s);
+        }
+        default: return staged_launch(args, layout, epilogue, plan.big, plan.exact, f16, s);
     }
-    return staged_launch(args, layout, epilogue, big, exact, f16, s);
 }
 
 }  // namespace cw

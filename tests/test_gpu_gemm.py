@@ -301,3 +301,50 @@ def test_relu_epilogue_keeps_nan(shape, dtype):
     assert torch.isnan(want[5]).all() and torch.equal(torch.isnan(got), torch.isnan(want))
     ok = ~torch.isnan(want)
     assert_parity(got[ok], want[ok], dtype, "relu epilogue beside a NaN row")
+
+
+def test_ring_kernel_order_of_summation_is_fixed_per_shape_and_bounded_across_shapes():
+    """The ring kernel starts each tile's reduction at a k offset that depends on the tile's position (an eighth
+    of the range per XCD), and only where M and N are tile multiples. So: (1) the same call twice gives the same
+    bits; (2) the same logical product reached another way - as rows of a product whose M is not a tile multiple
+    (no rotated start), or with CW_GEMM_IMPL=onelaunch in a fresh process for a shape whose last round of tiles
+    is otherwise peeled off into a second launch - may differ in the last bits, by no more than fp32
+    reassociation of the K-term sums allows: here at most one bf16 step of the largest magnitude, in few
+    elements."""
+    import os
+    import subprocess
+    import sys
+    from cubework_amd import ops
+
+    M, N, K = 4096, 4096, 2048       # 256 tiles: the ring kernel, rotated starts
+    a = randn((M + 8, K), torch.bfloat16, 71).to(DEV)
+    b = randn((K, N), torch.bfloat16, 72, 0.05).to(DEV)
+    c1 = ops.gemm_ksteps("NN", [a[:M]], [b])
+    c2 = ops.gemm_ksteps("NN", [a[:M]], [b])
+    assert torch.equal(c1, c2)
+    ragged = ops.gemm_ksteps("NN", [a], [b])[:M]          # M + 8 rows: overlapping last tiles, no rotation
+    step = c1.float().abs().max().item() * 2.0 ** -8      # one bf16 step at the largest magnitude
+    diff = (c1.float() - ragged.float()).abs()
+    assert diff.max().item() <= step
+    assert (diff > 0).float().mean().item() < 0.05
+    # the second launch for a mostly empty last round, against the one launch (read once per process: a fresh one)
+    Ms, Ns, Ks = 4096, 4376, 128
+    a2 = randn((Ms, Ks), torch.bfloat16, 73)
+    b2 = randn((Ks, Ns), torch.bfloat16, 74, 0.05)
+    here = ops.gemm_ksteps("NN", [a2.to(DEV)], [b2.to(DEV)]).cpu()
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    code = ("import sys, torch; sys.path.insert(0, %r)\n"
+            "from tests.util import randn\nfrom cubework_amd import ops\n"
+            "a = randn((%d, %d), torch.bfloat16, 73).to('cuda:0'); b = randn((%d, %d), torch.bfloat16, 74, 0.05).to('cuda:0')\n"
+            "torch.save(ops.gemm_ksteps('NN', [a], [b]).cpu(), sys.argv[1])\n" % (root, Ms, Ks, Ks, Ns))
+    import tempfile
+    with tempfile.TemporaryDirectory() as tmp:
+        path = os.path.join(tmp, "c.pt")
+        env = dict(os.environ, CW_GEMM_IMPL="onelaunch")
+        proc = subprocess.run([sys.executable, "-c", code, path], capture_output=True, text=True, timeout=300, env=env)
+        assert proc.returncode == 0, proc.stdout + proc.stderr
+        other = torch.load(path, weights_only=True)
+    step = here.float().abs().max().item() * 2.0 ** -8
+    diff = (here.float() - other.float()).abs()
+    assert diff.max().item() <= step
+    assert (diff > 0).float().mean().item() < 0.05
