@@ -294,7 +294,7 @@ def graph_time_us(fn, calls, replays=3, min_ms=100.0):
     return timed(n) if n > replays else pilot
 
 
-def bench_bandwidth_kernels(device):
+def bench_bandwidth_kernels(device, parts=("ln", "ln_wide", "ce")):
     """LayerNorm2D (config 3) and vocab-parallel CE (config 4) kernels: algorithmic
     bytes per launch / average launch duration. Each call below is one C-ABI
     entry point; the launches are replayed from a HIP graph. The LayerNorm2D
@@ -338,15 +338,17 @@ def bench_bandwidth_kernels(device):
         ("ln_backward_fused", 3 * 33554432 + 2 * 131072 + 8192,
          lambda: ops.ln_backward_fused(rot(dys), xs[i[0] % nb], mr_whole, gamma)),
     ]
-    for name, nbytes, fn in cases:
+    for name, nbytes, fn in cases if "ln" in parts else ():
         us = graph_time_us(fn, 2 * nb)
         out[name] = {"us": round(us, 2), "GBps": round(nbytes / us / 1e3, 1), "frac": round(nbytes / us / 1e3 / HBM_PEAK_GBPS, 3),
                      "bytes": nbytes}
     del xs, dys
+    if "ln_wide" not in parts and "ce" not in parts:
+        return out
     # wide rows held whole by the rank: the fp32 residual stream under autocast (hidden 2048 and 4096) and a
     # 16-bit hidden size of 4096; fused forward (x read, y written) and fused backward (dy, x read, dx written)
     for tag, Rw, Cw, dt in (("fp32_8192x2048", 8192, 2048, torch.float32), ("fp32_4096x4096", 4096, 4096, torch.float32),
-                            ("bf16_8192x4096", 8192, 4096, torch.bfloat16)):
+                            ("bf16_8192x4096", 8192, 4096, torch.bfloat16)) if "ln_wide" in parts else ():
         nw = 6
         es = 4 if dt == torch.float32 else 2
         xw = [_seeded((Rw, Cw), 400 + k, 1.0, dt).to(device) for k in range(nw)]
@@ -363,6 +365,8 @@ def bench_bandwidth_kernels(device):
             out[name] = {"us": round(us, 2), "GBps": round(nbytes / us / 1e3, 1),
                          "frac": round(nbytes / us / 1e3 / HBM_PEAK_GBPS, 3), "bytes": nbytes}
         del xw, dw
+    if "ce" not in parts:
+        return out
     T, V, V0 = 8192, 12568, 12568
     lg = [_seeded((T, V), 300 + k, 2.0, torch.bfloat16).to(device) for k in range(3)]  # 3 x 196 MiB
     tg = torch.randint(0, 50272, (T,), generator=torch.Generator().manual_seed(9)).to(device)

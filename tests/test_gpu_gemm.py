@@ -11,6 +11,7 @@ from tests.util import assert_parity, randn
 pytestmark = pytest.mark.gpu
 
 LAYOUTS = ["NN", "NT", "TN"]
+DEV = "cuda:0"
 
 
 def _operands(layout, M, N, K, steps, dtype, seed, pad_a=0, pad_b=0):

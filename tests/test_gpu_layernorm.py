@@ -364,3 +364,24 @@ def test_dx_close_argument_checks_and_no_rows():
                                   out[1].data_ptr(), 1, 0, None) == 0
     torch.cuda.synchronize()
     assert torch.equal(out, torch.zeros_like(out))
+
+
+def test_partial_stats_into_a_result_buffer_that_is_only_8_byte_aligned():
+    """The one-tile-per-wavefront statistics kernel writes two rows' results as one 16-byte piece when the
+    result buffer allows it; a buffer that is 8-byte but not 16-byte aligned takes per-row stores. Same bits."""
+    import ctypes
+    from cubework_amd import _lib, ops
+
+    lib = _lib.load()
+    for R, C in ((64, 1024), (37, 512), (1001, 2048)):
+        x = randn((R, C), torch.bfloat16, R).to(DEV)
+        want = ops.ln_partial_stats(x)
+        buf = torch.full((2 * R + 2,), float("nan"), dtype=torch.float32, device=DEV)
+        view = buf[2:]
+        assert view.data_ptr() % 16 == 8
+        stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+        _lib.check(lib.cw_ln_partial_stats(R, C, x.data_ptr(), C, _lib.CW_LN_ONE_PASS, None, view.data_ptr(), _lib.CW_BF16, stream),
+                   "cw_ln_partial_stats")
+        torch.cuda.synchronize()
+        assert torch.equal(view.view(R, 2), want)
+        assert torch.isnan(buf[:2]).all()
