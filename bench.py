@@ -436,11 +436,11 @@ class AbiCallTimer:
         if name == "cw_ln_forward_fused":
             return ("%dx%d" % (a[0], a[1]), "bytes", 2.0 * a[0] * a[1] * es(a[11]))
         if name == "cw_ln_backward_fused":
-            return ("%dx%d" % (a[0], a[1]), "bytes", 3.0 * a[0] * a[1] * es(a[15]))
+            return ("%dx%d" % (a[0], a[1]), "bytes", (4.0 if a[11] else 3.0) * a[0] * a[1] * es(a[18]))
         if name == "cw_colsum":
-            return ("%dx%d" % (a[0], a[1]), "bytes", 1.0 * a[0] * a[1] * es(a[7]))
+            return ("%dx%d" % (a[0], a[1]), "bytes", 1.0 * a[0] * a[1] * es(a[8]))
         if name == "cw_act_bwd_colsum":
-            return ("%dx%d" % (a[1], a[2]), "bytes", 3.0 * a[1] * a[2] * es(a[12]))
+            return ("%dx%d" % (a[1], a[2]), "bytes", 3.0 * a[1] * a[2] * es(a[13]))
         return ("", None, 0.0)
 
     def __getattr__(self, name):
@@ -550,6 +550,21 @@ def bench_other_configs(device, sets):
                       "comparison line only, nothing on the product path calls it")
     out["vendor_anchor_8192x8192x8192"] = anchor
     del big, o_big
+    # the four weight-gradient products of the OPT-1.3B-shaped block (config 5): dW = X^T dY over 8192 tokens (TN),
+    # [in, out] = qkv 2048 x 6144 (192 tiles of 256 x 256: three quarters of the compute units), out 2048 x 2048
+    # (64 tiles: split along k), fc1 2048 x 8192 and fc2 8192 x 2048 (256 tiles each)
+    tok = 8192
+    x_in = {2048: _seeded((tok, 2048), 71, 1.0, torch.bfloat16).to(device), 8192: _seeded((tok, 8192), 72, 1.0, torch.bfloat16).to(device)}
+    dy_out = {n_: _seeded((tok, n_), 73 + k_, 1.0, torch.bfloat16).to(device) for k_, n_ in enumerate((2048, 6144, 8192))}
+    for name, k_in, n_out in (("qkv_2048x6144", 2048, 6144), ("out_2048x2048", 2048, 2048), ("fc1_2048x8192", 2048, 8192),
+                              ("fc2_8192x2048", 8192, 2048)):
+        xa, dya = x_in[k_in], dy_out[n_out]
+        flop = 2.0 * tok * k_in * n_out
+        us = event_time_us(lambda: ops.gemm_ksteps("TN", [xa], [dya]), 20, 5)
+        out["config5_dW_" + name] = {"us": round(us, 2), "TFLOPs": round(flop / us / 1e6, 1),
+                                     "frac": round(flop / us / 1e6 / MFMA_BF16_PEAK_TFLOPS, 4),
+                                     "tiles_256": (k_in // 256) * (n_out // 256)}
+    del x_in, dy_out
     # config 2's product with float16 operands (what a plain torch.autocast hands the GEMM-type operators):
     # the same kernel with the other MFMA opcode and conversion
     a16 = [t.to(torch.float16) for t in sets[0][0]]
@@ -932,7 +947,26 @@ def stream_ceiling(device):
         us = graph_time_us(fill, 2 * nbuf)
         out["fill_%dMiB" % mib] = {"us": round(us, 2), "bytes": 2 * n, "GBps": round(2 * n / us / 1e3, 1),
                                    "frac": round(2 * n / us / 1e3 / HBM_PEAK_GBPS, 3)}
-        del src, dst
+        # read-only: torch's row reductions over the same buffers viewed as rows of 1024 (what a statistics kernel
+        # does: read everything, write one value per row)
+        rows = [t.view(-1, 1024) for t in src]
+        red = torch.empty(rows[0].shape[0], device=device, dtype=torch.float32)
+        redb = torch.empty(rows[0].shape[0], device=device, dtype=torch.bfloat16)
+
+        def row_sum():
+            i[0] += 1
+            torch.sum(rows[i[0] % nbuf], dim=1, dtype=torch.float32, out=red)
+
+        def row_amax():
+            i[0] += 1
+            torch.amax(rows[i[0] % nbuf], dim=1, out=redb)
+        for name, fn in (("row_sum", row_sum), ("row_amax", row_amax)):
+            if mib > 64:
+                continue
+            us = graph_time_us(fn, 2 * nbuf)
+            out["%s_%dMiB" % (name, mib)] = {"us": round(us, 2), "bytes": 2 * n, "GBps": round(2 * n / us / 1e3, 1),
+                                            "frac": round(2 * n / us / 1e3 / HBM_PEAK_GBPS, 3)}
+        del src, dst, rows
     return out
 
 

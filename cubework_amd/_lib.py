@@ -64,8 +64,8 @@ SIGNATURES = {
     "cw_ln_forward_fused": (_int, [_i64, _i64, _ptr, _i64, _int, _f32, _ptr, _ptr, _ptr, _i64, _ptr, _int, _ptr]),
     "cw_ln_bwd_partials": (_int, [_i64, _i64, _ptr, _i64, _ptr, _i64, _ptr, _ptr, _ptr, _ptr, _ptr, _int, _ptr, _i64, _int,
                                   _ptr]),
-    "cw_ln_backward_fused": (_int, [_i64, _i64, _ptr, _i64, _ptr, _i64, _ptr, _ptr, _ptr, _ptr, _i64, _ptr, _ptr, _int, _ptr,
-                                    _i64, _int, _ptr]),
+    "cw_ln_backward_fused": (_int, [_i64, _i64, _ptr, _i64, _ptr, _i64, _ptr, _ptr, _ptr, _ptr, _i64, _ptr, _i64, _ptr, _ptr,
+                                    _int, _ptr, _i64, _int, _ptr]),
     "cw_ln_bwd_dx": (_int, [_i64, _i64, _ptr, _i64, _ptr, _i64, _ptr, _ptr, _ptr, _i64, _ptr, _i64, _int, _ptr]),
     "cw_ln_bwd_partials_open": (_int, [_i64, _i64, _ptr, _i64, _ptr, _i64, _ptr, _ptr, _ptr, _ptr, _i64, _ptr, _int, _ptr]),
     "cw_ln_bwd_dx_close": (_int, [_i64, _i64, _ptr, _i64, _ptr, _i64, _ptr, _ptr, _ptr, _i64, _ptr, _i64, _ptr, _i64, _ptr,

@@ -652,7 +652,8 @@ template <typename T, int NCH, int NWAVES, int NR, bool FUSE_DX>
 __global__ __launch_bounds__(NWAVES * 64) void ln_bwd_partials_kernel(
     int64_t R, int64_t C, const T* __restrict__ dY, int64_t ld_dy, const T* __restrict__ x, int64_t ld_x,
     const float* __restrict__ mean_rstd, const T* __restrict__ gamma, float* __restrict__ row_sums,
-    float* __restrict__ col_ws, int want_cols, T* __restrict__ dx, int64_t ld_dx, float inv_h) {
+    float* __restrict__ col_ws, int want_cols, T* __restrict__ dx, int64_t ld_dx, float inv_h,
+    const T* __restrict__ dx_add, int64_t ld_add) {
     constexpr int V = elem<T>::kVec;
     extern __shared__ float lds_red[];
     const int lane = threadIdx.x & 63;
@@ -713,8 +714,15 @@ __global__ __launch_bounds__(NWAVES * 64) void ln_bwd_partials_kernel(
                         const float gg = gamma != nullptr ? dy[e] * g[e] : dy[e];
                         dy[e] = (gg - xh * c2 - c1) * rstd;
                     }
-                    if (row < R && chunk_valid<T>(j, lane, C))
+                    if (row < R && chunk_valid<T>(j, lane, C)) {
+                        if (FUSE_DX && dx_add != nullptr) {  // the gradient arriving along the residual branch
+                            float av[V];
+                            unpack_raw(load_raw_stream(dx_add + row * ld_add + ((int64_t)j * 64 + lane) * V), av, (const T*)nullptr);
+#pragma unroll
+                            for (int e = 0; e < V; ++e) dy[e] += av[e];
+                        }
                         store_raw_stream(dx + row * ld_dx + ((int64_t)j * 64 + lane) * V, pack_raw(dy, (const T*)nullptr));
+                    }
                 }
             }
         }
@@ -741,7 +749,8 @@ template <typename T, int NCH, int MAXW, bool FUSE_DX>
 __global__ __launch_bounds__(MAXW * 64, 4) void ln_bwd_split_kernel(
     int64_t R, int64_t C, const T* __restrict__ dY, int64_t ld_dy, const T* __restrict__ x, int64_t ld_x,
     const float* __restrict__ mean_rstd, const T* __restrict__ gamma, float* __restrict__ row_sums,
-    float* __restrict__ col_ws, int want_cols, T* __restrict__ dx, int64_t ld_dx, float inv_h, int wpr) {
+    float* __restrict__ col_ws, int want_cols, T* __restrict__ dx, int64_t ld_dx, float inv_h, int wpr,
+    const T* __restrict__ dx_add, int64_t ld_add) {
     constexpr int V = elem<T>::kVec;
     constexpr int kSeg = NCH * 64 * V;
     constexpr int NA = NCH * V;  // accumulators of one set (dgamma or dbeta) in a lane
@@ -759,6 +768,7 @@ __global__ __launch_bounds__(MAXW * 64, 4) void ln_bwd_split_kernel(
     x += col0;
     if (gamma != nullptr) gamma += col0;
     if (FUSE_DX) dx += col0;
+    if (FUSE_DX && dx_add != nullptr) dx_add += col0;
 
     raw16_t g_raw[NCH];
     load_param_chunks<T, NCH>(gamma, Cs, lane, g_raw);
@@ -834,8 +844,15 @@ __global__ __launch_bounds__(MAXW * 64, 4) void ln_bwd_split_kernel(
                     const float gg = gamma != nullptr ? dy[e] * g[e] : dy[e];
                     dy[e] = (gg - xh * c2 - c1) * rstd;
                 }
-                if (live && chunk_valid<T>(j, lane, Cs))
+                if (live && chunk_valid<T>(j, lane, Cs)) {
+                    if (dx_add != nullptr) {  // the gradient arriving along the residual branch
+                        float av[V];
+                        unpack_raw(load_raw_stream(dx_add + row * ld_add + ((int64_t)j * 64 + lane) * V), av, (const T*)nullptr);
+#pragma unroll
+                        for (int e = 0; e < V; ++e) dy[e] += av[e];
+                    }
                     store_raw_stream(dx + row * ld_dx + ((int64_t)j * 64 + lane) * V, pack_raw(dy, (const T*)nullptr));
+                }
             }
         }
         if (more) {
@@ -1106,6 +1123,13 @@ int normalize_impl(int64_t R, int64_t C, const void* x, int64_t ld, const float*
     return check_launch("ln_normalize_kernel");
 }
 
+// The gradient that reaches x along a residual branch, added to dx by the kernels that write dx from the row they
+// hold (p == nullptr: none).
+struct DxAdd {
+    const void* p = nullptr;
+    int64_t ld = 0;
+};
+
 // Number of blocks (= column partials) of the vector backward kernel.
 int64_t bwd_blocks(int64_t R, int nwaves) {
     int64_t nb = (R + nwaves - 1) / nwaves;
@@ -1117,7 +1141,7 @@ int64_t bwd_blocks(int64_t R, int nwaves) {
 template <typename T, int NCH, int NWAVES, int NR, bool FUSE_DX>
 int bwd_partials_launch_as(int64_t R, int64_t C, const void* dY, int64_t ld_dy, const void* x, int64_t ld_x,
                            const float* mean_rstd, const void* gamma, float* row_sums, float* ws, int want_cols,
-                           void* dx, int64_t ld_dx, hipStream_t s) {
+                           void* dx, int64_t ld_dx, hipStream_t s, DxAdd add = {}) {
     constexpr int V = elem<T>::kVec;
     const int64_t nb = bwd_blocks(R, NWAVES * NR);
     const size_t lds = flat_reduce_lds_bytes(2 * NCH * V, NWAVES);
@@ -1126,17 +1150,18 @@ int bwd_partials_launch_as(int64_t R, int64_t C, const void* dY, int64_t ld_dy, 
         if (const int lrc = ensure_dynamic_lds((const void*)kern, (int)((int)lds), "ln_bwd_partials"); lrc != CW_OK) return lrc;
     }
     hipLaunchKernelGGL(kern, dim3((unsigned)nb), dim3(NWAVES * 64), lds, s, R, C, (const T*)dY, ld_dy, (const T*)x,
-                       ld_x, mean_rstd, (const T*)gamma, row_sums, ws, want_cols, (T*)dx, ld_dx, 1.0f / (float)C);
+                       ld_x, mean_rstd, (const T*)gamma, row_sums, ws, want_cols, (T*)dx, ld_dx, 1.0f / (float)C,
+                       (const T*)add.p, add.ld);
     return check_launch("ln_bwd_partials_kernel");
 }
 
 template <typename T, int NCH, int NWAVES, int NR>
 int bwd_partials_launch(int64_t R, int64_t C, const void* dY, int64_t ld_dy, const void* x, int64_t ld_x,
                         const float* mean_rstd, const void* gamma, float* row_sums, float* ws, int want_cols,
-                        void* dx, int64_t ld_dx, hipStream_t s) {
+                        void* dx, int64_t ld_dx, hipStream_t s, DxAdd add = {}) {
     if (dx != nullptr)
         return bwd_partials_launch_as<T, NCH, NWAVES, NR, true>(R, C, dY, ld_dy, x, ld_x, mean_rstd, gamma, row_sums, ws,
-                                                                want_cols, dx, ld_dx, s);
+                                                                want_cols, dx, ld_dx, s, add);
     return bwd_partials_launch_as<T, NCH, NWAVES, NR, false>(R, C, dY, ld_dy, x, ld_x, mean_rstd, gamma, row_sums, ws,
                                                              want_cols, nullptr, 0, s);
 }
@@ -1181,23 +1206,24 @@ SplitShape split_shape(int64_t R, int64_t nch, int chunks) {
 template <typename T, int NCH, int MAXW, bool FUSE_DX>
 int bwd_split_launch_as(const SplitShape& sh, int64_t R, int64_t C, const void* dY, int64_t ld_dy, const void* x,
                         int64_t ld_x, const float* mean_rstd, const void* gamma, float* row_sums, float* ws,
-                        int want_cols, void* dx, int64_t ld_dx, hipStream_t s) {
+                        int want_cols, void* dx, int64_t ld_dx, hipStream_t s, DxAdd add = {}) {
     constexpr int V = elem<T>::kVec;
     const size_t lds = sh.nrg > 1 ? (size_t)sh.wpr * NCH * V * 64 * sizeof(float) : 0;
     hipLaunchKernelGGL((ln_bwd_split_kernel<T, NCH, MAXW, FUSE_DX>), dim3((unsigned)sh.blocks),
                        dim3(sh.wpr * sh.nrg * 64), lds, s, R, C, (const T*)dY, ld_dy, (const T*)x, ld_x, mean_rstd,
-                       (const T*)gamma, row_sums, ws, want_cols, (T*)dx, ld_dx, 1.0f / (float)C, sh.wpr);
+                       (const T*)gamma, row_sums, ws, want_cols, (T*)dx, ld_dx, 1.0f / (float)C, sh.wpr,
+                       (const T*)(FUSE_DX ? add.p : nullptr), add.ld);
     return check_launch("ln_bwd_split_kernel");
 }
 
 template <typename T>
 int bwd_split_launch(const SplitShape& sh, int64_t R, int64_t C, const void* dY, int64_t ld_dy, const void* x,
                      int64_t ld_x, const float* mean_rstd, const void* gamma, float* row_sums, float* ws,
-                     int want_cols, void* dx, int64_t ld_dx, hipStream_t s) {
+                     int want_cols, void* dx, int64_t ld_dx, hipStream_t s, DxAdd add = {}) {
     const bool wide = sh.wpr * sh.nrg > kSplitBlockWaves;
 #define CW_SPLIT(NCH, MAXW, FUSE)                                                                               \
     bwd_split_launch_as<T, NCH, MAXW, FUSE>(sh, R, C, dY, ld_dy, x, ld_x, mean_rstd, gamma, row_sums, ws, want_cols, \
-                                            dx, ld_dx, s)
+                                            dx, ld_dx, s, add)
     if constexpr (sizeof(T) == 4) {
         // three or four chunks: only rows that need more than eight such wavefronts, in one row group
         if (sh.chunks == 3) return dx != nullptr ? CW_SPLIT(3, 16, true) : CW_SPLIT(3, 16, false);
@@ -1216,14 +1242,14 @@ template <typename T>
 int bwd_partials_impl(int64_t R, int64_t C, const void* dY, int64_t ld_dy, const void* x, int64_t ld_x,
                       const float* mean_rstd, const void* gamma, float* row_sums, void* dgamma, void* dbeta,
                       int param_dtype, void* workspace, int64_t workspace_bytes, hipStream_t s, void* dx = nullptr,
-                      int64_t ld_dx = 0, bool* dx_done = nullptr, int64_t* open_parts = nullptr) {
+                      int64_t ld_dx = 0, bool* dx_done = nullptr, int64_t* open_parts = nullptr, DxAdd add = {}) {
     // open_parts: the column partials are left in the workspace, their count is reported, and whoever launches next
     // on the stream adds them up (bwd_dx_impl with a FinishCols)
     constexpr int V = elem<T>::kVec;
     if (dx_done != nullptr) *dx_done = false;
     const int want_cols = (dgamma != nullptr || dbeta != nullptr || open_parts != nullptr) ? 1 : 0;
     const bool vec = rows_vec_ok<T>(dY, ld_dy) && rows_vec_ok<T>(x, ld_x) && (gamma == nullptr || aligned16(gamma)) &&
-                     (C % V) == 0;
+                     (C % V) == 0 && (add.p == nullptr || rows_vec_ok<T>(add.p, add.ld));
     const int64_t nch = (C + 64 * V - 1) / (64 * V);
     int64_t nparts = 0;
     int rc;
@@ -1234,7 +1260,7 @@ int bwd_partials_impl(int64_t R, int64_t C, const void* dY, int64_t ld_dy, const
             return fail(CW_ERR_INVALID, "cw_ln_bwd_partials: workspace too small (%lld bytes)", (long long)workspace_bytes);
         void* fdx = (dx != nullptr && rows_vec_ok<T>(dx, ld_dx)) ? dx : nullptr;
         rc = bwd_split_launch<T>(sh, R, C, dY, ld_dy, x, ld_x, mean_rstd, gamma, row_sums, (float*)workspace, want_cols,
-                                 fdx, ld_dx, s);
+                                 fdx, ld_dx, s, add);
         if (rc != CW_OK) return rc;
         if (dx_done != nullptr) *dx_done = fdx != nullptr;
     } else if (vec && nch <= 8) {
@@ -1245,13 +1271,13 @@ int bwd_partials_impl(int64_t R, int64_t C, const void* dY, int64_t ld_dy, const
         float* ws = (float*)workspace;
         void* fdx = (dx != nullptr && rows_vec_ok<T>(dx, ld_dx)) ? dx : nullptr;
         if (nch <= 1)
-            rc = bwd_partials_launch<T, 1, 16, 2>(R, C, dY, ld_dy, x, ld_x, mean_rstd, gamma, row_sums, ws, want_cols, fdx, ld_dx, s);
+            rc = bwd_partials_launch<T, 1, 16, 2>(R, C, dY, ld_dy, x, ld_x, mean_rstd, gamma, row_sums, ws, want_cols, fdx, ld_dx, s, add);
         else if (nch <= 2)
-            rc = bwd_partials_launch<T, 2, 16, 1>(R, C, dY, ld_dy, x, ld_x, mean_rstd, gamma, row_sums, ws, want_cols, fdx, ld_dx, s);
+            rc = bwd_partials_launch<T, 2, 16, 1>(R, C, dY, ld_dy, x, ld_x, mean_rstd, gamma, row_sums, ws, want_cols, fdx, ld_dx, s, add);
         else if (nch <= 4)
-            rc = bwd_partials_launch<T, 4, 8, 1>(R, C, dY, ld_dy, x, ld_x, mean_rstd, gamma, row_sums, ws, want_cols, fdx, ld_dx, s);
+            rc = bwd_partials_launch<T, 4, 8, 1>(R, C, dY, ld_dy, x, ld_x, mean_rstd, gamma, row_sums, ws, want_cols, fdx, ld_dx, s, add);
         else
-            rc = bwd_partials_launch<T, 8, 4, 1>(R, C, dY, ld_dy, x, ld_x, mean_rstd, gamma, row_sums, ws, want_cols, fdx, ld_dx, s);
+            rc = bwd_partials_launch<T, 8, 4, 1>(R, C, dY, ld_dy, x, ld_x, mean_rstd, gamma, row_sums, ws, want_cols, fdx, ld_dx, s, add);
         if (rc != CW_OK) return rc;
         if (dx_done != nullptr) *dx_done = fdx != nullptr;
     } else {
@@ -1413,10 +1439,22 @@ template <typename T>
 int backward_fused_impl(int64_t R, int64_t C, const void* dY, int64_t ld_dy, const void* x, int64_t ld_x,
                         const float* mean_rstd, const void* gamma, float* row_sums, void* dx, int64_t ld_dx,
                         void* dgamma, void* dbeta, int param_dtype, void* workspace, int64_t workspace_bytes,
-                        hipStream_t s) {
+                        hipStream_t s, DxAdd add) {
+    // the residual gradient rides only the kernels that write dx from the row they hold: shapes that take the
+    // two-kernel path are refused before anything is launched (the caller adds it itself)
+    if (add.p != nullptr) {
+        constexpr int V = elem<T>::kVec;
+        const int64_t nch = (C + 64 * V - 1) / (64 * V);
+        const bool one_pass = rows_vec_ok<T>(dY, ld_dy) && rows_vec_ok<T>(x, ld_x) && rows_vec_ok<T>(dx, ld_dx) &&
+                              rows_vec_ok<T>(add.p, add.ld) && (gamma == nullptr || aligned16(gamma)) && (C % V) == 0 &&
+                              (split_chunks<T>(nch) != 0 || nch <= 8);
+        if (!one_pass)
+            return fail(CW_ERR_UNSUPPORTED, "cw_ln_backward_fused: dx_addend is taken by the one-pass kernels only (16-byte "
+                                            "aligned rows, C a multiple of the 16-byte vector, rows within their width)");
+    }
     bool dx_done = false;
     int rc = bwd_partials_impl<T>(R, C, dY, ld_dy, x, ld_x, mean_rstd, gamma, row_sums, dgamma, dbeta, param_dtype,
-                                  workspace, workspace_bytes, s, dx, ld_dx, &dx_done);
+                                  workspace, workspace_bytes, s, dx, ld_dx, &dx_done, nullptr, add);
     if (rc != CW_OK || dx_done) return rc;
     return bwd_dx_impl<T>(R, C, dY, ld_dy, x, ld_x, mean_rstd, gamma, row_sums, C, dx, ld_dx, s);
 }
@@ -1425,10 +1463,13 @@ int backward_fused_impl(int64_t R, int64_t C, const void* dY, int64_t ld_dy, con
 
 extern "C" int cw_ln_backward_fused(int64_t R, int64_t C, const void* dY, int64_t ld_dy, const void* x, int64_t ld_x,
                                     const float* mean_rstd, const void* gamma, float* row_sums, void* dx,
-                                    int64_t ld_dx, void* dgamma, void* dbeta, int param_dtype, void* workspace,
-                                    int64_t workspace_bytes, int io_dtype, void* stream) {
+                                    int64_t ld_dx, const void* dx_addend, int64_t ld_add, void* dgamma, void* dbeta,
+                                    int param_dtype, void* workspace, int64_t workspace_bytes, int io_dtype,
+                                    void* stream) {
     int rc = check_rc("cw_ln_backward_fused", R, C, io_dtype);
     if (rc != CW_OK) return rc;
+    if (dx_addend != nullptr && ld_add < C)
+        return fail(CW_ERR_INVALID, "cw_ln_backward_fused: ld_add < C");
     if (dgamma != nullptr && !col_out_dtype_ok(param_dtype))
         return fail(CW_ERR_INVALID, "cw_ln_backward_fused: bad param_dtype %d", param_dtype);
     if ((dgamma == nullptr) != (dbeta == nullptr))
@@ -1440,10 +1481,13 @@ extern "C" int cw_ln_backward_fused(int64_t R, int64_t C, const void* dY, int64_
     if (dgamma != nullptr && workspace == nullptr) return fail(CW_ERR_INVALID, "cw_ln_backward_fused: workspace is NULL");
     if (const int drc = require_gfx950("cw_ln_backward_fused"); drc != CW_OK) return drc;
     hipStream_t s = (hipStream_t)stream;
+    DxAdd add;
+    add.p = R > 0 ? dx_addend : nullptr;
+    add.ld = ld_add;
     return with_elem_type(io_dtype, [&](auto* tag) {
         return backward_fused_impl<std::remove_pointer_t<decltype(tag)>>(R, C, dY, ld_dy, x, ld_x, mean_rstd, gamma, row_sums,
                                                                          dx, ld_dx, dgamma, dbeta, param_dtype,
-                                                                         workspace, workspace_bytes, s);
+                                                                         workspace, workspace_bytes, s, add);
     });
 }
 

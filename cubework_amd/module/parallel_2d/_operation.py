@@ -205,7 +205,7 @@ class _Layernorm2D(torch.autograd.Function):
 
     @staticmethod
     @fp32_fwd()
-    def forward(ctx, input_, weight, bias, hidden_size, eps, row_parallel_mode, col_parallel_mode):
+    def forward(ctx, input_, weight, bias, hidden_size, eps, row_parallel_mode, col_parallel_mode, fork_residual=False):
         gamma = all_gather(weight, -1, col_parallel_mode)
         beta = all_gather(bias, -1, col_parallel_mode)
         if row_parallel_mode.world_size == 1:
@@ -215,32 +215,42 @@ class _Layernorm2D(torch.autograd.Function):
             out, mean_rstd = ops.ln_normalize(input_, stats, hidden_size, eps, gamma, beta, mode=CW_LN_ONE_PASS)
         ctx.save_for_backward(input_, gamma, mean_rstd)
         ctx.meta = (hidden_size, row_parallel_mode, col_parallel_mode, weight.dtype, bias.dtype)
+        if fork_residual:
+            # the input goes out again beside the result, for the residual branch around the layers that follow:
+            # the gradients of the two branches then meet in this operator's backward, where the kernel that writes
+            # dx adds the residual branch's in the same pass, instead of in an accumulation pass of autograd
+            return out, input_.view_as(input_)
         return out
 
     @staticmethod
     @bwd()
-    def backward(ctx, output_grad):
+    def backward(ctx, output_grad, residual_grad=None):
         x, gamma, mean_rstd = ctx.saved_tensors
         hidden_size, row_mode, col_mode, w_dtype, b_dtype = ctx.meta
         # dgamma / dbeta: fp32 sums, stored in the parameters' dtype at once where no reduce-scatter follows
         pd = w_dtype if col_mode.world_size == 1 and w_dtype == b_dtype else None
         with torch.no_grad():
             if row_mode.world_size == 1:
-                input_grad, dgamma, dbeta = ops.ln_backward_fused(output_grad, x, mean_rstd, gamma, param_dtype=pd)
+                input_grad, dgamma, dbeta = ops.ln_backward_fused(output_grad, x, mean_rstd, gamma, param_dtype=pd,
+                                                                  dx_addend=residual_grad)
+                residual_grad = None
             else:
                 # the dx launch also finishes the column sums that the first launch leaves as partial rows
                 row_sums, pending = ops.ln_bwd_partials_open(output_grad, x, mean_rstd, gamma)
                 row_sums = all_reduce(row_sums, row_mode)
                 input_grad, dgamma, dbeta = ops.ln_bwd_dx_close(output_grad, x, mean_rstd, row_sums, hidden_size, pending,
                                                                 gamma, param_dtype=pd)
+            if residual_grad is not None:
+                input_grad = input_grad + residual_grad
             weight_grad = reduce_scatter(dgamma, -1, col_mode).to(w_dtype)
             bias_grad = reduce_scatter(dbeta, -1, col_mode).to(b_dtype)
-        return input_grad, weight_grad, bias_grad, None, None, None, None
+        return input_grad, weight_grad, bias_grad, None, None, None, None, None
 
 
 def layernorm_2d(input_: Tensor, weight: Tensor, bias: Tensor, hidden_size: int, eps: float,
-                 row_parallel_mode: ParallelMode, col_parallel_mode: ParallelMode) -> Tensor:
-    return _Layernorm2D.apply(input_, weight, bias, hidden_size, eps, row_parallel_mode, col_parallel_mode)
+                 row_parallel_mode: ParallelMode, col_parallel_mode: ParallelMode, fork_residual: bool = False):
+    """fork_residual (additive option, default off): returns (normalised, input) - see _Layernorm2D.forward."""
+    return _Layernorm2D.apply(input_, weight, bias, hidden_size, eps, row_parallel_mode, col_parallel_mode, fork_residual)
 
 
 class _Classifier2D(torch.autograd.Function):

@@ -101,9 +101,12 @@ class LayerNorm2D(nn.Module):
         set_tensor_parallel_attribute_by_partition(self.weight, self.summa_dim ** 2)
         set_tensor_parallel_attribute_by_partition(self.bias, self.summa_dim ** 2)
 
-    def forward(self, x: Tensor) -> Tensor:
+    def forward(self, x: Tensor, fork_residual: bool = False):
+        """fork_residual (additive option, default off): returns (normalised x, x) for a pre-LayerNorm block whose
+        residual branch starts at this layer's input (benchmark/opt/opt.py:170-174, 193-197): take the residual from
+        the second result, and the gradients of both branches are summed inside this layer's backward kernel."""
         return layernorm_2d(x, self.weight, self.bias, self.normalized_shape, self.variance_epsilon,
-                            pm.PARALLEL_2D_ROW, pm.PARALLEL_2D_COL)
+                            pm.PARALLEL_2D_ROW, pm.PARALLEL_2D_COL, fork_residual)
 
 
 class Classifier2D(nn.Module):

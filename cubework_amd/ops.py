@@ -367,10 +367,11 @@ def ln_bwd_dx_close(dy: torch.Tensor, x: torch.Tensor, mean_rstd: torch.Tensor, 
 
 def ln_backward_fused(dy: torch.Tensor, x: torch.Tensor, mean_rstd: torch.Tensor,
                       gamma: Optional[torch.Tensor] = None, want_param_grads: bool = True,
-                      param_dtype: Optional[torch.dtype] = None):
+                      param_dtype: Optional[torch.dtype] = None, dx_addend: Optional[torch.Tensor] = None):
     """Backward of LayerNorm over rows this rank holds whole: (dx, dgamma [C] or None, dbeta [C] or None) in
     one pass over dy and x; the parameter gradients are fp32 sums stored as param_dtype (default float32).
-    See cw_ln_backward_fused."""
+    dx_addend: the gradient reaching x along a residual branch, added to dx in the same pass where the kernel
+    offers it (else by a separate addition here). See cw_ln_backward_fused."""
     lib = _lib.load()
     shape = x.shape
     dy, x = _rows(dy), _rows(x)
@@ -387,9 +388,24 @@ def ln_backward_fused(dy: torch.Tensor, x: torch.Tensor, mean_rstd: torch.Tensor
         dgamma = torch.empty(C, dtype=param_dtype, device=x.device)
         dbeta = torch.empty(C, dtype=param_dtype, device=x.device)
         ws = _workspace(R, C, x.device)
-    rc = lib.cw_ln_backward_fused(R, C, _p(dy), _ld(dy), _p(x), _ld(x), _p(mean_rstd), _p(gamma), _p(row_sums), _p(dx),
-                                  _ld(dx), _p(dgamma), _p(dbeta), _TORCH_CODE[param_dtype], _p(ws),
-                                  ws.numel() if ws is not None else 0, _dtype_code(x), _stream())
+    add = None
+    if dx_addend is not None:
+        add = _rows(dx_addend)
+        if add.shape != x.shape or add.dtype != x.dtype:
+            raise ValueError("dx_addend must agree with x in shape and dtype")
+        _require_device(add)
+
+    def call(a):
+        return lib.cw_ln_backward_fused(R, C, _p(dy), _ld(dy), _p(x), _ld(x), _p(mean_rstd), _p(gamma), _p(row_sums), _p(dx),
+                                        _ld(dx), _p(a), _ld(a) if a is not None else 0, _p(dgamma), _p(dbeta),
+                                        _TORCH_CODE[param_dtype], _p(ws), ws.numel() if ws is not None else 0,
+                                        _dtype_code(x), _stream())
+    rc = call(add)
+    if rc == _lib.CW_ERR_UNSUPPORTED and add is not None:   # a shape of the two-kernel path: add separately
+        rc = call(None)
+        _lib.check(rc, "cw_ln_backward_fused")
+        dx = dx + add
+        return dx.reshape(shape), dgamma, dbeta
     _lib.check(rc, "cw_ln_backward_fused")
     return dx.reshape(shape), dgamma, dbeta
 

@@ -19,7 +19,7 @@ import torch.nn.functional as F
 
 from . import module as cube_nn
 from . import ops
-from .module.parallel_2d import Linear2D
+from .module.parallel_2d import LayerNorm2D, Linear2D
 
 
 class OPTBlock(nn.Module):
@@ -52,16 +52,28 @@ class OPTBlock(nn.Module):
         """residual + layer(inp) (benchmark/opt/opt.py:184,206): in the GEMM's epilogue where the layer offers it
         (Linear2D's `residual` option), as a separate addition elsewhere."""
         inner = getattr(layer, "linear", layer)
-        if isinstance(inner, Linear2D) and inner.activation is None and not inner.skip_bias_add:
+        # not under autocast: the operator would cast the residual stream to the 16-bit type with its other inputs
+        if (isinstance(inner, Linear2D) and inner.activation is None and not inner.skip_bias_add
+                and residual.dtype == inp.dtype == inner.weight.dtype and not torch.is_autocast_enabled("cuda")):
             return layer(inp, residual=residual)
         return residual + layer(inp)
 
+    @staticmethod
+    def _norm_fork(layer, x: torch.Tensor):
+        """(layer(x), x for the residual branch): through LayerNorm2D's `fork_residual` option where the layer is
+        one, so that the two branches' gradients are added inside its backward kernel."""
+        inner = getattr(layer, "norm", layer)
+        if isinstance(inner, LayerNorm2D) and x.dtype == inner.weight.dtype and not torch.is_autocast_enabled("cuda"):
+            return layer(x, fork_residual=True)
+        return layer(x), x
+
     def forward(self, x: torch.Tensor) -> torch.Tensor:
-        h = self.self_attn_layer_norm(x)
+        h, x = self._norm_fork(self.self_attn_layer_norm, x)
         x = self._linear_plus(self.out_proj, self._attention_core(self.qkv_proj(h)), x)
         shape = x.shape
         r = x.reshape(-1, shape[-1])
-        h = self.fc1(self.final_layer_norm(r))
+        h, r = self._norm_fork(self.final_layer_norm, r)
+        h = self.fc1(h)
         if not self.fuse_activation:
             h = _ACT[self.activation](h)
         return self._linear_plus(self.fc2, h, r).view(shape)

@@ -277,10 +277,15 @@ int cw_ln_bwd_dx_close(int64_t R, int64_t C, const void* dY, int64_t ld_dy, cons
  * _Layernorm3D.backward (parallel_3d/_operation.py:294-311) compute when the group their sums are
  * all-reduced over has one member. The counterpart of cw_ln_forward_fused. row_sums ([R,2] fp32) is
  * written as by cw_ln_bwd_partials; shapes the one-pass kernel does not take run the two kernels.
+ * dx_addend (may be NULL; [R,C] of the io dtype, leading dimension ld_add): the gradient that reaches x along
+ * a residual branch around the layer (benchmark/opt/opt.py:170,184 and :193,206), added to dx before its one
+ * rounding: what autograd's accumulation of the two branches computes with a pass of its own. Taken by the
+ * one-pass kernels only; a shape that runs the two kernels is refused with CW_ERR_UNSUPPORTED before any launch.
  */
 int cw_ln_backward_fused(int64_t R, int64_t C, const void* dY, int64_t ld_dy,
                          const void* x, int64_t ld_x, const float* mean_rstd, const void* gamma,
-                         float* row_sums, void* dx, int64_t ld_dx, void* dgamma, void* dbeta, int param_dtype,
+                         float* row_sums, void* dx, int64_t ld_dx, const void* dx_addend, int64_t ld_add,
+                         void* dgamma, void* dbeta, int param_dtype,
                          void* workspace, int64_t workspace_bytes, int io_dtype, void* stream);
 
 /* ---- vocab-parallel cross-entropy -------------------------------------- */

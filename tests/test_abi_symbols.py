@@ -98,7 +98,7 @@ def test_scratch_sizes_and_refusals_of_the_later_entry_points():
     args[3], args[17] = 64, F32
     assert lib.cw_attn_fwd(*args) == -3
     # fused LayerNorm backward: the two column outputs come together
-    assert lib.cw_ln_backward_fused(4, 8, None, 8, None, 8, None, None, None, None, 8, None, C.c_void_p(16), F32, None, 0, BF16, None) == -1
+    assert lib.cw_ln_backward_fused(4, 8, None, 8, None, 8, None, None, None, None, 8, None, 0, None, C.c_void_p(16), F32, None, 0, BF16, None) == -1
     assert b"both" in lib.cw_last_error()
 
 

@@ -82,12 +82,15 @@ def test_opt_block_full_size_operator_by_operator(activation):
         mod = getattr(blk, n)
 
         def fwd(m, args, kwargs, out, n=n):
-            cap[n]["in"], cap[n]["out"] = args[0].detach(), out.detach()
+            # the LayerNorms are called with fork_residual=True: (normalised, input again for the residual branch)
+            cap[n]["in"], cap[n]["out"] = args[0].detach(), (out[0] if isinstance(out, tuple) else out).detach()
             res = kwargs.get("residual")   # out_proj and fc2 add the residual stream in their epilogue
             cap[n]["residual"] = None if res is None else res.detach()
 
         def bwd(m, gin, gout, n=n):
             cap[n]["d_in"], cap[n]["d_out"] = gin[0].detach(), gout[0].detach()
+            # a forked LayerNorm also receives the residual branch's gradient, which its kernel adds to dx
+            cap[n]["d_res"] = gout[1].detach() if len(gout) > 1 and gout[1] is not None else None
         hooks += [mod.register_forward_hook(fwd, with_kwargs=True), mod.register_full_backward_hook(bwd)]
     y = blk(x)
     y.backward(dy)
@@ -117,7 +120,8 @@ def test_opt_block_full_size_operator_by_operator(activation):
         ref = F.layer_norm(xr, (hidden,), gr, br, 1e-5)
         ref.backward(_rows(c["d_out"], rows))
         assert_parity(_rows(c["out"], rows), ref.detach(), BF, n + " forward rows")
-        assert_parity(_rows(c["d_in"], rows), xr.grad, BF, n + " dX rows")
+        assert c["d_res"] is not None, "the residual branch's gradient did not reach the LayerNorm's backward"
+        assert_parity(_rows(c["d_in"], rows), xr.grad + _rows(c["d_res"], rows), BF, n + " dX rows (+ residual branch)")
         xa = c["in"].detach().reshape(T, hidden).double().cpu()
         da = c["d_out"].detach().reshape(T, hidden).double().cpu()
         mu = xa.mean(-1, keepdim=True)

@@ -385,3 +385,58 @@ def test_partial_stats_into_a_result_buffer_that_is_only_8_byte_aligned():
         torch.cuda.synchronize()
         assert torch.equal(view.view(R, 2), want)
         assert torch.isnan(buf[:2]).all()
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32, torch.float16])
+@pytest.mark.parametrize("shape", [(64, 1024), (300, 2048), (33, 4096), (17, 200), (5, 1001), (70, 8192), (9, 12288)])
+def test_ln_backward_fused_with_the_residual_branch_gradient(shape, dtype):
+    """cw_ln_backward_fused with dx_addend: dx = LayerNorm backward + the gradient arriving along the residual
+    branch, rounded once (expected: the oracle's dx in float64 plus the addend); dgamma / dbeta / row sums are
+    the same bits as without it. Shapes cover the whole-row kernel, the split kernel for wide rows, and the
+    two-kernel path (ragged / unaligned rows), where the wrapper adds separately."""
+    import oracle
+    from cubework_amd import ops
+
+    R, C = shape
+    x, dy, gamma, _ = _inputs(R, C, dtype, 11)
+    add = randn((R, C), dtype, 15)
+    xd, dyd, gd, ad = (t.to(DEV) for t in (x, dy, gamma, add))
+    _, mr = ops.ln_forward_fused(xd, 1e-5, gd, None)
+    dx0, dg0, db0 = ops.ln_backward_fused(dyd, xd, mr, gd)
+    dx1, dg1, db1 = ops.ln_backward_fused(dyd, xd, mr, gd, dx_addend=ad)
+    assert torch.equal(dg0, dg1) and torch.equal(db0, db1)
+    with oracle.precision(torch.float64):
+        want, _, _ = oracle.ln_backward_full(dy, x, mr.cpu(), gamma)
+        want = want.double() + add.double()
+    assert_parity(dx1, _rounded(want, dtype), dtype, "fused backward + residual gradient %s" % (shape,))
+
+
+def test_layernorm2d_fork_residual_option():
+    """LayerNorm2D(x, fork_residual=True) returns (LN(x), x): a block y = x + f(LN(x)) built on it has the same
+    output and the same gradients as the plain composition, the sum of the two branches' gradients being formed
+    in the layer's backward kernel."""
+    from cubework_amd.distributed import initialize
+    from cubework_amd.module.parallel_2d import LayerNorm2D
+
+    initialize("2d", 1)
+    norm = LayerNorm2D(1024).to(torch.bfloat16).to(DEV)
+    with torch.no_grad():
+        norm.weight.copy_(rand_uniform((1024,), torch.bfloat16, 1, 0.9, 1.1))
+        norm.bias.copy_(randn((1024,), torch.bfloat16, 2, 0.02))
+    w = randn((1024, 1024), torch.bfloat16, 3, 0.03).to(DEV)
+    dy = randn((6, 50, 1024), torch.bfloat16, 4).to(DEV)
+    outs = []
+    for fork in (False, True):
+        x = randn((6, 50, 1024), torch.bfloat16, 5).to(DEV).requires_grad_(True)
+        norm.zero_grad(set_to_none=True)
+        if fork:
+            h, res = norm(x, fork_residual=True)
+        else:
+            h, res = norm(x), x
+        y = res + torch.tanh(h @ w)
+        y.backward(dy)
+        outs.append((y.detach(), x.grad, norm.weight.grad.clone(), norm.bias.grad.clone()))
+    assert torch.equal(outs[0][0], outs[1][0])
+    assert torch.equal(outs[0][2], outs[1][2]) and torch.equal(outs[0][3], outs[1][3])
+    # one rounding instead of two: equal up to a bf16 step
+    assert_parity(outs[1][1], outs[0][1].double(), torch.bfloat16, "x.grad with the branches summed in the kernel")
