@@ -686,10 +686,23 @@ def bench_other_configs(device, sets):
     out["clip_grad_norm_block"] = {"us": round(us_clip, 2), "bytes": 3 * grad_bytes, "tensors": len(params),
                                    "GBps": round(3 * grad_bytes / us_clip / 1e3, 1),
                                    "frac": round(3 * grad_bytes / us_clip / 1e3 / HBM_PEAK_GBPS, 3)}
+    # the same step with the residual additions as separate passes (torch's add after out_proj / fc2, autograd's
+    # accumulation at the two LayerNorm forks) instead of the GEMM epilogue / LayerNorm backward kernel: same process,
+    # right after the figure above
+    fused_plus, fused_fork = OPTBlock.__dict__["_linear_plus"], OPTBlock.__dict__["_norm_fork"]
+    try:
+        OPTBlock._linear_plus = staticmethod(lambda layer, inp, residual: residual + layer(inp))
+        OPTBlock._norm_fork = staticmethod(lambda layer, x_: (layer(x_), x_))
+        us_plain = event_time_us(block_step, 10, 3)
+    finally:
+        OPTBlock._linear_plus, OPTBlock._norm_fork = fused_plus, fused_fork
+    us_again = event_time_us(block_step, 10, 3)
     lin_flop = 3 * 2.0 * 8192 * 2048 * (6144 + 2048 + 8192 + 8192)
     out["opt_block_fwd_bwd"] = {"ms": round(us / 1e3, 3), "linear_flop": lin_flop,
                                 "linear_TFLOPs_if_all_time_were_linears": round(lin_flop / us / 1e6, 1),
                                 "note": "four Linear2D, two LayerNorm2D and the fused attention core (cw_attn_fwd / cw_attn_bwd), tp=1",
+                                "same_run_ab": {"residual_additions_as_separate_passes_ms": round(us_plain / 1e3, 3),
+                                                "in_epilogue_and_ln_backward_again_ms": round(us_again / 1e3, 3)},
                                 "per_kernel": per_kernel,
                                 "per_kernel_source": "events around every C-ABI call during %d instrumented passes of the same "
                                                      "step in this run; the last row is the step's time minus their sum" % passes}
