@@ -848,7 +848,8 @@ def mfma_rate_ceiling(device, seconds=0.4):
     sink = torch.empty(65536, dtype=torch.float32, device=device)
     stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
     out = {}
-    for name, mode in (("random_operands", 0), ("zero_operands", 1), ("random_operands_read_from_lds", 2)):
+    for name, mode in (("random_operands", 0), ("zero_operands", 1), ("random_operands_read_from_lds", 2),
+                       ("random_operands_16x16x32_instruction", 3)):
         def call():
             rc = lib.cw_diag_mfma_rate(iters, mode, sink.data_ptr(), stream)
             if rc != 0:
@@ -863,7 +864,8 @@ def mfma_rate_ceiling(device, seconds=0.4):
                 gm["pJ_per_FLOP"] = round(gm["socket_power_W_from_energy_counter"] / (flop / us / 1e6), 4)
     out["note"] = ("register-only loop of v_mfma_f32_32x32x16_bf16 on all 1024 SIMDs: what the board's power management "
                    "leaves of the data-sheet rate for operands that toggle like the workload's; read_from_lds: the same "
-                   "loop with the ring kernel's fragment reads from LDS (8 KB per 16 MFMAs), no global loads")
+                   "loop with the ring kernel's fragment reads from LDS (8 KB per 16 MFMAs), no global loads; "
+                   "16x16x32_instruction: the register-only loop with the other bf16 matrix instruction, same FLOP per trip")
     return out
 
 

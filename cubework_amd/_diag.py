@@ -3,7 +3,8 @@ csrc/diag.hip and csrc/diag_gemm.hip. Not part of the product: nothing under cub
 it, the operators never call it, and libcubework_hip.so exports none of its symbols.
 
   cw_diag_mfma_rate(iters, mode, sink, stream)   the GEMM's matrix instruction back to back from registers
-                                                 (mode 0 random operands, 1 zeros, 2 random operands read from LDS)
+                                                 (mode 0 random operands, 1 zeros, 2 random operands read from LDS,
+                                                 3 random operands, the 16 x 16 x 32 instruction)
   cw_diag_mfma_rate_flop(iters)                  FLOP of one such call
   cw_diag_gemm_part(part, M, N, K, n_steps, A_steps, lda, B_steps, ldb, bias, C, ldc, stream)
                                                  the ring kernel of the block GEMM (NN, bf16, bias + GeLU-tanh) whole

@@ -7,7 +7,7 @@
 // LDS traffic of the ring kernel's k loop: 8 KB per wavefront and 16 MFMAs. The result says what the power
 // management of the board leaves of the 2516.6 TFLOP/s that the data sheet quotes at 2.4 GHz, for operands that
 // toggle like the workload's, and what it leaves a kernel that also has to fetch them from LDS; bench.py reports
-// both beside the GEMM kernel's own rate.
+// both beside the GEMM kernel's own rate. Mode 3 is the register-only loop with the 16 x 16 x 32 instruction.
 #include "cw_common.h"
 #include "gemm_bf16_kernel.h"
 
@@ -111,23 +111,70 @@ __global__ __launch_bounds__(256) void mfma_rate_kernel(int iters, int zeros, fl
     if (sink != nullptr) sink[gid] = s;  // keeps the products alive
 }
 
+// The same FLOP per trip from the other bf16 matrix instruction, v_mfma_f32_16x16x32_bf16: 8 x 4 accumulator
+// tiles of 16 x 16 and 32 instructions per trip, random operands in registers. Says whether the choice of
+// instruction shape changes what the board sustains (time and energy per FLOP).
+__global__ __launch_bounds__(256) void mfma16_rate_kernel(int iters, float* __restrict__ sink) {
+    const uint32_t gid = blockIdx.x * 256u + threadIdx.x;
+    typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+    typedef float f32x4_t __attribute__((ext_vector_type(4)));
+    bf16x8_t a[8], b[4];
+#pragma unroll
+    for (int t = 0; t < 8; ++t) {
+        uint32_t w[4];
+#pragma unroll
+        for (int d = 0; d < 4; ++d) w[d] = random_bf16_pair(gid * 64u + t * 4u + d, 1.0f);
+        a[t] = __builtin_bit_cast(bf16x8_t, (u32x4){w[0], w[1], w[2], w[3]});
+    }
+#pragma unroll
+    for (int t = 0; t < 4; ++t) {
+        uint32_t w[4];
+#pragma unroll
+        for (int d = 0; d < 4; ++d) w[d] = random_bf16_pair(gid * 64u + 32u + t * 4u + d, 0.02f);
+        b[t] = __builtin_bit_cast(bf16x8_t, (u32x4){w[0], w[1], w[2], w[3]});
+    }
+    f32x4_t acc[8][4];
+#pragma unroll
+    for (int i = 0; i < 8; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) acc[i][j] = (f32x4_t){0.0f, 0.0f, 0.0f, 0.0f};
+    for (int it = 0; it < iters; ++it) {
+#pragma unroll
+        for (int i = 0; i < 8; ++i)
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const int js = (i & 1) ? 3 - j : j;
+                acc[i][js] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(b[js], a[i], acc[i][js], 0, 0, 0);
+            }
+    }
+    float s = 0.0f;
+#pragma unroll
+    for (int i = 0; i < 8; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+#pragma unroll
+            for (int e = 0; e < 4; ++e) s += acc[i][j][e];
+    if (sink != nullptr) sink[gid] = s;
+}
+
 }  // namespace
 }  // namespace cw
 
 using namespace cw;
 
 extern "C" int64_t cw_diag_mfma_rate_flop(int iters) {
-    // 1024 wavefronts x 16 instructions per trip x 32 x 32 x 16 x 2
+    // 1024 wavefronts x 16 instructions per trip x 32 x 32 x 16 x 2 (mode 3: 32 instructions x 16 x 16 x 32 x 2)
     return iters <= 0 ? 0 : (int64_t)iters * 1024 * 16 * 32768;
 }
 
 extern "C" int cw_diag_mfma_rate(int iters, int mode, float* sink, void* stream) {
-    if (mode < 0 || mode > 2) return fail(CW_ERR_INVALID, "cw_diag_mfma_rate: mode %d outside [0, 2]", mode);
+    if (mode < 0 || mode > 3) return fail(CW_ERR_INVALID, "cw_diag_mfma_rate: mode %d outside [0, 3]", mode);
     if (iters <= 0 || iters > (1 << 24)) return fail(CW_ERR_INVALID, "cw_diag_mfma_rate: iters=%d outside [1, 2^24]", iters);
     if (const int drc = require_gfx950("cw_diag_mfma_rate"); drc != CW_OK) return drc;
     hipStream_t s = (hipStream_t)stream;
     // one workgroup of four wavefronts per compute unit, one wavefront per SIMD: 256 x 256 threads
-    if (mode == 2) hipLaunchKernelGGL(mfma_rate_kernel<true>, dim3(256), dim3(256), 0, s, iters, 0, sink);
+    if (mode == 3) hipLaunchKernelGGL(mfma16_rate_kernel, dim3(256), dim3(256), 0, s, iters, sink);
+    else if (mode == 2) hipLaunchKernelGGL(mfma_rate_kernel<true>, dim3(256), dim3(256), 0, s, iters, 0, sink);
     else hipLaunchKernelGGL(mfma_rate_kernel<false>, dim3(256), dim3(256), 0, s, iters, mode, sink);
     return check_launch("mfma_rate_kernel");
 }

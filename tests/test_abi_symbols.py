@@ -137,7 +137,7 @@ def test_measurement_library_is_separate_from_the_boundary():
             assert not hasattr(product, name), name
     diag = _diag.load()
     assert diag.cw_diag_mfma_rate(0, 0, None, None) == -1
-    assert diag.cw_diag_mfma_rate(10, 3, None, None) == -1
+    assert diag.cw_diag_mfma_rate(10, 4, None, None) == -1
     assert b"mode" in diag.cw_last_error()
     assert diag.cw_diag_mfma_rate_flop(2) == 2 * 1024 * 16 * 32768
     assert diag.cw_diag_gemm_part(7, 8192, 2048, 2048, 2, None, 2048, None, 2048, None, None, 2048, None) == -1
