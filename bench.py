@@ -869,6 +869,84 @@ def mfma_rate_ceiling(device, seconds=0.4):
     return out
 
 
+def hw_probes(device):
+    """Two facts about the hardware that the attention kernels are priced against. (1) A SIMD with two wavefronts, one
+    issuing 4 independent 32x32x16 MFMAs per trip (128 cycles of the matrix pipe), the other 32 vector instructions
+    per trip (v_fma_f32, or the transcendental v_exp_f32): time of each alone and of both together. (2) The rate at
+    which a compute unit reads LDS with ds_read_b128 and with ds_read_b64_tr_b16 (8 wavefronts, no bank conflicts)."""
+    import ctypes
+    import torch
+    from cubework_amd import _diag
+    lib = _diag.load()
+    stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+    sink = torch.empty(256 * 512, dtype=torch.float32, device=device)
+    isink = torch.empty(256 * 512, dtype=torch.int32, device=device)
+    iters = 20000
+    out = {"matrix_and_vector_instructions_of_two_wavefronts_on_one_simd": {}, "lds_read_rate_per_compute_unit": {}}
+
+    def check(rc):
+        if rc != 0:
+            raise RuntimeError(lib.cw_last_error().decode())
+    for vop, name in ((0, "v_fma_f32"), (1, "v_exp_f32")):
+        t = {}
+        for roles, key in ((1, "mfma_only"), (2, "vector_only"), (3, "both")):
+            us = event_time_us(lambda: check(lib.cw_diag_overlap(iters, roles, vop, sink.data_ptr(), stream)), 10, 3, min_ms=300)
+            t[key] = us / iters * 1e3  # ns per trip
+        row = {"ns_per_trip_" + k: round(v, 2) for k, v in t.items()}
+        # both = vector_only + x * mfma_only: x = 0 would be complete overlap, 1 none
+        row["share_of_the_mfma_time_not_hidden_under_the_vector_wavefront"] = round((t["both"] - t["vector_only"]) / t["mfma_only"], 3)
+        row["vector_ns_per_instruction_alone"] = round(t["vector_only"] / 32, 3)
+        row["mfma_ns_per_instruction_alone"] = round(t["mfma_only"] / 4, 3)
+        out["matrix_and_vector_instructions_of_two_wavefronts_on_one_simd"][name] = row
+    li = 4000
+    nbytes = lib.cw_diag_lds_rate_bytes(li)
+    for tr, name in ((0, "ds_read_b128"), (1, "ds_read_b64_tr_b16")):
+        us = event_time_us(lambda: check(lib.cw_diag_lds_rate(li, tr, isink.data_ptr(), stream)), 10, 3, min_ms=300)
+        out["lds_read_rate_per_compute_unit"][name] = {"us_per_call": round(us, 1), "GB_per_s": round(nbytes / us / 1e3, 1)}
+    a = out["lds_read_rate_per_compute_unit"]
+    a["b128_over_transposing"] = round(a["ds_read_b128"]["GB_per_s"] / a["ds_read_b64_tr_b16"]["GB_per_s"], 2)
+    return out
+
+
+def gemm_k_sweep(device):
+    """Time of one launch of the block GEMM against its reduction length, at an output of one tile per compute
+    unit (8192 x 2048 = 256 tiles of 256 x 256): slope = the k loop, intercept = what every round of tiles costs
+    besides (the gap between launches, the first tiles' way from HBM into the ring, the epilogue and the write of
+    C, during which no matrix instruction runs). Operands rotate through more than the Infinity Cache holds."""
+    import torch
+    from cubework_amd import ops
+    m_, n_ = 8192, 2048
+    out = {"M": m_, "N": n_, "tiles_256": (m_ // 256) * (n_ // 256), "rows": []}
+    for layout in ("NT", "NN"):
+        for epi in (None, "relu"):
+            pts = []
+            for k_ in (512, 1024, 2048, 4096, 8192):
+                nrot = min(6, max(2, int(600e6 // ((m_ + n_) * k_ * 2))))
+                a_ = [_seeded((m_, k_), 10 + i, 1.0, torch.bfloat16).to(device) for i in range(nrot)]
+                b_ = [_seeded((n_, k_) if layout == "NT" else (k_, n_), 20 + i, 0.02, torch.bfloat16).to(device)
+                      for i in range(nrot)]
+                bias = _seeded((n_,), 5, 0.02, torch.bfloat16).to(device) if epi else None
+                c_ = torch.empty((m_, n_), dtype=torch.bfloat16, device=device)
+                j = [0]
+
+                def fn():
+                    j[0] += 1
+                    ops.gemm_ksteps(layout, [a_[j[0] % nrot]], [b_[j[0] % nrot]], bias, epi, out=c_)
+                pts.append((k_, event_time_us(fn, 30, 5, min_ms=400)))
+                del a_, b_
+            (k1, t1), (k2, t2) = pts[2], pts[4]
+            slope = (t2 - t1) / (k2 - k1)
+            flop_per_k = 2.0 * m_ * n_
+            out["rows"].append({"layout": layout, "epilogue": epi or "none",
+                                "us_by_k": {str(k_): round(t, 2) for k_, t in pts},
+                                "us_per_1024_k": round(slope * 1024, 2),
+                                "k_loop_frac_of_mfma_peak": round(flop_per_k / slope / 1e6 / MFMA_BF16_PEAK_TFLOPS, 4),
+                                "us_per_launch_beyond_the_k_loop": round(t1 - slope * k1, 2)})
+    out["note"] = ("slope and intercept from K = 2048 and 8192; the intercept holds the launch-to-launch gap of back-to-back "
+                   "launches, the ring's fill from HBM and the epilogue with the write of the 32 MiB of C")
+    return out
+
+
 def energy_table(device, sets, bias, outs, seconds):
     """Where a launch of the headline GEMM spends its energy: the ring kernel whole and with one part taken out
     (cw_diag_gemm_part of the measurement library: the same kernel source, parts 1-3 not computing anything
@@ -1013,6 +1091,20 @@ def main():
                     help="instead of the benchmark: launch the fp32 ring kernels (config 1 forward and input "
                          "gradient) and the small-tile 16-bit ring kernel (2048^3) six times each, interleaved with "
                          "torch.matmul on the same operands - the program of the hardware-counter comparison")
+    ap.add_argument("--attention-counter-run", action="store_true",
+                    help="instead of the benchmark: launch the attention core's forward and backward kernels four "
+                         "times at config 5's shape (batch 4, 32 heads of 64, 2048 tokens, causal) - the program of "
+                         "the hardware-counter passes over those kernels")
+    ap.add_argument("--hw-probes", action="store_true",
+                    help="instead of the benchmark: two probes of the measurement library that bound the attention "
+                         "kernels - how far matrix instructions of one wavefront and vector instructions of another "
+                         "overlap on a SIMD, and the LDS read rate of a compute unit with 16-byte reads and with the "
+                         "transposing 8-byte reads")
+    ap.add_argument("--gemm-k-sweep", action="store_true",
+                    help="instead of the benchmark: the 16-bit block GEMM at 8192 x 2048 outputs (256 tiles, one round "
+                         "of the chip) for reduction lengths 512 ... 8192, NT and NN, plain and bias + ReLU: the time "
+                         "per 1024 of k and what a launch costs beyond its k loop (launch gap, filling the ring from "
+                         "HBM, writing the 32 MiB of C)")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         sys.stderr.write("bench.py measures one rank's share on ONE GPU; --gpus N with N > 1 is not part of this "
@@ -1046,8 +1138,28 @@ def main():
         torch.cuda.synchronize()
         return
 
+    if args.attention_counter_run:
+        b_, s_, h_, d_ = 4, 2048, 32, 64
+        t4 = _seeded((b_, s_, h_ * 3 * d_), 21, 1.0, torch.bfloat16).to(device).view(b_, s_, h_, 3 * d_)
+        q_, k_, v_ = t4[..., :d_], t4[..., d_:2 * d_], t4[..., 2 * d_:]
+        do_ = _seeded((b_, s_, h_ * d_), 22, 1.0, torch.bfloat16).to(device)
+        g_ = torch.empty_like(t4)
+        for _ in range(4):
+            o_, lse_ = ops.attn_fwd(q_, k_, v_, want_lse=True)
+            ops.attn_bwd(q_, k_, v_, o_, do_, lse_, g_[..., :d_], g_[..., d_:2 * d_], g_[..., 2 * d_:])
+        torch.cuda.synchronize()
+        return
+
     if args.stream_ceiling:
         print(json.dumps({"stream_ceiling": stream_ceiling(device)}))
+        return
+
+    if args.gemm_k_sweep:
+        print(json.dumps({"gemm_k_sweep": gemm_k_sweep(device)}))
+        return
+
+    if args.hw_probes:
+        print(json.dumps({"hw_probes": hw_probes(device)}))
         return
 
     # The bandwidth-bound kernels of the same path run first: the headline's warm-up and timed steps then find the

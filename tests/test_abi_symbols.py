@@ -139,6 +139,9 @@ def test_measurement_library_is_separate_from_the_boundary():
     assert diag.cw_diag_mfma_rate(0, 0, None, None) == -1
     assert diag.cw_diag_mfma_rate(10, 4, None, None) == -1
     assert b"mode" in diag.cw_last_error()
+    assert diag.cw_diag_overlap(10, 0, 0, None, None) == -1
+    assert diag.cw_diag_lds_rate(10, 2, None, None) == -1
+    assert diag.cw_diag_lds_rate_bytes(3) == 3 * 65536
     assert diag.cw_diag_mfma_rate_flop(2) == 2 * 1024 * 16 * 32768
     assert diag.cw_diag_gemm_part(7, 8192, 2048, 2048, 2, None, 2048, None, 2048, None, None, 2048, None) == -1
     tab = (ctypes.c_void_p * 2)(256, 256)
