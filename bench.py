@@ -645,6 +645,18 @@ def bench_other_configs(device, sets):
     us = event_time_us(lambda: ops.attn_bwd(q_, k_, v_, o_, do_, lse_, g_[..., :d_], g_[..., d_:2 * d_], g_[..., 2 * d_:]), 30, 5)
     out["attention_bwd_causal"] = {"us": round(us, 2), "TFLOPs": round(2.5 * attn_flop / us / 1e6, 1),
                                    "frac": round(2.5 * attn_flop / us / 1e6 / MFMA_BF16_PEAK_TFLOPS, 4)}
+    # the same launches back to back for 3.5 s each: what holds the clock while these kernels run (clock, socket power,
+    # share of the firmware's samples in which the package-power limiter was active, energy per launch)
+    for key, fn in (("attention_fwd_causal", lambda: ops.attn_fwd(q_, k_, v_)),
+                    ("attention_bwd_causal", lambda: ops.attn_bwd(q_, k_, v_, o_, do_, lse_, g_[..., :d_], g_[..., d_:2 * d_],
+                                                                  g_[..., 2 * d_:]))):
+        us_s, smi = sustained_us(fn, int(3.5e6 / out[key]["us"]) + 1)
+        row = {"us": round(us_s, 2)}
+        if smi:
+            row.update({k: smi[k] for k in ("shader_clock_MHz", "socket_power_W") if k in smi})
+            gm = smi.get("gpu_metrics") or {}
+            row.update({k: gm[k] for k in ("energy_mJ_per_launch", "limiter_residency") if k in gm})
+        out[key]["sustained"] = row
     del qkv, t4, o_, do_, g_
     # config 5: OPT-1.3B-shaped block, batch 4 x seq 2048, bf16, forward + backward
     initialize("2d", 1)
