@@ -529,6 +529,27 @@ def attn_bwd(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, out: torch.Tenso
     _lib.check(rc, "cw_attn_bwd")
 
 
+def _attn_padded_head(d: int) -> int:
+    """Head size the kernels run at for a model head size d: 64 and 128 are native; smaller ones and those in
+    between (the reference's opt_125m has 768 / 16 = 48, opt_2_7b and opt_13b have 80, benchmark/opt/opt.py:419-495)
+    are zero-padded up - zero columns add nothing to q.k, and the matching output and gradient columns are dropped."""
+    if d in (64, 128):
+        return d
+    if 0 < d < 64:
+        return 64
+    if 64 < d < 128:
+        return 128
+    raise NotImplementedError("attention_core: head size %d (the kernels cover head sizes up to 128)" % d)
+
+
+def _pad_last(t: torch.Tensor, d: int, dp: int) -> torch.Tensor:
+    """[..., n*d] -> [..., n*dp] with every group of d columns followed by dp - d zeros."""
+    lead, n = t.shape[:-1], t.shape[-1] // d
+    out = t.new_zeros(lead + (n, dp))
+    out[..., :d] = t.reshape(lead + (n, d))
+    return out.view(lead + (n * dp,))
+
+
 class _AttentionCore(torch.autograd.Function):
     """qkv [b, s, heads*3*d] (per head: q, k, v side by side, benchmark/opt/opt.py:72-76) -> [b, s, heads*d]."""
 
@@ -536,22 +557,31 @@ class _AttentionCore(torch.autograd.Function):
     def forward(ctx, qkv: torch.Tensor, heads: int, scale: Optional[float], causal: bool):
         b, s, w = qkv.shape
         d = w // (3 * heads)
+        dp = _attn_padded_head(d)
+        if dp != d:
+            scale = d ** -0.5 if scale is None else scale  # of the model's head size, not the padded one
+            qkv = _pad_last(qkv, d, dp)
         qkv = qkv if qkv.stride(-1) == 1 else qkv.contiguous()
-        t = qkv.view(b, s, heads, 3 * d) if qkv.is_contiguous() else qkv.reshape(b, s, heads, 3 * d)
-        q, k, v = t[..., :d], t[..., d:2 * d], t[..., 2 * d:]
+        t = qkv.view(b, s, heads, 3 * dp) if qkv.is_contiguous() else qkv.reshape(b, s, heads, 3 * dp)
+        q, k, v = t[..., :dp], t[..., dp:2 * dp], t[..., 2 * dp:]
         out, lse = attn_fwd(q, k, v, scale, causal, want_lse=True)
         ctx.save_for_backward(t, out, lse)
-        ctx.meta = (heads, d, scale, causal)
+        ctx.meta = (heads, d, dp, scale, causal)
+        if dp != d:
+            return out.view(b, s, heads, dp)[..., :d].reshape(b, s, heads * d)
         return out
 
     @staticmethod
     def backward(ctx, d_out: torch.Tensor):
         t, out, lse = ctx.saved_tensors
-        heads, d, scale, causal = ctx.meta
+        heads, d, dp, scale, causal = ctx.meta
         b, s = t.shape[0], t.shape[1]
-        q, k, v = t[..., :d], t[..., d:2 * d], t[..., 2 * d:]
-        g = torch.empty((b, s, heads, 3 * d), dtype=t.dtype, device=t.device)
-        attn_bwd(q, k, v, out, d_out.contiguous(), lse, g[..., :d], g[..., d:2 * d], g[..., 2 * d:], scale, causal)
+        q, k, v = t[..., :dp], t[..., dp:2 * dp], t[..., 2 * dp:]
+        g = torch.empty((b, s, heads, 3 * dp), dtype=t.dtype, device=t.device)
+        d_out = d_out.contiguous() if dp == d else _pad_last(d_out, d, dp)
+        attn_bwd(q, k, v, out, d_out, lse, g[..., :dp], g[..., dp:2 * dp], g[..., 2 * dp:], scale, causal)
+        if dp != d:
+            return g.view(b, s, heads, 3, dp)[..., :d].reshape(b, s, heads * 3 * d), None, None, None
         return g.view(b, s, heads * 3 * d), None, None, None
 
 

@@ -8,9 +8,9 @@ causal attention -> out Linear -> residual -> LayerNorm -> fc1 -> activation ->
 fc2 -> residual. The four Linears and two LayerNorms are cubework_amd.module
 layers (HIP path). The attention core (scaled QK^T, causal mask, softmax, PV:
 benchmark/opt/opt.py:84-117) is the fused HIP kernel pair cw_attn_fwd /
-cw_attn_bwd for the shapes it provides (bf16, head size 64 or 128: every OPT size but 2.7B);
-other head sizes or dtypes use torch's scaled_dot_product_attention, as model
-code would.
+cw_attn_bwd for 16-bit inputs and head sizes up to 128 (64 and 128 natively, the 48 of
+opt_125m and the 80 of opt_2_7b / opt_13b zero-padded, benchmark/opt/opt.py:419-495); fp32
+inputs or larger heads use torch's scaled_dot_product_attention, as model code would.
 """
 
 import torch
@@ -39,7 +39,7 @@ class OPTBlock(nn.Module):
         self.fc2 = cube_nn.Linear(ffn, hidden, dtype=dtype)
 
     def _attention_core(self, qkv: torch.Tensor) -> torch.Tensor:
-        if self.head_dim in (64, 128) and qkv.dtype in (torch.bfloat16, torch.float16) and qkv.is_cuda:
+        if self.head_dim <= 128 and qkv.dtype in (torch.bfloat16, torch.float16) and qkv.is_cuda:
             return ops.attention_core(qkv, self.heads)
         b, s, _ = qkv.shape
         qkv = qkv.view(b, s, self.heads, 3 * self.head_dim).permute(0, 2, 1, 3)

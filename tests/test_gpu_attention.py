@@ -175,6 +175,41 @@ def test_attention_head_size_128(shape, causal):
         assert_parity(got.permute(0, 2, 1, 3), ref, torch.bfloat16, "attention %s d=128 %s causal=%s" % (name, shape, causal))
 
 
+@pytest.mark.parametrize("d", [48, 80, 8])
+@pytest.mark.parametrize("causal", [True, False])
+def test_attention_core_head_sizes_between_the_kernels(d, causal):
+    """Head sizes of the reference's model list that are neither 64 nor 128 (opt_125m: 768 / 16 = 48; opt_2_7b and
+    opt_13b: 80, benchmark/opt/opt.py:419-495) go through the same kernels zero-padded to 64 / 128, with the softmax
+    scale of the model's own head size: forward and the gradient of the whole qkv tensor against the oracle."""
+    import oracle
+    from cubework_amd import ops
+
+    b, s, h = 2, 200, 3
+    qkv = _qkv(b, s, h, d, seed=41 + d)
+    d_out = randn((b, s, h * d), torch.bfloat16, seed=42 + d)
+    x = qkv.to(DEV).requires_grad_(True)
+    y = ops.attention_core(x, h, None, causal)
+    assert y.shape == (b, s, h * d)
+    y.backward(d_out.to(DEV))
+    g1 = x.grad.clone()
+    x.grad = None
+    ops.attention_core(x, h, None, causal).backward(d_out.to(DEV))
+    assert torch.equal(g1, x.grad)
+    qc, kc, vc = oracle.split_qkv(qkv, h)
+    assert_parity(y, oracle.attention_core(qc, kc, vc, causal=causal), torch.bfloat16, "attention_core forward, head size %d" % d)
+    dq, dk, dv = oracle.attention_core_backward(qc, kc, vc, d_out, causal=causal)
+    want = torch.cat([dq, dk, dv], dim=-1).permute(0, 2, 1, 3).reshape(b, s, h * 3 * d)
+    assert_parity(g1, want, torch.bfloat16, "d qkv, head size %d" % d)
+
+
+def test_attention_core_rejects_head_sizes_above_128():
+    from cubework_amd import ops
+
+    x = torch.zeros((1, 8, 3 * 160), dtype=torch.bfloat16, device=DEV)
+    with pytest.raises(NotImplementedError):
+        ops.attention_core(x, 1)
+
+
 def test_attention_head_size_128_autograd():
     import oracle
     from cubework_amd import ops
