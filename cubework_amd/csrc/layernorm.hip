@@ -1456,6 +1456,8 @@ int backward_fused_impl(int64_t R, int64_t C, const void* dY, int64_t ld_dy, con
     int rc = bwd_partials_impl<T>(R, C, dY, ld_dy, x, ld_x, mean_rstd, gamma, row_sums, dgamma, dbeta, param_dtype,
                                   workspace, workspace_bytes, s, dx, ld_dx, &dx_done, nullptr, add);
     if (rc != CW_OK || dx_done) return rc;
+    if (add.p != nullptr)  // the check above and the choice of kernel have come apart: never drop the addend silently
+        return fail(CW_ERR_UNSUPPORTED, "cw_ln_backward_fused: this shape took the two-kernel path, which does not add dx_addend");
     return bwd_dx_impl<T>(R, C, dY, ld_dy, x, ld_x, mean_rstd, gamma, row_sums, C, dx, ld_dx, s);
 }
 }  // namespace
