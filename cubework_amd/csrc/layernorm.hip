@@ -646,9 +646,11 @@ int tile_grid(int64_t R, int nr) {
 // (j*64 + l)*V .. +V-1, j < NCH, for every row its wavefront visits, so the
 // dgamma/dbeta accumulators stay in registers for the whole kernel. A
 // wavefront holds NR rows of dY and x at a time.
-// FUSE_DX: the rows are complete on this rank (C is the whole hidden size), so the row sums are final and
-// dx is written from the registers that hold the row, in the same pass.
-template <typename T, int NCH, int NWAVES, int NR, bool FUSE_DX>
+// FUSE_DX != 0: the rows are complete on this rank (C is the whole hidden size), so the row sums are final and
+// dx is written from the registers that hold the row, in the same pass. FUSE_DX == 2: the same rows of dx_add
+// (the gradient arriving along a residual branch) are loaded with the tiles and added before the store; an
+// instantiation of its own, so that the kernel without an addend carries neither the loads nor a test for them.
+template <typename T, int NCH, int NWAVES, int NR, int FUSE_DX>
 __global__ __launch_bounds__(NWAVES * 64) void ln_bwd_partials_kernel(
     int64_t R, int64_t C, const T* __restrict__ dY, int64_t ld_dy, const T* __restrict__ x, int64_t ld_x,
     const float* __restrict__ mean_rstd, const T* __restrict__ gamma, float* __restrict__ row_sums,
@@ -667,9 +669,10 @@ __global__ __launch_bounds__(NWAVES * 64) void ln_bwd_partials_kernel(
 
     const int64_t step = (int64_t)gridDim.x * NWAVES * NR;
     for (int64_t row0 = ((int64_t)blockIdx.x * NWAVES + wave) * NR; row0 < R; row0 += step) {
-        RowTile<T, NCH, NR> tdy, tx;
+        RowTile<T, NCH, NR> tdy, tx, tadd;
         tdy.load(dY, ld_dy, row0, R, C, lane);
         tx.load(x, ld_x, row0, R, C, lane);
+        if constexpr (FUSE_DX == 2) tadd.load(dx_add, ld_add, row0, R, C, lane);
         tdy.zero_dead_rows(row0, R);  // a zero dY row adds nothing to the column sums
 #pragma unroll
         for (int r = 0; r < NR; ++r) {            const int64_t row = row0 + r;
@@ -714,15 +717,14 @@ __global__ __launch_bounds__(NWAVES * 64) void ln_bwd_partials_kernel(
                         const float gg = gamma != nullptr ? dy[e] * g[e] : dy[e];
                         dy[e] = (gg - xh * c2 - c1) * rstd;
                     }
-                    if (row < R && chunk_valid<T>(j, lane, C)) {
-                        if (FUSE_DX && dx_add != nullptr) {  // the gradient arriving along the residual branch
-                            float av[V];
-                            unpack_raw(load_raw_stream(dx_add + row * ld_add + ((int64_t)j * 64 + lane) * V), av, (const T*)nullptr);
+                    if constexpr (FUSE_DX == 2) {  // the gradient arriving along the residual branch
+                        float av[V];
+                        unpack_raw(tadd.raw[r][j], av, (const T*)nullptr);
 #pragma unroll
-                            for (int e = 0; e < V; ++e) dy[e] += av[e];
-                        }
-                        store_raw_stream(dx + row * ld_dx + ((int64_t)j * 64 + lane) * V, pack_raw(dy, (const T*)nullptr));
+                        for (int e = 0; e < V; ++e) dy[e] += av[e];
                     }
+                    if (row < R && chunk_valid<T>(j, lane, C))
+                        store_raw_stream(dx + row * ld_dx + ((int64_t)j * 64 + lane) * V, pack_raw(dy, (const T*)nullptr));
                 }
             }
         }
@@ -745,7 +747,7 @@ __global__ __launch_bounds__(NWAVES * 64) void ln_bwd_partials_kernel(
 // segment of dx from the registers that hold the row. The next trip's rows are loaded before the barrier.
 // The dgamma/dbeta accumulators of the row groups are added through LDS at the end, in a fixed order.
 // The launcher chooses wpr so that every segment starts inside the row.
-template <typename T, int NCH, int MAXW, bool FUSE_DX>
+template <typename T, int NCH, int MAXW, int FUSE_DX>
 __global__ __launch_bounds__(MAXW * 64, 4) void ln_bwd_split_kernel(
     int64_t R, int64_t C, const T* __restrict__ dY, int64_t ld_dy, const T* __restrict__ x, int64_t ld_x,
     const float* __restrict__ mean_rstd, const T* __restrict__ gamma, float* __restrict__ row_sums,
@@ -768,7 +770,7 @@ __global__ __launch_bounds__(MAXW * 64, 4) void ln_bwd_split_kernel(
     x += col0;
     if (gamma != nullptr) gamma += col0;
     if (FUSE_DX) dx += col0;
-    if (FUSE_DX && dx_add != nullptr) dx_add += col0;
+    if constexpr (FUSE_DX == 2) dx_add += col0;
 
     raw16_t g_raw[NCH];
     load_param_chunks<T, NCH>(gamma, Cs, lane, g_raw);
@@ -795,6 +797,9 @@ __global__ __launch_bounds__(MAXW * 64, 4) void ln_bwd_split_kernel(
         const int64_t row_c = live ? row : R - 1;
         const float mean = mean_rstd[2 * row_c];
         const float rstd = mean_rstd[2 * row_c + 1];
+        // the residual branch's gradient of this row: on its way while the row sums are formed and exchanged
+        RowTile<T, NCH, 1> tadd;
+        if constexpr (FUSE_DX == 2) tadd.load(dx_add, ld_add, row, R, Cs, lane);
         float s1 = 0.0f, s2 = 0.0f;
 #pragma unroll
         for (int j = 0; j < NCH; ++j) {
@@ -844,15 +849,14 @@ __global__ __launch_bounds__(MAXW * 64, 4) void ln_bwd_split_kernel(
                     const float gg = gamma != nullptr ? dy[e] * g[e] : dy[e];
                     dy[e] = (gg - xh * c2 - c1) * rstd;
                 }
-                if (live && chunk_valid<T>(j, lane, Cs)) {
-                    if (dx_add != nullptr) {  // the gradient arriving along the residual branch
-                        float av[V];
-                        unpack_raw(load_raw_stream(dx_add + row * ld_add + ((int64_t)j * 64 + lane) * V), av, (const T*)nullptr);
+                if constexpr (FUSE_DX == 2) {  // the gradient arriving along the residual branch
+                    float av[V];
+                    unpack_raw(tadd.raw[0][j], av, (const T*)nullptr);
 #pragma unroll
-                        for (int e = 0; e < V; ++e) dy[e] += av[e];
-                    }
-                    store_raw_stream(dx + row * ld_dx + ((int64_t)j * 64 + lane) * V, pack_raw(dy, (const T*)nullptr));
+                    for (int e = 0; e < V; ++e) dy[e] += av[e];
                 }
+                if (live && chunk_valid<T>(j, lane, Cs))
+                    store_raw_stream(dx + row * ld_dx + ((int64_t)j * 64 + lane) * V, pack_raw(dy, (const T*)nullptr));
             }
         }
         if (more) {
@@ -1138,7 +1142,7 @@ int64_t bwd_blocks(int64_t R, int nwaves) {
     return nb;
 }
 
-template <typename T, int NCH, int NWAVES, int NR, bool FUSE_DX>
+template <typename T, int NCH, int NWAVES, int NR, int FUSE_DX>
 int bwd_partials_launch_as(int64_t R, int64_t C, const void* dY, int64_t ld_dy, const void* x, int64_t ld_x,
                            const float* mean_rstd, const void* gamma, float* row_sums, float* ws, int want_cols,
                            void* dx, int64_t ld_dx, hipStream_t s, DxAdd add = {}) {
@@ -1159,11 +1163,14 @@ template <typename T, int NCH, int NWAVES, int NR>
 int bwd_partials_launch(int64_t R, int64_t C, const void* dY, int64_t ld_dy, const void* x, int64_t ld_x,
                         const float* mean_rstd, const void* gamma, float* row_sums, float* ws, int want_cols,
                         void* dx, int64_t ld_dx, hipStream_t s, DxAdd add = {}) {
+    if (dx != nullptr && add.p != nullptr)
+        return bwd_partials_launch_as<T, NCH, NWAVES, NR, 2>(R, C, dY, ld_dy, x, ld_x, mean_rstd, gamma, row_sums, ws,
+                                                             want_cols, dx, ld_dx, s, add);
     if (dx != nullptr)
-        return bwd_partials_launch_as<T, NCH, NWAVES, NR, true>(R, C, dY, ld_dy, x, ld_x, mean_rstd, gamma, row_sums, ws,
-                                                                want_cols, dx, ld_dx, s, add);
-    return bwd_partials_launch_as<T, NCH, NWAVES, NR, false>(R, C, dY, ld_dy, x, ld_x, mean_rstd, gamma, row_sums, ws,
-                                                             want_cols, nullptr, 0, s);
+        return bwd_partials_launch_as<T, NCH, NWAVES, NR, 1>(R, C, dY, ld_dy, x, ld_x, mean_rstd, gamma, row_sums, ws,
+                                                             want_cols, dx, ld_dx, s);
+    return bwd_partials_launch_as<T, NCH, NWAVES, NR, 0>(R, C, dY, ld_dy, x, ld_x, mean_rstd, gamma, row_sums, ws,
+                                                         want_cols, nullptr, 0, s);
 }
 
 // Rows of more than kSplitMinChunks chunks go to the split kernel: kSplitChunks chunks per wavefront (three
@@ -1203,7 +1210,7 @@ SplitShape split_shape(int64_t R, int64_t nch, int chunks) {
     return sh;
 }
 
-template <typename T, int NCH, int MAXW, bool FUSE_DX>
+template <typename T, int NCH, int MAXW, int FUSE_DX>
 int bwd_split_launch_as(const SplitShape& sh, int64_t R, int64_t C, const void* dY, int64_t ld_dy, const void* x,
                         int64_t ld_x, const float* mean_rstd, const void* gamma, float* row_sums, float* ws,
                         int want_cols, void* dx, int64_t ld_dx, hipStream_t s, DxAdd add = {}) {
@@ -1212,7 +1219,7 @@ int bwd_split_launch_as(const SplitShape& sh, int64_t R, int64_t C, const void* 
     hipLaunchKernelGGL((ln_bwd_split_kernel<T, NCH, MAXW, FUSE_DX>), dim3((unsigned)sh.blocks),
                        dim3(sh.wpr * sh.nrg * 64), lds, s, R, C, (const T*)dY, ld_dy, (const T*)x, ld_x, mean_rstd,
                        (const T*)gamma, row_sums, ws, want_cols, (T*)dx, ld_dx, 1.0f / (float)C, sh.wpr,
-                       (const T*)(FUSE_DX ? add.p : nullptr), add.ld);
+                       (const T*)(FUSE_DX == 2 ? add.p : nullptr), add.ld);
     return check_launch("ln_bwd_split_kernel");
 }
 
@@ -1224,13 +1231,15 @@ int bwd_split_launch(const SplitShape& sh, int64_t R, int64_t C, const void* dY,
 #define CW_SPLIT(NCH, MAXW, FUSE)                                                                               \
     bwd_split_launch_as<T, NCH, MAXW, FUSE>(sh, R, C, dY, ld_dy, x, ld_x, mean_rstd, gamma, row_sums, ws, want_cols, \
                                             dx, ld_dx, s, add)
+#define CW_SPLIT_MODE(NCH, MAXW) \
+    (dx == nullptr ? CW_SPLIT(NCH, MAXW, 0) : (add.p != nullptr ? CW_SPLIT(NCH, MAXW, 2) : CW_SPLIT(NCH, MAXW, 1)))
     if constexpr (sizeof(T) == 4) {
         // three or four chunks: only rows that need more than eight such wavefronts, in one row group
-        if (sh.chunks == 3) return dx != nullptr ? CW_SPLIT(3, 16, true) : CW_SPLIT(3, 16, false);
-        if (sh.chunks == 4) return dx != nullptr ? CW_SPLIT(4, 16, true) : CW_SPLIT(4, 16, false);
+        if (sh.chunks == 3) return CW_SPLIT_MODE(3, 16);
+        if (sh.chunks == 4) return CW_SPLIT_MODE(4, 16);
     }
-    if (dx != nullptr) return wide ? CW_SPLIT(kSplitChunks, 16, true) : CW_SPLIT(kSplitChunks, kSplitBlockWaves, true);
-    return wide ? CW_SPLIT(kSplitChunks, 16, false) : CW_SPLIT(kSplitChunks, kSplitBlockWaves, false);
+    return wide ? CW_SPLIT_MODE(kSplitChunks, 16) : CW_SPLIT_MODE(kSplitChunks, kSplitBlockWaves);
+#undef CW_SPLIT_MODE
 #undef CW_SPLIT
 }
 
