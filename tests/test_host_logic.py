@@ -186,3 +186,25 @@ def test_bench_refuses_more_than_one_gpu_and_has_no_cpu_path():
         r = subprocess.run([sys.executable, bench, "--steps", "1", "--warmup", "0"], capture_output=True, text=True,
                            timeout=300)
         assert r.returncode == 3 and "no CPU fallback" in r.stderr and r.stdout.strip() == ""
+
+
+def test_attention_head_padding_is_exact_on_the_host():
+    """Head sizes between the kernels' 64 and 128 are zero-padded (cubework_amd.ops._pad_last): the padded q.k
+    products equal the unpadded ones, slicing the padded columns away gives the input back, and sizes above
+    128 are refused (benchmark/opt/opt.py:419-495 lists 48, 64, 80 and 128)."""
+    from cubework_amd import ops
+
+    assert [ops._attn_padded_head(d) for d in (8, 48, 64, 80, 127, 128)] == [64, 64, 64, 128, 128, 128]
+    with pytest.raises(NotImplementedError):
+        ops._attn_padded_head(160)
+    b, s, h, d, dp = 2, 5, 3, 80, 128
+    qkv = torch.randn((b, s, h * 3 * d), generator=torch.Generator().manual_seed(1)).to(torch.bfloat16)
+    padded = ops._pad_last(qkv, d, dp)
+    assert padded.shape == (b, s, h * 3 * dp)
+    t, tp = qkv.view(b, s, h, 3, d), padded.view(b, s, h, 3, dp)
+    assert torch.equal(tp[..., :d], t) and torch.count_nonzero(tp[..., d:]) == 0
+    q, k = t[..., 0, :].float(), t[..., 1, :].float()
+    qp, kp = tp[..., 0, :].float(), tp[..., 1, :].float()
+    # zeros add nothing to q.k (compared in float64: the order of a float32 sum may differ with the length)
+    assert torch.equal(torch.einsum("bshd,bthd->bhst", q.double(), k.double()),
+                       torch.einsum("bshd,bthd->bhst", qp.double(), kp.double()))
