@@ -1018,6 +1018,12 @@ def energy_table(device, sets, bias, outs, seconds):
         }
         parts["rest_launch_gap_prologue_barriers_waits"] = round(whole - sum(parts.values()), 2)
         out["energy_mJ_per_launch"] = {"whole_kernel": whole, **parts}
+        if pj["zero_operands"]:
+            # the matrix instructions' energy in two parts: what the same instructions cost on all-zero operands
+            # (clocks, control, leakage: there whether or not the data toggle) and what the operands' switching adds
+            idle = round(pj["zero_operands"] * GEMM_FLOP * 1e-9, 2)
+            out["energy_mJ_per_launch"]["matrix_instructions_on_zero_operands"] = idle
+            out["energy_mJ_per_launch"]["matrix_instructions_operand_switching"] = round(parts["matrix_instructions"] - idle, 2)
         if pj["random_operands_read_from_lds"]:
             out["energy_mJ_per_launch"]["cross_check_lds_reads_from_the_matrix_loops"] = round(
                 (pj["random_operands_read_from_lds"] - pj["random_operands"]) * GEMM_FLOP * 1e-9, 2)
