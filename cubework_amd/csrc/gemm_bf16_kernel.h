@@ -361,6 +361,16 @@ __device__ __forceinline__ void gemm_epilogue_slabs(f32x16_t (&acc)[4][4], const
         constexpr bool ACT = decltype(activated)::value;
         const int mrow = m0 + wm * 128 + I * 32 + (lane & 31);
         uint16_t* dst = lds + buf * BUF + lrow * CP + col_l;
+        // the first addend's 16 pieces of this slab are requested together, ahead of the arithmetic (a load in
+        // front of each use would expose its latency sixteen times); further addends, rare, are read where used
+        u32x2_t add0[4][4];
+        if (args.n_addends > 0) {
+            const uint16_t* ap = reinterpret_cast<const uint16_t*>(pick_ptr(args.addend, 0)) + (int64_t)mrow * args.ldadd + n0 + col_l;
+#pragma unroll
+            for (int j = 0; j < 4; ++j)
+#pragma unroll
+                for (int g = 0; g < 4; ++g) add0[j][g] = *reinterpret_cast<const u32x2_t*>(ap + j * 32 + 8 * g);
+        }
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
 #pragma unroll
@@ -373,8 +383,12 @@ __device__ __forceinline__ void gemm_epilogue_slabs(f32x16_t (&acc)[4][4], const
                 v[3] = acc[I][j][4 * g + 3] + half_conv<E>::hi(b.y);
                 if (args.n_addends > 0) {
                     const int ncol = n0 + col_l + j * 32 + 8 * g;
+                    v[0] += half_conv<E>::lo(add0[j][g].x);
+                    v[1] += half_conv<E>::hi(add0[j][g].x);
+                    v[2] += half_conv<E>::lo(add0[j][g].y);
+                    v[3] += half_conv<E>::hi(add0[j][g].y);
 #pragma unroll 1
-                    for (int a = 0; a < args.n_addends; ++a) {
+                    for (int a = 1; a < args.n_addends; ++a) {
                         float t[4];
                         load4_half<E>(reinterpret_cast<const uint16_t*>(pick_ptr(args.addend, a)) + (int64_t)mrow * args.ldadd + ncol,
                                       4, true, t);
