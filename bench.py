@@ -709,12 +709,33 @@ def bench_other_configs(device, sets):
     finally:
         OPTBlock._linear_plus, OPTBlock._norm_fork = fused_plus, fused_fork
     us_again = event_time_us(block_step, 10, 3)
+    # the same step recorded into a HIP graph and replayed: what the launch gaps of the eager step cost (the entry
+    # points neither allocate nor synchronise, so forward + autograd backward capture whole)
+    us_graph = None
+    try:
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            for _ in range(3):
+                block_step()
+        torch.cuda.current_stream().wait_stream(side)
+        torch.cuda.synchronize()
+        blk.zero_grad(set_to_none=True)
+        xb.grad = None
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            blk(xb).backward(dyb)
+        us_graph = event_time_us(graph.replay, 10, 3)
+        del graph
+    except RuntimeError as exc:  # a torch build that cannot capture: the eager figures stand
+        sys.stderr.write("bench.py: the block step was not captured (%s)\n" % exc)
     lin_flop = 3 * 2.0 * 8192 * 2048 * (6144 + 2048 + 8192 + 8192)
     out["opt_block_fwd_bwd"] = {"ms": round(us / 1e3, 3), "linear_flop": lin_flop,
                                 "linear_TFLOPs_if_all_time_were_linears": round(lin_flop / us / 1e6, 1),
                                 "note": "four Linear2D, two LayerNorm2D and the fused attention core (cw_attn_fwd / cw_attn_bwd), tp=1",
                                 "same_run_ab": {"residual_additions_as_separate_passes_ms": round(us_plain / 1e3, 3),
-                                                "in_epilogue_and_ln_backward_again_ms": round(us_again / 1e3, 3)},
+                                                "in_epilogue_and_ln_backward_again_ms": round(us_again / 1e3, 3),
+                                                "replayed_from_a_hip_graph_ms": None if us_graph is None else round(us_graph / 1e3, 3)},
                                 "per_kernel": per_kernel,
                                 "per_kernel_source": "events around every C-ABI call during %d instrumented passes of the same "
                                                      "step in this run; the last row is the step's time minus their sum" % passes}
